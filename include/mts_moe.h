@@ -1,0 +1,151 @@
+/*
+ * C ABI of the MI355X (gfx950) fused top-k MoE kernels.
+ *
+ * The reference reaches this path through a Python operator interface and has
+ * no C ABI of its own; every entry point below names the reference function it
+ * stands in for (paths relative to the reference root).  A binding only needs
+ * raw device pointers, sizes and a HIP stream: there are no framework types in
+ * any signature.
+ *
+ * Conventions
+ *   - every pointer is a device pointer unless the comment says "host";
+ *   - `stream` is a `hipStream_t` passed as `void*` (NULL = the null stream);
+ *   - kernels are enqueued on `stream`; no entry point synchronises, allocates
+ *     or frees device memory; scratch is passed in by the caller and sized with
+ *     the matching `*_workspace_bytes` function;
+ *   - return value: 0 on success, a negative MTS_ERR_* for a contract violation
+ *     (nothing was launched), a positive `hipError_t` if a launch failed;
+ *   - T tokens, K experts per token, E experts, H model width, I expert width,
+ *     TK = T*K routes; "entry" = t*K+k; "row" = position in the expert-sorted
+ *     order; tensors are dense row-major.
+ */
+#ifndef MTS_MOE_H
+#define MTS_MOE_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MTS_VERSION 1
+
+/* element types of activations / weights / weight gradients */
+#define MTS_BF16 0
+#define MTS_F32 1
+
+#define MTS_OK 0
+#define MTS_ERR_NULL (-1)        /* a required pointer is NULL                      */
+#define MTS_ERR_SHAPE (-2)       /* sizes out of the supported range                */
+#define MTS_ERR_DTYPE (-3)       /* unknown or unsupported element type             */
+#define MTS_ERR_WORKSPACE (-4)   /* workspace too small                             */
+#define MTS_ERR_ALIGN (-5)       /* a pointer or leading dimension is not 16-byte aligned */
+
+#define MTS_MAX_EXPERTS 1024
+#define MTS_MAX_TOP_K 8
+
+int mts_version(void);
+const char* mts_error_string(int code);
+
+/* ---- router post-process ------------------------------------------------
+ * Replaces TorchOpsBackend.router_postprocess (minitrain/kernels/torch_ops.py:87-120)
+ * and _router_forward_kernel (minitrain/kernels/triton/router.py:62-152).
+ * logits [T,E] f32 -> weights [T,K] f32, indices [T,K] i32 (rank order, ties to
+ * the lower expert index), prob_mean [E], z_loss [1], entropy [1].
+ * The statistics are reduced in a fixed order (no float atomics).            */
+int64_t mts_router_workspace_bytes(int64_t T, int E);
+int mts_router_fwd(const float* logits, int64_t T, int E, int K, int normalize,
+                   float* weights, int32_t* indices, float* prob_mean, float* z_loss,
+                   float* entropy, void* workspace, int64_t workspace_bytes, void* stream);
+
+/* Replaces _router_backward_kernel (minitrain/kernels/triton/router.py:155-259).
+ * g_weights [T,K], g_prob_mean [E], g_z_loss [1] -> dlogits [T,E].            */
+int mts_router_bwd(const float* logits, const float* weights, const int32_t* indices,
+                   const float* g_weights, const float* g_prob_mean, const float* g_z_loss,
+                   int64_t T, int E, int K, int normalize, float* dlogits, void* stream);
+
+/* ---- routing metadata ---------------------------------------------------
+ * Replaces compute_routing_metadata (minitrain/kernels/triton/fused_moe.py:74-154)
+ * and its three kernels (fused_moe_kernels.py:25-234): per-expert counts [E],
+ * expert_start [E+1], the stable expert-major permutation (s_scatter [TK]: row ->
+ * entry, s_reverse [TK]: entry -> row, x_gather [TK]: row -> token) and, when
+ * tile_row_start/tile_expert/tile_count are not NULL, the list of block_m-row
+ * tiles (capacity min(TK, ceil(TK/block_m)+E-1) each, tile_count [1]).
+ * Returns MTS_ERR_SHAPE if E > MTS_MAX_EXPERTS; indices outside [0,E) are a
+ * caller error: they are clamped into range (memory-safe, result undefined).                        */
+int64_t mts_moe_route_workspace_bytes(int64_t T, int K, int E);
+int mts_moe_route(const int32_t* top_k_index, int64_t T, int K, int E, int block_m,
+                  int32_t* counts, int32_t* expert_start, int32_t* s_scatter,
+                  int32_t* s_reverse, int32_t* x_gather, int32_t* tile_row_start,
+                  int32_t* tile_expert, int32_t* tile_count, void* workspace,
+                  int64_t workspace_bytes, void* stream);
+
+/* ---- weight staging -----------------------------------------------------
+ * src [E,R,C] of src_dtype -> dst bf16, [E,R,C] (transpose=0) or [E,C,R]
+ * (transpose=1).  Stands in for the in-kernel weight casts of the reference
+ * (fused_moe_kernels.py:343,351) and stages the transposed operands of the
+ * backward GEMMs.                                                            */
+int mts_moe_stage_weights(const void* src, int src_dtype, void* dst_bf16, int E, int64_t R,
+                          int64_t C, int transpose, void* stream);
+
+/* ---- forward ------------------------------------------------------------
+ * Replaces _fused_up_proj_swiglu_kernel (fused_moe_kernels.py:264-367):
+ * for every row r (token x_gather[r], expert e): [g;u] = W1[e] x ; a = silu(g)*u.
+ * x [T,H], w1 [E,2I,H] bf16, pre_act [TK,2I], post_act [TK,I] (act_dtype).     */
+int mts_moe_fwd_gateup_swiglu(const void* x, const void* w1, const int32_t* x_gather,
+                              const int32_t* expert_start, int64_t T, int K, int E, int H,
+                              int I, int act_dtype, void* pre_act, void* post_act,
+                              void* stream);
+
+/* Replaces _fused_down_proj_kernel (fused_moe_kernels.py:369-437):
+ * y[r] = W2[e] a[r];  post_act [TK,I], w2 [E,H,I] bf16 -> y [TK,H].           */
+int mts_moe_fwd_down(const void* post_act, const void* w2, const int32_t* expert_start,
+                     int64_t TK, int E, int H, int I, int act_dtype, void* y, void* stream);
+
+/* Replaces _token_gather_weighted_sum_kernel (fused_moe_kernels.py:451-498):
+ * out[t] = sum_k w[t,k] * y[s_reverse[t*K+k]]  (fp32 sum, one rounding);
+ * weights == NULL gives the unweighted sum used for dx.                      */
+int mts_moe_combine(const void* y, const void* weights, const int32_t* s_reverse, int64_t T,
+                    int K, int H, int act_dtype, void* out, void* stream);
+
+/* ---- backward -----------------------------------------------------------
+ * Replaces _moe_bwd_down_proj_kernel (fused_moe_kernels.py:500-600):
+ * A = W2[e]^T dO[t];  dS = <A,a>;  weighted_act = s*a;  [dg;du] = d(s*A)/d[g;u].
+ * w2t is W2 staged as [E,I,H] bf16.  ds_partial is [TK, mts_moe_ds_partials(I)]
+ * f32 scratch reduced by mts_moe_bwd_ds (fixed order, no atomics).            */
+int mts_moe_ds_partials(int I);
+int mts_moe_bwd_dy1(const void* d_out, const void* w2t, const void* pre_act,
+                    const void* weights, const int32_t* x_gather, const int32_t* s_scatter,
+                    const int32_t* expert_start, int64_t T, int K, int E, int H, int I,
+                    int act_dtype, void* d_pre_act, void* weighted_act, float* ds_partial,
+                    void* stream);
+
+/* dS[entry] = sum of the partials of row s_reverse[entry], cast to act_dtype
+ * (fused_moe.py:437-443 returns dS as [T,K] in the weights' dtype).          */
+int mts_moe_bwd_ds(const float* ds_partial, const int32_t* s_reverse, int64_t TK, int I,
+                   int act_dtype, void* d_weights, void* stream);
+
+/* Replaces _moe_bwd_dX_expanded_kernel (fused_moe_kernels.py:674-756):
+ * dx_expanded[r] = W1[e]^T [dg;du][r];  w1t is W1 staged as [E,H,2I] bf16.
+ * The per-token sum is mts_moe_combine with weights == NULL.                 */
+int mts_moe_bwd_dx(const void* d_pre_act, const void* w1t, const int32_t* expert_start,
+                   int64_t TK, int E, int H, int I, int act_dtype, void* dx_expanded,
+                   void* stream);
+
+/* Replaces _moe_bwd_dW2_kernel (fused_moe_kernels.py:602-672):
+ * dW2[e] = sum_{r in e} dO[x_gather[r]] (x) weighted_act[r]   -> [E,H,I] grad_dtype.
+ * Experts without routes receive zeros.                                      */
+int mts_moe_bwd_dw2(const void* d_out, const void* weighted_act, const int32_t* x_gather,
+                    const int32_t* expert_start, int64_t T, int K, int E, int H, int I,
+                    int act_dtype, int grad_dtype, void* d_w2, void* stream);
+
+/* Replaces _moe_bwd_dW1_kernel (fused_moe_kernels.py:758-828):
+ * dW1[e] = sum_{r in e} [dg;du][r] (x) x[x_gather[r]]        -> [E,2I,H] grad_dtype. */
+int mts_moe_bwd_dw1(const void* d_pre_act, const void* x, const int32_t* x_gather,
+                    const int32_t* expert_start, int64_t T, int K, int E, int H, int I,
+                    int act_dtype, int grad_dtype, void* d_w1, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MTS_MOE_H */

@@ -1,0 +1,182 @@
+// HBM-bound helpers around the grouped GEMMs: the per-token weighted sum of
+// expert rows (combine), the routing-weight gradient reduction and the staging
+// (cast / transpose) of expert weights to bf16.
+#include "mts_common.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+
+// ---- combine -------------------------------------------------------------
+// One thread produces 8 consecutive columns (16 bytes of bf16) of one token:
+// K row loads of 16 bytes each, fp32 accumulation, one rounding.
+__global__ __launch_bounds__(kThreads) void combine_bf16_kernel(
+    const bf16_t* __restrict__ y, const bf16_t* __restrict__ w, const int32_t* __restrict__ s_rev,
+    int64_t T, int K, int H, bf16_t* __restrict__ out) {
+    const int vec_per_row = H / 8;
+    const int64_t total = T * (int64_t)vec_per_row;
+    for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total;
+         i += (int64_t)gridDim.x * kThreads) {
+        const int64_t t = i / vec_per_row;
+        const int c = (int)(i - t * vec_per_row);
+        float acc[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+        for (int k = 0; k < K; ++k) {
+            const int64_t row = s_rev[t * K + k];
+            const float s = w ? (float)w[t * K + k] : 1.0f;
+            const bf16x8 v = *reinterpret_cast<const bf16x8*>(y + row * H + c * 8);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) acc[j] += s * (float)v[j];
+        }
+        bf16x8 o;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) o[j] = (bf16_t)acc[j];
+        *reinterpret_cast<bf16x8*>(out + t * H + c * 8) = o;
+    }
+}
+
+__global__ __launch_bounds__(kThreads) void combine_f32_kernel(
+    const float* __restrict__ y, const float* __restrict__ w, const int32_t* __restrict__ s_rev,
+    int64_t T, int K, int H, float* __restrict__ out) {
+    const int vec_per_row = H / 4;
+    const int64_t total = T * (int64_t)vec_per_row;
+    for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total;
+         i += (int64_t)gridDim.x * kThreads) {
+        const int64_t t = i / vec_per_row;
+        const int c = (int)(i - t * vec_per_row);
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        for (int k = 0; k < K; ++k) {
+            const int64_t row = s_rev[t * K + k];
+            const float s = w ? w[t * K + k] : 1.0f;
+            const f32x4 v = *reinterpret_cast<const f32x4*>(y + row * H + c * 4);
+            acc += s * v;
+        }
+        *reinterpret_cast<f32x4*>(out + t * H + c * 4) = acc;
+    }
+}
+
+// ---- routing-weight gradient ---------------------------------------------
+template <typename OutT>
+__global__ __launch_bounds__(kThreads) void ds_reduce_kernel(const float* __restrict__ part,
+                                                             const int32_t* __restrict__ s_rev,
+                                                             int64_t TK, int np,
+                                                             OutT* __restrict__ d_w) {
+    for (int64_t n = (int64_t)blockIdx.x * kThreads + threadIdx.x; n < TK;
+         n += (int64_t)gridDim.x * kThreads) {
+        const float* p = part + (int64_t)s_rev[n] * np;
+        float v = 0.f;
+        for (int j = 0; j < np; ++j) v += p[j];
+        d_w[n] = (OutT)v;
+    }
+}
+
+// ---- weight staging --------------------------------------------------------
+// 64x64 tiles through LDS; reads and writes are both row-contiguous.
+template <typename SrcT, bool TRANSPOSE>
+__global__ __launch_bounds__(kThreads) void stage_weights_kernel(const SrcT* __restrict__ src,
+                                                                 bf16_t* __restrict__ dst,
+                                                                 int64_t R, int64_t C) {
+    __shared__ bf16_t tile[64][64 + 2];
+    const int64_t e = blockIdx.z;
+    const int64_t r0 = (int64_t)blockIdx.y * 64, c0 = (int64_t)blockIdx.x * 64;
+    const SrcT* s = src + e * R * C;
+    bf16_t* d = dst + e * R * C;
+    const int tx = threadIdx.x % 64, ty = threadIdx.x / 64;
+    for (int i = ty; i < 64; i += kThreads / 64) {
+        int64_t r = r0 + i, c = c0 + tx;
+        if (r < R && c < C) {
+            bf16_t v = (bf16_t)(float)s[r * C + c];
+            if (TRANSPOSE) tile[i][tx] = v;
+            else d[r * C + c] = v;
+        }
+    }
+    if (!TRANSPOSE) return;
+    __syncthreads();
+    for (int i = ty; i < 64; i += kThreads / 64) {
+        int64_t c = c0 + i, r = r0 + tx;  // output row = source column
+        if (r < R && c < C) d[c * R + r] = tile[tx][i];
+    }
+}
+
+int grid_1d(int64_t total) {
+    int64_t b = (total + kThreads - 1) / kThreads;
+    const int64_t cap = 256 * 32;
+    return (int)(b < cap ? (b > 0 ? b : 1) : cap);
+}
+
+}  // namespace
+
+extern "C" int mts_moe_combine(const void* y, const void* weights, const int32_t* s_reverse,
+                               int64_t T, int K, int H, int act_dtype, void* out, void* stream) {
+    if (!y || !s_reverse || !out) return MTS_ERR_NULL;
+    if (T <= 0 || K < 1 || H < 1) return MTS_ERR_SHAPE;
+    if (!mts_aligned16(y) || !mts_aligned16(out)) return MTS_ERR_ALIGN;
+    hipStream_t s = (hipStream_t)stream;
+    if (act_dtype == MTS_BF16) {
+        if (H % 8) return MTS_ERR_SHAPE;
+        combine_bf16_kernel<<<grid_1d(T * (int64_t)(H / 8)), kThreads, 0, s>>>(
+            (const bf16_t*)y, (const bf16_t*)weights, s_reverse, T, K, H, (bf16_t*)out);
+    } else if (act_dtype == MTS_F32) {
+        if (H % 4) return MTS_ERR_SHAPE;
+        combine_f32_kernel<<<grid_1d(T * (int64_t)(H / 4)), kThreads, 0, s>>>(
+            (const float*)y, (const float*)weights, s_reverse, T, K, H, (float*)out);
+    } else {
+        return MTS_ERR_DTYPE;
+    }
+    MTS_CHECK_LAUNCH();
+    return MTS_OK;
+}
+
+extern "C" int mts_moe_bwd_ds(const float* ds_partial, const int32_t* s_reverse, int64_t TK, int I,
+                              int act_dtype, void* d_weights, void* stream) {
+    if (!ds_partial || !s_reverse || !d_weights) return MTS_ERR_NULL;
+    if (TK <= 0 || I < 1) return MTS_ERR_SHAPE;
+    hipStream_t s = (hipStream_t)stream;
+    const int np = mts_moe_ds_partials(I);
+    if (act_dtype == MTS_BF16)
+        ds_reduce_kernel<bf16_t><<<grid_1d(TK), kThreads, 0, s>>>(ds_partial, s_reverse, TK, np,
+                                                                  (bf16_t*)d_weights);
+    else if (act_dtype == MTS_F32)
+        ds_reduce_kernel<float><<<grid_1d(TK), kThreads, 0, s>>>(ds_partial, s_reverse, TK, np,
+                                                                 (float*)d_weights);
+    else
+        return MTS_ERR_DTYPE;
+    MTS_CHECK_LAUNCH();
+    return MTS_OK;
+}
+
+extern "C" int mts_moe_stage_weights(const void* src, int src_dtype, void* dst_bf16, int E,
+                                     int64_t R, int64_t C, int transpose, void* stream) {
+    if (!src || !dst_bf16) return MTS_ERR_NULL;
+    if (E < 1 || R < 1 || C < 1 || E > 65535) return MTS_ERR_SHAPE;
+    hipStream_t s = (hipStream_t)stream;
+    dim3 grid((unsigned)((C + 63) / 64), (unsigned)((R + 63) / 64), (unsigned)E);
+    if (grid.y > 65535) return MTS_ERR_SHAPE;
+    bf16_t* d = (bf16_t*)dst_bf16;
+    if (src_dtype == MTS_F32) {
+        if (transpose) stage_weights_kernel<float, true><<<grid, kThreads, 0, s>>>((const float*)src, d, R, C);
+        else stage_weights_kernel<float, false><<<grid, kThreads, 0, s>>>((const float*)src, d, R, C);
+    } else if (src_dtype == MTS_BF16) {
+        if (transpose) stage_weights_kernel<bf16_t, true><<<grid, kThreads, 0, s>>>((const bf16_t*)src, d, R, C);
+        else stage_weights_kernel<bf16_t, false><<<grid, kThreads, 0, s>>>((const bf16_t*)src, d, R, C);
+    } else {
+        return MTS_ERR_DTYPE;
+    }
+    MTS_CHECK_LAUNCH();
+    return MTS_OK;
+}
+
+extern "C" int mts_version(void) { return MTS_VERSION; }
+
+extern "C" const char* mts_error_string(int code) {
+    switch (code) {
+        case MTS_OK: return "ok";
+        case MTS_ERR_NULL: return "a required pointer is NULL";
+        case MTS_ERR_SHAPE: return "sizes outside the supported range";
+        case MTS_ERR_DTYPE: return "unsupported element type";
+        case MTS_ERR_WORKSPACE: return "workspace too small";
+        case MTS_ERR_ALIGN: return "pointer or leading dimension not 16-byte aligned";
+        default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error";
+    }
+}

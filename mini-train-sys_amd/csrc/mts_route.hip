@@ -1,0 +1,187 @@
+// Routing metadata: per-expert counts, exclusive prefix sums and the stable
+// expert-major permutation of the T*K routes.  Integer work only.
+//
+// The flat entry array is cut into chunks of kChunk entries, one chunk per wave.
+//   1. histogram:  cnt[chunk][e]               (LDS atomics, order-free)
+//   2. scan:       cnt[chunk][e] <- number of routes of e in earlier chunks;
+//                  counts[e], expert_start[e] and the optional tile list
+//   3. scatter:    a wave walks its chunk 64 entries at a time; lanes holding the
+//                  same expert are found with ballots, rank inside the group is a
+//                  popcount of the lower lanes, so entries keep ascending order
+//                  inside every expert (a stable sort by expert).
+#include "mts_common.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / MTS_WAVE;
+constexpr int kChunk = 1024;  // entries per wave
+
+// Expert ids outside [0,E) are a caller error; they are clamped so that no
+// address derived from them can leave the output arrays.
+__device__ __forceinline__ int clamp_expert(int e, int E) { return e < 0 ? 0 : (e >= E ? E - 1 : e); }
+
+__global__ __launch_bounds__(kThreads) void route_hist_kernel(const int32_t* __restrict__ idx,
+                                                              int64_t TK, int E,
+                                                              int32_t* __restrict__ cnt) {
+    extern __shared__ int32_t lds[];  // [kWaves][E]
+    for (int i = threadIdx.x; i < kWaves * E; i += kThreads) lds[i] = 0;
+    __syncthreads();
+    const int wave = threadIdx.x / MTS_WAVE, lane = threadIdx.x % MTS_WAVE;
+    const int64_t chunk = (int64_t)blockIdx.x * kWaves + wave;
+    const int64_t base = chunk * kChunk;
+    int32_t* mine = lds + wave * E;
+    for (int i = lane; i < kChunk; i += MTS_WAVE) {
+        int64_t n = base + i;
+        if (n < TK) atomicAdd(&mine[clamp_expert(idx[n], E)], 1);
+    }
+    __syncthreads();
+    if (base < TK) {
+        for (int e = lane; e < E; e += MTS_WAVE) cnt[chunk * E + e] = mine[e];
+    }
+}
+
+// One block.  Wave w owns experts w, w+nw, ...: exclusive scan over chunks in
+// groups of 64, then an exclusive scan of the totals over experts.
+__global__ __launch_bounds__(1024) void route_scan_kernel(
+    int32_t* __restrict__ cnt, int64_t n_chunks, int E, int64_t TK, int block_m,
+    int32_t* __restrict__ counts, int32_t* __restrict__ expert_start,
+    int32_t* __restrict__ tile_row_start, int32_t* __restrict__ tile_expert,
+    int32_t* __restrict__ tile_count) {
+    __shared__ int32_t total[MTS_MAX_EXPERTS];
+    __shared__ int32_t start[MTS_MAX_EXPERTS + 1];
+    __shared__ int32_t tile_off[MTS_MAX_EXPERTS + 1];
+    const int wave = threadIdx.x / MTS_WAVE, lane = threadIdx.x % MTS_WAVE;
+    const int nw = blockDim.x / MTS_WAVE;
+    for (int e = wave; e < E; e += nw) {
+        int32_t carry = 0;
+        for (int64_t c0 = 0; c0 < n_chunks; c0 += MTS_WAVE) {
+            int64_t c = c0 + lane;
+            int32_t v = (c < n_chunks) ? cnt[c * E + e] : 0;
+            int32_t incl = v;
+#pragma unroll
+            for (int o = 1; o < MTS_WAVE; o <<= 1) {
+                int32_t up = __shfl_up(incl, o, MTS_WAVE);
+                if (lane >= o) incl += up;
+            }
+            if (c < n_chunks) cnt[c * E + e] = carry + incl - v;
+            carry += __shfl(incl, MTS_WAVE - 1, MTS_WAVE);
+        }
+        if (lane == 0) total[e] = carry;
+    }
+    __syncthreads();
+    if (wave == 0) {
+        int32_t carry = 0, tcarry = 0;
+        for (int e0 = 0; e0 < E; e0 += MTS_WAVE) {
+            int e = e0 + lane;
+            int32_t v = (e < E) ? total[e] : 0;
+            int32_t tv = (v + block_m - 1) / block_m;
+            int32_t incl = v, tincl = tv;
+#pragma unroll
+            for (int o = 1; o < MTS_WAVE; o <<= 1) {
+                int32_t up = __shfl_up(incl, o, MTS_WAVE);
+                int32_t tup = __shfl_up(tincl, o, MTS_WAVE);
+                if (lane >= o) {
+                    incl += up;
+                    tincl += tup;
+                }
+            }
+            if (e < E) {
+                start[e] = carry + incl - v;
+                tile_off[e] = tcarry + tincl - tv;
+                counts[e] = v;
+                expert_start[e] = carry + incl - v;
+            }
+            carry += __shfl(incl, MTS_WAVE - 1, MTS_WAVE);
+            tcarry += __shfl(tincl, MTS_WAVE - 1, MTS_WAVE);
+        }
+        if (lane == 0) {
+            start[E] = carry;
+            tile_off[E] = tcarry;
+            expert_start[E] = (int32_t)TK;
+            if (tile_count) tile_count[0] = tcarry;
+        }
+    }
+    __syncthreads();
+    if (tile_row_start && tile_expert) {
+        for (int e = wave; e < E; e += nw) {
+            int32_t nt = tile_off[e + 1] - tile_off[e];
+            for (int j = lane; j < nt; j += MTS_WAVE) {
+                tile_row_start[tile_off[e] + j] = start[e] + j * block_m;
+                tile_expert[tile_off[e] + j] = e;
+            }
+        }
+    }
+}
+
+__global__ __launch_bounds__(kThreads) void route_scatter_kernel(
+    const int32_t* __restrict__ idx, int64_t TK, int K, int E, const int32_t* __restrict__ cnt,
+    const int32_t* __restrict__ expert_start, int32_t* __restrict__ s_scatter,
+    int32_t* __restrict__ s_reverse, int32_t* __restrict__ x_gather) {
+    extern __shared__ int32_t lds[];  // [kWaves][E] next free row per expert
+    const int wave = threadIdx.x / MTS_WAVE, lane = threadIdx.x % MTS_WAVE;
+    const int64_t chunk = (int64_t)blockIdx.x * kWaves + wave;
+    const int64_t base = chunk * kChunk;
+    if (base >= TK) return;  // whole wave leaves; no block barrier below
+    volatile int32_t* next = lds + wave * E;
+    for (int e = lane; e < E; e += MTS_WAVE) next[e] = expert_start[e] + cnt[chunk * E + e];
+    const uint64_t lt = lanemask_lt();
+    for (int i = 0; i < kChunk; i += MTS_WAVE) {
+        int64_t n = base + i + lane;
+        bool valid = n < TK;
+        int e = valid ? clamp_expert(idx[n], E) : -1;
+        int pos = 0;
+        uint64_t todo = __ballot(valid);
+        while (todo) {
+            int leader = __ffsll((unsigned long long)todo) - 1;
+            int el = __shfl(e, leader, MTS_WAVE);
+            uint64_t same = __ballot(e == el);
+            int first = next[el];  // every lane reads before the leader updates
+            if (e == el) pos = first + __popcll(same & lt);
+            if (lane == leader) next[el] = first + __popcll(same);
+            todo &= ~same;
+        }
+        if (valid) {
+            s_reverse[n] = pos;
+            s_scatter[pos] = (int32_t)n;
+            x_gather[pos] = (int32_t)(n / K);
+        }
+    }
+}
+
+}  // namespace
+
+extern "C" int64_t mts_moe_route_workspace_bytes(int64_t T, int K, int E) {
+    int64_t TK = T * K;
+    int64_t n_chunks = (TK + kChunk - 1) / kChunk;
+    return n_chunks * E * (int64_t)sizeof(int32_t);
+}
+
+extern "C" int mts_moe_route(const int32_t* top_k_index, int64_t T, int K, int E, int block_m,
+                             int32_t* counts, int32_t* expert_start, int32_t* s_scatter,
+                             int32_t* s_reverse, int32_t* x_gather, int32_t* tile_row_start,
+                             int32_t* tile_expert, int32_t* tile_count, void* workspace,
+                             int64_t workspace_bytes, void* stream) {
+    if (!top_k_index || !counts || !expert_start || !s_scatter || !s_reverse || !x_gather ||
+        !workspace)
+        return MTS_ERR_NULL;
+    if (T <= 0 || K < 1 || E < 1 || E > MTS_MAX_EXPERTS || block_m < 1 ||
+        T * (int64_t)K > 0x7fffffffLL)
+        return MTS_ERR_SHAPE;
+    if (workspace_bytes < mts_moe_route_workspace_bytes(T, K, E)) return MTS_ERR_WORKSPACE;
+    hipStream_t s = (hipStream_t)stream;
+    const int64_t TK = T * K;
+    const int64_t n_chunks = (TK + kChunk - 1) / kChunk;
+    const int grid = (int)((n_chunks + kWaves - 1) / kWaves);
+    const size_t lds = (size_t)kWaves * E * sizeof(int32_t);
+    int32_t* cnt = (int32_t*)workspace;
+    route_hist_kernel<<<grid, kThreads, lds, s>>>(top_k_index, TK, E, cnt);
+    MTS_CHECK_LAUNCH();
+    route_scan_kernel<<<1, 1024, 0, s>>>(cnt, n_chunks, E, TK, block_m, counts, expert_start,
+                                         tile_row_start, tile_expert, tile_count);
+    MTS_CHECK_LAUNCH();
+    route_scatter_kernel<<<grid, kThreads, lds, s>>>(top_k_index, TK, K, E, cnt, expert_start,
+                                                     s_scatter, s_reverse, x_gather);
+    MTS_CHECK_LAUNCH();
+    return MTS_OK;
+}

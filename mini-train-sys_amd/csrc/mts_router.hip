@@ -1,0 +1,348 @@
+// Router post-process for fp32 logits: softmax, top-k on the logits with the
+// lower expert index winning a tie, selected-weight normalisation, mean
+// probability, z-loss and entropy; and its backward.
+//
+// A row of E logits is held by G adjacent lanes, EP values per lane
+// (expert e = j*G + g).  E <= 8 is one thread per row with two 16-byte loads.
+// Row statistics are summed per lane over a grid-stride loop, reduced over the
+// wave with a fixed shuffle tree, over the block through LDS and over blocks by a
+// second one-block kernel, so that results are bit-stable from run to run.
+#include "mts_common.h"
+
+#include <math.h>
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kMaxBlocks = 256;
+constexpr float kLogFloor = -20.72326583694641f;  // log(1e-9): the entropy clamps p at 1e-9
+
+template <int G>
+__device__ __forceinline__ float group_sum(float v) {
+#pragma unroll
+    for (int o = G / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, MTS_WAVE);
+    return v;
+}
+template <int G>
+__device__ __forceinline__ float group_max(float v) {
+#pragma unroll
+    for (int o = G / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, MTS_WAVE));
+    return v;
+}
+
+template <int EP, int G>
+struct RowState {
+    float l[EP];
+    float p[EP];
+    float m, s, L;
+};
+
+template <int EP, int G>
+__device__ __forceinline__ void load_row(const float* __restrict__ logits, int64_t row, int E, int g,
+                                         RowState<EP, G>& r) {
+    const float* src = logits + row * (int64_t)E;
+    if (G == 1 && EP == 8 && E == 8) {
+        const f32x4* v = reinterpret_cast<const f32x4*>(src);
+        f32x4 a = v[0], b = v[1];
+        r.l[0] = a[0]; r.l[1] = a[1]; r.l[2] = a[2]; r.l[3] = a[3];
+        r.l[4 % EP] = b[0]; r.l[5 % EP] = b[1]; r.l[6 % EP] = b[2]; r.l[7 % EP] = b[3];
+    } else {
+#pragma unroll
+        for (int j = 0; j < EP; ++j) {
+            int e = j * G + g;
+            r.l[j] = (e < E) ? src[e] : -INFINITY;
+        }
+    }
+    float m = r.l[0];
+#pragma unroll
+    for (int j = 1; j < EP; ++j) m = fmaxf(m, r.l[j]);
+    m = group_max<G>(m);
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < EP; ++j) {
+        r.p[j] = expf(r.l[j] - m);
+        s += r.p[j];
+    }
+    s = group_sum<G>(s);
+    float inv = 1.0f / s;
+#pragma unroll
+    for (int j = 0; j < EP; ++j) r.p[j] *= inv;
+    r.m = m;
+    r.s = s;
+    r.L = m + logf(s);
+}
+
+template <int EP, int G>
+__global__ __launch_bounds__(kThreads) void router_fwd_kernel(
+    const float* __restrict__ logits, int64_t T, int E, int K, int normalize,
+    float* __restrict__ weights, int32_t* __restrict__ indices, float* __restrict__ partial) {
+    constexpr int ROWS = kThreads / G;
+    const int g = threadIdx.x % G;
+    const int rl = threadIdx.x / G;
+    float psum[EP];
+#pragma unroll
+    for (int j = 0; j < EP; ++j) psum[j] = 0.f;
+    float zsum = 0.f, hsum = 0.f;
+
+    for (int64_t row0 = (int64_t)blockIdx.x * ROWS; row0 < T; row0 += (int64_t)gridDim.x * ROWS) {
+        int64_t row = row0 + rl;
+        bool live = row < T;
+        RowState<EP, G> r;
+        load_row<EP, G>(logits, live ? row : 0, E, g, r);
+
+        uint32_t taken = 0;
+#pragma unroll
+        for (int j = 0; j < EP; ++j)
+            if (j * G + g >= E) taken |= 1u << j;
+
+        float sel_p[MTS_MAX_TOP_K];
+        int sel_e[MTS_MAX_TOP_K];
+        float mass = 0.f;
+#pragma unroll
+        for (int k = 0; k < MTS_MAX_TOP_K; ++k) {
+            sel_p[k] = 0.f;
+            sel_e[k] = 0;
+            if (k < K) {
+                float bv = -INFINITY;
+                int be = 0x7fffffff;
+#pragma unroll
+                for (int j = 0; j < EP; ++j) {
+                    int e = j * G + g;
+                    bool free_slot = !((taken >> j) & 1u);
+                    if (free_slot && (r.l[j] > bv || (r.l[j] == bv && e < be))) {
+                        bv = r.l[j];
+                        be = e;
+                    }
+                }
+#pragma unroll
+                for (int o = G / 2; o > 0; o >>= 1) {
+                    float ov = __shfl_xor(bv, o, MTS_WAVE);
+                    int oe = __shfl_xor(be, o, MTS_WAVE);
+                    if (ov > bv || (ov == bv && oe < be)) {
+                        bv = ov;
+                        be = oe;
+                    }
+                }
+                if (be % G == g) taken |= 1u << (be / G);
+                float pk = expf(bv - r.m) / r.s;
+                sel_p[k] = pk;
+                sel_e[k] = be;
+                mass += pk;
+            }
+        }
+        if (live && g == 0) {
+            float inv = normalize ? 1.0f / fmaxf(mass, 1.1920928955078125e-07f) : 1.0f;
+#pragma unroll
+            for (int k = 0; k < MTS_MAX_TOP_K; ++k) {
+                if (k < K) {
+                    weights[row * K + k] = sel_p[k] * inv;
+                    indices[row * K + k] = sel_e[k];
+                }
+            }
+        }
+        if (live) {
+#pragma unroll
+            for (int j = 0; j < EP; ++j) {
+                psum[j] += r.p[j];
+                // p * log(max(p, 1e-9)); p == 0 (padding or underflow) contributes 0
+                float lp = fmaxf(r.l[j] - r.L, kLogFloor);
+                hsum -= (r.p[j] > 0.f) ? r.p[j] * lp : 0.f;
+            }
+            if (g == 0) zsum += r.L * r.L;
+        }
+    }
+
+    // wave: sum lanes that hold the same experts (same g)
+#pragma unroll
+    for (int j = 0; j < EP; ++j) {
+#pragma unroll
+        for (int o = 32; o >= G; o >>= 1) psum[j] += __shfl_xor(psum[j], o, MTS_WAVE);
+    }
+    zsum = wave_sum(zsum);
+    hsum = wave_sum(hsum);
+
+    __shared__ float red[kThreads / MTS_WAVE][EP * G + 2];
+    const int wave = threadIdx.x / MTS_WAVE, lane = threadIdx.x % MTS_WAVE;
+    if (lane < G) {
+#pragma unroll
+        for (int j = 0; j < EP; ++j) red[wave][j * G + lane] = psum[j];
+    }
+    if (lane == 0) {
+        red[wave][EP * G] = zsum;
+        red[wave][EP * G + 1] = hsum;
+    }
+    __syncthreads();
+    float* out = partial + (int64_t)blockIdx.x * (E + 2);
+    for (int i = threadIdx.x; i < E + 2; i += kThreads) {
+        int src = i < E ? i : EP * G + (i - E);
+        float v = 0.f;
+#pragma unroll
+        for (int w = 0; w < kThreads / MTS_WAVE; ++w) v += red[w][src];
+        out[i] = v;
+    }
+}
+
+__global__ __launch_bounds__(kThreads) void router_stats_kernel(
+    const float* __restrict__ partial, int nblocks, int E, float inv_t,
+    float* __restrict__ prob_mean, float* __restrict__ z_loss, float* __restrict__ entropy) {
+    for (int i = threadIdx.x; i < E + 2; i += kThreads) {
+        float v = 0.f;
+        for (int b = 0; b < nblocks; ++b) v += partial[(int64_t)b * (E + 2) + i];
+        v *= inv_t;
+        if (i < E) prob_mean[i] = v;
+        else if (i == E) z_loss[0] = v;
+        else entropy[0] = v;
+    }
+}
+
+template <int EP, int G>
+__global__ __launch_bounds__(kThreads) void router_bwd_kernel(
+    const float* __restrict__ logits, const float* __restrict__ weights,
+    const int32_t* __restrict__ indices, const float* __restrict__ g_w,
+    const float* __restrict__ g_p, const float* __restrict__ g_z, int64_t T, int E, int K,
+    int normalize, float* __restrict__ dlogits) {
+    constexpr int ROWS = kThreads / G;
+    const int g = threadIdx.x % G;
+    const int rl = threadIdx.x / G;
+    const float inv_t = 1.0f / (float)T;
+    const float gz = g_z[0] * 2.0f * inv_t;
+    float gp[EP];
+#pragma unroll
+    for (int j = 0; j < EP; ++j) {
+        int e = j * G + g;
+        gp[j] = (e < E) ? g_p[e] * inv_t : 0.f;
+    }
+    for (int64_t row0 = (int64_t)blockIdx.x * ROWS; row0 < T; row0 += (int64_t)gridDim.x * ROWS) {
+        int64_t row = row0 + rl;
+        bool live = row < T;
+        int64_t rr = live ? row : 0;
+        RowState<EP, G> r;
+        load_row<EP, G>(logits, rr, E, g, r);
+        float dp[EP], extra[EP];
+#pragma unroll
+        for (int j = 0; j < EP; ++j) {
+            dp[j] = gp[j];
+            extra[j] = 0.f;
+        }
+        float wdot = 0.f;
+        if (normalize) {
+            for (int k = 0; k < K; ++k) wdot += weights[rr * K + k] * g_w[rr * K + k];
+        }
+        for (int k = 0; k < K; ++k) {
+            int e = indices[rr * K + k];
+            float gw = g_w[rr * K + k];
+            float w = weights[rr * K + k];
+#pragma unroll
+            for (int j = 0; j < EP; ++j) {
+                if (j * G + g == e) {
+                    if (normalize) extra[j] += w * (gw - wdot);
+                    else dp[j] += gw;
+                }
+            }
+        }
+        float dot = 0.f;
+#pragma unroll
+        for (int j = 0; j < EP; ++j) dot += r.p[j] * dp[j];
+        dot = group_sum<G>(dot);
+        if (live) {
+            float* dst = dlogits + row * (int64_t)E;
+            float o[EP];
+#pragma unroll
+            for (int j = 0; j < EP; ++j) o[j] = r.p[j] * (dp[j] - dot) + gz * r.L * r.p[j] + extra[j];
+            if (G == 1 && EP == 8 && E == 8) {
+                f32x4* v = reinterpret_cast<f32x4*>(dst);
+                v[0] = f32x4{o[0], o[1], o[2], o[3]};
+                v[1] = f32x4{o[4 % EP], o[5 % EP], o[6 % EP], o[7 % EP]};
+            } else {
+#pragma unroll
+                for (int j = 0; j < EP; ++j) {
+                    int e = j * G + g;
+                    if (e < E) dst[e] = o[j];
+                }
+            }
+        }
+    }
+}
+
+int grid_for(int64_t T, int G) {
+    int64_t rows = kThreads / G;
+    int64_t b = (T + rows - 1) / rows;
+    return (int)(b < kMaxBlocks ? b : kMaxBlocks);
+}
+
+// lanes per row: E <= 8 -> 1, then the smallest power of two with 8*G >= E; 16 per lane above 512
+int lanes_for(int E) {
+    int G = 1;
+    while (G < 64 && 8 * G < E) G <<= 1;
+    return G;
+}
+
+#define MTS_ROUTER_DISPATCH(FN, ...)                                              \
+    do {                                                                          \
+        if (E > 512) { FN<16, 64> __VA_ARGS__; break; }                           \
+        switch (lanes_for(E)) {                                                   \
+            case 1: FN<8, 1> __VA_ARGS__; break;                                  \
+            case 2: FN<8, 2> __VA_ARGS__; break;                                  \
+            case 4: FN<8, 4> __VA_ARGS__; break;                                  \
+            case 8: FN<8, 8> __VA_ARGS__; break;                                  \
+            case 16: FN<8, 16> __VA_ARGS__; break;                                \
+            case 32: FN<8, 32> __VA_ARGS__; break;                                \
+            default: FN<8, 64> __VA_ARGS__; break;                                \
+        }                                                                         \
+    } while (0)
+
+int check_router(const void* logits, int64_t T, int E, int K) {
+    if (!logits) return MTS_ERR_NULL;
+    if (T <= 0 || T > (int64_t)1 << 40 || E < 1 || E > MTS_MAX_EXPERTS || K < 1 || K > E ||
+        K > MTS_MAX_TOP_K)
+        return MTS_ERR_SHAPE;
+    if (E == 8 && !mts_aligned16(logits)) return MTS_ERR_ALIGN;
+    return MTS_OK;
+}
+
+}  // namespace
+
+extern "C" int64_t mts_router_workspace_bytes(int64_t T, int E) {
+    (void)T;
+    return (int64_t)kMaxBlocks * (E + 2) * (int64_t)sizeof(float);
+}
+
+extern "C" int mts_router_fwd(const float* logits, int64_t T, int E, int K, int normalize,
+                              float* weights, int32_t* indices, float* prob_mean, float* z_loss,
+                              float* entropy, void* workspace, int64_t workspace_bytes,
+                              void* stream) {
+    int rc = check_router(logits, T, E, K);
+    if (rc) return rc;
+    if (!weights || !indices || !prob_mean || !z_loss || !entropy || !workspace) return MTS_ERR_NULL;
+    if (workspace_bytes < mts_router_workspace_bytes(T, E)) return MTS_ERR_WORKSPACE;
+    hipStream_t s = (hipStream_t)stream;
+    float* partial = (float*)workspace;
+    int G = E > 512 ? 64 : lanes_for(E);
+    int grid = grid_for(T, G);
+    MTS_ROUTER_DISPATCH(router_fwd_kernel,
+                        <<<grid, kThreads, 0, s>>>(logits, T, E, K, normalize, weights, indices, partial));
+    MTS_CHECK_LAUNCH();
+    router_stats_kernel<<<1, kThreads, 0, s>>>(partial, grid, E, 1.0f / (float)T, prob_mean, z_loss,
+                                               entropy);
+    MTS_CHECK_LAUNCH();
+    return MTS_OK;
+}
+
+extern "C" int mts_router_bwd(const float* logits, const float* weights, const int32_t* indices,
+                              const float* g_weights, const float* g_prob_mean,
+                              const float* g_z_loss, int64_t T, int E, int K, int normalize,
+                              float* dlogits, void* stream) {
+    int rc = check_router(logits, T, E, K);
+    if (rc) return rc;
+    if (!weights || !indices || !g_weights || !g_prob_mean || !g_z_loss || !dlogits)
+        return MTS_ERR_NULL;
+    if (E == 8 && !mts_aligned16(dlogits)) return MTS_ERR_ALIGN;
+    hipStream_t s = (hipStream_t)stream;
+    int G = E > 512 ? 64 : lanes_for(E);
+    int grid = grid_for(T, G);
+    MTS_ROUTER_DISPATCH(router_bwd_kernel,
+                        <<<grid, kThreads, 0, s>>>(logits, weights, indices, g_weights, g_prob_mean,
+                                                   g_z_loss, T, E, K, normalize, dlogits));
+    MTS_CHECK_LAUNCH();
+    return MTS_OK;
+}

@@ -1,0 +1,89 @@
+"""Compile the gfx950 HIP sources into ``lib/libmts_moe.so`` with hipcc.
+
+``python -m minitrain_amd.build`` (or ``build_library()``) always recompiles.  The
+library is linked against the HIP runtime by soname only, with no run path, so a
+process that has already imported torch resolves it to the runtime torch loaded.
+"""
+
+from __future__ import annotations
+
+import os
+import re
+import shutil
+import subprocess
+import sys
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(os.path.dirname(PKG_DIR), "csrc")
+INCLUDE = os.path.join(os.path.dirname(os.path.dirname(PKG_DIR)), "include")
+LIB_DIR = os.path.join(PKG_DIR, "lib")
+LIB_PATH = os.path.join(LIB_DIR, "libmts_moe.so")
+SOURCES = ("mts_router.hip", "mts_route.hip", "mts_combine.hip", "mts_gemm.hip")
+
+FLAGS = [
+    "-O3",
+    "--offload-arch=gfx950",
+    "-fPIC",
+    "-shared",
+    "-std=c++17",
+    # packed fp32 arithmetic is kept off for every kernel in this library
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def find_hipcc() -> str:
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.exists(cand):
+            return cand
+    raise RuntimeError("hipcc not found; set HIPCC or install ROCm")
+
+
+def build_library(verbose: bool = False, resource_report: bool = False) -> str:
+    os.makedirs(LIB_DIR, exist_ok=True)
+    cmd = [find_hipcc(), *FLAGS, f"-I{INCLUDE}", f"-I{CSRC}"]
+    if resource_report:
+        cmd.append("-Rpass-analysis=kernel-resource-usage")
+    cmd += [os.path.join(CSRC, s) for s in SOURCES]
+    tmp = LIB_PATH + ".tmp"
+    cmd += ["-o", tmp]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    err = "\n".join(l for l in proc.stderr.splitlines() if "packed-fp32-ops" not in l)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{err}")
+    os.replace(tmp, LIB_PATH)
+    if resource_report:
+        print(summarise_resources(proc.stderr))
+    elif verbose and err.strip():
+        print(err)
+    return LIB_PATH
+
+
+def summarise_resources(text: str) -> str:
+    rows, cur = [], {}
+    for line in text.splitlines():
+        m = re.search(r"remark: .*?:\d+:\d+: (.*) \[-Rpass", line) or re.search(r"remark:\s+(.*) \[-Rpass", line)
+        if not m:
+            continue
+        item = m.group(1).strip()
+        if item.startswith("Function Name:"):
+            cur = {"name": item.split(":", 1)[1].strip()}
+            rows.append(cur)
+        elif ":" in item and cur is not None:
+            k, v = item.split(":", 1)
+            cur[k.strip()] = v.strip()
+    out = []
+    for r in rows:
+        name = subprocess.run(["c++filt", r["name"]], capture_output=True, text=True).stdout.strip()
+        name = re.sub(r"\(anonymous namespace\)::", "", name).split("(")[0]
+        out.append(
+            f"{name[:90]:<90} vgpr={r.get('VGPRs', '?'):>4} agpr={r.get('AGPRs', '?'):>4} "
+            f"spill={r.get('VGPRs Spill', r.get('VGPR Spill', '?')):>3} scratch={r.get('ScratchSize [bytes/lane]', '?'):>4} "
+            f"occ={r.get('Occupancy [waves/SIMD]', '?'):>2} lds={r.get('LDS Size [bytes/block]', '?')}"
+        )
+    return "\n".join(out)
+
+
+if __name__ == "__main__":
+    path = build_library(verbose=True, resource_report="--resources" in sys.argv)
+    print("built", path)

@@ -1,0 +1,29 @@
+"""`hip` operator backend: MoE operators on hand-written gfx950 kernels.
+
+Counterpart of the reference's ``TritonOpsBackend``
+(minitrain/kernels/triton/__init__.py:36-113) for the two MoE methods.  Unlike
+that class there is no fallback: an unsupported tensor contract raises.
+"""
+
+from minitrain_amd.kernels.dense_ops import DenseTorchOps
+from minitrain_amd.kernels.hip.fused_moe import fused_moe, is_fused_moe_supported
+from minitrain_amd.kernels.hip.router import is_router_postprocess_supported, router_postprocess
+
+
+class HipOpsBackend(DenseTorchOps):
+    name = "hip"
+
+    def router_postprocess(self, logits, top_k, *, normalize):
+        return router_postprocess(logits, top_k, normalize=normalize)
+
+    def fused_moe(self, x, gate_up_proj, down_proj, top_k_index, top_k_weights):
+        return fused_moe(x, gate_up_proj, down_proj, top_k_index, top_k_weights)
+
+
+__all__ = [
+    "HipOpsBackend",
+    "fused_moe",
+    "is_fused_moe_supported",
+    "is_router_postprocess_supported",
+    "router_postprocess",
+]

@@ -1,0 +1,261 @@
+"""Fused top-k MoE (dispatch -> grouped SwiGLU experts -> weighted combine).
+
+Counterpart of minitrain/kernels/triton/fused_moe.py:37-449: the support
+predicate, the routing-metadata step, the autograd function and the module-level
+entry point.  Every buffer is a torch tensor on the caller's device; kernels are
+enqueued on the current stream through the C ABI and nothing synchronises.
+"""
+
+import functools
+
+import torch
+
+from minitrain_amd import _lib
+
+_MAX_EXPERTS = 1024
+BLOCK_M_TOKEN = 64
+
+
+def ensure_contiguous(fn):
+    @functools.wraps(fn)
+    def wrapper(ctx, *args, **kwargs):
+        args = [a.contiguous() if isinstance(a, torch.Tensor) else a for a in args]
+        return fn(ctx, *args, **kwargs)
+
+    return wrapper
+
+
+def is_fused_moe_supported(x, gate_up_proj, down_proj, top_k_index, top_k_weights) -> bool:
+    tensors = (x, gate_up_proj, down_proj, top_k_index, top_k_weights)
+    if not all(t.is_cuda for t in tensors):
+        return False
+    if len({t.device for t in tensors}) != 1:
+        return False
+    if x.ndim != 2 or gate_up_proj.ndim != 3 or down_proj.ndim != 3:
+        return False
+    if top_k_index.ndim != 2 or top_k_weights.shape != top_k_index.shape:
+        return False
+    tokens, hidden = x.shape
+    experts, twice_intermediate, weight_hidden = gate_up_proj.shape
+    intermediate = twice_intermediate // 2
+    weight_dtypes = (torch.bfloat16, torch.float32)
+    return (
+        tokens > 0
+        and 0 < experts <= _MAX_EXPERTS
+        and twice_intermediate % 2 == 0
+        and weight_hidden == hidden
+        and down_proj.shape == (experts, hidden, intermediate)
+        and top_k_index.shape[0] == tokens
+        and 0 < top_k_index.shape[1] <= min(experts, 32768)
+        and tokens * top_k_index.shape[1] < 2**31
+        and top_k_index.dtype == torch.int32
+        and top_k_weights.dtype == x.dtype
+        and x.dtype == torch.bfloat16
+        and gate_up_proj.dtype in weight_dtypes
+        and down_proj.dtype in weight_dtypes
+        and hidden % 8 == 0
+        and intermediate % 8 == 0
+    )
+
+
+def compute_routing_metadata(topk_indices: torch.Tensor, E: int, block_m_token: int = BLOCK_M_TOKEN):
+    """Counts, expert offsets, the stable expert-major permutation and the tile list.
+
+    Returns the same eight tensors, in the same order, as the reference's
+    ``compute_routing_metadata`` (minitrain/kernels/triton/fused_moe.py:74-154).
+    """
+    lib = _lib.load()
+    topk_indices = topk_indices.contiguous()
+    T, K = topk_indices.shape
+    TK = T * K
+    dev = topk_indices.device
+    i32 = dict(dtype=torch.int32, device=dev)
+    expert_token_count = torch.empty(E, **i32)
+    expert_start_idx = torch.empty(E + 1, **i32)
+    s_scatter_idx = torch.empty(TK, **i32)
+    s_reverse_scatter_idx = torch.empty(TK, **i32)
+    x_gather_idx = torch.empty(TK, **i32)
+    max_m_tiles = min(TK, -(-TK // block_m_token) + E - 1)
+    tile_row_start = torch.empty(max_m_tiles, **i32)
+    tile_expert = torch.empty(max_m_tiles, **i32)
+    tile_count = torch.empty(1, **i32)
+    ws_bytes = lib.mts_moe_route_workspace_bytes(T, K, E)
+    ws = torch.empty(max(ws_bytes, 4), dtype=torch.uint8, device=dev)
+    _lib.check(
+        lib.mts_moe_route(
+            topk_indices.data_ptr(), T, K, E, block_m_token, expert_token_count.data_ptr(),
+            expert_start_idx.data_ptr(), s_scatter_idx.data_ptr(), s_reverse_scatter_idx.data_ptr(),
+            x_gather_idx.data_ptr(), tile_row_start.data_ptr(), tile_expert.data_ptr(),
+            tile_count.data_ptr(), ws.data_ptr(), ws_bytes, _lib.stream_of(topk_indices),
+        ),
+        "mts_moe_route",
+    )
+    return (
+        expert_token_count,
+        expert_start_idx,
+        x_gather_idx,
+        s_scatter_idx,
+        s_reverse_scatter_idx,
+        tile_row_start,
+        tile_expert,
+        tile_count,
+    )
+
+
+def _stage(lib, w: torch.Tensor, transpose: bool) -> torch.Tensor:
+    """bf16 copy of an expert weight ``[E,R,C]``, optionally as ``[E,C,R]``."""
+    if not transpose and w.dtype == torch.bfloat16:
+        return w
+    E, R, C = w.shape
+    out = torch.empty((E, C, R) if transpose else (E, R, C), dtype=torch.bfloat16, device=w.device)
+    _lib.check(
+        lib.mts_moe_stage_weights(
+            w.data_ptr(), _lib.dtype_code(w.dtype), out.data_ptr(), E, R, C, int(transpose), _lib.stream_of(w)
+        ),
+        "mts_moe_stage_weights",
+    )
+    return out
+
+
+class _FusedMoEFunction(torch.autograd.Function):
+    @staticmethod
+    @ensure_contiguous
+    def forward(ctx, x, gate_up_proj, down_proj, top_k_index, top_k_weights):
+        lib = _lib.load()
+        T, K = top_k_index.shape
+        E = gate_up_proj.shape[0]
+        H = x.shape[1]
+        I = gate_up_proj.shape[1] // 2
+        TK = T * K
+        dev = x.device
+        act = _lib.dtype_code(x.dtype)
+        stream = _lib.stream_of(x)
+
+        with torch.no_grad():
+            (_, expert_start, x_gather, s_scatter, s_reverse, _, _, _) = compute_routing_metadata(top_k_index, E)
+
+        w1 = _stage(lib, gate_up_proj, False)
+        w2 = _stage(lib, down_proj, False)
+        pre_act = torch.empty(TK, 2 * I, dtype=x.dtype, device=dev)
+        post_act = torch.empty(TK, I, dtype=x.dtype, device=dev)
+        _lib.check(
+            lib.mts_moe_fwd_gateup_swiglu(
+                x.data_ptr(), w1.data_ptr(), x_gather.data_ptr(), expert_start.data_ptr(), T, K, E, H, I, act,
+                pre_act.data_ptr(), post_act.data_ptr(), stream,
+            ),
+            "mts_moe_fwd_gateup_swiglu",
+        )
+        y = torch.empty(TK, H, dtype=x.dtype, device=dev)
+        _lib.check(
+            lib.mts_moe_fwd_down(
+                post_act.data_ptr(), w2.data_ptr(), expert_start.data_ptr(), TK, E, H, I, act, y.data_ptr(), stream
+            ),
+            "mts_moe_fwd_down",
+        )
+        weights_flat = top_k_weights.flatten().contiguous()
+        out = torch.empty(T, H, dtype=x.dtype, device=dev)
+        _lib.check(
+            lib.mts_moe_combine(
+                y.data_ptr(), weights_flat.data_ptr(), s_reverse.data_ptr(), T, K, H, act, out.data_ptr(), stream
+            ),
+            "mts_moe_combine",
+        )
+
+        ctx.save_for_backward(
+            x, gate_up_proj, down_proj, pre_act, weights_flat, expert_start, x_gather, s_scatter, s_reverse
+        )
+        ctx.dims = (T, K, E, H, I)
+        ctx.mark_non_differentiable(top_k_index)
+        ctx.set_materialize_grads(False)
+        return out
+
+    @staticmethod
+    @ensure_contiguous
+    def backward(ctx, dO):
+        if dO is None:
+            return None, None, None, None, None
+        lib = _lib.load()
+        (x, gate_up_proj, down_proj, pre_act, weights_flat, expert_start, x_gather, s_scatter, s_reverse) = (
+            ctx.saved_tensors
+        )
+        T, K, E, H, I = ctx.dims
+        TK = T * K
+        dev = dO.device
+        if dO.dtype != x.dtype:
+            dO = dO.to(x.dtype)
+        act = _lib.dtype_code(x.dtype)
+        stream = _lib.stream_of(dO)
+        need_x, need_w1, need_w2, _, need_s = ctx.needs_input_grad
+
+        w2t = _stage(lib, down_proj, True)  # [E, I, H]
+        d_pre_act = torch.empty(TK, 2 * I, dtype=x.dtype, device=dev)
+        weighted_act = torch.empty(TK, I, dtype=x.dtype, device=dev)
+        n_part = lib.mts_moe_ds_partials(I)
+        ds_part = torch.empty(TK, n_part, dtype=torch.float32, device=dev)
+        _lib.check(
+            lib.mts_moe_bwd_dy1(
+                dO.data_ptr(), w2t.data_ptr(), pre_act.data_ptr(), weights_flat.data_ptr(), x_gather.data_ptr(),
+                s_scatter.data_ptr(), expert_start.data_ptr(), T, K, E, H, I, act, d_pre_act.data_ptr(),
+                weighted_act.data_ptr(), ds_part.data_ptr(), stream,
+            ),
+            "mts_moe_bwd_dy1",
+        )
+        del w2t
+
+        d_weights = None
+        if need_s:
+            d_weights = torch.empty(T, K, dtype=weights_flat.dtype, device=dev)
+            _lib.check(
+                lib.mts_moe_bwd_ds(ds_part.data_ptr(), s_reverse.data_ptr(), TK, I, act, d_weights.data_ptr(), stream),
+                "mts_moe_bwd_ds",
+            )
+
+        ddown_proj = None
+        if need_w2:
+            ddown_proj = torch.empty_like(down_proj)
+            _lib.check(
+                lib.mts_moe_bwd_dw2(
+                    dO.data_ptr(), weighted_act.data_ptr(), x_gather.data_ptr(), expert_start.data_ptr(), T, K, E, H,
+                    I, act, _lib.dtype_code(down_proj.dtype), ddown_proj.data_ptr(), stream,
+                ),
+                "mts_moe_bwd_dw2",
+            )
+        del weighted_act
+
+        dx = None
+        if need_x:
+            w1t = _stage(lib, gate_up_proj, True)  # [E, H, 2I]
+            dx_expanded = torch.empty(TK, H, dtype=x.dtype, device=dev)
+            _lib.check(
+                lib.mts_moe_bwd_dx(
+                    d_pre_act.data_ptr(), w1t.data_ptr(), expert_start.data_ptr(), TK, E, H, I, act,
+                    dx_expanded.data_ptr(), stream,
+                ),
+                "mts_moe_bwd_dx",
+            )
+            dx = torch.empty(T, H, dtype=x.dtype, device=dev)
+            _lib.check(
+                lib.mts_moe_combine(
+                    dx_expanded.data_ptr(), None, s_reverse.data_ptr(), T, K, H, act, dx.data_ptr(), stream
+                ),
+                "mts_moe_combine",
+            )
+
+        dgate_up_proj = None
+        if need_w1:
+            dgate_up_proj = torch.empty_like(gate_up_proj)
+            _lib.check(
+                lib.mts_moe_bwd_dw1(
+                    d_pre_act.data_ptr(), x.data_ptr(), x_gather.data_ptr(), expert_start.data_ptr(), T, K, E, H, I,
+                    act, _lib.dtype_code(gate_up_proj.dtype), dgate_up_proj.data_ptr(), stream,
+                ),
+                "mts_moe_bwd_dw1",
+            )
+
+        return dx, dgate_up_proj, ddown_proj, None, d_weights
+
+
+def fused_moe(x, gate_up_proj, down_proj, top_k_index, top_k_weights):
+    if not is_fused_moe_supported(x, gate_up_proj, down_proj, top_k_index, top_k_weights):
+        raise RuntimeError("Unsupported tensor contract for hip fused MoE")
+    return _FusedMoEFunction.apply(x, gate_up_proj, down_proj, top_k_index, top_k_weights)

@@ -1,0 +1,110 @@
+"""Router post-process on the GPU: one pass over the fp32 logits.
+
+Counterpart of minitrain/kernels/triton/router.py:262-357 (autograd wrapper and
+module-level entry point) with the argument checks of
+minitrain/kernels/torch_ops.py:96-101.  Top-k is taken on the logits with the
+lower expert index winning ties, and the statistics are reduced in a fixed
+order, so the operator is deterministic and needs no deterministic-mode opt-out.
+"""
+
+import torch
+
+from minitrain_amd import _lib
+from minitrain_amd.model.ops import RouterPostprocessOutput
+
+_MAX_EXPERTS = 1024
+_MAX_TOP_K = 8
+
+
+def is_router_postprocess_supported(logits: torch.Tensor, top_k: int, normalize: bool) -> bool:
+    del normalize  # both normalised and raw full-softmax weights are supported
+    return (
+        logits.is_cuda
+        and logits.ndim == 2
+        and logits.dtype == torch.float32
+        and logits.shape[0] > 0
+        and 1 <= top_k <= min(logits.shape[1], _MAX_TOP_K)
+        and logits.shape[1] <= _MAX_EXPERTS
+    )
+
+
+class _RouterPostprocessFunction(torch.autograd.Function):
+    @staticmethod
+    @torch.amp.custom_fwd(device_type="cuda")
+    def forward(ctx, logits: torch.Tensor, top_k: int, normalize: bool):
+        lib = _lib.load()
+        logits = logits.contiguous()
+        T, E = logits.shape
+        dev = logits.device
+        weights = torch.empty((T, top_k), device=dev, dtype=torch.float32)
+        indices = torch.empty((T, top_k), device=dev, dtype=torch.int32)
+        stats = torch.empty(E + 2, device=dev, dtype=torch.float32)
+        ws_bytes = lib.mts_router_workspace_bytes(T, E)
+        ws = torch.empty(ws_bytes, device=dev, dtype=torch.uint8)
+        prob_mean, z_loss, entropy = stats[:E], stats[E], stats[E + 1]
+        _lib.check(
+            lib.mts_router_fwd(
+                logits.data_ptr(), T, E, top_k, int(normalize), weights.data_ptr(), indices.data_ptr(),
+                prob_mean.data_ptr(), z_loss.data_ptr(), entropy.data_ptr(), ws.data_ptr(), ws_bytes,
+                _lib.stream_of(logits),
+            ),
+            "mts_router_fwd",
+        )
+        ctx.save_for_backward(logits, weights, indices)
+        ctx.top_k = top_k
+        ctx.normalize = normalize
+        ctx.mark_non_differentiable(indices, entropy)
+        return weights, indices, prob_mean, z_loss, entropy
+
+    @staticmethod
+    @torch.amp.custom_bwd(device_type="cuda")
+    def backward(ctx, grad_weights, _grad_indices, grad_probability_mean, grad_z_loss, _grad_entropy):
+        lib = _lib.load()
+        logits, weights, indices = ctx.saved_tensors
+        T, E = logits.shape
+        dev = logits.device
+
+        def dense(g, shape):
+            if g is None:
+                return torch.zeros(shape, device=dev, dtype=torch.float32)
+            return g.to(torch.float32).contiguous()
+
+        g_w = dense(grad_weights, (T, ctx.top_k))
+        g_p = dense(grad_probability_mean, (E,))
+        g_z = dense(grad_z_loss, ())
+        grad_logits = torch.empty_like(logits)
+        _lib.check(
+            lib.mts_router_bwd(
+                logits.data_ptr(), weights.data_ptr(), indices.data_ptr(), g_w.data_ptr(), g_p.data_ptr(),
+                g_z.data_ptr(), T, E, ctx.top_k, int(ctx.normalize), grad_logits.data_ptr(),
+                _lib.stream_of(logits),
+            ),
+            "mts_router_bwd",
+        )
+        return grad_logits, None, None
+
+
+def router_postprocess(logits: torch.Tensor, top_k: int, *, normalize: bool) -> RouterPostprocessOutput:
+    """Process router logits without materialising the full probability matrix."""
+
+    if logits.ndim != 2 or logits.dtype != torch.float32:
+        raise ValueError("router logits must be a 2D fp32 tensor")
+    if logits.shape[0] == 0:
+        raise ValueError("router logits must contain at least one token")
+    if not 1 <= top_k <= logits.shape[1]:
+        raise ValueError(f"top_k must be in [1, {logits.shape[1]}], got {top_k}")
+    if not is_router_postprocess_supported(logits, top_k, normalize):
+        raise RuntimeError(
+            "hip router postprocess requires non-empty 2D fp32 logits on the GPU, "
+            f"1 <= top_k <= {_MAX_TOP_K} and at most {_MAX_EXPERTS} experts"
+        )
+    weights, indices, probability_mean, z_loss, entropy = _RouterPostprocessFunction.apply(
+        logits, top_k, normalize
+    )
+    return RouterPostprocessOutput(
+        expert_weights=weights,
+        expert_indices=indices,
+        probability_per_expert=probability_mean,
+        z_loss=z_loss,
+        entropy=entropy,
+    )

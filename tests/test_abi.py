@@ -1,0 +1,65 @@
+"""The C-ABI library loads and exports every symbol the public header declares (no GPU needed)."""
+
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "mts_moe.h")
+
+
+def _declared():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mts_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    names = _declared()
+    for must in ("mts_router_fwd", "mts_router_bwd", "mts_moe_route", "mts_moe_fwd_gateup_swiglu", "mts_moe_fwd_down",
+                 "mts_moe_combine", "mts_moe_bwd_dy1", "mts_moe_bwd_dx", "mts_moe_bwd_dw1", "mts_moe_bwd_dw2"):
+        assert must in names
+
+
+def test_library_exports_every_declared_symbol():
+    from minitrain_amd import _lib
+
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.fail(f"{_lib.LIB_PATH} not built: run `python -c 'import __graft_entry__ as g; g.build()'`")
+    lib = _lib.load()
+    for name in _declared():
+        assert hasattr(lib, name), f"{name} is declared in mts_moe.h but not exported"
+        assert name in _lib.SIGNATURES, f"{name} has no ctypes prototype"
+    assert lib.mts_version() == 1
+    assert lib.mts_error_string(0) == b"ok"
+    # argument checks run on the host before any launch: safe without a GPU
+    assert lib.mts_router_fwd(None, 4, 8, 2, 1, None, None, None, None, None, None, 0, None) == -1
+    assert lib.mts_moe_route_workspace_bytes(24576, 2, 8) == 48 * 8 * 4
+    assert lib.mts_moe_ds_partials(1024) > 0
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    from minitrain_amd import _lib
+
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(_lib.MtsError):
+        _lib.load()
+
+
+def test_cpu_tensors_are_rejected_not_served_by_a_fallback():
+    import torch
+
+    from minitrain_amd.model.ops import get_ops_backend
+
+    ops = get_ops_backend("hip")
+    with pytest.raises(RuntimeError):
+        ops.router_postprocess(torch.zeros(4, 8), 2, normalize=True)
+    with pytest.raises(RuntimeError):
+        ops.fused_moe(torch.zeros(4, 8, dtype=torch.bfloat16), torch.zeros(2, 16, 8, dtype=torch.bfloat16),
+                      torch.zeros(2, 8, 8, dtype=torch.bfloat16), torch.zeros(4, 1, dtype=torch.int32),
+                      torch.zeros(4, 1, dtype=torch.bfloat16))
+    with pytest.raises(ValueError):
+        get_ops_backend("triton")

@@ -1,0 +1,168 @@
+"""HIP fused MoE (forward and backward, through the C ABI) against the oracle."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import moe_oracle as O
+from tests.helpers import BF16_TOL, assert_close_scaled, hip_backend, hip_moe_grads, oracle_moe_grads, routed_case
+
+pytestmark = pytest.mark.gpu
+
+NAMES = ("dx", "dW1", "dW2", "dS")
+
+
+def _compare(case, *, device="cpu", tol=BF16_TOL):
+    out, grads = hip_moe_grads(case["x"], case["w1"], case["w2"], case["idx"], case["w"], case["g"])
+    ref_out, ref_grads = oracle_moe_grads(case["x"], case["w1"], case["w2"], case["idx"], case["w"], case["g"],
+                                          device=device)
+    assert out.dtype == case["x"].dtype and out.shape == case["x"].shape
+    stats = {"out": assert_close_scaled(out, ref_out, tol, "out")}
+    for name, got, want, leaf in zip(NAMES, grads, ref_grads, (case["x"], case["w1"], case["w2"], case["w"])):
+        assert got.dtype == leaf.dtype and got.shape == leaf.shape, name
+        stats[name] = assert_close_scaled(got, want, tol, name)
+    # the reference's own acceptance for this operator: relative L2 and cosine
+    for name, st in stats.items():
+        assert st["relative_l2"] <= 1e-2 and st["cosine"] >= 0.9999, (name, st)
+    return stats
+
+
+@pytest.mark.parametrize("T,H,E,I,K", [(256, 64, 4, 128, 2), (33, 128, 8, 64, 2), (1, 64, 4, 64, 1),
+                                       (257, 192, 8, 320, 2), (700, 72, 3, 40, 2), (129, 32, 4, 24, 3)])
+def test_small_shapes(T, H, E, I, K):
+    print(f"moe small T={T} H={H} E={E} I={I} K={K}", flush=True)
+    _compare(routed_case(10 + T, T, H, E, I, K))
+
+
+def test_reference_edge_probe():
+    """T=33, K=3, only experts {0,1} of 8 used, repeated experts inside a token and
+    zero weights on [::2, -1]; zero-weight routes must still receive a gradient."""
+    print("moe edge probe", flush=True)
+    T, H, E, I, K = 33, 128, 8, 64, 3
+    case = routed_case(5, T, H, E, I, K)
+    idx = torch.stack([(torch.arange(T) + s) % 2 for s in range(K)], dim=1).to(torch.int32)
+    w = torch.rand(T, K, generator=torch.Generator().manual_seed(1)).bfloat16()
+    w[::2, -1] = 0
+    case.update(idx=idx, w=w)
+    _compare(case)
+    out, grads = hip_moe_grads(case["x"], case["w1"], case["w2"], idx, w, case["g"])
+    assert float(grads[3][::2, -1].float().abs().min()) > 0
+    for e in range(2, E):
+        assert not grads[1][e].any() and not grads[2][e].any(), "experts without routes get zero gradients"
+
+
+def test_fp32_master_weights_bf16_activations():
+    """Parameters stay fp32 under autocast: weight gradients come back in fp32."""
+    print("moe fp32 weights", flush=True)
+    case = routed_case(21, 300, 128, 4, 192, 2)
+    _, w_r, w1, w2, _ = O.make_inputs(21, 300, 128, 4, 192)
+    case.update(w1=w1, w2=w2)
+    _compare(case)
+
+
+def test_non_contiguous_inputs_and_no_grad_paths():
+    print("moe non-contiguous", flush=True)
+    ops = hip_backend()
+    case = routed_case(31, 200, 128, 4, 128, 2)
+    x = torch.zeros(200, 256, dtype=torch.bfloat16)
+    x[:, ::2] = case["x"]
+    xs = x.cuda()[:, ::2]
+    assert not xs.is_contiguous()
+    got = ops.fused_moe(xs, case["w1"].cuda(), case["w2"].cuda(), case["idx"].cuda(), case["w"].cuda())
+    want = ops.fused_moe(case["x"].cuda(), case["w1"].cuda(), case["w2"].cuda(), case["idx"].cuda(), case["w"].cuda())
+    assert torch.equal(got, want)
+    # only x requires grad
+    xg = case["x"].cuda().requires_grad_(True)
+    ops.fused_moe(xg, case["w1"].cuda(), case["w2"].cuda(), case["idx"].cuda(), case["w"].cuda()).sum().backward()
+    assert xg.grad is not None
+    # unsupported contracts raise instead of falling back
+    with pytest.raises(RuntimeError):
+        ops.fused_moe(case["x"], case["w1"], case["w2"], case["idx"], case["w"])               # CPU tensors
+    with pytest.raises(RuntimeError):
+        ops.fused_moe(case["x"].cuda(), case["w1"].cuda(), case["w2"].cuda(), case["idx"].cuda().long(),
+                      case["w"].cuda())                                                        # int64 indices
+    with pytest.raises(RuntimeError):
+        ops.fused_moe(case["x"].cuda(), case["w1"].cuda(), case["w2"].cuda(), case["idx"].cuda(),
+                      case["w"].cuda().float())                                                # weight dtype != x dtype
+
+
+def test_run_to_run_determinism():
+    print("moe determinism", flush=True)
+    case = routed_case(41, 1000, 128, 8, 256, 2)
+    a = hip_moe_grads(case["x"], case["w1"], case["w2"], case["idx"], case["w"], case["g"])
+    b = hip_moe_grads(case["x"], case["w1"], case["w2"], case["idx"], case["w"], case["g"])
+    assert torch.equal(a[0], b[0])
+    for u, v in zip(a[1], b[1]):
+        assert torch.equal(u, v)
+
+
+def test_layer_shape_subset_of_tokens():
+    """293M-class layer dims at 2048 tokens: the whole oracle still runs on the CPU in seconds."""
+    print("moe 2048x768x1024", flush=True)
+    _compare(routed_case(1, 2048, 768, 8, 1024, 2))
+
+
+@pytest.mark.parametrize("name,seed,T,imbalanced", [("config2", 1, 24576, False), ("config4", 3, 24576, True),
+                                                    ("config3", 2, 98304, False)])
+def test_full_size_configs(name, seed, T, imbalanced):
+    """Full benchmark sizes.  The checker is the oracle's expert loop evaluated in
+    fp32 on the GPU (same code, library matmuls); in addition the rows of a sample
+    of tokens are checked against the oracle on the CPU (tokens are independent)."""
+    print(f"moe {name} T={T}", flush=True)
+    H, E, I, K = 768, 8, 1024, 2
+    bias = O.zipf_log_bias(E) if imbalanced else None
+    case = routed_case(seed, T, H, E, I, K, bias=bias, tie_fraction=0.01 if imbalanced else 0.0)
+    if imbalanced:
+        share = np.bincount(case["idx"].flatten().numpy(), minlength=E) / case["idx"].numel()
+        assert share.max() > 0.3
+    stats = _compare(case, device="cuda")
+    print({k: (round(v["max_rel_scaled"], 5), round(v["relative_l2"], 5)) for k, v in stats.items()}, flush=True)
+    # sample of tokens against the CPU oracle
+    ops = hip_backend()
+    out = ops.fused_moe(*(case[k].cuda() for k in ("x", "w1", "w2", "idx", "w"))).cpu()
+    pick = torch.from_numpy(np.random.Generator(np.random.Philox(seed)).choice(T, size=192, replace=False))
+    ref = O.fused_moe(case["x"][pick], case["w1"], case["w2"], case["idx"][pick], case["w"][pick],
+                      compute_dtype=torch.float32)
+    assert_close_scaled(out[pick], ref, BF16_TOL, "sampled tokens vs CPU oracle")
+    if name == "config3":
+        print("peak HBM allocated (MB):", torch.cuda.max_memory_allocated() / 2**20, flush=True)
+
+
+def test_moe_block_end_to_end():
+    """Router + fused MoE through the block that owns the parameters, with the aux and
+    z losses in the objective so that all three router-gradient inlets are used."""
+    print("moe block end to end", flush=True)
+    from minitrain_amd.model.blocks import MoEFeedForward
+    from minitrain_amd.model.config import ModelConfig
+
+    T, H, E, I, K = 512, 128, 8, 256, 2
+    cfg = ModelConfig(hidden_size=H, intermediate_size=I, num_experts=E, experts_per_token=K, n_layers=12)
+    x, w_r, w1, w2, g = O.make_inputs(7, T, H, E, I)
+    block = MoEFeedForward(cfg).cuda()
+    with torch.no_grad():
+        block.router.weight.copy_(w_r)
+        block.gate_up_proj.copy_(w1)
+        block.down_proj.copy_(w2)
+    xg = x.bfloat16().cuda().requires_grad_(True)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        out = block(xg.view(4, T // 4, H), hip_backend())
+    loss = (out.hidden_states.float() * g.cuda().view(4, T // 4, H)).sum() + 0.01 * out.router_aux_loss \
+        + 0.001 * out.router_z_loss
+    loss.backward()
+    # oracle: same arithmetic on the CPU, fp32-accumulated experts
+    leaves = [t.clone().requires_grad_(True) for t in (x.bfloat16().float(), w_r, w1, w2)]
+    hidden, r = O.moe_feed_forward(leaves[0].bfloat16(), leaves[1], leaves[2].bfloat16(), leaves[3].bfloat16(), K,
+                                   compute_dtype=torch.float32)
+    ref_loss = (hidden * g).sum() + 0.01 * r.auxiliary_loss + 0.001 * r.z_loss
+    ref_loss.backward()
+    assert torch.equal(out.router_metrics["moe/expert_load_fraction"].cpu() * T * K,
+                       torch.bincount(r.expert_indices.flatten().long(), minlength=E).float())
+    assert_close_scaled(out.hidden_states.view(T, H), hidden, BF16_TOL, "hidden")
+    torch.testing.assert_close(out.router_aux_loss.cpu(), r.auxiliary_loss, rtol=1e-4, atol=1e-6)
+    torch.testing.assert_close(out.router_z_loss.cpu(), r.z_loss, rtol=1e-4, atol=1e-6)
+    assert_close_scaled(xg.grad, leaves[0].grad, BF16_TOL, "dx")
+    assert_close_scaled(block.router.weight.grad, leaves[1].grad, BF16_TOL, "dRouter")
+    assert_close_scaled(block.gate_up_proj.grad, leaves[2].grad, BF16_TOL, "dW1")
+    assert_close_scaled(block.down_proj.grad, leaves[3].grad, BF16_TOL, "dW2")
+    for key in ("moe/router_entropy", "moe/dropped_route_fraction", "moe/max_expert_load", "moe/min_expert_load"):
+        assert key in out.router_metrics
