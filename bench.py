@@ -1,0 +1,268 @@
+#!/usr/bin/env python3
+"""MoE-layer forward+backward benchmark on one MI355X.
+
+A step is one pass of the hot path over one batch of synthetic input: fp32 router
+GEMM -> router post-process -> fused top-2 MoE, then the full backward (dX,
+dRouter, dW1, dW2).  The workload is the 293M-class layer shape: 24 x 1024
+tokens, d_model 768, 8 experts, top-2, expert d_ff 1024, bf16 tensors with fp32
+accumulation, seed 1, all inputs resident in HBM before the timed region.
+
+One JSON line is printed.  Besides the whole-layer tokens/s it carries
+  * ``kernels``: every kernel stage timed on its own with HIP events on the stream
+    it is launched on, with its algorithmic FLOPs or bytes and roofline fraction;
+  * ``roofline``: the same figures for the stage that takes the most time;
+  * ``gemm_roofline`` / ``combine_roofline``: all expert GEMMs together against the
+    dense bf16 MFMA peak, and the combine kernels against peak HBM bandwidth;
+  * ``cpu_baseline``: the CPU restatement of the reference's PyTorch path timed on
+    the host cores of the same box on a bounded sample of the same workload.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "mini-train-sys_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+import numpy as np
+import torch
+import torch.nn.functional as F
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+
+WORKLOAD = dict(name="moe_layer_24x1024_d768_e8_top2_ff1024_bf16", seed=1, T=24576, H=768, E=8, K=2, I=1024)
+
+
+def make_inputs(seed, T, H, E, I):
+    """x, W_r, gate_up_proj, down_proj, G drawn in that order from a Philox stream."""
+    rng = np.random.Generator(np.random.Philox(seed))
+    x = rng.standard_normal((T, H), dtype=np.float32)
+    w_r = rng.standard_normal((E, H), dtype=np.float32) * np.float32(0.02)
+    w1 = rng.standard_normal((E, 2 * I, H), dtype=np.float32) * np.float32(0.02)
+    w2 = rng.standard_normal((E, H, I), dtype=np.float32) * np.float32(0.02)
+    g = rng.standard_normal((T, H), dtype=np.float32)
+    return tuple(torch.from_numpy(a) for a in (x, w_r, w1, w2, g))
+
+
+class Layer:
+    """The layer as the MoE block runs it, with leaves that collect gradients."""
+
+    def __init__(self, ops, x, w_r, w1, w2, g, K):
+        self.ops, self.K = ops, K
+        self.x = x.cuda().bfloat16().requires_grad_(True)
+        self.w_r = w_r.cuda().requires_grad_(True)
+        self.w1 = w1.cuda().bfloat16().requires_grad_(True)
+        self.w2 = w2.cuda().bfloat16().requires_grad_(True)
+        self.g = g.cuda().bfloat16()
+        self.E = w_r.shape[0]
+
+    def step(self):
+        for t in (self.x, self.w_r, self.w1, self.w2):
+            t.grad = None
+        logits = F.linear(self.x.float(), self.w_r)
+        route = self.ops.router_postprocess(logits, self.K, normalize=True)
+        counts = torch.bincount(route.expert_indices.flatten().long(), minlength=self.E)
+        aux = self.E * torch.sum(counts.float() / route.expert_indices.numel() * route.probability_per_expert)
+        out = self.ops.fused_moe(self.x, self.w1, self.w2, route.expert_indices, route.expert_weights.to(self.x.dtype))
+        loss_side = 0.01 * aux + 0.001 * route.z_loss
+        torch.autograd.backward([out, loss_side], [self.g, torch.ones_like(loss_side)])
+        return out
+
+
+def time_layer(layer, steps, warmup):
+    for _ in range(warmup):
+        layer.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        layer.step()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def stage_breakdown(layer, steps):
+    """Launch every kernel stage through the C ABI with HIP events around each launch."""
+    from minitrain_amd import _lib
+    from minitrain_amd.kernels.hip.fused_moe import compute_routing_metadata
+
+    lib = _lib.load()
+    w = WORKLOAD
+    T, H, E, K, I = w["T"], w["H"], w["E"], w["K"], w["I"]
+    TK = T * K
+    dev = layer.x.device
+    bf = dict(dtype=torch.bfloat16, device=dev)
+    x, w1, w2, g = layer.x.detach(), layer.w1.detach(), layer.w2.detach(), layer.g
+    logits = F.linear(x.float(), layer.w_r.detach())
+    route = layer.ops.router_postprocess(logits, K, normalize=True)
+    idx, wts = route.expert_indices, route.expert_weights.bfloat16().flatten().contiguous()
+    (_, es, xg, ss, sr, _, _, _) = compute_routing_metadata(idx, E)
+    pre, post, y, out = torch.empty(TK, 2 * I, **bf), torch.empty(TK, I, **bf), torch.empty(TK, H, **bf), torch.empty(T, H, **bf)
+    dpre, wact, dxe, dx = torch.empty(TK, 2 * I, **bf), torch.empty(TK, I, **bf), torch.empty(TK, H, **bf), torch.empty(T, H, **bf)
+    npart = lib.mts_moe_ds_partials(I)
+    dsp = torch.empty(TK, npart, dtype=torch.float32, device=dev)
+    dwts = torch.empty(T, K, **bf)
+    w2t, w1t = torch.empty(E, I, H, **bf), torch.empty(E, H, 2 * I, **bf)
+    dw1, dw2 = torch.empty_like(w1), torch.empty_like(w2)
+    rw = torch.empty(lib.mts_router_workspace_bytes(T, E), dtype=torch.uint8, device=dev)
+    rws = torch.empty(max(4, lib.mts_moe_route_workspace_bytes(T, K, E)), dtype=torch.uint8, device=dev)
+    r_w, r_i = torch.empty(T, K, dtype=torch.float32, device=dev), torch.empty(T, K, dtype=torch.int32, device=dev)
+    r_stats = torch.empty(E + 2, dtype=torch.float32, device=dev)
+    i32 = dict(dtype=torch.int32, device=dev)
+    cnt, es2, a1, a2, a3 = torch.empty(E, **i32), torch.empty(E + 1, **i32), torch.empty(TK, **i32), torch.empty(TK, **i32), torch.empty(TK, **i32)
+    dlog = torch.empty_like(logits)
+    gw, gp, gz = torch.randn(T, K, device=dev), torch.randn(E, device=dev), torch.ones((), device=dev)
+    st = torch.cuda.current_stream().cuda_stream
+    p = lambda t: t.data_ptr()
+    B = _lib.MTS_BF16
+    gemm = lambda mult: 2.0 * TK * H * I * mult
+    esz = 2
+    stages = [
+        ("router_fwd", "hbm", T * E * 4 + T * K * 8,
+         lambda: lib.mts_router_fwd(p(logits), T, E, K, 1, p(r_w), p(r_i), p(r_stats), p(r_stats) + 4 * E, p(r_stats) + 4 * E + 4, p(rw), rw.numel(), st)),
+        ("route_metadata", "hbm", TK * 4 * 2 + 3 * TK * 4,
+         lambda: lib.mts_moe_route(p(idx), T, K, E, 64, p(cnt), p(es2), p(a1), p(a2), p(a3), None, None, None, p(rws), rws.numel(), st)),
+        ("fwd_gateup_swiglu", "mfma", gemm(2),
+         lambda: lib.mts_moe_fwd_gateup_swiglu(p(x), p(w1), p(xg), p(es), T, K, E, H, I, B, p(pre), p(post), st)),
+        ("fwd_down", "mfma", gemm(1), lambda: lib.mts_moe_fwd_down(p(post), p(w2), p(es), TK, E, H, I, B, p(y), st)),
+        ("combine", "hbm", TK * H * esz + T * H * esz + TK * 4 + TK * esz,
+         lambda: lib.mts_moe_combine(p(y), p(wts), p(sr), T, K, H, B, p(out), st)),
+        ("stage_w2_transposed", "hbm", 2 * E * H * I * esz, lambda: lib.mts_moe_stage_weights(p(w2), B, p(w2t), E, H, I, 1, st)),
+        ("bwd_dy1", "mfma", gemm(1),
+         lambda: lib.mts_moe_bwd_dy1(p(g), p(w2t), p(pre), p(wts), p(xg), p(ss), p(es), T, K, E, H, I, B, p(dpre), p(wact), p(dsp), st)),
+        ("bwd_ds", "hbm", TK * npart * 4 + TK * 4 + TK * esz, lambda: lib.mts_moe_bwd_ds(p(dsp), p(sr), TK, I, B, p(dwts), st)),
+        ("bwd_dw2", "mfma", gemm(1), lambda: lib.mts_moe_bwd_dw2(p(g), p(wact), p(xg), p(es), T, K, E, H, I, B, B, p(dw2), st)),
+        ("stage_w1_transposed", "hbm", 2 * E * 2 * I * H * esz, lambda: lib.mts_moe_stage_weights(p(w1), B, p(w1t), E, 2 * I, H, 1, st)),
+        ("bwd_dx", "mfma", gemm(2), lambda: lib.mts_moe_bwd_dx(p(dpre), p(w1t), p(es), TK, E, H, I, B, p(dxe), st)),
+        ("dx_combine", "hbm", TK * H * esz + T * H * esz + TK * 4,
+         lambda: lib.mts_moe_combine(p(dxe), None, p(sr), T, K, H, B, p(dx), st)),
+        ("bwd_dw1", "mfma", gemm(2), lambda: lib.mts_moe_bwd_dw1(p(dpre), p(x), p(xg), p(es), T, K, E, H, I, B, B, p(dw1), st)),
+        ("router_bwd", "hbm", T * E * 4 * 2 + T * K * 12,
+         lambda: lib.mts_router_bwd(p(logits), p(r_w), p(r_i), p(gw), p(gp), p(gz), T, E, K, 1, p(dlog), st)),
+    ]
+    ev = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in stages] for _ in range(steps)]
+    for it in range(2 + steps):
+        for j, (name, _, _, fn) in enumerate(stages):
+            if it >= 2:
+                ev[it - 2][j][0].record()
+            rc = fn()
+            if it >= 2:
+                ev[it - 2][j][1].record()
+            if rc != 0:
+                raise RuntimeError(f"{name} returned {rc}")
+    torch.cuda.synchronize()
+    rows = []
+    for j, (name, bound, work, _) in enumerate(stages):
+        ms = float(np.mean([ev[i][j][0].elapsed_time(ev[i][j][1]) for i in range(steps)]))
+        if bound == "mfma":
+            ach = work / (ms * 1e-3) / 1e12
+            rows.append(dict(stage=name, bound=bound, avg_ms=round(ms, 4), achieved=round(ach, 2), peak=PEAK_BF16_TFLOPS,
+                             unit="TFLOP/s", frac=round(ach / PEAK_BF16_TFLOPS, 4), work=work))
+        else:
+            ach = work / (ms * 1e-3) / 1e9
+            rows.append(dict(stage=name, bound=bound, avg_ms=round(ms, 4), achieved=round(ach, 1), peak=PEAK_HBM_GBS,
+                             unit="GB/s", frac=round(ach / PEAK_HBM_GBS, 4), work=work))
+    return rows
+
+
+def cpu_baseline(budget_s=20.0):
+    """The oracle's restatement of the reference's PyTorch path (input-dtype arithmetic,
+    autograd backward) on the host cores, on the first ``sample`` tokens of the workload."""
+    from oracle import moe_oracle as O
+
+    w = WORKLOAD
+    sample = w["T"]
+    x, w_r, w1, w2, g = O.make_inputs(w["seed"], w["T"], w["H"], w["E"], w["I"])
+    x, g = x[:sample].bfloat16(), g[:sample].bfloat16()
+    w1, w2 = w1.bfloat16(), w2.bfloat16()
+
+    def step():
+        leaves = [t.clone().requires_grad_(True) for t in (x, w_r, w1, w2)]
+        hidden, r = O.moe_feed_forward(leaves[0], leaves[1], leaves[2], leaves[3], w["K"])
+        loss = (hidden.float() * g.float()).sum() + 0.01 * r.auxiliary_loss + 0.001 * r.z_loss
+        loss.backward()
+
+    step()
+    times = []
+    t_end = time.perf_counter() + budget_s
+    while len(times) < 10 and (time.perf_counter() < t_end or len(times) < 3):
+        t0 = time.perf_counter()
+        step()
+        times.append(time.perf_counter() - t0)
+    p50 = float(np.median(times))
+    return dict(value=round(sample / p50, 1), unit="tokens/s", cores=torch.get_num_threads(), kind="port",
+                sample=f"{sample} of {w['T']} tokens of the same workload, bf16 tensors, fwd+bwd, p50 of {len(times)} runs",
+                host_cpus=os.cpu_count(), p50_s=round(p50, 4))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-breakdown", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (there is no CPU fallback for the hip backend)", file=sys.stderr)
+        sys.exit(2)
+
+    from minitrain_amd.model.ops import get_ops_backend
+
+    w = WORKLOAD
+    ops = get_ops_backend("hip")
+    layer = Layer(ops, *make_inputs(w["seed"], w["T"], w["H"], w["E"], w["I"]), w["K"])
+    sec = time_layer(layer, args.steps, args.warmup)
+    tokens_per_s = w["T"] / sec
+    gemm_flops = 18.0 * w["T"] * w["K"] * w["H"] * w["I"]
+
+    result = {
+        "metric": "MoE layer fwd+bwd tokens/s (24x1024, bf16)",
+        "value": round(tokens_per_s, 1),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(sec * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": w["name"], "tokens": w["T"], "d_model": w["H"], "experts": w["E"], "top_k": w["K"],
+                   "d_ff": w["I"], "seed": w["seed"], "step": "router GEMM + router post-process + fused MoE, fwd + full bwd"},
+        "layer_gemm_tflops": round(gemm_flops / sec / 1e12, 2),
+    }
+    if not args.no_breakdown:
+        rows = stage_breakdown(layer, max(5, min(args.steps, 20)))
+        result["kernels"] = rows
+        dom = max(rows, key=lambda r: r["avg_ms"])
+        result["roofline"] = {"kernel": dom["stage"], "bound": dom["bound"], "achieved": dom["achieved"], "peak": dom["peak"],
+                              "unit": dom["unit"], "frac": dom["frac"], "traffic": None}
+        gemm_rows = [r for r in rows if r["bound"] == "mfma"]
+        g_ms = sum(r["avg_ms"] for r in gemm_rows)
+        g_ach = sum(r["work"] for r in gemm_rows) / (g_ms * 1e-3) / 1e12
+        result["gemm_roofline"] = {"bound": "mfma", "achieved": round(g_ach, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                                   "frac": round(g_ach / PEAK_BF16_TFLOPS, 4), "sum_ms": round(g_ms, 4)}
+        c_rows = [r for r in rows if r["stage"] in ("combine", "dx_combine")]
+        c_ms = sum(r["avg_ms"] for r in c_rows)
+        c_ach = sum(r["work"] for r in c_rows) / (c_ms * 1e-3) / 1e9
+        result["combine_roofline"] = {"bound": "hbm", "achieved": round(c_ach, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                                      "frac": round(c_ach / PEAK_HBM_GBS, 4), "sum_ms": round(c_ms, 4)}
+        result["kernel_sum_ms"] = round(sum(r["avg_ms"] for r in rows), 4)
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()
