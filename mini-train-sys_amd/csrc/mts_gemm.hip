@@ -10,9 +10,14 @@
 //       operands arrive "k-major" and are transposed 8x8 in registers on their
 //       way into LDS.
 //
-// LDS tiles are [rows][BK + 8] bf16 (the 16-byte pad makes the 16-byte MFMA
-// fragment reads of 16 consecutive rows hit distinct banks), double buffered:
-// the global loads of tile k+1 are issued before the MFMAs of tile k.
+// Global reads are raw buffer loads: a lane that must contribute zeros (row past
+// the expert's end, column past N, k past K) is given an offset beyond the buffer
+// and the hardware returns 0, so the main loop has no divergent branches.
+//
+// LDS tiles are [rows][64] bf16 with the 16-byte chunk index XOR-swizzled by
+// (row >> 1) & 7: the 16-byte MFMA fragment reads of 16 consecutive rows, and the
+// row-contiguous tile writes, are both bank-conflict free without padding.  Two
+// stages: the global loads of tile k+1 are in flight during the MFMAs of tile k.
 //
 // MFMA 32x32x16 register layout used below (lane l):
 //   A/B fragment: row (l % 32) of the 32-row operand, k = 8*(l/32) .. 8*(l/32)+7
@@ -23,8 +28,24 @@
 
 namespace {
 
-constexpr int BK = 64;
-constexpr int LDS_LD = BK + 8;
+constexpr int BK = 64;                       // k extent of an LDS tile (8 chunks of 8 bf16)
+constexpr uint32_t kInvalid = 0x80000000u;   // buffer offset that is out of range for every operand
+constexpr int64_t kMaxOperandBytes = 0x7fffffffLL;
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, int64_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ u32x4 buf_load16(__amdgpu_buffer_rsrc_t r, uint32_t byte_off) {
+    return __builtin_amdgcn_raw_buffer_load_b128(r, (int)byte_off, 0, 0);
+}
+__device__ __forceinline__ int buf_load4(__amdgpu_buffer_rsrc_t r, uint32_t byte_off) {
+    return (int)__builtin_amdgcn_raw_buffer_load_b32(r, (int)byte_off, 0, 0);
+}
+
+// element offset of 16-byte chunk `chunk` of row `row` inside a swizzled tile
+__device__ __forceinline__ int lds_off(int row, int chunk) {
+    return row * BK + ((chunk ^ ((row >> 1) & 7)) << 3);
+}
 
 template <int BM_, int BN_, int WAVES_M_, int WAVES_N_>
 struct Tile {
@@ -33,7 +54,8 @@ struct Tile {
     static constexpr int NT = NWAVES * MTS_WAVE;
     static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
     static constexpr int MF = WM / 32, NF = WN / 32;
-    static constexpr int LDS_ELEMS = 2 * (BM + BN) * LDS_LD;
+    static constexpr int STAGE = (BM + BN) * BK;   // elements per pipeline stage
+    static constexpr int LDS_ELEMS = 2 * STAGE;
     static_assert(WM % 32 == 0 && WN % 64 == 0, "wave tile must hold whole 32x32 fragments");
     static_assert((BM * 8) % NT == 0 && (BN * 8) % NT == 0, "loader split");
 };
@@ -42,10 +64,11 @@ enum Epilogue { EPI_PLAIN = 0, EPI_SWIGLU = 1, EPI_DY1 = 2 };
 
 struct RowsParams {
     const bf16_t* A;           // activations, row-major, leading dimension lda
-    int64_t lda;
+    int64_t a_rows;            // rows of A (for the buffer range)
+    int lda;
     const int32_t* a_gather;   // row -> source row of A, or NULL for identity
-    const bf16_t* B;           // [E][n_rows_b][Kdim] bf16
-    int64_t b_expert_stride;
+    const bf16_t* B;           // [E][b_rows][Kdim] bf16
+    int b_rows;
     int N;                     // output columns (SwiGLU: I, B holds 2I rows)
     int Kdim;
     const int32_t* expert_start;
@@ -57,6 +80,7 @@ struct RowsParams {
     const int32_t* s_scatter;  // DY1: row -> entry
     float* ds_part;            // DY1: [TK][np]
     int np;
+    int64_t TK;                // rows of every output
 };
 
 // ---------------------------------------------------------------------------
@@ -65,40 +89,42 @@ struct RowsParams {
 template <int ROWS, int NT>
 struct KMajorLoader {
     static constexpr int LOADS = ROWS * (BK / 8) / NT;
-    const bf16_t* ptr[LOADS];  // row base + this thread's 8-element column, NULL = zero row
+    __amdgpu_buffer_rsrc_t rsrc;
+    uint32_t voff[LOADS];  // byte offset of this thread's chunk at k = 0, or kInvalid
     u32x4 reg[LOADS];
-    int col;                   // element offset of this thread's vector inside the k-tile
+    int chunk;             // this thread's 16-byte chunk inside the k-tile
 
     __device__ __forceinline__ void fetch(int k0, int Kdim) {
+        const bool kok = k0 + chunk * 8 < Kdim;
 #pragma unroll
-        for (int p = 0; p < LOADS; ++p) {
-            u32x4 v = {0u, 0u, 0u, 0u};
-            if (ptr[p] != nullptr && k0 + col < Kdim)
-                v = *reinterpret_cast<const u32x4*>(ptr[p] + k0);
-            reg[p] = v;
-        }
+        for (int p = 0; p < LOADS; ++p)
+            reg[p] = buf_load16(rsrc, kok ? voff[p] + (uint32_t)k0 * 2u : kInvalid);
     }
     __device__ __forceinline__ void commit(bf16_t* lds) const {
         const int r = threadIdx.x / 8;
 #pragma unroll
         for (int p = 0; p < LOADS; ++p)
-            *reinterpret_cast<u32x4*>(lds + (p * (NT / 8) + r) * LDS_LD + col) = reg[p];
+            *reinterpret_cast<u32x4*>(lds + lds_off(p * (NT / 8) + r, chunk)) = reg[p];
     }
 };
 
 // one MFMA sweep over a staged k-tile
-template <class T, bool SWIGLU>
+// (ROWLEN = k extent of the LDS rows: 64 with swizzle (row>>1)&7, 32 with (row>>2)&3)
+template <class T, bool SWIGLU, int ROWLEN = BK, bool WEIGHT_FIRST = true>
 __device__ __forceinline__ void mma_tile(const bf16_t* As, const bf16_t* Bs, int wm, int wn,
                                          f32x16 (&acc)[T::MF][T::NF]) {
     const int lane = threadIdx.x % MTS_WAVE;
-    const int frow = lane % 32, fk = (lane / 32) * 8;
+    const int frow = lane % 32, kb = lane / 32;
+    const int swz = ROWLEN == 64 ? (frow >> 1) & 7 : (frow >> 2) & 3;
+    const bf16_t* a_base = As + (wm * T::WM + frow) * ROWLEN;
+    const bf16_t* b_base = Bs + frow * ROWLEN;
 #pragma unroll
-    for (int ks = 0; ks < BK / 16; ++ks) {
+    for (int ks = 0; ks < ROWLEN / 16; ++ks) {
+        const int coff = ((ks * 2 + kb) ^ swz) << 3;
         bf16x8 a[T::MF], b[T::NF];
 #pragma unroll
         for (int mf = 0; mf < T::MF; ++mf)
-            a[mf] = *reinterpret_cast<const bf16x8*>(As + (wm * T::WM + mf * 32 + frow) * LDS_LD +
-                                                    ks * 16 + fk);
+            a[mf] = *reinterpret_cast<const bf16x8*>(a_base + mf * 32 * ROWLEN + coff);
 #pragma unroll
         for (int nf = 0; nf < T::NF; ++nf) {
             int brow;
@@ -108,24 +134,182 @@ __device__ __forceinline__ void mma_tile(const bf16_t* As, const bf16_t* Bs, int
             } else {
                 brow = wn * T::WN + nf * 32;
             }
-            b[nf] = *reinterpret_cast<const bf16x8*>(Bs + (brow + frow) * LDS_LD + ks * 16 + fk);
+            b[nf] = *reinterpret_cast<const bf16x8*>(b_base + brow * ROWLEN + coff);
         }
 #pragma unroll
         for (int mf = 0; mf < T::MF; ++mf)
 #pragma unroll
             for (int nf = 0; nf < T::NF; ++nf)
-                acc[mf][nf] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[mf], b[nf], acc[mf][nf], 0, 0, 0);
+                acc[mf][nf] = WEIGHT_FIRST
+                                  ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[nf], a[mf], acc[mf][nf], 0, 0, 0)
+                                  : __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[mf], b[nf], acc[mf][nf], 0, 0, 0);
     }
 }
 
 __device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + __expf(-x)); }
+
+template <class T>
+__device__ __forceinline__ void zero_acc(f32x16 (&acc)[T::MF][T::NF]) {
+#pragma unroll
+    for (int mf = 0; mf < T::MF; ++mf)
+#pragma unroll
+        for (int nf = 0; nf < T::NF; ++nf)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[mf][nf][i] = 0.f;
+}
+
+// ---------------------------------------------------------------------------
+// epilogues of rows_gemm (accumulators -> global memory)
+//
+// The MFMAs of rows_gemm take the weight fragment as the first operand, so a lane
+// holds, for ONE activation row (lane % 32), four runs of four consecutive output
+// columns: element i of fragment nf is column 32*nf + 8*(i/4) + 4*(lane/32) + i%4.
+// Per-row quantities (routing weight, dS) therefore live in one lane pair, and
+// the bf16 results are staged through a per-wave LDS tile [32][COLS+8] with 8-byte
+// writes and flushed with 16-byte, row-contiguous buffer stores; rows past the
+// expert's end and columns past N get an out-of-range offset and are dropped by
+// the hardware, so there are no divergent branches.
+// ---------------------------------------------------------------------------
+template <class T, int EPI>
+struct EpiShape {
+    static constexpr int COLS = (EPI == EPI_SWIGLU) ? T::WN / 2 : T::WN;  // contiguous columns per staged tile
+    static constexpr int NBUF = (EPI == EPI_PLAIN) ? 1 : 3;
+    static constexpr int LDW = COLS + 8;
+    static constexpr int ELEMS = T::NWAVES * NBUF * 32 * LDW;
+};
+
+__device__ __forceinline__ void stage4(bf16_t* dst, float a, float b, float c, float d) {
+    bf16x4 v = {(bf16_t)a, (bf16_t)b, (bf16_t)c, (bf16_t)d};
+    *reinterpret_cast<bf16x4*>(dst) = v;
+}
+
+// staged [32][COLS] tile -> global rows rowg0.., columns col.. of a matrix with leading dimension ldc
+template <int COLS>
+__device__ __forceinline__ void flush_tile(const bf16_t* buf, __amdgpu_buffer_rsrc_t rs, uint32_t ldc, uint32_t col,
+                                           int rowg0, int rend, int ncol0, int N) {
+    constexpr int LPR = COLS / 8, RPI = MTS_WAVE / LPR, LDW = COLS + 8;
+    const int lane = threadIdx.x % MTS_WAVE;
+    const int c = (lane % LPR) * 8;
+#pragma unroll
+    for (int it = 0; it < 32 / RPI; ++it) {
+        const int r = it * RPI + lane / LPR;
+        const u32x4 v = *reinterpret_cast<const u32x4*>(buf + r * LDW + c);
+        const int row = rowg0 + r;
+        const bool ok = row < rend && ncol0 + c < N;
+        const uint32_t off = ok ? ((uint32_t)row * ldc + col + (uint32_t)c) * 2u : kInvalid;
+        __builtin_amdgcn_raw_buffer_store_b128(v, rs, (int)off, 0, 0);
+    }
+}
+
+template <class T, int EPI>
+__device__ __forceinline__ void rows_epilogue(const RowsParams& p, f32x16 (&acc)[T::MF][T::NF], bf16_t* smem,
+                                              int row0, int rend, int n0, int wm, int wn) {
+    typedef EpiShape<T, EPI> ES;
+    constexpr int COLS = ES::COLS, LDW = ES::LDW;
+    const int wave = threadIdx.x / MTS_WAVE, lane = threadIdx.x % MTS_WAVE;
+    const int ml = lane % 32, nq = (lane / 32) * 4;
+    bf16_t* buf0 = smem + wave * ES::NBUF * 32 * LDW;
+    bf16_t* buf1 = buf0 + 32 * LDW;
+    bf16_t* buf2 = buf1 + 32 * LDW;
+    const int ncol0 = n0 + wn * COLS;  // first output column of this wave
+    const uint32_t N = (uint32_t)p.N;
+    const __amdgpu_buffer_rsrc_t rs_c = make_rsrc(p.C, p.TK * (int64_t)(EPI == EPI_PLAIN ? N : 2 * N) * 2);
+    const __amdgpu_buffer_rsrc_t rs_c2 = make_rsrc(p.C2, EPI == EPI_PLAIN ? 0 : p.TK * (int64_t)N * 2);
+    const __amdgpu_buffer_rsrc_t rs_pre = make_rsrc(p.pre_act, EPI == EPI_DY1 ? p.TK * (int64_t)N * 4 : 0);
+
+#pragma unroll
+    for (int mf = 0; mf < T::MF; ++mf) {
+        const int rowg0 = row0 + wm * T::WM + mf * 32;
+        if (EPI == EPI_PLAIN) {
+#pragma unroll
+            for (int nf = 0; nf < T::NF; ++nf)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    stage4(buf0 + ml * LDW + nf * 32 + 8 * j + nq, acc[mf][nf][4 * j], acc[mf][nf][4 * j + 1],
+                           acc[mf][nf][4 * j + 2], acc[mf][nf][4 * j + 3]);
+            flush_tile<COLS>(buf0, rs_c, N, ncol0, rowg0, rend, ncol0, p.N);
+        } else if (EPI == EPI_SWIGLU) {
+            constexpr int HALF = T::NF / 2;
+#pragma unroll
+            for (int f = 0; f < HALF; ++f)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    float g[4], u[4], a[4];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        g[q] = acc[mf][f][4 * j + q];
+                        u[q] = acc[mf][f + HALF][4 * j + q];
+                        a[q] = g[q] * sigmoidf_(g[q]) * u[q];
+                    }
+                    const int o = ml * LDW + f * 32 + 8 * j + nq;
+                    stage4(buf0 + o, g[0], g[1], g[2], g[3]);
+                    stage4(buf1 + o, u[0], u[1], u[2], u[3]);
+                    stage4(buf2 + o, a[0], a[1], a[2], a[3]);
+                }
+            flush_tile<COLS>(buf0, rs_c, 2 * N, ncol0, rowg0, rend, ncol0, p.N);
+            flush_tile<COLS>(buf1, rs_c, 2 * N, N + ncol0, rowg0, rend, ncol0, p.N);
+            flush_tile<COLS>(buf2, rs_c2, N, ncol0, rowg0, rend, ncol0, p.N);
+        } else {  // EPI_DY1
+            const int row = rowg0 + ml;
+            const bool rok = row < rend;
+            float s = 0.f;
+            if (rok) s = (float)p.route_w[p.s_scatter[row]];
+            float dsp = 0.f;
+#pragma unroll
+            for (int nf = 0; nf < T::NF; ++nf)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int nl = nf * 32 + 8 * j + nq;   // column inside the wave tile
+                    const int n = ncol0 + nl;
+                    const uint32_t po = (rok && n < p.N) ? ((uint32_t)row * 2u * N + (uint32_t)n) * 2u : kInvalid;
+                    const uint2 gr = __builtin_bit_cast(uint2, __builtin_amdgcn_raw_buffer_load_b64(rs_pre, (int)po, 0, 0));
+                    const uint2 ur = __builtin_bit_cast(
+                        uint2, __builtin_amdgcn_raw_buffer_load_b64(rs_pre, (int)(po == kInvalid ? kInvalid : po + N * 2u), 0, 0));
+                    float wa[4], dg[4], du[4];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const uint32_t gw = q < 2 ? gr.x : gr.y, uw = q < 2 ? ur.x : ur.y;
+                        const float g = bf16_bits_to_f32((q & 1) ? gw >> 16 : gw & 0xffffu);
+                        const float u = bf16_bits_to_f32((q & 1) ? uw >> 16 : uw & 0xffffu);
+                        const float a = acc[mf][nf][4 * j + q];
+                        const float sig = sigmoidf_(g);
+                        const float silu = g * sig;
+                        const float y1 = silu * u;
+                        dsp += a * y1;
+                        wa[q] = s * y1;
+                        const float da = a * s;
+                        dg[q] = da * (silu * (1.0f - sig) + sig) * u;
+                        du[q] = da * silu;
+                    }
+                    const int o = ml * LDW + nl;
+                    stage4(buf0 + o, wa[0], wa[1], wa[2], wa[3]);
+                    stage4(buf1 + o, dg[0], dg[1], dg[2], dg[3]);
+                    stage4(buf2 + o, du[0], du[1], du[2], du[3]);
+                }
+            dsp += __shfl_xor(dsp, 32, MTS_WAVE);
+            // one partial per 64 output columns, whatever the tile shape: a wave that
+            // covers 128 columns writes its sum to the first slot and 0 to the second
+            if (rok && lane < 32) {
+                const int slot = ncol0 / 64;
+#pragma unroll
+                for (int q = 0; q < T::WN / 64; ++q)
+                    if (slot + q < p.np) p.ds_part[(int64_t)row * p.np + slot + q] = q == 0 ? dsp : 0.f;
+            }
+            flush_tile<COLS>(buf0, rs_c2, N, ncol0, rowg0, rend, ncol0, p.N);
+            flush_tile<COLS>(buf1, rs_c, 2 * N, ncol0, rowg0, rend, ncol0, p.N);
+            flush_tile<COLS>(buf2, rs_c, 2 * N, N + ncol0, rowg0, rend, ncol0, p.N);
+        }
+    }
+}
 
 // ---------------------------------------------------------------------------
 // rows_gemm
 // ---------------------------------------------------------------------------
 template <class T, int EPI>
 __global__ __launch_bounds__(T::NT) void rows_gemm_kernel(RowsParams p) {
-    __shared__ __attribute__((aligned(16))) bf16_t smem[T::LDS_ELEMS];
+    constexpr int LDS_ELEMS = T::LDS_ELEMS > EpiShape<T, EPI>::ELEMS ? T::LDS_ELEMS : EpiShape<T, EPI>::ELEMS;
+    static_assert(LDS_ELEMS * 2 <= 160 * 1024, "LDS capacity");
+    __shared__ __attribute__((aligned(16))) bf16_t smem[LDS_ELEMS];
     constexpr bool SWIGLU = (EPI == EPI_SWIGLU);
 
     // which expert does this m-tile belong to
@@ -151,20 +335,18 @@ __global__ __launch_bounds__(T::NT) void rows_gemm_kernel(RowsParams p) {
 
     KMajorLoader<T::BM, T::NT> la;
     KMajorLoader<T::BN, T::NT> lb;
-    la.col = lb.col = (threadIdx.x % 8) * 8;
+    la.chunk = lb.chunk = threadIdx.x % 8;
+    la.rsrc = make_rsrc(p.A, p.a_rows * p.lda * 2);
+    lb.rsrc = make_rsrc(p.B + (int64_t)e * p.b_rows * p.Kdim, (int64_t)p.b_rows * p.Kdim * 2);
     {
         const int r = threadIdx.x / 8;
 #pragma unroll
         for (int q = 0; q < la.LOADS; ++q) {
             int row = row0 + q * (T::NT / 8) + r;
-            const bf16_t* ptr = nullptr;
-            if (row < rend) {
-                int64_t src = p.a_gather ? (int64_t)p.a_gather[row] : (int64_t)row;
-                ptr = p.A + src * p.lda + la.col;
-            }
-            la.ptr[q] = ptr;
+            int lrow = row < rend ? row : rend - 1;          // keep the index load in range
+            int src = p.a_gather ? p.a_gather[lrow] : lrow;
+            la.voff[q] = row < rend ? ((uint32_t)src * (uint32_t)p.lda + la.chunk * 8) * 2u : kInvalid;
         }
-        const bf16_t* Be = p.B + (int64_t)e * p.b_expert_stride;
 #pragma unroll
         for (int q = 0; q < lb.LOADS; ++q) {
             int br = q * (T::NT / 8) + r;  // row inside the B tile
@@ -177,22 +359,16 @@ __global__ __launch_bounds__(T::NT) void rows_gemm_kernel(RowsParams p) {
                 n = n0 + br;
                 grow = n;
             }
-            lb.ptr[q] = (n < p.N) ? Be + (int64_t)grow * p.Kdim + lb.col : nullptr;
+            lb.voff[q] = (n < p.N) ? ((uint32_t)grow * (uint32_t)p.Kdim + lb.chunk * 8) * 2u : kInvalid;
         }
     }
 
     const int wave = threadIdx.x / MTS_WAVE, lane = threadIdx.x % MTS_WAVE;
     const int wm = wave / T::WAVES_N, wn = wave % T::WAVES_N;
     f32x16 acc[T::MF][T::NF];
-#pragma unroll
-    for (int mf = 0; mf < T::MF; ++mf)
-#pragma unroll
-        for (int nf = 0; nf < T::NF; ++nf)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) acc[mf][nf][i] = 0.f;
+    zero_acc<T>(acc);
 
-    constexpr int STAGE = (T::BM + T::BN) * LDS_LD;  // one buffer: A tile then B tile
-    constexpr int B_OFF = T::BM * LDS_LD;
+    constexpr int B_OFF = T::BM * BK;
     const int nk = (p.Kdim + BK - 1) / BK;
     la.fetch(0, p.Kdim);
     lb.fetch(0, p.Kdim);
@@ -200,8 +376,8 @@ __global__ __launch_bounds__(T::NT) void rows_gemm_kernel(RowsParams p) {
     lb.commit(smem + B_OFF);
     __syncthreads();
     for (int kt = 0; kt < nk; ++kt) {
-        bf16_t* cur = smem + (kt & 1) * STAGE;
-        bf16_t* nxt = smem + ((kt & 1) ^ 1) * STAGE;
+        bf16_t* cur = smem + (kt & 1) * T::STAGE;
+        bf16_t* nxt = smem + ((kt & 1) ^ 1) * T::STAGE;
         if (kt + 1 < nk) {
             la.fetch((kt + 1) * BK, p.Kdim);
             lb.fetch((kt + 1) * BK, p.Kdim);
@@ -214,86 +390,189 @@ __global__ __launch_bounds__(T::NT) void rows_gemm_kernel(RowsParams p) {
         __syncthreads();
     }
 
-    // ---- epilogue ----
-    const int fcol = lane % 32, frow4 = (lane / 32) * 4;
-#pragma unroll
-    for (int mf = 0; mf < T::MF; ++mf) {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const int row = row0 + wm * T::WM + mf * 32 + 8 * (i / 4) + frow4 + (i % 4);
-            const bool rok = row < rend;
-            if (EPI == EPI_PLAIN) {
-#pragma unroll
-                for (int nf = 0; nf < T::NF; ++nf) {
-                    int n = n0 + wn * T::WN + nf * 32 + fcol;
-                    if (rok && n < p.N) p.C[(int64_t)row * p.N + n] = (bf16_t)acc[mf][nf][i];
-                }
-            } else if (EPI == EPI_SWIGLU) {
-                constexpr int HALF = T::NF / 2;
-#pragma unroll
-                for (int f = 0; f < HALF; ++f) {
-                    int n = n0 + wn * (T::WN / 2) + f * 32 + fcol;
-                    float g = acc[mf][f][i], u = acc[mf][f + HALF][i];
-                    if (rok && n < p.N) {
-                        p.C[(int64_t)row * (2 * p.N) + n] = (bf16_t)g;
-                        p.C[(int64_t)row * (2 * p.N) + p.N + n] = (bf16_t)u;
-                        p.C2[(int64_t)row * p.N + n] = (bf16_t)(g * sigmoidf_(g) * u);
-                    }
-                }
-            } else {  // EPI_DY1
-                float s = 0.f;
-                if (rok) s = (float)p.route_w[p.s_scatter[row]];
-                float dsp = 0.f;
-#pragma unroll
-                for (int nf = 0; nf < T::NF; ++nf) {
-                    int n = n0 + wn * T::WN + nf * 32 + fcol;
-                    if (rok && n < p.N) {
-                        const int64_t o = (int64_t)row * (2 * p.N) + n;
-                        float g = (float)p.pre_act[o], u = (float)p.pre_act[o + p.N];
-                        float a = acc[mf][nf][i];
-                        float sig = sigmoidf_(g);
-                        float silu = g * sig;
-                        float y1 = silu * u;
-                        dsp += a * y1;
-                        p.C2[(int64_t)row * p.N + n] = (bf16_t)(s * y1);
-                        float da = a * s;
-                        p.C[o] = (bf16_t)(da * (silu * (1.0f - sig) + sig) * u);
-                        p.C[o + p.N] = (bf16_t)(da * silu);
-                    }
-                }
-#pragma unroll
-                for (int o = 16; o > 0; o >>= 1) dsp += __shfl_xor(dsp, o, MTS_WAVE);
-                if (rok && fcol == 0) p.ds_part[(int64_t)row * p.np + ntile * T::WAVES_N + wn] = dsp;
+    rows_epilogue<T, EPI>(p, acc, smem, row0, rend, n0, wm, wn);
+}
+
+// ---------------------------------------------------------------------------
+// rows_gemm, ring pipeline.  Tiles go from global memory straight into LDS with
+// `buffer_load_dwordx4 ... lds` (16 bytes per lane, one KiB per wave instruction),
+// STAGES deep, so the loads of tiles k+1 .. k+STAGES-1 are in flight during the
+// MFMAs of tile k and no VGPRs or ds_write instructions are spent on staging.
+// The LDS image of a wave instruction is fixed (lane l lands at byte 16*l), so
+// the swizzle is applied on the global side: lane l fetches the chunk that
+// belongs at its landing slot.  Requires Kdim % BKS == 0.
+// ---------------------------------------------------------------------------
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int BKS_, int STAGES_>
+struct RingTile {
+    static constexpr int BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
+    static constexpr int BKS = BKS_, STAGES = STAGES_;
+    static constexpr int NWAVES = WAVES_M * WAVES_N;
+    static constexpr int NT = NWAVES * MTS_WAVE;
+    static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+    static constexpr int MF = WM / 32, NF = WN / 32;
+    static constexpr int CHUNKS = BKS / 8;          // 16-byte chunks per LDS row
+    static constexpr int RPI = MTS_WAVE / CHUNKS;   // rows covered by one wave instruction
+    static constexpr int A_INSTR = BM / RPI / NWAVES, B_INSTR = BN / RPI / NWAVES;
+    static constexpr int STAGE = (BM + BN) * BKS;
+    static constexpr int LDS_ELEMS = STAGES * STAGE;
+    static_assert(BKS == 32 || BKS == 64, "LDS rows are 64 or 128 bytes");
+    static_assert(WM % 32 == 0 && WN % 64 == 0, "wave tile must hold whole 32x32 fragments");
+    static_assert(A_INSTR * RPI * NWAVES == BM && B_INSTR * RPI * NWAVES == BN, "loader split");
+    static_assert(STAGES >= 2 && STAGES <= 4 && (A_INSTR + B_INSTR) * (STAGES - 2) <= 63, "vmcnt range");
+    static_assert(LDS_ELEMS * 2 <= 160 * 1024, "LDS capacity");
+};
+
+#define MTS_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+
+// s_waitcnt vmcnt(N) only (gfx9 encoding: vmcnt = simm16[15:14,3:0], expcnt [6:4], lgkmcnt [11:8])
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | 0x0F70);
+}
+
+template <class T, int EPI>
+__global__ __launch_bounds__(T::NT) void rows_gemm_ring_kernel(RowsParams p) {
+    constexpr int LDS_ELEMS = T::LDS_ELEMS > EpiShape<T, EPI>::ELEMS ? T::LDS_ELEMS : EpiShape<T, EPI>::ELEMS;
+    static_assert(LDS_ELEMS * 2 <= 160 * 1024, "LDS capacity");
+    __shared__ __attribute__((aligned(1024))) bf16_t smem[LDS_ELEMS];
+    constexpr bool SWIGLU = (EPI == EPI_SWIGLU);
+    constexpr int S = T::STAGES, L = T::A_INSTR + T::B_INSTR;
+
+    int e = 0, row0 = 0, rend = 0;
+    {
+        int tile = blockIdx.x, seen = 0;
+        bool found = false;
+        for (e = 0; e < p.E; ++e) {
+            int s0 = p.expert_start[e], s1 = p.expert_start[e + 1];
+            int nt = (s1 - s0 + T::BM - 1) / T::BM;
+            if (tile < seen + nt) {
+                row0 = s0 + (tile - seen) * T::BM;
+                rend = s1;
+                found = true;
+                break;
             }
+            seen += nt;
+        }
+        if (!found) return;
+    }
+    const int ntile = blockIdx.y;
+    const int n0 = ntile * (SWIGLU ? T::BN / 2 : T::BN);
+    const int wave = threadIdx.x / MTS_WAVE, lane = threadIdx.x % MTS_WAVE;
+    const int wm = wave / T::WAVES_N, wn = wave % T::WAVES_N;
+
+    const __amdgpu_buffer_rsrc_t rs_a = make_rsrc(p.A, p.a_rows * p.lda * 2);
+    const __amdgpu_buffer_rsrc_t rs_b =
+        make_rsrc(p.B + (int64_t)e * p.b_rows * p.Kdim, (int64_t)p.b_rows * p.Kdim * 2);
+    uint32_t voff_a[T::A_INSTR], voff_b[T::B_INSTR];
+    {
+        const int slot = lane % T::CHUNKS, rin = lane / T::CHUNKS;
+#pragma unroll
+        for (int j = 0; j < T::A_INSTR; ++j) {
+            const int tr = (wave * T::A_INSTR + j) * T::RPI + rin;   // row inside the A tile
+            const int chunk = slot ^ (T::CHUNKS == 8 ? (tr >> 1) & 7 : (tr >> 2) & 3);
+            const int row = row0 + tr;
+            const int lrow = row < rend ? row : rend - 1;
+            const int src = p.a_gather ? p.a_gather[lrow] : lrow;
+            voff_a[j] = row < rend ? ((uint32_t)src * (uint32_t)p.lda + chunk * 8) * 2u : kInvalid;
+        }
+#pragma unroll
+        for (int j = 0; j < T::B_INSTR; ++j) {
+            const int br = (wave * T::B_INSTR + j) * T::RPI + rin;   // row inside the B tile
+            const int chunk = slot ^ (T::CHUNKS == 8 ? (br >> 1) & 7 : (br >> 2) & 3);
+            int n, grow;
+            if (SWIGLU) {
+                n = n0 + br % (T::BN / 2);
+                grow = (br / (T::BN / 2)) * p.N + n;
+            } else {
+                n = n0 + br;
+                grow = n;
+            }
+            voff_b[j] = (n < p.N) ? ((uint32_t)grow * (uint32_t)p.Kdim + chunk * 8) * 2u : kInvalid;
         }
     }
+
+    auto issue = [&](int stage, int kt) {
+        bf16_t* sa = smem + stage * T::STAGE + wave * T::A_INSTR * 512;
+        bf16_t* sb = smem + stage * T::STAGE + T::BM * T::BKS + wave * T::B_INSTR * 512;
+        const int soff = kt * T::BKS * 2;
+#pragma unroll
+        for (int j = 0; j < T::A_INSTR; ++j)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, MTS_LDS_PTR(sa + j * 512), 16, (int)voff_a[j], soff, 0, 0);
+#pragma unroll
+        for (int j = 0; j < T::B_INSTR; ++j)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_b, MTS_LDS_PTR(sb + j * 512), 16, (int)voff_b[j], soff, 0, 0);
+    };
+
+    f32x16 acc[T::MF][T::NF];
+    zero_acc<T>(acc);
+
+    const int nk = p.Kdim / T::BKS;
+#pragma unroll
+    for (int s = 0; s < S - 1; ++s)
+        if (s < nk) issue(s, s);
+    int stage = 0;
+    for (int kt = 0; kt < nk; ++kt) {
+        // tile kt must have landed; up to S-2 younger tiles may stay in flight
+        const int younger = nk - 1 - kt;
+        if (S >= 4 && younger >= 2) wait_vmcnt<L * (S >= 4 ? 2 : 0)>();
+        else if (S >= 3 && younger >= 1) wait_vmcnt<L>();
+        else wait_vmcnt<0>();
+        __builtin_amdgcn_s_barrier();
+        // every wave is past the MFMAs of tile kt-1: its stage can be refilled
+        if (kt + S - 1 < nk) issue(stage == 0 ? S - 1 : stage - 1, kt + S - 1);
+        const bf16_t* cur = smem + stage * T::STAGE;
+        mma_tile<T, SWIGLU, T::BKS>(cur, cur + T::BM * T::BKS, wm, wn, acc);
+        stage = stage + 1 == S ? 0 : stage + 1;
+    }
+    __builtin_amdgcn_s_barrier();  // every wave is done reading the ring before it is reused
+    rows_epilogue<T, EPI>(p, acc, smem, row0, rend, n0, wm, wn);
 }
 
 // ---------------------------------------------------------------------------
 // dw_gemm
 // ---------------------------------------------------------------------------
 struct DwParams {
-    const bf16_t* P;  // rows -> M side, row-major [*, M]
-    int64_t ldp;
+    const bf16_t* P;  // rows -> M side, row-major [p_rows, M]
+    int64_t p_rows;
     const int32_t* p_gather;
-    const bf16_t* Q;  // rows -> N side, row-major [*, N]
-    int64_t ldq;
+    const bf16_t* Q;  // rows -> N side, row-major [q_rows, N]
+    int64_t q_rows;
     const int32_t* q_gather;
     int M, N;
+    int64_t TK;
     const int32_t* expert_start;
     void* C;  // [E][M][N], bf16 or f32
 };
 
 // Stages a [64 k][64 m] block per wave-item: lane = (kgrp = lane%8, mc = lane/8) loads
 // rows k = 8*kgrp+i, columns 8*mc..8*mc+7, transposes the 8x8 block in registers
-// and writes 8 rows of LDS (m-major, 16 bytes of k each).
+// and writes 8 rows of LDS (m-major, 16 bytes of k each).  Gathered operands take
+// their source rows from one index load per k-tile (lane j holds the index of row
+// j), fetched one tile ahead and spread with cross-lane reads.
 template <class T>
 struct MMajorLoader {
     static constexpr int ITEMS_A = T::BM / 64, ITEMS_B = T::BN / 64;
     static constexpr int ITEMS = ITEMS_A + ITEMS_B;
     static constexpr int PER_WAVE = (ITEMS + T::NWAVES - 1) / T::NWAVES;
+    __amdgpu_buffer_rsrc_t rs_p, rs_q, rs_gp, rs_gq;
+    bool gp, gq;
+    int tok_p, tok_q;  // source row of k-row `lane` of the tile that is fetched next
     u32x4 reg[PER_WAVE][8];
 
+    __device__ __forceinline__ void init(const DwParams& p) {
+        rs_p = make_rsrc(p.P, p.p_rows * p.M * 2);
+        rs_q = make_rsrc(p.Q, p.q_rows * p.N * 2);
+        gp = p.p_gather != nullptr;
+        gq = p.q_gather != nullptr;
+        rs_gp = make_rsrc(p.p_gather, gp ? p.TK * 4 : 0);
+        rs_gq = make_rsrc(p.q_gather, gq ? p.TK * 4 : 0);
+    }
+    // source rows for the tile starting at row r0 (rows past the end read index 0; they are masked later)
+    __device__ __forceinline__ void fetch_index(int r0) {
+        const int lane = threadIdx.x % MTS_WAVE;
+        tok_p = gp ? buf_load4(rs_gp, (uint32_t)(r0 + lane) * 4u) : r0 + lane;
+        tok_q = gq ? buf_load4(rs_gq, (uint32_t)(r0 + lane) * 4u) : r0 + lane;
+    }
     __device__ __forceinline__ void fetch(const DwParams& p, int m0, int n0, int r0, int rend) {
         const int wave = threadIdx.x / MTS_WAVE, lane = threadIdx.x % MTS_WAVE;
         const int kgrp = lane % 8, mc = lane / 8;
@@ -302,20 +581,16 @@ struct MMajorLoader {
             const int item = q * T::NWAVES + wave;
             if (item >= ITEMS) break;
             const bool isA = item < ITEMS_A;
-            const bf16_t* base = isA ? p.P : p.Q;
-            const int64_t ld = isA ? p.ldp : p.ldq;
-            const int32_t* gather = isA ? p.p_gather : p.q_gather;
             const int dim = isA ? p.M : p.N;
             const int c = (isA ? m0 + item * 64 : n0 + (item - ITEMS_A) * 64) + mc * 8;
+            const int tok = isA ? tok_p : tok_q;
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                const int r = r0 + kgrp * 8 + i;
-                u32x4 v = {0u, 0u, 0u, 0u};
-                if (r < rend && c < dim) {
-                    int64_t src = gather ? (int64_t)gather[r] : (int64_t)r;
-                    v = *reinterpret_cast<const u32x4*>(base + src * ld + c);
-                }
-                reg[q][i] = v;
+                const int kr = kgrp * 8 + i;
+                const int src = __shfl(tok, kr, MTS_WAVE);
+                const bool ok = (r0 + kr < rend) && (c < dim);
+                const uint32_t off = ok ? ((uint32_t)src * (uint32_t)dim + (uint32_t)c) * 2u : kInvalid;
+                reg[q][i] = buf_load16(isA ? rs_p : rs_q, off);
             }
         }
     }
@@ -328,8 +603,8 @@ struct MMajorLoader {
             const int item = q * T::NWAVES + wave;
             if (item >= ITEMS) break;
             const bool isA = item < ITEMS_A;
-            bf16_t* dst = (isA ? As + (item * 64) * LDS_LD : Bs + ((item - ITEMS_A) * 64) * LDS_LD) +
-                          (mc * 8) * LDS_LD + kgrp * 8;
+            bf16_t* dst = isA ? As : Bs;
+            const int rbase = (isA ? item : item - ITEMS_A) * 64 + mc * 8;
 #pragma unroll
             for (int md = 0; md < 4; ++md) {
                 u32x4 lo, hi;  // columns 2*md and 2*md+1 of the 8x8 block, k = 0..7
@@ -339,8 +614,8 @@ struct MMajorLoader {
                     lo[kp] = (a & 0xffffu) | (b << 16);
                     hi[kp] = (a >> 16) | (b & 0xffff0000u);
                 }
-                *reinterpret_cast<u32x4*>(dst + (2 * md) * LDS_LD) = lo;
-                *reinterpret_cast<u32x4*>(dst + (2 * md + 1) * LDS_LD) = hi;
+                *reinterpret_cast<u32x4*>(dst + lds_off(rbase + 2 * md, kgrp)) = lo;
+                *reinterpret_cast<u32x4*>(dst + lds_off(rbase + 2 * md + 1, kgrp)) = hi;
             }
         }
     }
@@ -356,27 +631,27 @@ __global__ __launch_bounds__(T::NT) void dw_gemm_kernel(DwParams p) {
     const int wave = threadIdx.x / MTS_WAVE, lane = threadIdx.x % MTS_WAVE;
     const int wm = wave / T::WAVES_N, wn = wave % T::WAVES_N;
     f32x16 acc[T::MF][T::NF];
-#pragma unroll
-    for (int mf = 0; mf < T::MF; ++mf)
-#pragma unroll
-        for (int nf = 0; nf < T::NF; ++nf)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) acc[mf][nf][i] = 0.f;
+    zero_acc<T>(acc);
 
-    constexpr int STAGE = (T::BM + T::BN) * LDS_LD;
-    constexpr int B_OFF = T::BM * LDS_LD;
+    constexpr int B_OFF = T::BM * BK;
     const int nk = (rend - rbeg + BK - 1) / BK;
     MMajorLoader<T> ld;
+    ld.init(p);
     if (nk > 0) {
+        ld.fetch_index(rbeg);
         ld.fetch(p, m0, n0, rbeg, rend);
+        ld.fetch_index(rbeg + BK);
         ld.commit(smem, smem + B_OFF);
     }
     __syncthreads();
     for (int kt = 0; kt < nk; ++kt) {
-        bf16_t* cur = smem + (kt & 1) * STAGE;
-        bf16_t* nxt = smem + ((kt & 1) ^ 1) * STAGE;
-        if (kt + 1 < nk) ld.fetch(p, m0, n0, rbeg + (kt + 1) * BK, rend);
-        mma_tile<T, false>(cur, cur + B_OFF, wm, wn, acc);
+        bf16_t* cur = smem + (kt & 1) * T::STAGE;
+        bf16_t* nxt = smem + ((kt & 1) ^ 1) * T::STAGE;
+        if (kt + 1 < nk) {
+            ld.fetch(p, m0, n0, rbeg + (kt + 1) * BK, rend);
+            ld.fetch_index(rbeg + (kt + 2) * BK);
+        }
+        mma_tile<T, false, BK, false>(cur, cur + B_OFF, wm, wn, acc);
         if (kt + 1 < nk) ld.commit(nxt, nxt + B_OFF);
         __syncthreads();
     }
@@ -399,21 +674,46 @@ __global__ __launch_bounds__(T::NT) void dw_gemm_kernel(DwParams p) {
 // ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
-typedef Tile<128, 128, 2, 2> TileS;
-typedef Tile<256, 256, 2, 2> TileL;
+typedef Tile<128, 128, 2, 2> Tile0;   // 4 waves of 64x64
+typedef Tile<256, 256, 2, 2> Tile1;   // 4 waves of 128x128
+typedef Tile<256, 256, 2, 4> Tile2;   // 8 waves of 128x64
+typedef Tile<256, 128, 2, 2> Tile3;   // 4 waves of 128x64
+typedef Tile<256, 128, 4, 2> Tile4;   // 8 waves of 64x64
 
-int tile_choice() {
-    static int choice = -1;
-    if (choice < 0) {
-        const char* s = getenv("MTS_GEMM_TILE");
-        choice = (s && atoi(s) == 256) ? 1 : 0;
+typedef RingTile<256, 256, 2, 2, 32, 4> Ring0;   // 4 waves of 128x128, 4 x 32 KiB stages
+typedef RingTile<256, 256, 2, 4, 32, 4> Ring1;   // 8 waves of 128x64
+typedef RingTile<256, 128, 2, 2, 64, 3> Ring2;   // 4 waves of 128x64, 3 x 48 KiB stages
+typedef RingTile<256, 128, 4, 2, 64, 3> Ring3;   // 8 waves of 64x64
+typedef RingTile<128, 128, 2, 2, 64, 4> Ring4;   // 4 waves of 64x64, 4 x 32 KiB stages
+typedef RingTile<256, 128, 2, 2, 32, 4> Ring5;   // 4 waves of 128x64, 4 x 24 KiB stages
+typedef RingTile<256, 128, 4, 2, 32, 4> Ring6;   // 8 waves of 64x64
+typedef RingTile<256, 256, 2, 4, 64, 2> Ring7;   // 8 waves of 128x64, 2 x 64 KiB stages
+
+enum Kind { K_GATEUP = 0, K_DOWN, K_DY1, K_DX, K_DW2, K_DW1, K_COUNT };
+const char* const kKindEnv[K_COUNT] = {"MTS_TILE_GATEUP", "MTS_TILE_DOWN", "MTS_TILE_DY1",
+                                       "MTS_TILE_DX",     "MTS_TILE_DW2",  "MTS_TILE_DW1"};
+const int kDefaultTile[K_COUNT] = {0, 0, 0, 0, 0, 0};
+
+// tile shape per GEMM; the environment overrides exist for tuning runs only
+int tile_choice(int kind) {
+    static int choice[K_COUNT] = {-1, -1, -1, -1, -1, -1};
+    if (choice[kind] < 0) {
+        int c = kDefaultTile[kind];
+        const char* s = getenv(kKindEnv[kind]);
+        if (!s) s = getenv("MTS_GEMM_TILE");
+        if (s) c = atoi(s);
+        choice[kind] = (c >= 0 && c <= 17) ? c : 0;
     }
-    return choice;
+    return choice[kind];
 }
 
 int check_common(int64_t TK, int E, int H, int I) {
     if (TK <= 0 || TK > 0x7fffffffLL || E < 1 || E > MTS_MAX_EXPERTS || H < 8 || I < 8 || H % 8 ||
         I % 8)
+        return MTS_ERR_SHAPE;
+    // every operand is addressed through a 32-bit buffer offset
+    if (TK * (int64_t)(2 * I) * 2 > kMaxOperandBytes || TK * (int64_t)H * 2 > kMaxOperandBytes ||
+        (int64_t)2 * I * H * 2 > kMaxOperandBytes)
         return MTS_ERR_SHAPE;
     return MTS_OK;
 }
@@ -433,9 +733,35 @@ int launch_rows(const RowsParams& p, int64_t TK, hipStream_t s) {
     return MTS_OK;
 }
 
+template <class T, int EPI>
+int launch_ring(const RowsParams& p, int64_t TK, hipStream_t s) {
+    const int per_block = (EPI == EPI_SWIGLU) ? T::BN / 2 : T::BN;
+    dim3 grid((unsigned)m_tiles<T>(TK, p.E), (unsigned)((p.N + per_block - 1) / per_block));
+    rows_gemm_ring_kernel<T, EPI><<<grid, T::NT, 0, s>>>(p);
+    MTS_CHECK_LAUNCH();
+    return MTS_OK;
+}
+
 template <int EPI>
-int launch_rows_any(const RowsParams& p, int64_t TK, hipStream_t s) {
-    return tile_choice() ? launch_rows<TileL, EPI>(p, TK, s) : launch_rows<TileS, EPI>(p, TK, s);
+int launch_rows_any(int kind, const RowsParams& p, int64_t TK, hipStream_t s) {
+    int choice = tile_choice(kind);
+    // ring kernels (choices 10..17) need whole k-tiles; other shapes use the staged kernel
+    if (choice >= 10 && p.Kdim % 64 != 0) choice = 0;
+    switch (choice) {
+        case 10: return launch_ring<Ring0, EPI>(p, TK, s);
+        case 11: return launch_ring<Ring1, EPI>(p, TK, s);
+        case 12: return launch_ring<Ring2, EPI>(p, TK, s);
+        case 13: return launch_ring<Ring3, EPI>(p, TK, s);
+        case 14: return launch_ring<Ring4, EPI>(p, TK, s);
+        case 15: return launch_ring<Ring5, EPI>(p, TK, s);
+        case 16: return launch_ring<Ring6, EPI>(p, TK, s);
+        case 17: return launch_ring<Ring7, EPI>(p, TK, s);
+        case 1: return launch_rows<Tile1, EPI>(p, TK, s);
+        case 2: return launch_rows<Tile2, EPI>(p, TK, s);
+        case 3: return launch_rows<Tile3, EPI>(p, TK, s);
+        case 4: return launch_rows<Tile4, EPI>(p, TK, s);
+        default: return launch_rows<Tile0, EPI>(p, TK, s);
+    }
 }
 
 template <class T>
@@ -448,16 +774,23 @@ int launch_dw(const DwParams& p, int E, int grad_dtype, hipStream_t s) {
     return MTS_OK;
 }
 
-int launch_dw_any(const DwParams& p, int E, int grad_dtype, hipStream_t s) {
-    return tile_choice() ? launch_dw<TileL>(p, E, grad_dtype, s) : launch_dw<TileS>(p, E, grad_dtype, s);
+int launch_dw_any(int kind, const DwParams& p, int E, int grad_dtype, hipStream_t s) {
+    int choice = tile_choice(kind);
+    if (choice > 4) choice = 0;
+    switch (choice) {
+        case 1: return launch_dw<Tile1>(p, E, grad_dtype, s);
+        case 2: return launch_dw<Tile2>(p, E, grad_dtype, s);
+        case 3: return launch_dw<Tile3>(p, E, grad_dtype, s);
+        case 4: return launch_dw<Tile4>(p, E, grad_dtype, s);
+        default: return launch_dw<Tile0>(p, E, grad_dtype, s);
+    }
 }
+
+int dy1_partials(int I) { return (I + 63) / 64; }
 
 }  // namespace
 
-extern "C" int mts_moe_ds_partials(int I) {
-    if (tile_choice()) return ((I + TileL::BN - 1) / TileL::BN) * TileL::WAVES_N;
-    return ((I + TileS::BN - 1) / TileS::BN) * TileS::WAVES_N;
-}
+extern "C" int mts_moe_ds_partials(int I) { return dy1_partials(I); }
 
 extern "C" int mts_moe_fwd_gateup_swiglu(const void* x, const void* w1, const int32_t* x_gather,
                                          const int32_t* expert_start, int64_t T, int K, int E,
@@ -470,11 +803,11 @@ extern "C" int mts_moe_fwd_gateup_swiglu(const void* x, const void* w1, const in
     if (rc) return rc;
     if (!mts_aligned16(x) || !mts_aligned16(w1)) return MTS_ERR_ALIGN;
     RowsParams p = {};
-    p.A = (const bf16_t*)x; p.lda = H; p.a_gather = x_gather;
-    p.B = (const bf16_t*)w1; p.b_expert_stride = (int64_t)2 * I * H;
+    p.A = (const bf16_t*)x; p.a_rows = T; p.lda = H; p.a_gather = x_gather;
+    p.B = (const bf16_t*)w1; p.b_rows = 2 * I;
     p.N = I; p.Kdim = H; p.expert_start = expert_start; p.E = E;
-    p.C = (bf16_t*)pre_act; p.C2 = (bf16_t*)post_act;
-    return launch_rows_any<EPI_SWIGLU>(p, T * K, (hipStream_t)stream);
+    p.C = (bf16_t*)pre_act; p.C2 = (bf16_t*)post_act; p.TK = T * K;
+    return launch_rows_any<EPI_SWIGLU>(K_GATEUP, p, T * K, (hipStream_t)stream);
 }
 
 extern "C" int mts_moe_fwd_down(const void* post_act, const void* w2, const int32_t* expert_start,
@@ -486,11 +819,11 @@ extern "C" int mts_moe_fwd_down(const void* post_act, const void* w2, const int3
     if (rc) return rc;
     if (!mts_aligned16(post_act) || !mts_aligned16(w2)) return MTS_ERR_ALIGN;
     RowsParams p = {};
-    p.A = (const bf16_t*)post_act; p.lda = I; p.a_gather = nullptr;
-    p.B = (const bf16_t*)w2; p.b_expert_stride = (int64_t)H * I;
+    p.A = (const bf16_t*)post_act; p.a_rows = TK; p.lda = I; p.a_gather = nullptr;
+    p.B = (const bf16_t*)w2; p.b_rows = H;
     p.N = H; p.Kdim = I; p.expert_start = expert_start; p.E = E;
-    p.C = (bf16_t*)y;
-    return launch_rows_any<EPI_PLAIN>(p, TK, (hipStream_t)stream);
+    p.C = (bf16_t*)y; p.TK = TK;
+    return launch_rows_any<EPI_PLAIN>(K_DOWN, p, TK, (hipStream_t)stream);
 }
 
 extern "C" int mts_moe_bwd_dy1(const void* d_out, const void* w2t, const void* pre_act,
@@ -507,13 +840,13 @@ extern "C" int mts_moe_bwd_dy1(const void* d_out, const void* w2t, const void* p
     if (rc) return rc;
     if (!mts_aligned16(d_out) || !mts_aligned16(w2t)) return MTS_ERR_ALIGN;
     RowsParams p = {};
-    p.A = (const bf16_t*)d_out; p.lda = H; p.a_gather = x_gather;
-    p.B = (const bf16_t*)w2t; p.b_expert_stride = (int64_t)H * I;
+    p.A = (const bf16_t*)d_out; p.a_rows = T; p.lda = H; p.a_gather = x_gather;
+    p.B = (const bf16_t*)w2t; p.b_rows = I;
     p.N = I; p.Kdim = H; p.expert_start = expert_start; p.E = E;
     p.C = (bf16_t*)d_pre_act; p.C2 = (bf16_t*)weighted_act;
     p.pre_act = (const bf16_t*)pre_act; p.route_w = (const bf16_t*)weights;
-    p.s_scatter = s_scatter; p.ds_part = ds_partial; p.np = mts_moe_ds_partials(I);
-    return launch_rows_any<EPI_DY1>(p, T * K, (hipStream_t)stream);
+    p.s_scatter = s_scatter; p.ds_part = ds_partial; p.np = mts_moe_ds_partials(I); p.TK = T * K;
+    return launch_rows_any<EPI_DY1>(K_DY1, p, T * K, (hipStream_t)stream);
 }
 
 extern "C" int mts_moe_bwd_dx(const void* d_pre_act, const void* w1t, const int32_t* expert_start,
@@ -525,11 +858,11 @@ extern "C" int mts_moe_bwd_dx(const void* d_pre_act, const void* w1t, const int3
     if (rc) return rc;
     if (!mts_aligned16(d_pre_act) || !mts_aligned16(w1t)) return MTS_ERR_ALIGN;
     RowsParams p = {};
-    p.A = (const bf16_t*)d_pre_act; p.lda = (int64_t)2 * I; p.a_gather = nullptr;
-    p.B = (const bf16_t*)w1t; p.b_expert_stride = (int64_t)2 * I * H;
+    p.A = (const bf16_t*)d_pre_act; p.a_rows = TK; p.lda = 2 * I; p.a_gather = nullptr;
+    p.B = (const bf16_t*)w1t; p.b_rows = H;
     p.N = H; p.Kdim = 2 * I; p.expert_start = expert_start; p.E = E;
-    p.C = (bf16_t*)dx_expanded;
-    return launch_rows_any<EPI_PLAIN>(p, TK, (hipStream_t)stream);
+    p.C = (bf16_t*)dx_expanded; p.TK = TK;
+    return launch_rows_any<EPI_PLAIN>(K_DX, p, TK, (hipStream_t)stream);
 }
 
 extern "C" int mts_moe_bwd_dw2(const void* d_out, const void* weighted_act, const int32_t* x_gather,
@@ -542,10 +875,10 @@ extern "C" int mts_moe_bwd_dw2(const void* d_out, const void* weighted_act, cons
     if (rc) return rc;
     if (!mts_aligned16(d_out) || !mts_aligned16(weighted_act)) return MTS_ERR_ALIGN;
     DwParams p = {};
-    p.P = (const bf16_t*)d_out; p.ldp = H; p.p_gather = x_gather;
-    p.Q = (const bf16_t*)weighted_act; p.ldq = I; p.q_gather = nullptr;
-    p.M = H; p.N = I; p.expert_start = expert_start; p.C = d_w2;
-    return launch_dw_any(p, E, grad_dtype, (hipStream_t)stream);
+    p.P = (const bf16_t*)d_out; p.p_rows = T; p.p_gather = x_gather;
+    p.Q = (const bf16_t*)weighted_act; p.q_rows = T * K; p.q_gather = nullptr;
+    p.M = H; p.N = I; p.TK = T * K; p.expert_start = expert_start; p.C = d_w2;
+    return launch_dw_any(K_DW2, p, E, grad_dtype, (hipStream_t)stream);
 }
 
 extern "C" int mts_moe_bwd_dw1(const void* d_pre_act, const void* x, const int32_t* x_gather,
@@ -558,8 +891,8 @@ extern "C" int mts_moe_bwd_dw1(const void* d_pre_act, const void* x, const int32
     if (rc) return rc;
     if (!mts_aligned16(d_pre_act) || !mts_aligned16(x)) return MTS_ERR_ALIGN;
     DwParams p = {};
-    p.P = (const bf16_t*)d_pre_act; p.ldp = (int64_t)2 * I; p.p_gather = nullptr;
-    p.Q = (const bf16_t*)x; p.ldq = H; p.q_gather = x_gather;
-    p.M = 2 * I; p.N = H; p.expert_start = expert_start; p.C = d_w1;
-    return launch_dw_any(p, E, grad_dtype, (hipStream_t)stream);
+    p.P = (const bf16_t*)d_pre_act; p.p_rows = T * K; p.p_gather = nullptr;
+    p.Q = (const bf16_t*)x; p.q_rows = T; p.q_gather = x_gather;
+    p.M = 2 * I; p.N = H; p.TK = T * K; p.expert_start = expert_start; p.C = d_w1;
+    return launch_dw_any(K_DW1, p, E, grad_dtype, (hipStream_t)stream);
 }
