@@ -81,6 +81,7 @@ struct RowsParams {
     float* ds_part;            // DY1: [TK][np]
     int np;
     int64_t TK;                // rows of every output
+    int n_tiles;               // column tiles per m-tile (set by the launcher)
 };
 
 // ---------------------------------------------------------------------------
@@ -110,21 +111,29 @@ struct KMajorLoader {
 
 // one MFMA sweep over a staged k-tile
 // (ROWLEN = k extent of the LDS rows: 64 with swizzle (row>>1)&7, 32 with (row>>2)&3)
-template <class T, bool SWIGLU, int ROWLEN = BK, bool WEIGHT_FIRST = true>
+struct NoHook {
+    __device__ __forceinline__ void operator()(int) const {}
+};
+
+// `hook(ks)` runs once per 16-wide k-step, between the fragment reads and the MFMAs.
+// Fragments are double buffered: the LDS reads of k-step ks+1 are issued before the
+// MFMAs of k-step ks, so that their latency is covered by the matrix pipe.
+template <class T, bool SWIGLU, int ROWLEN = BK, bool WEIGHT_FIRST = true, class Hook = NoHook>
 __device__ __forceinline__ void mma_tile(const bf16_t* As, const bf16_t* Bs, int wm, int wn,
-                                         f32x16 (&acc)[T::MF][T::NF]) {
+                                         f32x16 (&acc)[T::MF][T::NF], Hook hook = Hook()) {
     const int lane = threadIdx.x % MTS_WAVE;
     const int frow = lane % 32, kb = lane / 32;
     const int swz = ROWLEN == 64 ? (frow >> 1) & 7 : (frow >> 2) & 3;
     const bf16_t* a_base = As + (wm * T::WM + frow) * ROWLEN;
     const bf16_t* b_base = Bs + frow * ROWLEN;
-#pragma unroll
-    for (int ks = 0; ks < ROWLEN / 16; ++ks) {
+    constexpr int KSTEPS = ROWLEN / 16;
+    bf16x8 a[2][T::MF], b[2][T::NF];
+
+    auto load_frags = [&](int ks, int buf) {
         const int coff = ((ks * 2 + kb) ^ swz) << 3;
-        bf16x8 a[T::MF], b[T::NF];
 #pragma unroll
         for (int mf = 0; mf < T::MF; ++mf)
-            a[mf] = *reinterpret_cast<const bf16x8*>(a_base + mf * 32 * ROWLEN + coff);
+            a[buf][mf] = *reinterpret_cast<const bf16x8*>(a_base + mf * 32 * ROWLEN + coff);
 #pragma unroll
         for (int nf = 0; nf < T::NF; ++nf) {
             int brow;
@@ -134,15 +143,23 @@ __device__ __forceinline__ void mma_tile(const bf16_t* As, const bf16_t* Bs, int
             } else {
                 brow = wn * T::WN + nf * 32;
             }
-            b[nf] = *reinterpret_cast<const bf16x8*>(b_base + brow * ROWLEN + coff);
+            b[buf][nf] = *reinterpret_cast<const bf16x8*>(b_base + brow * ROWLEN + coff);
         }
+    };
+
+    load_frags(0, 0);
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+        const int cur = ks & 1;
+        if (ks + 1 < KSTEPS) load_frags(ks + 1, cur ^ 1);
+        hook(ks);
 #pragma unroll
         for (int mf = 0; mf < T::MF; ++mf)
 #pragma unroll
             for (int nf = 0; nf < T::NF; ++nf)
                 acc[mf][nf] = WEIGHT_FIRST
-                                  ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[nf], a[mf], acc[mf][nf], 0, 0, 0)
-                                  : __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[mf], b[nf], acc[mf][nf], 0, 0, 0);
+                                  ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[cur][nf], a[cur][mf], acc[mf][nf], 0, 0, 0)
+                                  : __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[cur][mf], b[cur][nf], acc[mf][nf], 0, 0, 0);
     }
 }
 
@@ -303,6 +320,36 @@ __device__ __forceinline__ void rows_epilogue(const RowsParams& p, f32x16 (&acc)
 }
 
 // ---------------------------------------------------------------------------
+// block -> tile mapping.  Workgroups are handed to the 8 XCDs round-robin
+// (block b runs on XCD b % 8) and every XCD has its own L2, so the blocks that
+// share operand panels are given to one XCD back to back: the j-th block of XCD x
+// computes m-tile x + 8*(j / n_tiles), n-tile j % n_tiles, i.e. all n-tiles of an
+// m-tile (same activation rows) and a few m-tiles of the same expert (same
+// weights) are in flight on one XCD at the same time.
+// ---------------------------------------------------------------------------
+constexpr int kXcds = 8;
+
+template <int BM>
+__device__ __forceinline__ bool locate_rows_tile(const RowsParams& p, int& e, int& row0, int& rend, int& ntile) {
+    const int b = blockIdx.x;
+    const int xcd = b % kXcds, j = b / kXcds;
+    const int tile = xcd + kXcds * (j / p.n_tiles);
+    ntile = j % p.n_tiles;
+    int seen = 0;
+    for (e = 0; e < p.E; ++e) {
+        const int s0 = p.expert_start[e], s1 = p.expert_start[e + 1];
+        const int nt = (s1 - s0 + BM - 1) / BM;
+        if (tile < seen + nt) {
+            row0 = s0 + (tile - seen) * BM;
+            rend = s1;
+            return true;
+        }
+        seen += nt;
+    }
+    return false;
+}
+
+// ---------------------------------------------------------------------------
 // rows_gemm
 // ---------------------------------------------------------------------------
 template <class T, int EPI>
@@ -312,25 +359,8 @@ __global__ __launch_bounds__(T::NT) void rows_gemm_kernel(RowsParams p) {
     __shared__ __attribute__((aligned(16))) bf16_t smem[LDS_ELEMS];
     constexpr bool SWIGLU = (EPI == EPI_SWIGLU);
 
-    // which expert does this m-tile belong to
-    int e = 0, row0 = 0, rend = 0;
-    {
-        int tile = blockIdx.x, seen = 0;
-        bool found = false;
-        for (e = 0; e < p.E; ++e) {
-            int s0 = p.expert_start[e], s1 = p.expert_start[e + 1];
-            int nt = (s1 - s0 + T::BM - 1) / T::BM;
-            if (tile < seen + nt) {
-                row0 = s0 + (tile - seen) * T::BM;
-                rend = s1;
-                found = true;
-                break;
-            }
-            seen += nt;
-        }
-        if (!found) return;
-    }
-    const int ntile = blockIdx.y;
+    int e, row0, rend, ntile;
+    if (!locate_rows_tile<T::BM>(p, e, row0, rend, ntile)) return;
     const int n0 = ntile * (SWIGLU ? T::BN / 2 : T::BN);  // first output column of this block
 
     KMajorLoader<T::BM, T::NT> la;
@@ -402,8 +432,9 @@ __global__ __launch_bounds__(T::NT) void rows_gemm_kernel(RowsParams p) {
 // the swizzle is applied on the global side: lane l fetches the chunk that
 // belongs at its landing slot.  Requires Kdim % BKS == 0.
 // ---------------------------------------------------------------------------
-template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int BKS_, int STAGES_>
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int BKS_, int STAGES_, int WAVES_PER_EU_ = 1>
 struct RingTile {
+    static constexpr int WAVES_PER_EU = WAVES_PER_EU_;  // register budget: 512 / WAVES_PER_EU per lane
     static constexpr int BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
     static constexpr int BKS = BKS_, STAGES = STAGES_;
     static constexpr int NWAVES = WAVES_M * WAVES_N;
@@ -431,31 +462,15 @@ __device__ __forceinline__ void wait_vmcnt() {
 }
 
 template <class T, int EPI>
-__global__ __launch_bounds__(T::NT) void rows_gemm_ring_kernel(RowsParams p) {
+__global__ __launch_bounds__(T::NT, T::WAVES_PER_EU) void rows_gemm_ring_kernel(RowsParams p) {
     constexpr int LDS_ELEMS = T::LDS_ELEMS > EpiShape<T, EPI>::ELEMS ? T::LDS_ELEMS : EpiShape<T, EPI>::ELEMS;
     static_assert(LDS_ELEMS * 2 <= 160 * 1024, "LDS capacity");
     __shared__ __attribute__((aligned(1024))) bf16_t smem[LDS_ELEMS];
     constexpr bool SWIGLU = (EPI == EPI_SWIGLU);
     constexpr int S = T::STAGES, L = T::A_INSTR + T::B_INSTR;
 
-    int e = 0, row0 = 0, rend = 0;
-    {
-        int tile = blockIdx.x, seen = 0;
-        bool found = false;
-        for (e = 0; e < p.E; ++e) {
-            int s0 = p.expert_start[e], s1 = p.expert_start[e + 1];
-            int nt = (s1 - s0 + T::BM - 1) / T::BM;
-            if (tile < seen + nt) {
-                row0 = s0 + (tile - seen) * T::BM;
-                rend = s1;
-                found = true;
-                break;
-            }
-            seen += nt;
-        }
-        if (!found) return;
-    }
-    const int ntile = blockIdx.y;
+    int e, row0, rend, ntile;
+    if (!locate_rows_tile<T::BM>(p, e, row0, rend, ntile)) return;
     const int n0 = ntile * (SWIGLU ? T::BN / 2 : T::BN);
     const int wave = threadIdx.x / MTS_WAVE, lane = threadIdx.x % MTS_WAVE;
     const int wm = wave / T::WAVES_N, wn = wave % T::WAVES_N;
@@ -491,16 +506,20 @@ __global__ __launch_bounds__(T::NT) void rows_gemm_ring_kernel(RowsParams p) {
         }
     }
 
-    auto issue = [&](int stage, int kt) {
+    // loads of one stage; `part` of `parts` selects a slice so that the refill of a
+    // stage can be spread over the k-steps of the tile that is being multiplied
+    auto issue = [&](int stage, int kt, int part, int parts) {
         bf16_t* sa = smem + stage * T::STAGE + wave * T::A_INSTR * 512;
         bf16_t* sb = smem + stage * T::STAGE + T::BM * T::BKS + wave * T::B_INSTR * 512;
         const int soff = kt * T::BKS * 2;
 #pragma unroll
         for (int j = 0; j < T::A_INSTR; ++j)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, MTS_LDS_PTR(sa + j * 512), 16, (int)voff_a[j], soff, 0, 0);
+            if (j % parts == part)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, MTS_LDS_PTR(sa + j * 512), 16, (int)voff_a[j], soff, 0, 0);
 #pragma unroll
         for (int j = 0; j < T::B_INSTR; ++j)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_b, MTS_LDS_PTR(sb + j * 512), 16, (int)voff_b[j], soff, 0, 0);
+            if ((j + T::A_INSTR) % parts == part)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_b, MTS_LDS_PTR(sb + j * 512), 16, (int)voff_b[j], soff, 0, 0);
     };
 
     f32x16 acc[T::MF][T::NF];
@@ -509,7 +528,7 @@ __global__ __launch_bounds__(T::NT) void rows_gemm_ring_kernel(RowsParams p) {
     const int nk = p.Kdim / T::BKS;
 #pragma unroll
     for (int s = 0; s < S - 1; ++s)
-        if (s < nk) issue(s, s);
+        if (s < nk) issue(s, s, 0, 1);
     int stage = 0;
     for (int kt = 0; kt < nk; ++kt) {
         // tile kt must have landed; up to S-2 younger tiles may stay in flight
@@ -519,9 +538,13 @@ __global__ __launch_bounds__(T::NT) void rows_gemm_ring_kernel(RowsParams p) {
         else wait_vmcnt<0>();
         __builtin_amdgcn_s_barrier();
         // every wave is past the MFMAs of tile kt-1: its stage can be refilled
-        if (kt + S - 1 < nk) issue(stage == 0 ? S - 1 : stage - 1, kt + S - 1);
+        const bool refill = kt + S - 1 < nk;
+        const int rstage = stage == 0 ? S - 1 : stage - 1;
         const bf16_t* cur = smem + stage * T::STAGE;
-        mma_tile<T, SWIGLU, T::BKS>(cur, cur + T::BM * T::BKS, wm, wn, acc);
+        constexpr int KSTEPS = T::BKS / 16;
+        mma_tile<T, SWIGLU, T::BKS>(cur, cur + T::BM * T::BKS, wm, wn, acc, [&](int ks) {
+            if (refill) issue(rstage, kt + S - 1, ks, KSTEPS);
+        });
         stage = stage + 1 == S ? 0 : stage + 1;
     }
     __builtin_amdgcn_s_barrier();  // every wave is done reading the ring before it is reused
@@ -542,6 +565,7 @@ struct DwParams {
     int64_t TK;
     const int32_t* expert_start;
     void* C;  // [E][M][N], bf16 or f32
+    int E, n_tiles, tiles_per_expert;  // set by the launcher
 };
 
 // Stages a [64 k][64 m] block per wave-item: lane = (kgrp = lane%8, mc = lane/8) loads
@@ -624,8 +648,13 @@ struct MMajorLoader {
 template <class T, typename OutT>
 __global__ __launch_bounds__(T::NT) void dw_gemm_kernel(DwParams p) {
     __shared__ __attribute__((aligned(16))) bf16_t smem[T::LDS_ELEMS];
-    const int e = blockIdx.z;
-    const int m0 = blockIdx.x * T::BM, n0 = blockIdx.y * T::BN;
+    // all tiles of one expert run on one XCD (block b -> XCD b % 8), so the expert's
+    // activation rows stream through that XCD's L2 once and are shared by its tiles
+    const int xcd = blockIdx.x % kXcds, j = blockIdx.x / kXcds;
+    const int e = xcd + kXcds * (j / p.tiles_per_expert);
+    if (e >= p.E) return;
+    const int tile = j % p.tiles_per_expert;
+    const int m0 = (tile / p.n_tiles) * T::BM, n0 = (tile % p.n_tiles) * T::BN;
     const int rbeg = p.expert_start[e], rend = p.expert_start[e + 1];
 
     const int wave = threadIdx.x / MTS_WAVE, lane = threadIdx.x % MTS_WAVE;
@@ -672,6 +701,206 @@ __global__ __launch_bounds__(T::NT) void dw_gemm_kernel(DwParams p) {
 }
 
 // ---------------------------------------------------------------------------
+// dw_gemm, ring pipeline.  Both operands are k-major in memory (a row of the
+// operand is one k), so tiles are brought into LDS as they are, [BKS k][BM or BN]
+// with `buffer_load ... lds`, and the MFMA fragments (8 consecutive k per lane)
+// are read with the transposing LDS load ds_read_b64_tr_b16: within a group of 16
+// lanes, lane s addresses 4 consecutive columns of row s/4 and lane l receives the
+// 4 rows of column l.  The 16-byte chunk index of a row is XOR-swizzled with
+// 4*(row % 4) so that the 4 rows x 2 column halves read by 32 lanes cover all banks.
+// Source rows of a gathered operand come from scalar loads of the row index, one
+// k-tile ahead.  Rows past the expert's end are fetched with an out-of-range
+// offset and arrive as zeros.
+// ---------------------------------------------------------------------------
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int BKS_, int STAGES_, int WAVES_PER_EU_ = 1>
+struct DwRingTile {
+    static constexpr int BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
+    static constexpr int BKS = BKS_, STAGES = STAGES_, WAVES_PER_EU = WAVES_PER_EU_;
+    static constexpr int NWAVES = WAVES_M * WAVES_N;
+    static constexpr int NT = NWAVES * MTS_WAVE;
+    static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+    static constexpr int MF = WM / 32, NF = WN / 32;
+    static constexpr int CPR_A = BM / 8, CPR_B = BN / 8;                    // 16-byte chunks per LDS row
+    static constexpr int RPI_A = MTS_WAVE / CPR_A, RPI_B = MTS_WAVE / CPR_B;  // rows per wave instruction
+    static constexpr int A_INSTR = BKS / RPI_A / NWAVES, B_INSTR = BKS / RPI_B / NWAVES;
+    static constexpr int STAGE = BKS * (BM + BN);
+    static constexpr int LDS_ELEMS = STAGES * STAGE;
+    static_assert(BM <= 512 && BN <= 512 && BM % 64 == 0 && BN % 64 == 0, "tile width");
+    static_assert(A_INSTR >= 1 && B_INSTR >= 1 && A_INSTR * RPI_A * NWAVES == BKS && B_INSTR * RPI_B * NWAVES == BKS,
+                  "loader split");
+    static_assert(STAGES >= 2 && STAGES <= 4 && (A_INSTR + B_INSTR) * (STAGES - 2) <= 63, "vmcnt range");
+    static_assert(LDS_ELEMS * 2 <= 160 * 1024, "LDS capacity");
+};
+
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+
+// 32 (m) x 16 (k) MFMA fragment out of a k-major LDS tile with row length ROWLEN
+template <int ROWLEN>
+__device__ __forceinline__ bf16x8 read_frag_tr(const bf16_t* tile, int krow0, int col0) {
+    const int lane = threadIdx.x % MTS_WAVE;
+    const int col = col0 + 16 * ((lane / 16) % 2) + 4 * (lane % 4);
+    const int chunk = col / 8, within = col % 8;
+    s16x4 h[2];
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+        const int row = krow0 + 8 * (lane / 32) + 4 * q + (lane % 16) / 4;
+        const bf16_t* src = tile + row * ROWLEN + ((chunk ^ ((row & 3) << 2)) << 3) + within;
+        h[q] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(src));
+    }
+    typedef __attribute__((ext_vector_type(8))) short s16x8;
+    s16x8 v = {h[0][0], h[0][1], h[0][2], h[0][3], h[1][0], h[1][1], h[1][2], h[1][3]};
+    return __builtin_bit_cast(bf16x8, v);
+}
+
+template <class T, typename OutT>
+__global__ __launch_bounds__(T::NT, T::WAVES_PER_EU) void dw_gemm_ring_kernel(DwParams p) {
+    __shared__ __attribute__((aligned(1024))) bf16_t smem[T::LDS_ELEMS];
+    constexpr int S = T::STAGES, L = T::A_INSTR + T::B_INSTR;
+    const int xcd = blockIdx.x % kXcds, jb = blockIdx.x / kXcds;
+    const int e = xcd + kXcds * (jb / p.tiles_per_expert);
+    if (e >= p.E) return;
+    const int tile = jb % p.tiles_per_expert;
+    const int m0 = (tile / p.n_tiles) * T::BM, n0 = (tile % p.n_tiles) * T::BN;
+    const int rbeg = p.expert_start[e], rend = p.expert_start[e + 1];
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / MTS_WAVE), lane = threadIdx.x % MTS_WAVE;
+    const int wm = wave / T::WAVES_N, wn = wave % T::WAVES_N;
+
+    const __amdgpu_buffer_rsrc_t rs_p = make_rsrc(p.P, p.p_rows * p.M * 2);
+    const __amdgpu_buffer_rsrc_t rs_q = make_rsrc(p.Q, p.q_rows * p.N * 2);
+    const int32_t* __restrict__ gp = p.p_gather;
+    const int32_t* __restrict__ gq = p.q_gather;
+    const int last_row = (int)p.TK - 1;
+
+    // column part of this lane's offsets (constant over the k loop)
+    uint32_t col_a[T::A_INSTR], col_b[T::B_INSTR];
+    int rin_a[T::A_INSTR], rin_b[T::B_INSTR];   // this lane's row inside the k-tile, per instruction
+#pragma unroll
+    for (int j = 0; j < T::A_INSTR; ++j) {
+        const int tr = (wave * T::A_INSTR + j) * T::RPI_A + lane / T::CPR_A;
+        const int c = m0 + (((lane % T::CPR_A) ^ ((tr & 3) << 2)) << 3);
+        rin_a[j] = tr;
+        col_a[j] = c < p.M ? (uint32_t)c * 2u : kInvalid;
+    }
+#pragma unroll
+    for (int j = 0; j < T::B_INSTR; ++j) {
+        const int tr = (wave * T::B_INSTR + j) * T::RPI_B + lane / T::CPR_B;
+        const int c = n0 + (((lane % T::CPR_B) ^ ((tr & 3) << 2)) << 3);
+        rin_b[j] = tr;
+        col_b[j] = c < p.N ? (uint32_t)c * 2u : kInvalid;
+    }
+
+    // source rows of the next tile to be fetched (scalar registers; row index clamped into the array)
+    int src_a[T::A_INSTR][T::RPI_A], src_b[T::B_INSTR][T::RPI_B];
+    auto fetch_index = [&](int r0) {
+#pragma unroll
+        for (int j = 0; j < T::A_INSTR; ++j)
+#pragma unroll
+            for (int q = 0; q < T::RPI_A; ++q) {
+                int r = r0 + (wave * T::A_INSTR + j) * T::RPI_A + q;
+                r = r < last_row ? r : last_row;
+                src_a[j][q] = gp ? gp[r] : r;
+            }
+#pragma unroll
+        for (int j = 0; j < T::B_INSTR; ++j)
+#pragma unroll
+            for (int q = 0; q < T::RPI_B; ++q) {
+                int r = r0 + (wave * T::B_INSTR + j) * T::RPI_B + q;
+                r = r < last_row ? r : last_row;
+                src_b[j][q] = gq ? gq[r] : r;
+            }
+    };
+    uint32_t voff_a[T::A_INSTR], voff_b[T::B_INSTR];
+    auto make_offsets = [&](int r0) {
+#pragma unroll
+        for (int j = 0; j < T::A_INSTR; ++j) {
+            int src = src_a[j][0];
+#pragma unroll
+            for (int q = 1; q < T::RPI_A; ++q) src = (lane / T::CPR_A == q) ? src_a[j][q] : src;
+            const bool ok = r0 + rin_a[j] < rend && col_a[j] != kInvalid;
+            voff_a[j] = ok ? (uint32_t)src * (uint32_t)p.M * 2u + col_a[j] : kInvalid;
+        }
+#pragma unroll
+        for (int j = 0; j < T::B_INSTR; ++j) {
+            int src = src_b[j][0];
+#pragma unroll
+            for (int q = 1; q < T::RPI_B; ++q) src = (lane / T::CPR_B == q) ? src_b[j][q] : src;
+            const bool ok = r0 + rin_b[j] < rend && col_b[j] != kInvalid;
+            voff_b[j] = ok ? (uint32_t)src * (uint32_t)p.N * 2u + col_b[j] : kInvalid;
+        }
+    };
+    auto issue = [&](int stage, int part, int parts) {
+        bf16_t* sa = smem + stage * T::STAGE + wave * T::A_INSTR * 512;
+        bf16_t* sb = smem + stage * T::STAGE + T::BKS * T::BM + wave * T::B_INSTR * 512;
+#pragma unroll
+        for (int j = 0; j < T::A_INSTR; ++j)
+            if (j % parts == part)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_p, MTS_LDS_PTR(sa + j * 512), 16, (int)voff_a[j], 0, 0, 0);
+#pragma unroll
+        for (int j = 0; j < T::B_INSTR; ++j)
+            if ((j + T::A_INSTR) % parts == part)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_q, MTS_LDS_PTR(sb + j * 512), 16, (int)voff_b[j], 0, 0, 0);
+    };
+
+    f32x16 acc[T::MF][T::NF];
+    zero_acc<T>(acc);
+
+    const int nk = (rend - rbeg + T::BKS - 1) / T::BKS;
+#pragma unroll
+    for (int s = 0; s < S - 1; ++s) {
+        if (s < nk) {
+            fetch_index(rbeg + s * T::BKS);
+            make_offsets(rbeg + s * T::BKS);
+            issue(s, 0, 1);
+        }
+    }
+    if (S - 1 < nk) fetch_index(rbeg + (S - 1) * T::BKS);
+    int stage = 0;
+    for (int kt = 0; kt < nk; ++kt) {
+        const int younger = nk - 1 - kt;
+        if (S >= 4 && younger >= 2) wait_vmcnt<L * (S >= 4 ? 2 : 0)>();
+        else if (S >= 3 && younger >= 1) wait_vmcnt<L>();
+        else wait_vmcnt<0>();
+        __builtin_amdgcn_s_barrier();
+        const bool refill = kt + S - 1 < nk;
+        const int rstage = stage == 0 ? S - 1 : stage - 1;
+        if (refill) make_offsets(rbeg + (kt + S - 1) * T::BKS);
+        if (kt + S < nk) fetch_index(rbeg + (kt + S) * T::BKS);
+        const bf16_t* As = smem + stage * T::STAGE;
+        const bf16_t* Bs = As + T::BKS * T::BM;
+        constexpr int KSTEPS = T::BKS / 16;
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+            bf16x8 a[T::MF], b[T::NF];
+#pragma unroll
+            for (int mf = 0; mf < T::MF; ++mf) a[mf] = read_frag_tr<T::BM>(As, ks * 16, wm * T::WM + mf * 32);
+#pragma unroll
+            for (int nf = 0; nf < T::NF; ++nf) b[nf] = read_frag_tr<T::BN>(Bs, ks * 16, wn * T::WN + nf * 32);
+            if (refill) issue(rstage, ks, KSTEPS);
+#pragma unroll
+            for (int mf = 0; mf < T::MF; ++mf)
+#pragma unroll
+                for (int nf = 0; nf < T::NF; ++nf)
+                    acc[mf][nf] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[mf], b[nf], acc[mf][nf], 0, 0, 0);
+        }
+        stage = stage + 1 == S ? 0 : stage + 1;
+    }
+
+    OutT* C = reinterpret_cast<OutT*>(p.C) + (int64_t)e * p.M * p.N;
+    const int fcol = lane % 32, frow4 = (lane / 32) * 4;
+#pragma unroll
+    for (int mf = 0; mf < T::MF; ++mf)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int m = m0 + wm * T::WM + mf * 32 + 8 * (i / 4) + frow4 + (i % 4);
+#pragma unroll
+            for (int nf = 0; nf < T::NF; ++nf) {
+                const int n = n0 + wn * T::WN + nf * 32 + fcol;
+                if (m < p.M && n < p.N) C[(int64_t)m * p.N + n] = (OutT)acc[mf][nf][i];
+            }
+        }
+}
+
+// ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
 typedef Tile<128, 128, 2, 2> Tile0;   // 4 waves of 64x64
@@ -681,18 +910,28 @@ typedef Tile<256, 128, 2, 2> Tile3;   // 4 waves of 128x64
 typedef Tile<256, 128, 4, 2> Tile4;   // 8 waves of 64x64
 
 typedef RingTile<256, 256, 2, 2, 32, 4> Ring0;   // 4 waves of 128x128, 4 x 32 KiB stages
-typedef RingTile<256, 256, 2, 4, 32, 4> Ring1;   // 8 waves of 128x64
+typedef RingTile<256, 256, 2, 4, 32, 4, 2> Ring1;   // 8 waves of 128x64
 typedef RingTile<256, 128, 2, 2, 64, 3> Ring2;   // 4 waves of 128x64, 3 x 48 KiB stages
-typedef RingTile<256, 128, 4, 2, 64, 3> Ring3;   // 8 waves of 64x64
+typedef RingTile<256, 128, 4, 2, 64, 3, 2> Ring3;   // 8 waves of 64x64
 typedef RingTile<128, 128, 2, 2, 64, 4> Ring4;   // 4 waves of 64x64, 4 x 32 KiB stages
 typedef RingTile<256, 128, 2, 2, 32, 4> Ring5;   // 4 waves of 128x64, 4 x 24 KiB stages
-typedef RingTile<256, 128, 4, 2, 32, 4> Ring6;   // 8 waves of 64x64
-typedef RingTile<256, 256, 2, 4, 64, 2> Ring7;   // 8 waves of 128x64, 2 x 64 KiB stages
+typedef RingTile<256, 128, 4, 2, 32, 4, 2> Ring6;   // 8 waves of 64x64
+typedef RingTile<256, 256, 2, 4, 64, 2, 2> Ring7;   // 8 waves of 128x64, 2 x 64 KiB stages
+typedef RingTile<256, 128, 2, 2, 32, 3, 2> Ring8;   // 4 waves of 128x64, 3 x 24 KiB stages, two blocks per CU
+typedef RingTile<128, 256, 2, 2, 32, 3, 2> Ring9;   // 4 waves of 64x128, two blocks per CU
+typedef RingTile<256, 256, 2, 2, 64, 2> Ring10;  // 4 waves of 128x128, 2 x 64 KiB stages
+
+typedef DwRingTile<128, 128, 2, 2, 32, 4, 2> DwRing0;   // 4 waves of 64x64, 4 x 16 KiB stages, two blocks per CU
+typedef DwRingTile<256, 256, 2, 4, 32, 4, 2> DwRing1;   // 8 waves of 128x64, 4 x 32 KiB stages
+typedef DwRingTile<256, 128, 2, 2, 32, 4, 2> DwRing2;   // 4 waves of 128x64, 4 x 24 KiB stages
+typedef DwRingTile<256, 256, 2, 2, 32, 4> DwRing3;      // 4 waves of 128x128
+typedef DwRingTile<128, 128, 2, 2, 64, 3, 2> DwRing4;   // 4 waves of 64x64, 3 x 32 KiB stages
+typedef DwRingTile<256, 128, 4, 2, 64, 3, 2> DwRing5;   // 8 waves of 64x64, 3 x 48 KiB stages
 
 enum Kind { K_GATEUP = 0, K_DOWN, K_DY1, K_DX, K_DW2, K_DW1, K_COUNT };
 const char* const kKindEnv[K_COUNT] = {"MTS_TILE_GATEUP", "MTS_TILE_DOWN", "MTS_TILE_DY1",
                                        "MTS_TILE_DX",     "MTS_TILE_DW2",  "MTS_TILE_DW1"};
-const int kDefaultTile[K_COUNT] = {0, 0, 0, 0, 0, 0};
+const int kDefaultTile[K_COUNT] = {18, 18, 18, 18, 0, 11};
 
 // tile shape per GEMM; the environment overrides exist for tuning runs only
 int tile_choice(int kind) {
@@ -702,7 +941,7 @@ int tile_choice(int kind) {
         const char* s = getenv(kKindEnv[kind]);
         if (!s) s = getenv("MTS_GEMM_TILE");
         if (s) c = atoi(s);
-        choice[kind] = (c >= 0 && c <= 17) ? c : 0;
+        choice[kind] = (c >= 0 && c <= 20) ? c : 0;
     }
     return choice[kind];
 }
@@ -725,18 +964,22 @@ int64_t m_tiles(int64_t TK, int E) {
 }
 
 template <class T, int EPI>
-int launch_rows(const RowsParams& p, int64_t TK, hipStream_t s) {
+int launch_rows(RowsParams p, int64_t TK, hipStream_t s) {
     const int per_block = (EPI == EPI_SWIGLU) ? T::BN / 2 : T::BN;
-    dim3 grid((unsigned)m_tiles<T>(TK, p.E), (unsigned)((p.N + per_block - 1) / per_block));
+    p.n_tiles = (p.N + per_block - 1) / per_block;
+    const int64_t m_groups = (m_tiles<T>(TK, p.E) + kXcds - 1) / kXcds;
+    dim3 grid((unsigned)(m_groups * kXcds * p.n_tiles));
     rows_gemm_kernel<T, EPI><<<grid, T::NT, 0, s>>>(p);
     MTS_CHECK_LAUNCH();
     return MTS_OK;
 }
 
 template <class T, int EPI>
-int launch_ring(const RowsParams& p, int64_t TK, hipStream_t s) {
+int launch_ring(RowsParams p, int64_t TK, hipStream_t s) {
     const int per_block = (EPI == EPI_SWIGLU) ? T::BN / 2 : T::BN;
-    dim3 grid((unsigned)m_tiles<T>(TK, p.E), (unsigned)((p.N + per_block - 1) / per_block));
+    p.n_tiles = (p.N + per_block - 1) / per_block;
+    const int64_t m_groups = (m_tiles<T>(TK, p.E) + kXcds - 1) / kXcds;
+    dim3 grid((unsigned)(m_groups * kXcds * p.n_tiles));
     rows_gemm_ring_kernel<T, EPI><<<grid, T::NT, 0, s>>>(p);
     MTS_CHECK_LAUNCH();
     return MTS_OK;
@@ -756,6 +999,9 @@ int launch_rows_any(int kind, const RowsParams& p, int64_t TK, hipStream_t s) {
         case 15: return launch_ring<Ring5, EPI>(p, TK, s);
         case 16: return launch_ring<Ring6, EPI>(p, TK, s);
         case 17: return launch_ring<Ring7, EPI>(p, TK, s);
+        case 18: return launch_ring<Ring8, EPI>(p, TK, s);
+        case 19: return launch_ring<Ring9, EPI>(p, TK, s);
+        case 20: return launch_ring<Ring10, EPI>(p, TK, s);
         case 1: return launch_rows<Tile1, EPI>(p, TK, s);
         case 2: return launch_rows<Tile2, EPI>(p, TK, s);
         case 3: return launch_rows<Tile3, EPI>(p, TK, s);
@@ -765,8 +1011,11 @@ int launch_rows_any(int kind, const RowsParams& p, int64_t TK, hipStream_t s) {
 }
 
 template <class T>
-int launch_dw(const DwParams& p, int E, int grad_dtype, hipStream_t s) {
-    dim3 grid((unsigned)((p.M + T::BM - 1) / T::BM), (unsigned)((p.N + T::BN - 1) / T::BN), (unsigned)E);
+int launch_dw(DwParams p, int E, int grad_dtype, hipStream_t s) {
+    p.E = E;
+    p.n_tiles = (p.N + T::BN - 1) / T::BN;
+    p.tiles_per_expert = ((p.M + T::BM - 1) / T::BM) * p.n_tiles;
+    dim3 grid((unsigned)(((E + kXcds - 1) / kXcds) * kXcds * p.tiles_per_expert));
     if (grad_dtype == MTS_BF16) dw_gemm_kernel<T, bf16_t><<<grid, T::NT, 0, s>>>(p);
     else if (grad_dtype == MTS_F32) dw_gemm_kernel<T, float><<<grid, T::NT, 0, s>>>(p);
     else return MTS_ERR_DTYPE;
@@ -774,8 +1023,30 @@ int launch_dw(const DwParams& p, int E, int grad_dtype, hipStream_t s) {
     return MTS_OK;
 }
 
+template <class T>
+int launch_dw_ring(DwParams p, int E, int grad_dtype, hipStream_t s) {
+    p.E = E;
+    p.n_tiles = (p.N + T::BN - 1) / T::BN;
+    p.tiles_per_expert = ((p.M + T::BM - 1) / T::BM) * p.n_tiles;
+    dim3 grid((unsigned)(((E + kXcds - 1) / kXcds) * kXcds * p.tiles_per_expert));
+    if (grad_dtype == MTS_BF16) dw_gemm_ring_kernel<T, bf16_t><<<grid, T::NT, 0, s>>>(p);
+    else if (grad_dtype == MTS_F32) dw_gemm_ring_kernel<T, float><<<grid, T::NT, 0, s>>>(p);
+    else return MTS_ERR_DTYPE;
+    MTS_CHECK_LAUNCH();
+    return MTS_OK;
+}
+
 int launch_dw_any(int kind, const DwParams& p, int E, int grad_dtype, hipStream_t s) {
     int choice = tile_choice(kind);
+    switch (choice) {
+        case 10: return launch_dw_ring<DwRing0>(p, E, grad_dtype, s);
+        case 11: return launch_dw_ring<DwRing1>(p, E, grad_dtype, s);
+        case 12: return launch_dw_ring<DwRing2>(p, E, grad_dtype, s);
+        case 13: return launch_dw_ring<DwRing3>(p, E, grad_dtype, s);
+        case 14: return launch_dw_ring<DwRing4>(p, E, grad_dtype, s);
+        case 15: return launch_dw_ring<DwRing5>(p, E, grad_dtype, s);
+        default: break;
+    }
     if (choice > 4) choice = 0;
     switch (choice) {
         case 1: return launch_dw<Tile1>(p, E, grad_dtype, s);
