@@ -7,17 +7,18 @@
 //       so the permuted activations are never materialised.
 //   dw_gemm    C[e][m, n] = sum_{r in e} P[row(r), m] * Q[row(r), n]
 //       used for dW1 and dW2; the reduction runs over the expert's rows, so both
-//       operands arrive "k-major" and are transposed 8x8 in registers on their
-//       way into LDS.
+//       operands arrive "k-major"; the staged pipeline transposes them 8x8 in
+//       registers on their way into LDS, the ring pipeline keeps them k-major in
+//       LDS and reads fragments with the transposing LDS load.
 //
 // Global reads are raw buffer loads: a lane that must contribute zeros (row past
 // the expert's end, column past N, k past K) is given an offset beyond the buffer
-// and the hardware returns 0, so the main loop has no divergent branches.
+// and the hardware returns 0, so the main loops have no divergent branches.
 //
-// LDS tiles are [rows][64] bf16 with the 16-byte chunk index XOR-swizzled by
-// (row >> 1) & 7: the 16-byte MFMA fragment reads of 16 consecutive rows, and the
-// row-contiguous tile writes, are both bank-conflict free without padding.  Two
-// stages: the global loads of tile k+1 are in flight during the MFMAs of tile k.
+// Each family has two pipelines.  "staged": global -> VGPR -> LDS, two stages, any K
+// that is a multiple of 8.  "ring": global -> LDS directly (buffer_load ... lds),
+// two to four stages, whole k-tiles only.  LDS rows are XOR-swizzled instead of
+// padded, so fragment reads and tile writes are both bank-conflict free.
 //
 // MFMA 32x32x16 register layout used below (lane l):
 //   A/B fragment: row (l % 32) of the 32-row operand, k = 8*(l/32) .. 8*(l/32)+7
@@ -903,35 +904,21 @@ __global__ __launch_bounds__(T::NT, T::WAVES_PER_EU) void dw_gemm_ring_kernel(Dw
 // ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
-typedef Tile<128, 128, 2, 2> Tile0;   // 4 waves of 64x64
-typedef Tile<256, 256, 2, 2> Tile1;   // 4 waves of 128x128
-typedef Tile<256, 256, 2, 4> Tile2;   // 8 waves of 128x64
-typedef Tile<256, 128, 2, 2> Tile3;   // 4 waves of 128x64
-typedef Tile<256, 128, 4, 2> Tile4;   // 8 waves of 64x64
-
-typedef RingTile<256, 256, 2, 2, 32, 4> Ring0;   // 4 waves of 128x128, 4 x 32 KiB stages
-typedef RingTile<256, 256, 2, 4, 32, 4, 2> Ring1;   // 8 waves of 128x64
-typedef RingTile<256, 128, 2, 2, 64, 3> Ring2;   // 4 waves of 128x64, 3 x 48 KiB stages
-typedef RingTile<256, 128, 4, 2, 64, 3, 2> Ring3;   // 8 waves of 64x64
-typedef RingTile<128, 128, 2, 2, 64, 4> Ring4;   // 4 waves of 64x64, 4 x 32 KiB stages
-typedef RingTile<256, 128, 2, 2, 32, 4> Ring5;   // 4 waves of 128x64, 4 x 24 KiB stages
-typedef RingTile<256, 128, 4, 2, 32, 4, 2> Ring6;   // 8 waves of 64x64
-typedef RingTile<256, 256, 2, 4, 64, 2, 2> Ring7;   // 8 waves of 128x64, 2 x 64 KiB stages
-typedef RingTile<256, 128, 2, 2, 32, 3, 2> Ring8;   // 4 waves of 128x64, 3 x 24 KiB stages, two blocks per CU
-typedef RingTile<128, 256, 2, 2, 32, 3, 2> Ring9;   // 4 waves of 64x128, two blocks per CU
-typedef RingTile<256, 256, 2, 2, 64, 2> Ring10;  // 4 waves of 128x128, 2 x 64 KiB stages
-
-typedef DwRingTile<128, 128, 2, 2, 32, 4, 2> DwRing0;   // 4 waves of 64x64, 4 x 16 KiB stages, two blocks per CU
-typedef DwRingTile<256, 256, 2, 4, 32, 4, 2> DwRing1;   // 8 waves of 128x64, 4 x 32 KiB stages
-typedef DwRingTile<256, 128, 2, 2, 32, 4, 2> DwRing2;   // 4 waves of 128x64, 4 x 24 KiB stages
-typedef DwRingTile<256, 256, 2, 2, 32, 4> DwRing3;      // 4 waves of 128x128
-typedef DwRingTile<128, 128, 2, 2, 64, 3, 2> DwRing4;   // 4 waves of 64x64, 3 x 32 KiB stages
-typedef DwRingTile<256, 128, 4, 2, 64, 3, 2> DwRing5;   // 8 waves of 64x64, 3 x 48 KiB stages
+typedef Tile<128, 128, 2, 2> StagedSmall;                 // 4 waves of 64x64, any K that is a multiple of 8
+typedef Tile<256, 256, 2, 4> StagedLarge;                 // 8 waves of 128x64
+typedef RingTile<256, 128, 2, 2, 32, 3, 2> RingTwoPerCu;  // 4 waves of 128x64, 3 x 24 KiB stages, two blocks per CU
+typedef RingTile<256, 256, 2, 4, 64, 2, 2> RingLarge;     // 8 waves of 128x64, 2 x 64 KiB stages
+typedef RingTile<256, 256, 2, 4, 32, 4, 2> RingDeep;      // 8 waves of 128x64, 4 x 32 KiB stages
+typedef DwRingTile<256, 256, 2, 4, 32, 4, 2> DwRingLarge; // 8 waves of 128x64, 4 x 32 KiB stages
+typedef DwRingTile<256, 256, 2, 2, 32, 4> DwRingWide;     // 4 waves of 128x128
 
 enum Kind { K_GATEUP = 0, K_DOWN, K_DY1, K_DX, K_DW2, K_DW1, K_COUNT };
 const char* const kKindEnv[K_COUNT] = {"MTS_TILE_GATEUP", "MTS_TILE_DOWN", "MTS_TILE_DY1",
                                        "MTS_TILE_DX",     "MTS_TILE_DW2",  "MTS_TILE_DW1"};
-const int kDefaultTile[K_COUNT] = {18, 18, 18, 18, 0, 11};
+// rows_gemm: 0 StagedSmall, 1 RingTwoPerCu, 2 RingLarge, 3 RingDeep
+// dw_gemm:   0 StagedSmall, 1 StagedLarge,  2 DwRingLarge, 3 DwRingWide
+// Defaults are the fastest measured on the 24576-token, 768/1024, 8-expert layer.
+const int kDefaultTile[K_COUNT] = {1, 1, 1, 1, 0, 2};
 
 // tile shape per GEMM; the environment overrides exist for tuning runs only
 int tile_choice(int kind) {
@@ -939,9 +926,8 @@ int tile_choice(int kind) {
     if (choice[kind] < 0) {
         int c = kDefaultTile[kind];
         const char* s = getenv(kKindEnv[kind]);
-        if (!s) s = getenv("MTS_GEMM_TILE");
         if (s) c = atoi(s);
-        choice[kind] = (c >= 0 && c <= 20) ? c : 0;
+        choice[kind] = (c >= 0 && c <= 3) ? c : kDefaultTile[kind];
     }
     return choice[kind];
 }
@@ -988,25 +974,13 @@ int launch_ring(RowsParams p, int64_t TK, hipStream_t s) {
 template <int EPI>
 int launch_rows_any(int kind, const RowsParams& p, int64_t TK, hipStream_t s) {
     int choice = tile_choice(kind);
-    // ring kernels (choices 10..17) need whole k-tiles; other shapes use the staged kernel
-    if (choice >= 10 && p.Kdim % 64 != 0) choice = 0;
+    // the ring kernels need whole k-tiles; other shapes use the staged kernel
+    if (choice >= 1 && p.Kdim % 64 != 0) choice = 0;
     switch (choice) {
-        case 10: return launch_ring<Ring0, EPI>(p, TK, s);
-        case 11: return launch_ring<Ring1, EPI>(p, TK, s);
-        case 12: return launch_ring<Ring2, EPI>(p, TK, s);
-        case 13: return launch_ring<Ring3, EPI>(p, TK, s);
-        case 14: return launch_ring<Ring4, EPI>(p, TK, s);
-        case 15: return launch_ring<Ring5, EPI>(p, TK, s);
-        case 16: return launch_ring<Ring6, EPI>(p, TK, s);
-        case 17: return launch_ring<Ring7, EPI>(p, TK, s);
-        case 18: return launch_ring<Ring8, EPI>(p, TK, s);
-        case 19: return launch_ring<Ring9, EPI>(p, TK, s);
-        case 20: return launch_ring<Ring10, EPI>(p, TK, s);
-        case 1: return launch_rows<Tile1, EPI>(p, TK, s);
-        case 2: return launch_rows<Tile2, EPI>(p, TK, s);
-        case 3: return launch_rows<Tile3, EPI>(p, TK, s);
-        case 4: return launch_rows<Tile4, EPI>(p, TK, s);
-        default: return launch_rows<Tile0, EPI>(p, TK, s);
+        case 1: return launch_ring<RingTwoPerCu, EPI>(p, TK, s);
+        case 2: return launch_ring<RingLarge, EPI>(p, TK, s);
+        case 3: return launch_ring<RingDeep, EPI>(p, TK, s);
+        default: return launch_rows<StagedSmall, EPI>(p, TK, s);
     }
 }
 
@@ -1037,23 +1011,11 @@ int launch_dw_ring(DwParams p, int E, int grad_dtype, hipStream_t s) {
 }
 
 int launch_dw_any(int kind, const DwParams& p, int E, int grad_dtype, hipStream_t s) {
-    int choice = tile_choice(kind);
-    switch (choice) {
-        case 10: return launch_dw_ring<DwRing0>(p, E, grad_dtype, s);
-        case 11: return launch_dw_ring<DwRing1>(p, E, grad_dtype, s);
-        case 12: return launch_dw_ring<DwRing2>(p, E, grad_dtype, s);
-        case 13: return launch_dw_ring<DwRing3>(p, E, grad_dtype, s);
-        case 14: return launch_dw_ring<DwRing4>(p, E, grad_dtype, s);
-        case 15: return launch_dw_ring<DwRing5>(p, E, grad_dtype, s);
-        default: break;
-    }
-    if (choice > 4) choice = 0;
-    switch (choice) {
-        case 1: return launch_dw<Tile1>(p, E, grad_dtype, s);
-        case 2: return launch_dw<Tile2>(p, E, grad_dtype, s);
-        case 3: return launch_dw<Tile3>(p, E, grad_dtype, s);
-        case 4: return launch_dw<Tile4>(p, E, grad_dtype, s);
-        default: return launch_dw<Tile0>(p, E, grad_dtype, s);
+    switch (tile_choice(kind)) {
+        case 1: return launch_dw<StagedLarge>(p, E, grad_dtype, s);
+        case 2: return launch_dw_ring<DwRingLarge>(p, E, grad_dtype, s);
+        case 3: return launch_dw_ring<DwRingWide>(p, E, grad_dtype, s);
+        default: return launch_dw<StagedSmall>(p, E, grad_dtype, s);
     }
 }
 

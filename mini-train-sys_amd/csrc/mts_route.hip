@@ -15,7 +15,8 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / MTS_WAVE;
-constexpr int kChunk = 1024;  // entries per wave
+constexpr int kChunk = 256;   // entries per wave
+constexpr int kSteps = kChunk / MTS_WAVE;
 
 // Expert ids outside [0,E) are a caller error; they are clamped so that no
 // address derived from them can leave the output arrays.
@@ -126,10 +127,17 @@ __global__ __launch_bounds__(kThreads) void route_scatter_kernel(
     volatile int32_t* next = lds + wave * E;
     for (int e = lane; e < E; e += MTS_WAVE) next[e] = expert_start[e] + cnt[chunk * E + e];
     const uint64_t lt = lanemask_lt();
-    for (int i = 0; i < kChunk; i += MTS_WAVE) {
-        int64_t n = base + i + lane;
-        bool valid = n < TK;
-        int e = valid ? clamp_expert(idx[n], E) : -1;
+    int ev[kSteps];
+#pragma unroll
+    for (int s = 0; s < kSteps; ++s) {  // all of the chunk's loads are in flight together
+        const int64_t n = base + s * MTS_WAVE + lane;
+        ev[s] = n < TK ? clamp_expert(idx[n], E) : -1;
+    }
+#pragma unroll
+    for (int s = 0; s < kSteps; ++s) {
+        const int64_t n = base + s * MTS_WAVE + lane;
+        const bool valid = n < TK;
+        const int e = ev[s];
         int pos = 0;
         uint64_t todo = __ballot(valid);
         while (todo) {

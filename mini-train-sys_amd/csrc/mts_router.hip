@@ -182,16 +182,21 @@ __global__ __launch_bounds__(kThreads) void router_fwd_kernel(
     }
 }
 
+// One block: wave w reduces columns w, w+4, ...; lanes stride over the per-block
+// partials and the lane sums meet in a fixed shuffle tree (bit-stable).
 __global__ __launch_bounds__(kThreads) void router_stats_kernel(
     const float* __restrict__ partial, int nblocks, int E, float inv_t,
     float* __restrict__ prob_mean, float* __restrict__ z_loss, float* __restrict__ entropy) {
-    for (int i = threadIdx.x; i < E + 2; i += kThreads) {
+    const int wave = threadIdx.x / MTS_WAVE, lane = threadIdx.x % MTS_WAVE;
+    for (int i = wave; i < E + 2; i += kThreads / MTS_WAVE) {
         float v = 0.f;
-        for (int b = 0; b < nblocks; ++b) v += partial[(int64_t)b * (E + 2) + i];
-        v *= inv_t;
-        if (i < E) prob_mean[i] = v;
-        else if (i == E) z_loss[0] = v;
-        else entropy[0] = v;
+        for (int b = lane; b < nblocks; b += MTS_WAVE) v += partial[(int64_t)b * (E + 2) + i];
+        v = wave_sum(v) * inv_t;
+        if (lane == 0) {
+            if (i < E) prob_mean[i] = v;
+            else if (i == E) z_loss[0] = v;
+            else entropy[0] = v;
+        }
     }
 }
 
