@@ -37,6 +37,14 @@ import torch.nn.functional as F
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
+# HBM-side bytes per launch (fetch + write) of the GEMM and combine stages at this workload, from the
+# two rocprofv3 counter runs summarised in profiles/moe_layer_24x1024_hbm_traffic.txt (FETCH_SIZE
+# scaled by 2.0, WRITE_SIZE by 1.0 against a plain copy kernel of known size).  Not measured live.
+MEASURED_TRAFFIC_BYTES = {
+    "fwd_gateup_swiglu": 787.0e6, "fwd_down": 434.8e6, "bwd_dx": 434.8e6, "bwd_dy1": 732.0e6,
+    "bwd_dw2": 224.6e6, "bwd_dw1": 302.5e6, "combine": 114.8e6, "dx_combine": 114.8e6,
+}
+
 WORKLOAD = dict(name="moe_layer_24x1024_d768_e8_top2_ff1024_bf16", seed=1, T=24576, H=768, E=8, K=2, I=1024)
 
 
@@ -208,6 +216,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-breakdown", action="store_true")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run a plain 256 MiB -> 256 MiB elementwise copy (the known-size kernel that "
+                         "FETCH_SIZE / WRITE_SIZE counter runs are scaled by)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -247,7 +258,8 @@ def main():
         result["kernels"] = rows
         dom = max(rows, key=lambda r: r["avg_ms"])
         result["roofline"] = {"kernel": dom["stage"], "bound": dom["bound"], "achieved": dom["achieved"], "peak": dom["peak"],
-                              "unit": dom["unit"], "frac": dom["frac"], "traffic": None}
+                              "unit": dom["unit"], "frac": dom["frac"], "traffic": MEASURED_TRAFFIC_BYTES.get(dom["stage"]),
+                              "algorithmic": dom["work"], "avg_ms": dom["avg_ms"]}
         gemm_rows = [r for r in rows if r["bound"] == "mfma"]
         g_ms = sum(r["avg_ms"] for r in gemm_rows)
         g_ach = sum(r["work"] for r in gemm_rows) / (g_ms * 1e-3) / 1e12
@@ -259,6 +271,13 @@ def main():
         result["combine_roofline"] = {"bound": "hbm", "achieved": round(c_ach, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                                       "frac": round(c_ach / PEAK_HBM_GBS, 4), "sum_ms": round(c_ms, 4)}
         result["kernel_sum_ms"] = round(sum(r["avg_ms"] for r in rows), 4)
+    if args.copy_probe:
+        src = torch.ones(64 * 2**20, dtype=torch.float32, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.mul(src, 1.0, out=dst)
+        torch.cuda.synchronize()
+        result["copy_probe_bytes_each_way"] = src.numel() * 4
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline()
     print(json.dumps(result))
