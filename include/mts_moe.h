@@ -81,24 +81,26 @@ int mts_moe_route(const int32_t* top_k_index, int64_t T, int K, int E, int block
                   int64_t workspace_bytes, void* stream);
 
 /* ---- weight staging -----------------------------------------------------
- * src [E,R,C] of src_dtype -> dst bf16, [E,R,C] (transpose=0) or [E,C,R]
+ * src [E,R,C] of src_dtype -> dst of dst_dtype, [E,R,C] (transpose=0) or [E,C,R]
  * (transpose=1).  Stands in for the in-kernel weight casts of the reference
  * (fused_moe_kernels.py:343,351) and stages the transposed operands of the
- * backward GEMMs.                                                            */
-int mts_moe_stage_weights(const void* src, int src_dtype, void* dst_bf16, int E, int64_t R,
-                          int64_t C, int transpose, void* stream);
+ * backward GEMMs.  The GEMM entry points below take their weight operands in the
+ * activation dtype: bf16 weights with bf16 activations, fp32 with fp32.       */
+int mts_moe_stage_weights(const void* src, int src_dtype, void* dst, int dst_dtype, int E,
+                          int64_t R, int64_t C, int transpose, void* stream);
 
 /* ---- forward ------------------------------------------------------------
  * Replaces _fused_up_proj_swiglu_kernel (fused_moe_kernels.py:264-367):
  * for every row r (token x_gather[r], expert e): [g;u] = W1[e] x ; a = silu(g)*u.
- * x [T,H], w1 [E,2I,H] bf16, pre_act [TK,2I], post_act [TK,I] (act_dtype).     */
+ * x [T,H], w1 [E,2I,H], pre_act [TK,2I], post_act [TK,I], all of act_dtype
+ * (MTS_BF16: MFMA kernels, H and I multiples of 8; MTS_F32: plain fp32 kernels). */
 int mts_moe_fwd_gateup_swiglu(const void* x, const void* w1, const int32_t* x_gather,
                               const int32_t* expert_start, int64_t T, int K, int E, int H,
                               int I, int act_dtype, void* pre_act, void* post_act,
                               void* stream);
 
 /* Replaces _fused_down_proj_kernel (fused_moe_kernels.py:369-437):
- * y[r] = W2[e] a[r];  post_act [TK,I], w2 [E,H,I] bf16 -> y [TK,H].           */
+ * y[r] = W2[e] a[r];  post_act [TK,I], w2 [E,H,I] -> y [TK,H].                */
 int mts_moe_fwd_down(const void* post_act, const void* w2, const int32_t* expert_start,
                      int64_t TK, int E, int H, int I, int act_dtype, void* y, void* stream);
 
@@ -111,7 +113,7 @@ int mts_moe_combine(const void* y, const void* weights, const int32_t* s_reverse
 /* ---- backward -----------------------------------------------------------
  * Replaces _moe_bwd_down_proj_kernel (fused_moe_kernels.py:500-600):
  * A = W2[e]^T dO[t];  dS = <A,a>;  weighted_act = s*a;  [dg;du] = d(s*A)/d[g;u].
- * w2t is W2 staged as [E,I,H] bf16.  ds_partial is [TK, mts_moe_ds_partials(I)]
+ * w2t is W2 staged as [E,I,H].  ds_partial is [TK, mts_moe_ds_partials(I)]
  * f32 scratch reduced by mts_moe_bwd_ds (fixed order, no atomics).            */
 int mts_moe_ds_partials(int I);
 int mts_moe_bwd_dy1(const void* d_out, const void* w2t, const void* pre_act,
@@ -126,7 +128,7 @@ int mts_moe_bwd_ds(const float* ds_partial, const int32_t* s_reverse, int64_t TK
                    int act_dtype, void* d_weights, void* stream);
 
 /* Replaces _moe_bwd_dX_expanded_kernel (fused_moe_kernels.py:674-756):
- * dx_expanded[r] = W1[e]^T [dg;du][r];  w1t is W1 staged as [E,H,2I] bf16.
+ * dx_expanded[r] = W1[e]^T [dg;du][r];  w1t is W1 staged as [E,H,2I].
  * The per-token sum is mts_moe_combine with weights == NULL.                 */
 int mts_moe_bwd_dx(const void* d_pre_act, const void* w1t, const int32_t* expert_start,
                    int64_t TK, int E, int H, int I, int act_dtype, void* dx_expanded,

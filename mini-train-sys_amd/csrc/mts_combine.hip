@@ -73,20 +73,20 @@ __global__ __launch_bounds__(kThreads) void ds_reduce_kernel(const float* __rest
 
 // ---- weight staging --------------------------------------------------------
 // 64x64 tiles through LDS; reads and writes are both row-contiguous.
-template <typename SrcT, bool TRANSPOSE>
+template <typename SrcT, typename DstT, bool TRANSPOSE>
 __global__ __launch_bounds__(kThreads) void stage_weights_kernel(const SrcT* __restrict__ src,
-                                                                 bf16_t* __restrict__ dst,
+                                                                 DstT* __restrict__ dst,
                                                                  int64_t R, int64_t C) {
-    __shared__ bf16_t tile[64][64 + 2];
+    __shared__ DstT tile[64][64 + 2];
     const int64_t e = blockIdx.z;
     const int64_t r0 = (int64_t)blockIdx.y * 64, c0 = (int64_t)blockIdx.x * 64;
     const SrcT* s = src + e * R * C;
-    bf16_t* d = dst + e * R * C;
+    DstT* d = dst + e * R * C;
     const int tx = threadIdx.x % 64, ty = threadIdx.x / 64;
     for (int i = ty; i < 64; i += kThreads / 64) {
         int64_t r = r0 + i, c = c0 + tx;
         if (r < R && c < C) {
-            bf16_t v = (bf16_t)(float)s[r * C + c];
+            DstT v = (DstT)(float)s[r * C + c];
             if (TRANSPOSE) tile[i][tx] = v;
             else d[r * C + c] = v;
         }
@@ -146,23 +146,24 @@ extern "C" int mts_moe_bwd_ds(const float* ds_partial, const int32_t* s_reverse,
     return MTS_OK;
 }
 
-extern "C" int mts_moe_stage_weights(const void* src, int src_dtype, void* dst_bf16, int E,
+template <typename SrcT, typename DstT>
+void launch_stage(const void* src, void* dst, dim3 grid, int64_t R, int64_t C, int transpose, hipStream_t s) {
+    if (transpose) stage_weights_kernel<SrcT, DstT, true><<<grid, kThreads, 0, s>>>((const SrcT*)src, (DstT*)dst, R, C);
+    else stage_weights_kernel<SrcT, DstT, false><<<grid, kThreads, 0, s>>>((const SrcT*)src, (DstT*)dst, R, C);
+}
+
+extern "C" int mts_moe_stage_weights(const void* src, int src_dtype, void* dst, int dst_dtype, int E,
                                      int64_t R, int64_t C, int transpose, void* stream) {
-    if (!src || !dst_bf16) return MTS_ERR_NULL;
+    if (!src || !dst) return MTS_ERR_NULL;
     if (E < 1 || R < 1 || C < 1 || E > 65535) return MTS_ERR_SHAPE;
     hipStream_t s = (hipStream_t)stream;
     dim3 grid((unsigned)((C + 63) / 64), (unsigned)((R + 63) / 64), (unsigned)E);
     if (grid.y > 65535) return MTS_ERR_SHAPE;
-    bf16_t* d = (bf16_t*)dst_bf16;
-    if (src_dtype == MTS_F32) {
-        if (transpose) stage_weights_kernel<float, true><<<grid, kThreads, 0, s>>>((const float*)src, d, R, C);
-        else stage_weights_kernel<float, false><<<grid, kThreads, 0, s>>>((const float*)src, d, R, C);
-    } else if (src_dtype == MTS_BF16) {
-        if (transpose) stage_weights_kernel<bf16_t, true><<<grid, kThreads, 0, s>>>((const bf16_t*)src, d, R, C);
-        else stage_weights_kernel<bf16_t, false><<<grid, kThreads, 0, s>>>((const bf16_t*)src, d, R, C);
-    } else {
-        return MTS_ERR_DTYPE;
-    }
+    if (src_dtype == MTS_F32 && dst_dtype == MTS_BF16) launch_stage<float, bf16_t>(src, dst, grid, R, C, transpose, s);
+    else if (src_dtype == MTS_BF16 && dst_dtype == MTS_BF16) launch_stage<bf16_t, bf16_t>(src, dst, grid, R, C, transpose, s);
+    else if (src_dtype == MTS_F32 && dst_dtype == MTS_F32) launch_stage<float, float>(src, dst, grid, R, C, transpose, s);
+    else if (src_dtype == MTS_BF16 && dst_dtype == MTS_F32) launch_stage<bf16_t, float>(src, dst, grid, R, C, transpose, s);
+    else return MTS_ERR_DTYPE;
     MTS_CHECK_LAUNCH();
     return MTS_OK;
 }

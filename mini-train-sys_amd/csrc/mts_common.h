@@ -37,3 +37,11 @@ __device__ __forceinline__ uint64_t lanemask_lt() {
 }
 
 static inline bool mts_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// fp32 GEMM launchers (mts_gemm_f32.hip); epi: 0 plain, 1 SwiGLU, 2 dO*W2 with SwiGLU backward
+int mts_f32_rows(int epi, const float* A, int lda, const int32_t* a_gather, const float* B, int b_rows,
+                 int N, int Kdim, const int32_t* expert_start, int E, int64_t TK, float* C, float* C2,
+                 const float* pre_act, const float* route_w, const int32_t* s_scatter, float* ds_part,
+                 int np, hipStream_t s);
+int mts_f32_dw(const float* P, const int32_t* p_gather, const float* Q, const int32_t* q_gather, int M,
+               int N, const int32_t* expert_start, int E, int grad_dtype, void* C, hipStream_t s);

@@ -1030,8 +1030,14 @@ extern "C" int mts_moe_fwd_gateup_swiglu(const void* x, const void* w1, const in
                                          int H, int I, int act_dtype, void* pre_act,
                                          void* post_act, void* stream) {
     if (!x || !w1 || !x_gather || !expert_start || !pre_act || !post_act) return MTS_ERR_NULL;
-    if (act_dtype != MTS_BF16) return MTS_ERR_DTYPE;
     if (T <= 0 || K < 1) return MTS_ERR_SHAPE;
+    if (act_dtype == MTS_F32) {
+        if (E < 1 || E > MTS_MAX_EXPERTS || H < 1 || I < 1 || T * K > 0x7fffffffLL) return MTS_ERR_SHAPE;
+        return mts_f32_rows(1, (const float*)x, H, x_gather, (const float*)w1, 2 * I, I, H, expert_start, E, T * K,
+                            (float*)pre_act, (float*)post_act, nullptr, nullptr, nullptr, nullptr, 0,
+                            (hipStream_t)stream);
+    }
+    if (act_dtype != MTS_BF16) return MTS_ERR_DTYPE;
     int rc = check_common(T * K, E, H, I);
     if (rc) return rc;
     if (!mts_aligned16(x) || !mts_aligned16(w1)) return MTS_ERR_ALIGN;
@@ -1047,6 +1053,11 @@ extern "C" int mts_moe_fwd_down(const void* post_act, const void* w2, const int3
                                 int64_t TK, int E, int H, int I, int act_dtype, void* y,
                                 void* stream) {
     if (!post_act || !w2 || !expert_start || !y) return MTS_ERR_NULL;
+    if (act_dtype == MTS_F32) {
+        if (TK <= 0 || TK > 0x7fffffffLL || E < 1 || E > MTS_MAX_EXPERTS || H < 1 || I < 1) return MTS_ERR_SHAPE;
+        return mts_f32_rows(0, (const float*)post_act, I, nullptr, (const float*)w2, H, H, I, expert_start, E, TK,
+                            (float*)y, nullptr, nullptr, nullptr, nullptr, nullptr, 0, (hipStream_t)stream);
+    }
     if (act_dtype != MTS_BF16) return MTS_ERR_DTYPE;
     int rc = check_common(TK, E, H, I);
     if (rc) return rc;
@@ -1067,8 +1078,14 @@ extern "C" int mts_moe_bwd_dy1(const void* d_out, const void* w2t, const void* p
     if (!d_out || !w2t || !pre_act || !weights || !x_gather || !s_scatter || !expert_start ||
         !d_pre_act || !weighted_act || !ds_partial)
         return MTS_ERR_NULL;
-    if (act_dtype != MTS_BF16) return MTS_ERR_DTYPE;
     if (T <= 0 || K < 1) return MTS_ERR_SHAPE;
+    if (act_dtype == MTS_F32) {
+        if (E < 1 || E > MTS_MAX_EXPERTS || H < 1 || I < 1 || T * K > 0x7fffffffLL) return MTS_ERR_SHAPE;
+        return mts_f32_rows(2, (const float*)d_out, H, x_gather, (const float*)w2t, I, I, H, expert_start, E, T * K,
+                            (float*)d_pre_act, (float*)weighted_act, (const float*)pre_act, (const float*)weights,
+                            s_scatter, ds_partial, mts_moe_ds_partials(I), (hipStream_t)stream);
+    }
+    if (act_dtype != MTS_BF16) return MTS_ERR_DTYPE;
     int rc = check_common(T * K, E, H, I);
     if (rc) return rc;
     if (!mts_aligned16(d_out) || !mts_aligned16(w2t)) return MTS_ERR_ALIGN;
@@ -1086,6 +1103,12 @@ extern "C" int mts_moe_bwd_dx(const void* d_pre_act, const void* w1t, const int3
                               int64_t TK, int E, int H, int I, int act_dtype, void* dx_expanded,
                               void* stream) {
     if (!d_pre_act || !w1t || !expert_start || !dx_expanded) return MTS_ERR_NULL;
+    if (act_dtype == MTS_F32) {
+        if (TK <= 0 || TK > 0x7fffffffLL || E < 1 || E > MTS_MAX_EXPERTS || H < 1 || I < 1) return MTS_ERR_SHAPE;
+        return mts_f32_rows(0, (const float*)d_pre_act, 2 * I, nullptr, (const float*)w1t, H, H, 2 * I, expert_start, E,
+                            TK, (float*)dx_expanded, nullptr, nullptr, nullptr, nullptr, nullptr, 0,
+                            (hipStream_t)stream);
+    }
     if (act_dtype != MTS_BF16) return MTS_ERR_DTYPE;
     int rc = check_common(TK, E, H, I);
     if (rc) return rc;
@@ -1102,8 +1125,13 @@ extern "C" int mts_moe_bwd_dw2(const void* d_out, const void* weighted_act, cons
                                const int32_t* expert_start, int64_t T, int K, int E, int H, int I,
                                int act_dtype, int grad_dtype, void* d_w2, void* stream) {
     if (!d_out || !weighted_act || !x_gather || !expert_start || !d_w2) return MTS_ERR_NULL;
-    if (act_dtype != MTS_BF16) return MTS_ERR_DTYPE;
     if (T <= 0 || K < 1) return MTS_ERR_SHAPE;
+    if (act_dtype == MTS_F32) {
+        if (E < 1 || E > MTS_MAX_EXPERTS || H < 1 || I < 1) return MTS_ERR_SHAPE;
+        return mts_f32_dw((const float*)d_out, x_gather, (const float*)weighted_act, nullptr, H, I, expert_start, E,
+                          grad_dtype, d_w2, (hipStream_t)stream);
+    }
+    if (act_dtype != MTS_BF16) return MTS_ERR_DTYPE;
     int rc = check_common(T * K, E, H, I);
     if (rc) return rc;
     if (!mts_aligned16(d_out) || !mts_aligned16(weighted_act)) return MTS_ERR_ALIGN;
@@ -1118,8 +1146,13 @@ extern "C" int mts_moe_bwd_dw1(const void* d_pre_act, const void* x, const int32
                                const int32_t* expert_start, int64_t T, int K, int E, int H, int I,
                                int act_dtype, int grad_dtype, void* d_w1, void* stream) {
     if (!d_pre_act || !x || !x_gather || !expert_start || !d_w1) return MTS_ERR_NULL;
-    if (act_dtype != MTS_BF16) return MTS_ERR_DTYPE;
     if (T <= 0 || K < 1) return MTS_ERR_SHAPE;
+    if (act_dtype == MTS_F32) {
+        if (E < 1 || E > MTS_MAX_EXPERTS || H < 1 || I < 1) return MTS_ERR_SHAPE;
+        return mts_f32_dw((const float*)d_pre_act, nullptr, (const float*)x, x_gather, 2 * I, H, expert_start, E,
+                          grad_dtype, d_w1, (hipStream_t)stream);
+    }
+    if (act_dtype != MTS_BF16) return MTS_ERR_DTYPE;
     int rc = check_common(T * K, E, H, I);
     if (rc) return rc;
     if (!mts_aligned16(d_pre_act) || !mts_aligned16(x)) return MTS_ERR_ALIGN;

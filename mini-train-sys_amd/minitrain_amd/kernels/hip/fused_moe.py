@@ -50,11 +50,11 @@ def is_fused_moe_supported(x, gate_up_proj, down_proj, top_k_index, top_k_weight
         and tokens * top_k_index.shape[1] < 2**31
         and top_k_index.dtype == torch.int32
         and top_k_weights.dtype == x.dtype
-        and x.dtype == torch.bfloat16
+        and x.dtype in (torch.bfloat16, torch.float32)
         and gate_up_proj.dtype in weight_dtypes
         and down_proj.dtype in weight_dtypes
-        and hidden % 8 == 0
-        and intermediate % 8 == 0
+        and hidden % (8 if x.dtype == torch.bfloat16 else 4) == 0
+        and (intermediate % 8 == 0 or x.dtype == torch.float32)
     )
 
 
@@ -102,15 +102,16 @@ def compute_routing_metadata(topk_indices: torch.Tensor, E: int, block_m_token: 
     )
 
 
-def _stage(lib, w: torch.Tensor, transpose: bool) -> torch.Tensor:
-    """bf16 copy of an expert weight ``[E,R,C]``, optionally as ``[E,C,R]``."""
-    if not transpose and w.dtype == torch.bfloat16:
+def _stage(lib, w: torch.Tensor, transpose: bool, dtype: torch.dtype) -> torch.Tensor:
+    """Copy of an expert weight ``[E,R,C]`` in the activation dtype, optionally as ``[E,C,R]``."""
+    if not transpose and w.dtype == dtype:
         return w
     E, R, C = w.shape
-    out = torch.empty((E, C, R) if transpose else (E, R, C), dtype=torch.bfloat16, device=w.device)
+    out = torch.empty((E, C, R) if transpose else (E, R, C), dtype=dtype, device=w.device)
     _lib.check(
         lib.mts_moe_stage_weights(
-            w.data_ptr(), _lib.dtype_code(w.dtype), out.data_ptr(), E, R, C, int(transpose), _lib.stream_of(w)
+            w.data_ptr(), _lib.dtype_code(w.dtype), out.data_ptr(), _lib.dtype_code(dtype), E, R, C, int(transpose),
+            _lib.stream_of(w),
         ),
         "mts_moe_stage_weights",
     )
@@ -134,8 +135,8 @@ class _FusedMoEFunction(torch.autograd.Function):
         with torch.no_grad():
             (_, expert_start, x_gather, s_scatter, s_reverse, _, _, _) = compute_routing_metadata(top_k_index, E)
 
-        w1 = _stage(lib, gate_up_proj, False)
-        w2 = _stage(lib, down_proj, False)
+        w1 = _stage(lib, gate_up_proj, False, x.dtype)
+        w2 = _stage(lib, down_proj, False, x.dtype)
         pre_act = torch.empty(TK, 2 * I, dtype=x.dtype, device=dev)
         post_act = torch.empty(TK, I, dtype=x.dtype, device=dev)
         _lib.check(
@@ -187,7 +188,7 @@ class _FusedMoEFunction(torch.autograd.Function):
         stream = _lib.stream_of(dO)
         need_x, need_w1, need_w2, _, need_s = ctx.needs_input_grad
 
-        w2t = _stage(lib, down_proj, True)  # [E, I, H]
+        w2t = _stage(lib, down_proj, True, x.dtype)  # [E, I, H]
         d_pre_act = torch.empty(TK, 2 * I, dtype=x.dtype, device=dev)
         weighted_act = torch.empty(TK, I, dtype=x.dtype, device=dev)
         n_part = lib.mts_moe_ds_partials(I)
@@ -224,7 +225,7 @@ class _FusedMoEFunction(torch.autograd.Function):
 
         dx = None
         if need_x:
-            w1t = _stage(lib, gate_up_proj, True)  # [E, H, 2I]
+            w1t = _stage(lib, gate_up_proj, True, x.dtype)  # [E, H, 2I]
             dx_expanded = torch.empty(TK, H, dtype=x.dtype, device=dev)
             _lib.check(
                 lib.mts_moe_bwd_dx(
