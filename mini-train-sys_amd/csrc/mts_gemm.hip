@@ -330,22 +330,39 @@ __device__ __forceinline__ void rows_epilogue(const RowsParams& p, f32x16 (&acc)
 // ---------------------------------------------------------------------------
 constexpr int kXcds = 8;
 
+// The expert that owns m-tile `tile` is found with one vector load: lane l reads
+// expert_start[l] and [l+1], a wave scan turns tile counts into tile offsets, and a
+// ballot picks the first expert whose offset range contains the tile (63 experts per
+// round; more experts take more rounds).
 template <int BM>
 __device__ __forceinline__ bool locate_rows_tile(const RowsParams& p, int& e, int& row0, int& rend, int& ntile) {
     const int b = blockIdx.x;
     const int xcd = b % kXcds, j = b / kXcds;
     const int tile = xcd + kXcds * (j / p.n_tiles);
     ntile = j % p.n_tiles;
+    const int lane = threadIdx.x % MTS_WAVE;
     int seen = 0;
-    for (e = 0; e < p.E; ++e) {
-        const int s0 = p.expert_start[e], s1 = p.expert_start[e + 1];
+    for (int e0 = 0; e0 < p.E; e0 += MTS_WAVE) {
+        const int le = e0 + lane;
+        const int s0 = le < p.E ? p.expert_start[le] : 0;
+        const int s1 = le < p.E ? p.expert_start[le + 1] : 0;
         const int nt = (s1 - s0 + BM - 1) / BM;
-        if (tile < seen + nt) {
-            row0 = s0 + (tile - seen) * BM;
-            rend = s1;
+        int incl = nt;
+#pragma unroll
+        for (int o = 1; o < MTS_WAVE; o <<= 1) {
+            const int up = __shfl_up(incl, o, MTS_WAVE);
+            if (lane >= o) incl += up;
+        }
+        const uint64_t hit = __ballot(tile < seen + incl);
+        if (hit) {
+            const int w = __ffsll((unsigned long long)hit) - 1;
+            const int first = seen + __shfl(incl, w, MTS_WAVE) - __shfl(nt, w, MTS_WAVE);
+            e = e0 + w;
+            row0 = __shfl(s0, w, MTS_WAVE) + (tile - first) * BM;
+            rend = __shfl(s1, w, MTS_WAVE);
             return true;
         }
-        seen += nt;
+        seen += __shfl(incl, MTS_WAVE - 1, MTS_WAVE);
     }
     return false;
 }
@@ -544,11 +561,129 @@ __global__ __launch_bounds__(T::NT, T::WAVES_PER_EU) void rows_gemm_ring_kernel(
         const bf16_t* cur = smem + stage * T::STAGE;
         constexpr int KSTEPS = T::BKS / 16;
         mma_tile<T, SWIGLU, T::BKS>(cur, cur + T::BM * T::BKS, wm, wn, acc, [&](int ks) {
-            if (refill) issue(rstage, kt + S - 1, ks, KSTEPS);
+            if (refill && (T::NWAVES < 8 ? true : ks == (wave / 4) % KSTEPS)) {
+                if (T::NWAVES < 8) issue(rstage, kt + S - 1, ks, KSTEPS);
+                else issue(rstage, kt + S - 1, 0, 1);  // waves w and w+4 share a SIMD and take turns
+            }
         });
         stage = stage + 1 == S ? 0 : stage + 1;
     }
     __builtin_amdgcn_s_barrier();  // every wave is done reading the ring before it is reused
+    rows_epilogue<T, EPI>(p, acc, smem, row0, rend, n0, wm, wn);
+}
+
+// ---------------------------------------------------------------------------
+// rows_gemm, ring pipeline with specialised waves: consumer waves read fragments,
+// issue MFMAs and run the epilogue; producer waves compute the gather offsets and
+// issue every tile load, so that a load that cannot be queued (the L1 fill path
+// sustains about 25 B/clk/CU) stalls a wave that has no MFMAs to issue.  Pays off
+// for the longer reductions (down, dX).
+// ---------------------------------------------------------------------------
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int BKS_, int STAGES_, int PRODUCERS_, int WAVES_PER_EU_>
+struct WsTile {
+    static constexpr int BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
+    static constexpr int BKS = BKS_, STAGES = STAGES_, PRODUCERS = PRODUCERS_, WAVES_PER_EU = WAVES_PER_EU_;
+    static constexpr int NWAVES = WAVES_M * WAVES_N;   // consumer waves
+    static constexpr int NT = (NWAVES + PRODUCERS) * MTS_WAVE;
+    static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+    static constexpr int MF = WM / 32, NF = WN / 32;
+    static constexpr int CHUNKS = BKS / 8;
+    static constexpr int RPI = MTS_WAVE / CHUNKS;
+    static constexpr int A_INSTR = BM / RPI / PRODUCERS, B_INSTR = BN / RPI / PRODUCERS;   // per producer wave
+    static constexpr int STAGE = (BM + BN) * BKS;
+    static constexpr int LDS_ELEMS = STAGES * STAGE;
+    static_assert(BKS == 32 || BKS == 64, "LDS rows are 64 or 128 bytes");
+    static_assert(WM % 32 == 0 && WN % 64 == 0, "wave tile must hold whole 32x32 fragments");
+    static_assert(A_INSTR * RPI * PRODUCERS == BM && B_INSTR * RPI * PRODUCERS == BN, "loader split");
+    static_assert(STAGES >= 3 && STAGES <= 4 && (A_INSTR + B_INSTR) * (STAGES - 2) <= 63, "vmcnt range");
+    static_assert(LDS_ELEMS * 2 <= 160 * 1024, "LDS capacity");
+};
+
+template <class T, int EPI>
+__global__ __launch_bounds__(T::NT, T::WAVES_PER_EU) void rows_gemm_ws_kernel(RowsParams p) {
+    constexpr int LDS_ELEMS = T::LDS_ELEMS > EpiShape<T, EPI>::ELEMS ? T::LDS_ELEMS : EpiShape<T, EPI>::ELEMS;
+    static_assert(LDS_ELEMS * 2 <= 160 * 1024, "LDS capacity");
+    __shared__ __attribute__((aligned(1024))) bf16_t smem[LDS_ELEMS];
+    constexpr bool SWIGLU = (EPI == EPI_SWIGLU);
+    constexpr int S = T::STAGES, L = T::A_INSTR + T::B_INSTR;
+
+    int e, row0, rend, ntile;
+    if (!locate_rows_tile<T::BM>(p, e, row0, rend, ntile)) return;
+    const int n0 = ntile * (SWIGLU ? T::BN / 2 : T::BN);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / MTS_WAVE), lane = threadIdx.x % MTS_WAVE;
+    const int nk = p.Kdim / T::BKS;
+
+    if (wave >= T::NWAVES) {
+        // ------------------------------ producer ------------------------------
+        const int pw = wave - T::NWAVES;
+        const __amdgpu_buffer_rsrc_t rs_a = make_rsrc(p.A, p.a_rows * p.lda * 2);
+        const __amdgpu_buffer_rsrc_t rs_b =
+            make_rsrc(p.B + (int64_t)e * p.b_rows * p.Kdim, (int64_t)p.b_rows * p.Kdim * 2);
+        uint32_t voff_a[T::A_INSTR], voff_b[T::B_INSTR];
+        const int slot = lane % T::CHUNKS, rin = lane / T::CHUNKS;
+#pragma unroll
+        for (int j = 0; j < T::A_INSTR; ++j) {
+            const int tr = (pw * T::A_INSTR + j) * T::RPI + rin;
+            const int chunk = slot ^ (T::CHUNKS == 8 ? (tr >> 1) & 7 : (tr >> 2) & 3);
+            const int row = row0 + tr;
+            const int lrow = row < rend ? row : rend - 1;
+            const int src = p.a_gather ? p.a_gather[lrow] : lrow;
+            voff_a[j] = row < rend ? ((uint32_t)src * (uint32_t)p.lda + chunk * 8) * 2u : kInvalid;
+        }
+#pragma unroll
+        for (int j = 0; j < T::B_INSTR; ++j) {
+            const int br = (pw * T::B_INSTR + j) * T::RPI + rin;
+            const int chunk = slot ^ (T::CHUNKS == 8 ? (br >> 1) & 7 : (br >> 2) & 3);
+            int n, grow;
+            if (SWIGLU) {
+                n = n0 + br % (T::BN / 2);
+                grow = (br / (T::BN / 2)) * p.N + n;
+            } else {
+                n = n0 + br;
+                grow = n;
+            }
+            voff_b[j] = (n < p.N) ? ((uint32_t)grow * (uint32_t)p.Kdim + chunk * 8) * 2u : kInvalid;
+        }
+        auto issue = [&](int stage, int kt) {
+            bf16_t* sa = smem + stage * T::STAGE + pw * T::A_INSTR * 512;
+            bf16_t* sb = smem + stage * T::STAGE + T::BM * T::BKS + pw * T::B_INSTR * 512;
+            const int soff = kt * T::BKS * 2;
+#pragma unroll
+            for (int j = 0; j < T::A_INSTR; ++j)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, MTS_LDS_PTR(sa + j * 512), 16, (int)voff_a[j], soff, 0, 0);
+#pragma unroll
+            for (int j = 0; j < T::B_INSTR; ++j)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_b, MTS_LDS_PTR(sb + j * 512), 16, (int)voff_b[j], soff, 0, 0);
+        };
+#pragma unroll
+        for (int s = 0; s < S - 1; ++s)
+            if (s < nk) issue(s, s);
+        int stage = 0;
+        for (int kt = 0; kt < nk; ++kt) {
+            const int younger = nk - 1 - kt;
+            if (S >= 4 && younger >= 2) wait_vmcnt<L * (S >= 4 ? 2 : 0)>();
+            else if (younger >= 1) wait_vmcnt<L>();
+            else wait_vmcnt<0>();
+            __builtin_amdgcn_s_barrier();   // tile kt is visible; every consumer is done with tile kt-1
+            if (kt + S - 1 < nk) issue(stage == 0 ? S - 1 : stage - 1, kt + S - 1);
+            stage = stage + 1 == S ? 0 : stage + 1;
+        }
+        __builtin_amdgcn_s_barrier();       // matches the consumers' barrier before the epilogue
+        return;
+    }
+
+    // -------------------------------- consumer --------------------------------
+    const int wm = wave / T::WAVES_N, wn = wave % T::WAVES_N;
+    f32x16 acc[T::MF][T::NF];
+    zero_acc<T>(acc);
+    int stage = 0;
+    for (int kt = 0; kt < nk; ++kt) {
+        __builtin_amdgcn_s_barrier();
+        const bf16_t* cur = smem + stage * T::STAGE;
+        mma_tile<T, SWIGLU, T::BKS>(cur, cur + T::BM * T::BKS, wm, wn, acc);
+        stage = stage + 1 == S ? 0 : stage + 1;
+    }
+    __builtin_amdgcn_s_barrier();  // every consumer is done reading the ring before it is reused
     rows_epilogue<T, EPI>(p, acc, smem, row0, rend, n0, wm, wn);
 }
 
@@ -709,30 +844,24 @@ __global__ __launch_bounds__(T::NT) void dw_gemm_kernel(DwParams p) {
 // lanes, lane s addresses 4 consecutive columns of row s/4 and lane l receives the
 // 4 rows of column l.  The 16-byte chunk index of a row is XOR-swizzled with
 // 4*(row % 4) so that the 4 rows x 2 column halves read by 32 lanes cover all banks.
-// Source rows of a gathered operand come from scalar loads of the row index, one
-// k-tile ahead.  Rows past the expert's end are fetched with an out-of-range
-// offset and arrive as zeros.
+// Source rows of a gathered operand come from a per-lane load of the row index, one
+// k-tile ahead.  Rows past the expert's end are fetched with an out-of-range offset
+// and arrive as zeros.
+//
+// Waves are specialised.  A wave whose tile load cannot be queued stalls at that
+// instruction and, issue being in order, its MFMAs wait behind it; at about 25
+// B/clk/CU of L1 fill the load queue is full most of the time.  So 8 consumer waves
+// (two per SIMD) only read fragments and issue MFMAs, and 4 producer waves (one per
+// SIMD) only issue the tile loads, the row-index loads and an L2 prefetch, and a
+// blocked load never holds up the matrix pipe.  One barrier per k-tile joins them:
+// producers arrive once tile kt has landed, consumers once they are done reading
+// tile kt-1.
+//
+// L2 prefetch: all tiles of an expert run on one XCD in lockstep and ask for the same
+// rows, so the unique data in flight per XCD is only what the ring holds; one 4-byte
+// load per producer lane, PD tiles ahead, pulls the lines of the operand that is read
+// in place into that XCD's L2 early (it lands in 256 bytes of LDS that nobody reads).
 // ---------------------------------------------------------------------------
-template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int BKS_, int STAGES_, int WAVES_PER_EU_ = 1>
-struct DwRingTile {
-    static constexpr int BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
-    static constexpr int BKS = BKS_, STAGES = STAGES_, WAVES_PER_EU = WAVES_PER_EU_;
-    static constexpr int NWAVES = WAVES_M * WAVES_N;
-    static constexpr int NT = NWAVES * MTS_WAVE;
-    static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
-    static constexpr int MF = WM / 32, NF = WN / 32;
-    static constexpr int CPR_A = BM / 8, CPR_B = BN / 8;                    // 16-byte chunks per LDS row
-    static constexpr int RPI_A = MTS_WAVE / CPR_A, RPI_B = MTS_WAVE / CPR_B;  // rows per wave instruction
-    static constexpr int A_INSTR = BKS / RPI_A / NWAVES, B_INSTR = BKS / RPI_B / NWAVES;
-    static constexpr int STAGE = BKS * (BM + BN);
-    static constexpr int LDS_ELEMS = STAGES * STAGE;
-    static_assert(BM <= 512 && BN <= 512 && BM % 64 == 0 && BN % 64 == 0, "tile width");
-    static_assert(A_INSTR >= 1 && B_INSTR >= 1 && A_INSTR * RPI_A * NWAVES == BKS && B_INSTR * RPI_B * NWAVES == BKS,
-                  "loader split");
-    static_assert(STAGES >= 2 && STAGES <= 4 && (A_INSTR + B_INSTR) * (STAGES - 2) <= 63, "vmcnt range");
-    static_assert(LDS_ELEMS * 2 <= 160 * 1024, "LDS capacity");
-};
-
 typedef __attribute__((ext_vector_type(4))) short s16x4;
 
 // 32 (m) x 16 (k) MFMA fragment out of a k-major LDS tile with row length ROWLEN
@@ -753,10 +882,29 @@ __device__ __forceinline__ bf16x8 read_frag_tr(const bf16_t* tile, int krow0, in
     return __builtin_bit_cast(bf16x8, v);
 }
 
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int BKS_, int STAGES_, int PRODUCERS_>
+struct DwWsTile {
+    static constexpr int BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
+    static constexpr int BKS = BKS_, STAGES = STAGES_, PRODUCERS = PRODUCERS_;
+    static constexpr int NWAVES = WAVES_M * WAVES_N;              // consumer waves
+    static constexpr int NT = (NWAVES + PRODUCERS) * MTS_WAVE;
+    static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+    static constexpr int MF = WM / 32, NF = WN / 32;
+    static constexpr int CPR_A = BM / 8, CPR_B = BN / 8;
+    static constexpr int RPI_A = MTS_WAVE / CPR_A, RPI_B = MTS_WAVE / CPR_B;
+    static constexpr int A_INSTR = BKS / RPI_A / PRODUCERS, B_INSTR = BKS / RPI_B / PRODUCERS;  // per producer wave
+    static constexpr int STAGE = BKS * (BM + BN);
+    static constexpr int LDS_ELEMS = STAGES * STAGE;
+    static_assert(A_INSTR >= 1 && B_INSTR >= 1 && A_INSTR * RPI_A * PRODUCERS == BKS && B_INSTR * RPI_B * PRODUCERS == BKS,
+                  "loader split");
+    static_assert(STAGES >= 3 && STAGES <= 4 && (A_INSTR + B_INSTR + 1) * (STAGES - 2) <= 63, "vmcnt range");
+    static_assert(LDS_ELEMS * 2 + PRODUCERS * 256 <= 160 * 1024, "LDS capacity");
+};
+
 template <class T, typename OutT>
-__global__ __launch_bounds__(T::NT, T::WAVES_PER_EU) void dw_gemm_ring_kernel(DwParams p) {
-    __shared__ __attribute__((aligned(1024))) bf16_t smem[T::LDS_ELEMS];
-    constexpr int S = T::STAGES, L = T::A_INSTR + T::B_INSTR;
+__global__ __launch_bounds__(T::NT) void dw_gemm_ws_kernel(DwParams p) {
+    __shared__ __attribute__((aligned(1024))) bf16_t smem[T::LDS_ELEMS + T::PRODUCERS * 128];
+    constexpr int S = T::STAGES, L = T::A_INSTR + T::B_INSTR, PD = 8;
     const int xcd = blockIdx.x % kXcds, jb = blockIdx.x / kXcds;
     const int e = xcd + kXcds * (jb / p.tiles_per_expert);
     if (e >= p.E) return;
@@ -764,124 +912,120 @@ __global__ __launch_bounds__(T::NT, T::WAVES_PER_EU) void dw_gemm_ring_kernel(Dw
     const int m0 = (tile / p.n_tiles) * T::BM, n0 = (tile % p.n_tiles) * T::BN;
     const int rbeg = p.expert_start[e], rend = p.expert_start[e + 1];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / MTS_WAVE), lane = threadIdx.x % MTS_WAVE;
-    const int wm = wave / T::WAVES_N, wn = wave % T::WAVES_N;
+    const int nk = (rend - rbeg + T::BKS - 1) / T::BKS;
 
-    const __amdgpu_buffer_rsrc_t rs_p = make_rsrc(p.P, p.p_rows * p.M * 2);
-    const __amdgpu_buffer_rsrc_t rs_q = make_rsrc(p.Q, p.q_rows * p.N * 2);
-    const int32_t* __restrict__ gp = p.p_gather;
-    const int32_t* __restrict__ gq = p.q_gather;
-    const int last_row = (int)p.TK - 1;
-
-    // column part of this lane's offsets (constant over the k loop)
-    uint32_t col_a[T::A_INSTR], col_b[T::B_INSTR];
-    int rin_a[T::A_INSTR], rin_b[T::B_INSTR];   // this lane's row inside the k-tile, per instruction
-#pragma unroll
-    for (int j = 0; j < T::A_INSTR; ++j) {
-        const int tr = (wave * T::A_INSTR + j) * T::RPI_A + lane / T::CPR_A;
-        const int c = m0 + (((lane % T::CPR_A) ^ ((tr & 3) << 2)) << 3);
-        rin_a[j] = tr;
-        col_a[j] = c < p.M ? (uint32_t)c * 2u : kInvalid;
-    }
-#pragma unroll
-    for (int j = 0; j < T::B_INSTR; ++j) {
-        const int tr = (wave * T::B_INSTR + j) * T::RPI_B + lane / T::CPR_B;
-        const int c = n0 + (((lane % T::CPR_B) ^ ((tr & 3) << 2)) << 3);
-        rin_b[j] = tr;
-        col_b[j] = c < p.N ? (uint32_t)c * 2u : kInvalid;
-    }
-
-    // source rows of the next tile to be fetched (scalar registers; row index clamped into the array)
-    int src_a[T::A_INSTR][T::RPI_A], src_b[T::B_INSTR][T::RPI_B];
-    auto fetch_index = [&](int r0) {
-#pragma unroll
-        for (int j = 0; j < T::A_INSTR; ++j)
-#pragma unroll
-            for (int q = 0; q < T::RPI_A; ++q) {
-                int r = r0 + (wave * T::A_INSTR + j) * T::RPI_A + q;
-                r = r < last_row ? r : last_row;
-                src_a[j][q] = gp ? gp[r] : r;
-            }
-#pragma unroll
-        for (int j = 0; j < T::B_INSTR; ++j)
-#pragma unroll
-            for (int q = 0; q < T::RPI_B; ++q) {
-                int r = r0 + (wave * T::B_INSTR + j) * T::RPI_B + q;
-                r = r < last_row ? r : last_row;
-                src_b[j][q] = gq ? gq[r] : r;
-            }
-    };
-    uint32_t voff_a[T::A_INSTR], voff_b[T::B_INSTR];
-    auto make_offsets = [&](int r0) {
+    if (wave >= T::NWAVES) {
+        // ------------------------------ producer ------------------------------
+        const int pw = wave - T::NWAVES;
+        const __amdgpu_buffer_rsrc_t rs_p = make_rsrc(p.P, p.p_rows * p.M * 2);
+        const __amdgpu_buffer_rsrc_t rs_q = make_rsrc(p.Q, p.q_rows * p.N * 2);
+        const bool gath_p = p.p_gather != nullptr, gath_q = p.q_gather != nullptr;
+        const __amdgpu_buffer_rsrc_t rs_gp = make_rsrc(p.p_gather, gath_p ? p.TK * 4 : 0);
+        const __amdgpu_buffer_rsrc_t rs_gq = make_rsrc(p.q_gather, gath_q ? p.TK * 4 : 0);
+        uint32_t col_a[T::A_INSTR], col_b[T::B_INSTR];
+        int rin_a[T::A_INSTR], rin_b[T::B_INSTR];
 #pragma unroll
         for (int j = 0; j < T::A_INSTR; ++j) {
-            int src = src_a[j][0];
-#pragma unroll
-            for (int q = 1; q < T::RPI_A; ++q) src = (lane / T::CPR_A == q) ? src_a[j][q] : src;
-            const bool ok = r0 + rin_a[j] < rend && col_a[j] != kInvalid;
-            voff_a[j] = ok ? (uint32_t)src * (uint32_t)p.M * 2u + col_a[j] : kInvalid;
+            const int tr = (pw * T::A_INSTR + j) * T::RPI_A + lane / T::CPR_A;
+            const int c = m0 + (((lane % T::CPR_A) ^ ((tr & 3) << 2)) << 3);
+            rin_a[j] = tr;
+            col_a[j] = c < p.M ? (uint32_t)c * 2u : kInvalid;
         }
 #pragma unroll
         for (int j = 0; j < T::B_INSTR; ++j) {
-            int src = src_b[j][0];
-#pragma unroll
-            for (int q = 1; q < T::RPI_B; ++q) src = (lane / T::CPR_B == q) ? src_b[j][q] : src;
-            const bool ok = r0 + rin_b[j] < rend && col_b[j] != kInvalid;
-            voff_b[j] = ok ? (uint32_t)src * (uint32_t)p.N * 2u + col_b[j] : kInvalid;
+            const int tr = (pw * T::B_INSTR + j) * T::RPI_B + lane / T::CPR_B;
+            const int c = n0 + (((lane % T::CPR_B) ^ ((tr & 3) << 2)) << 3);
+            rin_b[j] = tr;
+            col_b[j] = c < p.N ? (uint32_t)c * 2u : kInvalid;
         }
-    };
-    auto issue = [&](int stage, int part, int parts) {
-        bf16_t* sa = smem + stage * T::STAGE + wave * T::A_INSTR * 512;
-        bf16_t* sb = smem + stage * T::STAGE + T::BKS * T::BM + wave * T::B_INSTR * 512;
+        int src_a[T::A_INSTR], src_b[T::B_INSTR];
+        auto fetch_index = [&](int r0) {
 #pragma unroll
-        for (int j = 0; j < T::A_INSTR; ++j)
-            if (j % parts == part)
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_p, MTS_LDS_PTR(sa + j * 512), 16, (int)voff_a[j], 0, 0, 0);
+            for (int j = 0; j < T::A_INSTR; ++j)
+                src_a[j] = gath_p ? buf_load4(rs_gp, (uint32_t)(r0 + rin_a[j]) * 4u) : r0 + rin_a[j];
 #pragma unroll
-        for (int j = 0; j < T::B_INSTR; ++j)
-            if ((j + T::A_INSTR) % parts == part)
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_q, MTS_LDS_PTR(sb + j * 512), 16, (int)voff_b[j], 0, 0, 0);
-    };
+            for (int j = 0; j < T::B_INSTR; ++j)
+                src_b[j] = gath_q ? buf_load4(rs_gq, (uint32_t)(r0 + rin_b[j]) * 4u) : r0 + rin_b[j];
+        };
+        auto issue = [&](int stage, int r0) {
+            bf16_t* sa = smem + stage * T::STAGE + pw * T::A_INSTR * 512;
+            bf16_t* sb = smem + stage * T::STAGE + T::BKS * T::BM + pw * T::B_INSTR * 512;
+#pragma unroll
+            for (int j = 0; j < T::A_INSTR; ++j) {
+                const bool ok = r0 + rin_a[j] < rend && col_a[j] != kInvalid;
+                const uint32_t off = ok ? (uint32_t)src_a[j] * (uint32_t)p.M * 2u + col_a[j] : kInvalid;
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_p, MTS_LDS_PTR(sa + j * 512), 16, (int)off, 0, 0, 0);
+            }
+#pragma unroll
+            for (int j = 0; j < T::B_INSTR; ++j) {
+                const bool ok = r0 + rin_b[j] < rend && col_b[j] != kInvalid;
+                const uint32_t off = ok ? (uint32_t)src_b[j] * (uint32_t)p.N * 2u + col_b[j] : kInvalid;
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_q, MTS_LDS_PTR(sb + j * 512), 16, (int)off, 0, 0, 0);
+            }
+        };
+        // L2 prefetch of the operand that is read in place, PD tiles ahead
+        const bool touch_p = !gath_p, touch_any = touch_p || !gath_q;
+        const __amdgpu_buffer_rsrc_t rs_t = touch_p ? rs_p : rs_q;
+        const int t_ld = touch_p ? p.M : p.N, t_col0 = touch_p ? m0 : n0, t_w = touch_p ? T::BM : T::BN;
+        constexpr int PPR = T::PRODUCERS * MTS_WAVE / T::BKS;
+        const int pt = pw * MTS_WAVE + lane;
+        const int t_row = pt / PPR, t_piece = (pt % PPR) * (t_w / PPR);
+        bf16_t* t_dst = smem + T::LDS_ELEMS + pw * 128;
+        auto touch = [&](int r0) {
+            const int r = r0 + t_row, c = t_col0 + t_piece;
+            const bool ok = touch_any && r < rend && c < t_ld;
+            const uint32_t off = ok ? ((uint32_t)r * (uint32_t)t_ld + (uint32_t)c) * 2u : kInvalid;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_t, MTS_LDS_PTR(t_dst), 4, (int)off, 0, 0, 0);
+        };
 
+#pragma unroll
+        for (int s = 0; s < S - 1; ++s) {
+            if (s < nk) {
+                fetch_index(rbeg + s * T::BKS);
+                issue(s, rbeg + s * T::BKS);
+            }
+        }
+        if (S - 1 < nk) fetch_index(rbeg + (S - 1) * T::BKS);
+        int stage = 0;
+        for (int kt = 0; kt < nk; ++kt) {
+            // tile kt has landed when at most the loads issued after it are outstanding: per later
+            // iteration one prefetch load and L tile loads (index loads are left out of the count,
+            // which only makes the wait a little longer)
+            const int younger = nk - 1 - kt;
+            if (S >= 4 && younger >= 2) wait_vmcnt<(L + 1) * (S >= 4 ? 2 : 0)>();
+            else if (younger >= 1) wait_vmcnt<L>();
+            else wait_vmcnt<0>();
+            __builtin_amdgcn_s_barrier();
+            const int rstage = stage == 0 ? S - 1 : stage - 1;
+            touch(rbeg + (kt + PD) * T::BKS);
+            if (kt + S - 1 < nk) issue(rstage, rbeg + (kt + S - 1) * T::BKS);
+            if (kt + S < nk) fetch_index(rbeg + (kt + S) * T::BKS);
+            stage = stage + 1 == S ? 0 : stage + 1;
+        }
+        return;
+    }
+
+    // -------------------------------- consumer --------------------------------
+    const int wm = wave / T::WAVES_N, wn = wave % T::WAVES_N;
     f32x16 acc[T::MF][T::NF];
     zero_acc<T>(acc);
-
-    const int nk = (rend - rbeg + T::BKS - 1) / T::BKS;
-#pragma unroll
-    for (int s = 0; s < S - 1; ++s) {
-        if (s < nk) {
-            fetch_index(rbeg + s * T::BKS);
-            make_offsets(rbeg + s * T::BKS);
-            issue(s, 0, 1);
-        }
-    }
-    if (S - 1 < nk) fetch_index(rbeg + (S - 1) * T::BKS);
     int stage = 0;
     for (int kt = 0; kt < nk; ++kt) {
-        const int younger = nk - 1 - kt;
-        if (S >= 4 && younger >= 2) wait_vmcnt<L * (S >= 4 ? 2 : 0)>();
-        else if (S >= 3 && younger >= 1) wait_vmcnt<L>();
-        else wait_vmcnt<0>();
         __builtin_amdgcn_s_barrier();
-        const bool refill = kt + S - 1 < nk;
-        const int rstage = stage == 0 ? S - 1 : stage - 1;
-        if (refill) make_offsets(rbeg + (kt + S - 1) * T::BKS);
-        if (kt + S < nk) fetch_index(rbeg + (kt + S) * T::BKS);
         const bf16_t* As = smem + stage * T::STAGE;
         const bf16_t* Bs = As + T::BKS * T::BM;
-        constexpr int KSTEPS = T::BKS / 16;
 #pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks) {
-            bf16x8 a[T::MF], b[T::NF];
-#pragma unroll
-            for (int mf = 0; mf < T::MF; ++mf) a[mf] = read_frag_tr<T::BM>(As, ks * 16, wm * T::WM + mf * 32);
+        for (int ks = 0; ks < T::BKS / 16; ++ks) {
+            bf16x8 b[T::NF];
 #pragma unroll
             for (int nf = 0; nf < T::NF; ++nf) b[nf] = read_frag_tr<T::BN>(Bs, ks * 16, wn * T::WN + nf * 32);
-            if (refill) issue(rstage, ks, KSTEPS);
 #pragma unroll
-            for (int mf = 0; mf < T::MF; ++mf)
+            for (int mf = 0; mf < T::MF; ++mf) {
+                const bf16x8 a = read_frag_tr<T::BM>(As, ks * 16, wm * T::WM + mf * 32);
 #pragma unroll
                 for (int nf = 0; nf < T::NF; ++nf)
-                    acc[mf][nf] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[mf], b[nf], acc[mf][nf], 0, 0, 0);
+                    acc[mf][nf] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b[nf], acc[mf][nf], 0, 0, 0);
+            }
         }
         stage = stage + 1 == S ? 0 : stage + 1;
     }
@@ -905,20 +1049,18 @@ __global__ __launch_bounds__(T::NT, T::WAVES_PER_EU) void dw_gemm_ring_kernel(Dw
 // host side
 // ---------------------------------------------------------------------------
 typedef Tile<128, 128, 2, 2> StagedSmall;                 // 4 waves of 64x64, any K that is a multiple of 8
-typedef Tile<256, 256, 2, 4> StagedLarge;                 // 8 waves of 128x64
 typedef RingTile<256, 128, 2, 2, 32, 3, 2> RingTwoPerCu;  // 4 waves of 128x64, 3 x 24 KiB stages, two blocks per CU
-typedef RingTile<256, 256, 2, 4, 64, 2, 2> RingLarge;     // 8 waves of 128x64, 2 x 64 KiB stages
-typedef RingTile<256, 256, 2, 4, 32, 4, 2> RingDeep;      // 8 waves of 128x64, 4 x 32 KiB stages
-typedef DwRingTile<256, 256, 2, 4, 32, 4, 2> DwRingLarge; // 8 waves of 128x64, 4 x 32 KiB stages
-typedef DwRingTile<256, 256, 2, 2, 32, 4> DwRingWide;     // 4 waves of 128x128
+typedef WsTile<256, 256, 2, 4, 32, 4, 4, 3> WsLarge;      // 8 consumer waves of 128x64 + 4 producers, 4 x 32 KiB stages
+typedef DwWsTile<256, 256, 2, 4, 32, 4, 4> DwWsLarge;     // same shape for the weight-gradient GEMMs
 
 enum Kind { K_GATEUP = 0, K_DOWN, K_DY1, K_DX, K_DW2, K_DW1, K_COUNT };
 const char* const kKindEnv[K_COUNT] = {"MTS_TILE_GATEUP", "MTS_TILE_DOWN", "MTS_TILE_DY1",
                                        "MTS_TILE_DX",     "MTS_TILE_DW2",  "MTS_TILE_DW1"};
-// rows_gemm: 0 StagedSmall, 1 RingTwoPerCu, 2 RingLarge, 3 RingDeep
-// dw_gemm:   0 StagedSmall, 1 StagedLarge,  2 DwRingLarge, 3 DwRingWide
-// Defaults are the fastest measured on the 24576-token, 768/1024, 8-expert layer.
-const int kDefaultTile[K_COUNT] = {1, 1, 1, 1, 0, 2};
+// rows_gemm: 0 StagedSmall, 1 RingTwoPerCu, 2 WsLarge;  dw_gemm: 0 StagedSmall, 2 DwWsLarge.
+// Defaults are the fastest measured on the 24576-token, 768/1024, 8-expert layer: the
+// kernels with heavy epilogues (gate/up, dY1) gain more from two co-resident blocks, the
+// longer reductions (down, dX, dW) from specialised waves.
+const int kDefaultTile[K_COUNT] = {1, 2, 1, 2, 2, 2};
 
 // tile shape per GEMM; the environment overrides exist for tuning runs only
 int tile_choice(int kind) {
@@ -927,7 +1069,7 @@ int tile_choice(int kind) {
         int c = kDefaultTile[kind];
         const char* s = getenv(kKindEnv[kind]);
         if (s) c = atoi(s);
-        choice[kind] = (c >= 0 && c <= 3) ? c : kDefaultTile[kind];
+        choice[kind] = (c >= 0 && c <= 2) ? c : kDefaultTile[kind];
     }
     return choice[kind];
 }
@@ -950,73 +1092,53 @@ int64_t m_tiles(int64_t TK, int E) {
 }
 
 template <class T, int EPI>
-int launch_rows(RowsParams p, int64_t TK, hipStream_t s) {
+dim3 rows_grid(RowsParams& p, int64_t TK) {
     const int per_block = (EPI == EPI_SWIGLU) ? T::BN / 2 : T::BN;
     p.n_tiles = (p.N + per_block - 1) / per_block;
     const int64_t m_groups = (m_tiles<T>(TK, p.E) + kXcds - 1) / kXcds;
-    dim3 grid((unsigned)(m_groups * kXcds * p.n_tiles));
-    rows_gemm_kernel<T, EPI><<<grid, T::NT, 0, s>>>(p);
-    MTS_CHECK_LAUNCH();
-    return MTS_OK;
-}
-
-template <class T, int EPI>
-int launch_ring(RowsParams p, int64_t TK, hipStream_t s) {
-    const int per_block = (EPI == EPI_SWIGLU) ? T::BN / 2 : T::BN;
-    p.n_tiles = (p.N + per_block - 1) / per_block;
-    const int64_t m_groups = (m_tiles<T>(TK, p.E) + kXcds - 1) / kXcds;
-    dim3 grid((unsigned)(m_groups * kXcds * p.n_tiles));
-    rows_gemm_ring_kernel<T, EPI><<<grid, T::NT, 0, s>>>(p);
-    MTS_CHECK_LAUNCH();
-    return MTS_OK;
+    return dim3((unsigned)(m_groups * kXcds * p.n_tiles));
 }
 
 template <int EPI>
-int launch_rows_any(int kind, const RowsParams& p, int64_t TK, hipStream_t s) {
+int launch_rows_any(int kind, RowsParams p, int64_t TK, hipStream_t s) {
     int choice = tile_choice(kind);
     // the ring kernels need whole k-tiles; other shapes use the staged kernel
     if (choice >= 1 && p.Kdim % 64 != 0) choice = 0;
-    switch (choice) {
-        case 1: return launch_ring<RingTwoPerCu, EPI>(p, TK, s);
-        case 2: return launch_ring<RingLarge, EPI>(p, TK, s);
-        case 3: return launch_ring<RingDeep, EPI>(p, TK, s);
-        default: return launch_rows<StagedSmall, EPI>(p, TK, s);
+    if (choice == 1) {
+        const dim3 grid = rows_grid<RingTwoPerCu, EPI>(p, TK);
+        rows_gemm_ring_kernel<RingTwoPerCu, EPI><<<grid, RingTwoPerCu::NT, 0, s>>>(p);
+    } else if (choice == 2) {
+        const dim3 grid = rows_grid<WsLarge, EPI>(p, TK);
+        rows_gemm_ws_kernel<WsLarge, EPI><<<grid, WsLarge::NT, 0, s>>>(p);
+    } else {
+        const dim3 grid = rows_grid<StagedSmall, EPI>(p, TK);
+        rows_gemm_kernel<StagedSmall, EPI><<<grid, StagedSmall::NT, 0, s>>>(p);
     }
-}
-
-template <class T>
-int launch_dw(DwParams p, int E, int grad_dtype, hipStream_t s) {
-    p.E = E;
-    p.n_tiles = (p.N + T::BN - 1) / T::BN;
-    p.tiles_per_expert = ((p.M + T::BM - 1) / T::BM) * p.n_tiles;
-    dim3 grid((unsigned)(((E + kXcds - 1) / kXcds) * kXcds * p.tiles_per_expert));
-    if (grad_dtype == MTS_BF16) dw_gemm_kernel<T, bf16_t><<<grid, T::NT, 0, s>>>(p);
-    else if (grad_dtype == MTS_F32) dw_gemm_kernel<T, float><<<grid, T::NT, 0, s>>>(p);
-    else return MTS_ERR_DTYPE;
     MTS_CHECK_LAUNCH();
     return MTS_OK;
 }
 
 template <class T>
-int launch_dw_ring(DwParams p, int E, int grad_dtype, hipStream_t s) {
+dim3 dw_grid(DwParams& p, int E) {
     p.E = E;
     p.n_tiles = (p.N + T::BN - 1) / T::BN;
     p.tiles_per_expert = ((p.M + T::BM - 1) / T::BM) * p.n_tiles;
-    dim3 grid((unsigned)(((E + kXcds - 1) / kXcds) * kXcds * p.tiles_per_expert));
-    if (grad_dtype == MTS_BF16) dw_gemm_ring_kernel<T, bf16_t><<<grid, T::NT, 0, s>>>(p);
-    else if (grad_dtype == MTS_F32) dw_gemm_ring_kernel<T, float><<<grid, T::NT, 0, s>>>(p);
-    else return MTS_ERR_DTYPE;
-    MTS_CHECK_LAUNCH();
-    return MTS_OK;
+    return dim3((unsigned)(((E + kXcds - 1) / kXcds) * kXcds * p.tiles_per_expert));
 }
 
-int launch_dw_any(int kind, const DwParams& p, int E, int grad_dtype, hipStream_t s) {
-    switch (tile_choice(kind)) {
-        case 1: return launch_dw<StagedLarge>(p, E, grad_dtype, s);
-        case 2: return launch_dw_ring<DwRingLarge>(p, E, grad_dtype, s);
-        case 3: return launch_dw_ring<DwRingWide>(p, E, grad_dtype, s);
-        default: return launch_dw<StagedSmall>(p, E, grad_dtype, s);
+int launch_dw_any(int kind, DwParams p, int E, int grad_dtype, hipStream_t s) {
+    if (grad_dtype != MTS_BF16 && grad_dtype != MTS_F32) return MTS_ERR_DTYPE;
+    if (tile_choice(kind) == 2) {
+        const dim3 grid = dw_grid<DwWsLarge>(p, E);
+        if (grad_dtype == MTS_BF16) dw_gemm_ws_kernel<DwWsLarge, bf16_t><<<grid, DwWsLarge::NT, 0, s>>>(p);
+        else dw_gemm_ws_kernel<DwWsLarge, float><<<grid, DwWsLarge::NT, 0, s>>>(p);
+    } else {
+        const dim3 grid = dw_grid<StagedSmall>(p, E);
+        if (grad_dtype == MTS_BF16) dw_gemm_kernel<StagedSmall, bf16_t><<<grid, StagedSmall::NT, 0, s>>>(p);
+        else dw_gemm_kernel<StagedSmall, float><<<grid, StagedSmall::NT, 0, s>>>(p);
     }
+    MTS_CHECK_LAUNCH();
+    return MTS_OK;
 }
 
 int dy1_partials(int I) { return (I + 63) / 64; }
