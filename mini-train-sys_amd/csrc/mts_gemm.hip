@@ -43,6 +43,25 @@ __device__ __forceinline__ int buf_load4(__amdgpu_buffer_rsrc_t r, uint32_t byte
     return (int)__builtin_amdgcn_raw_buffer_load_b32(r, (int)byte_off, 0, 0);
 }
 
+// Scalar buffer load of 8 consecutive dwords (read-only, through the scalar cache).  The
+// descriptor has the raw-buffer layout make_rsrc builds; offsets past `bytes` return 0.
+// The wait is part of the same statement: the compiler does not track the completion of a
+// load issued from inline assembly and may copy the result registers at any later point.
+typedef __attribute__((ext_vector_type(4))) int i32x4;
+__device__ __forceinline__ u32x4 scalar_rsrc(const void* p, int64_t bytes) {
+    const uint64_t a = (uint64_t)p;
+    u32x4 r = {(uint32_t)a, (uint32_t)(a >> 32) & 0xffffu, (uint32_t)bytes, 0x00020000u};
+    return r;
+}
+__device__ __forceinline__ void s_buffer_load8(u32x4 rsrc, int byte_off, i32x4& lo, i32x4& hi) {
+    asm volatile(
+        "s_buffer_load_dwordx4 %0, %2, %3\n\t"
+        "s_buffer_load_dwordx4 %1, %2, %4\n\t"
+        "s_waitcnt lgkmcnt(0)"
+        : "=&s"(lo), "=&s"(hi)
+        : "s"(rsrc), "s"(byte_off), "s"(byte_off + 16));
+}
+
 // element offset of 16-byte chunk `chunk` of row `row` inside a swizzled tile
 __device__ __forceinline__ int lds_off(int row, int chunk) {
     return row * BK + ((chunk ^ ((row >> 1) & 7)) << 3);
@@ -844,7 +863,7 @@ __global__ __launch_bounds__(T::NT) void dw_gemm_kernel(DwParams p) {
 // lanes, lane s addresses 4 consecutive columns of row s/4 and lane l receives the
 // 4 rows of column l.  The 16-byte chunk index of a row is XOR-swizzled with
 // 4*(row % 4) so that the 4 rows x 2 column halves read by 32 lanes cover all banks.
-// Source rows of a gathered operand come from a per-lane load of the row index, one
+// Source rows of a gathered operand come from a scalar load of the row indices, one
 // k-tile ahead.  Rows past the expert's end are fetched with an out-of-range offset
 // and arrive as zeros.
 //
@@ -852,15 +871,10 @@ __global__ __launch_bounds__(T::NT) void dw_gemm_kernel(DwParams p) {
 // instruction and, issue being in order, its MFMAs wait behind it; at about 25
 // B/clk/CU of L1 fill the load queue is full most of the time.  So 8 consumer waves
 // (two per SIMD) only read fragments and issue MFMAs, and 4 producer waves (one per
-// SIMD) only issue the tile loads, the row-index loads and an L2 prefetch, and a
-// blocked load never holds up the matrix pipe.  One barrier per k-tile joins them:
+// SIMD) only issue the tile loads and the row-index loads, and a blocked load never
+// holds up the matrix pipe.  One barrier per k-tile joins them:
 // producers arrive once tile kt has landed, consumers once they are done reading
 // tile kt-1.
-//
-// L2 prefetch: all tiles of an expert run on one XCD in lockstep and ask for the same
-// rows, so the unique data in flight per XCD is only what the ring holds; one 4-byte
-// load per producer lane, PD tiles ahead, pulls the lines of the operand that is read
-// in place into that XCD's L2 early (it lands in 256 bytes of LDS that nobody reads).
 // ---------------------------------------------------------------------------
 typedef __attribute__((ext_vector_type(4))) short s16x4;
 
@@ -897,14 +911,14 @@ struct DwWsTile {
     static constexpr int LDS_ELEMS = STAGES * STAGE;
     static_assert(A_INSTR >= 1 && B_INSTR >= 1 && A_INSTR * RPI_A * PRODUCERS == BKS && B_INSTR * RPI_B * PRODUCERS == BKS,
                   "loader split");
-    static_assert(STAGES >= 3 && STAGES <= 4 && (A_INSTR + B_INSTR + 1) * (STAGES - 2) <= 63, "vmcnt range");
-    static_assert(LDS_ELEMS * 2 + PRODUCERS * 256 <= 160 * 1024, "LDS capacity");
+    static_assert(STAGES >= 3 && STAGES <= 4 && (A_INSTR + B_INSTR) * (STAGES - 2) <= 63, "vmcnt range");
+    static_assert(LDS_ELEMS * 2 <= 160 * 1024, "LDS capacity");
 };
 
 template <class T, typename OutT>
 __global__ __launch_bounds__(T::NT) void dw_gemm_ws_kernel(DwParams p) {
-    __shared__ __attribute__((aligned(1024))) bf16_t smem[T::LDS_ELEMS + T::PRODUCERS * 128];
-    constexpr int S = T::STAGES, L = T::A_INSTR + T::B_INSTR, PD = 8;
+    __shared__ __attribute__((aligned(1024))) bf16_t smem[T::LDS_ELEMS];
+    constexpr int S = T::STAGES, L = T::A_INSTR + T::B_INSTR;
     const int xcd = blockIdx.x % kXcds, jb = blockIdx.x / kXcds;
     const int e = xcd + kXcds * (jb / p.tiles_per_expert);
     if (e >= p.E) return;
@@ -916,13 +930,23 @@ __global__ __launch_bounds__(T::NT) void dw_gemm_ws_kernel(DwParams p) {
 
     if (wave >= T::NWAVES) {
         // ------------------------------ producer ------------------------------
+        // The producer's own instruction count bounds the fill rate (a wave issues roughly one
+        // instruction per 4-8 clocks), so everything that does not change from tile to tile is
+        // computed once.  An operand that is read in place gets a descriptor that starts at the
+        // tile's first row and ends at the expert's last row, rebuilt with scalar instructions
+        // per tile: the per-lane offsets are constants and rows past the expert's end read as
+        // zeros.  A gathered operand takes its row indices through the scalar cache, fetched
+        // after the tile loads of the iteration were issued (a scalar load is counted by
+        // lgkmcnt, so waiting for it does not wait for the tile loads issued before it; vmcnt
+        // retires in order and a vector index load would drain the ring once per tile).
         const int pw = wave - T::NWAVES;
-        const __amdgpu_buffer_rsrc_t rs_p = make_rsrc(p.P, p.p_rows * p.M * 2);
-        const __amdgpu_buffer_rsrc_t rs_q = make_rsrc(p.Q, p.q_rows * p.N * 2);
         const bool gath_p = p.p_gather != nullptr, gath_q = p.q_gather != nullptr;
-        const __amdgpu_buffer_rsrc_t rs_gp = make_rsrc(p.p_gather, gath_p ? p.TK * 4 : 0);
-        const __amdgpu_buffer_rsrc_t rs_gq = make_rsrc(p.q_gather, gath_q ? p.TK * 4 : 0);
-        uint32_t col_a[T::A_INSTR], col_b[T::B_INSTR];
+        constexpr int ROWS_A = T::A_INSTR * T::RPI_A, ROWS_B = T::B_INSTR * T::RPI_B;
+        static_assert(T::RPI_A == 2 && T::RPI_B == 2 && T::CPR_A == T::CPR_B, "two rows per wave instruction");
+        static_assert(ROWS_A == 8 && ROWS_B == 8, "index fetch layout: 8 rows per producer wave");
+        const bool upper = lane >= T::CPR_A;
+        const uint32_t ld_a = (uint32_t)p.M * 2u, ld_b = (uint32_t)p.N * 2u;   // row pitch in bytes
+        uint32_t col_a[T::A_INSTR], col_b[T::B_INSTR], fix_a[T::A_INSTR], fix_b[T::B_INSTR];
         int rin_a[T::A_INSTR], rin_b[T::B_INSTR];
 #pragma unroll
         for (int j = 0; j < T::A_INSTR; ++j) {
@@ -930,6 +954,7 @@ __global__ __launch_bounds__(T::NT) void dw_gemm_ws_kernel(DwParams p) {
             const int c = m0 + (((lane % T::CPR_A) ^ ((tr & 3) << 2)) << 3);
             rin_a[j] = tr;
             col_a[j] = c < p.M ? (uint32_t)c * 2u : kInvalid;
+            fix_a[j] = c < p.M ? (uint32_t)tr * ld_a + (uint32_t)c * 2u : kInvalid;
         }
 #pragma unroll
         for (int j = 0; j < T::B_INSTR; ++j) {
@@ -937,45 +962,49 @@ __global__ __launch_bounds__(T::NT) void dw_gemm_ws_kernel(DwParams p) {
             const int c = n0 + (((lane % T::CPR_B) ^ ((tr & 3) << 2)) << 3);
             rin_b[j] = tr;
             col_b[j] = c < p.N ? (uint32_t)c * 2u : kInvalid;
+            fix_b[j] = c < p.N ? (uint32_t)tr * ld_b + (uint32_t)c * 2u : kInvalid;
         }
-        int src_a[T::A_INSTR], src_b[T::B_INSTR];
+        const __amdgpu_buffer_rsrc_t rs_p = make_rsrc(p.P, p.p_rows * p.M * 2);
+        const __amdgpu_buffer_rsrc_t rs_q = make_rsrc(p.Q, p.q_rows * p.N * 2);
+        const u32x4 rs_gp = scalar_rsrc(p.p_gather, gath_p ? p.TK * 4 : 0);
+        const u32x4 rs_gq = scalar_rsrc(p.q_gather, gath_q ? p.TK * 4 : 0);
+        i32x4 idx_a[ROWS_A / 4] = {}, idx_b[ROWS_B / 4] = {};
         auto fetch_index = [&](int r0) {
-#pragma unroll
-            for (int j = 0; j < T::A_INSTR; ++j)
-                src_a[j] = gath_p ? buf_load4(rs_gp, (uint32_t)(r0 + rin_a[j]) * 4u) : r0 + rin_a[j];
-#pragma unroll
-            for (int j = 0; j < T::B_INSTR; ++j)
-                src_b[j] = gath_q ? buf_load4(rs_gq, (uint32_t)(r0 + rin_b[j]) * 4u) : r0 + rin_b[j];
+            if (gath_p) s_buffer_load8(rs_gp, (r0 + pw * ROWS_A) * 4, idx_a[0], idx_a[1]);
+            if (gath_q) s_buffer_load8(rs_gq, (r0 + pw * ROWS_B) * 4, idx_b[0], idx_b[1]);
         };
         auto issue = [&](int stage, int r0) {
             bf16_t* sa = smem + stage * T::STAGE + pw * T::A_INSTR * 512;
             bf16_t* sb = smem + stage * T::STAGE + T::BKS * T::BM + pw * T::B_INSTR * 512;
+            const int left = rend - r0;   // rows of the expert from this tile on
+            if (gath_p) {
 #pragma unroll
-            for (int j = 0; j < T::A_INSTR; ++j) {
-                const bool ok = r0 + rin_a[j] < rend && col_a[j] != kInvalid;
-                const uint32_t off = ok ? (uint32_t)src_a[j] * (uint32_t)p.M * 2u + col_a[j] : kInvalid;
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_p, MTS_LDS_PTR(sa + j * 512), 16, (int)off, 0, 0, 0);
-            }
+                for (int j = 0; j < T::A_INSTR; ++j) {
+                    const uint32_t lo = (uint32_t)idx_a[(2 * j) / 4][(2 * j) % 4] * ld_a;
+                    const uint32_t hi = (uint32_t)idx_a[(2 * j + 1) / 4][(2 * j + 1) % 4] * ld_a;
+                    const uint32_t off = rin_a[j] < left ? (upper ? hi : lo) + col_a[j] : kInvalid;
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_p, MTS_LDS_PTR(sa + j * 512), 16, (int)off, 0, 0, 0);
+                }
+            } else {
+                const __amdgpu_buffer_rsrc_t rs = make_rsrc(p.P + (int64_t)r0 * p.M, (int64_t)left * p.M * 2);
 #pragma unroll
-            for (int j = 0; j < T::B_INSTR; ++j) {
-                const bool ok = r0 + rin_b[j] < rend && col_b[j] != kInvalid;
-                const uint32_t off = ok ? (uint32_t)src_b[j] * (uint32_t)p.N * 2u + col_b[j] : kInvalid;
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_q, MTS_LDS_PTR(sb + j * 512), 16, (int)off, 0, 0, 0);
+                for (int j = 0; j < T::A_INSTR; ++j)
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, MTS_LDS_PTR(sa + j * 512), 16, (int)fix_a[j], 0, 0, 0);
             }
-        };
-        // L2 prefetch of the operand that is read in place, PD tiles ahead
-        const bool touch_p = !gath_p, touch_any = touch_p || !gath_q;
-        const __amdgpu_buffer_rsrc_t rs_t = touch_p ? rs_p : rs_q;
-        const int t_ld = touch_p ? p.M : p.N, t_col0 = touch_p ? m0 : n0, t_w = touch_p ? T::BM : T::BN;
-        constexpr int PPR = T::PRODUCERS * MTS_WAVE / T::BKS;
-        const int pt = pw * MTS_WAVE + lane;
-        const int t_row = pt / PPR, t_piece = (pt % PPR) * (t_w / PPR);
-        bf16_t* t_dst = smem + T::LDS_ELEMS + pw * 128;
-        auto touch = [&](int r0) {
-            const int r = r0 + t_row, c = t_col0 + t_piece;
-            const bool ok = touch_any && r < rend && c < t_ld;
-            const uint32_t off = ok ? ((uint32_t)r * (uint32_t)t_ld + (uint32_t)c) * 2u : kInvalid;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_t, MTS_LDS_PTR(t_dst), 4, (int)off, 0, 0, 0);
+            if (gath_q) {
+#pragma unroll
+                for (int j = 0; j < T::B_INSTR; ++j) {
+                    const uint32_t lo = (uint32_t)idx_b[(2 * j) / 4][(2 * j) % 4] * ld_b;
+                    const uint32_t hi = (uint32_t)idx_b[(2 * j + 1) / 4][(2 * j + 1) % 4] * ld_b;
+                    const uint32_t off = rin_b[j] < left ? (upper ? hi : lo) + col_b[j] : kInvalid;
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_q, MTS_LDS_PTR(sb + j * 512), 16, (int)off, 0, 0, 0);
+                }
+            } else {
+                const __amdgpu_buffer_rsrc_t rs = make_rsrc(p.Q + (int64_t)r0 * p.N, (int64_t)left * p.N * 2);
+#pragma unroll
+                for (int j = 0; j < T::B_INSTR; ++j)
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, MTS_LDS_PTR(sb + j * 512), 16, (int)fix_b[j], 0, 0, 0);
+            }
         };
 
 #pragma unroll
@@ -988,17 +1017,13 @@ __global__ __launch_bounds__(T::NT) void dw_gemm_ws_kernel(DwParams p) {
         if (S - 1 < nk) fetch_index(rbeg + (S - 1) * T::BKS);
         int stage = 0;
         for (int kt = 0; kt < nk; ++kt) {
-            // tile kt has landed when at most the loads issued after it are outstanding: per later
-            // iteration one prefetch load and L tile loads (index loads are left out of the count,
-            // which only makes the wait a little longer)
+            // tile kt has landed when at most the L loads of each later tile are outstanding
             const int younger = nk - 1 - kt;
-            if (S >= 4 && younger >= 2) wait_vmcnt<(L + 1) * (S >= 4 ? 2 : 0)>();
+            if (S >= 4 && younger >= 2) wait_vmcnt<L * (S >= 4 ? 2 : 0)>();
             else if (younger >= 1) wait_vmcnt<L>();
             else wait_vmcnt<0>();
-            __builtin_amdgcn_s_barrier();
-            const int rstage = stage == 0 ? S - 1 : stage - 1;
-            touch(rbeg + (kt + PD) * T::BKS);
-            if (kt + S - 1 < nk) issue(rstage, rbeg + (kt + S - 1) * T::BKS);
+            __builtin_amdgcn_s_barrier();   // tile kt is visible; every consumer is done with tile kt-1
+            if (kt + S - 1 < nk) issue(stage == 0 ? S - 1 : stage - 1, rbeg + (kt + S - 1) * T::BKS);
             if (kt + S < nk) fetch_index(rbeg + (kt + S) * T::BKS);
             stage = stage + 1 == S ? 0 : stage + 1;
         }
