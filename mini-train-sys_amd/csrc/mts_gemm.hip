@@ -183,6 +183,63 @@ __device__ __forceinline__ void mma_tile(const bf16_t* As, const bf16_t* Bs, int
     }
 }
 
+// Fragment pipeline of a consumer wave that runs across k-tiles: the LDS reads of the next
+// 16-wide k-step (of this tile or of the next one) are in flight while the MFMAs of the
+// current step are issued, so the matrix pipe does not idle at the start of a k-tile.
+// Weight fragments are double buffered; an activation fragment is reloaded for the next
+// k-step right behind the MFMAs that used it.
+template <class T, bool SWIGLU, int ROWLEN>
+struct FragPipe {
+    static constexpr int KSTEPS = ROWLEN / 16;
+    static_assert(KSTEPS % 2 == 0, "weight fragment buffers alternate with the k-step");
+    bf16x8 a[T::MF], b[2][T::NF];
+    int a_off, b_off[T::NF], swz, kb;
+
+    __device__ __forceinline__ void init(int wm, int wn) {
+        const int lane = threadIdx.x % MTS_WAVE;
+        const int frow = lane % 32;
+        kb = lane / 32;
+        swz = ROWLEN == 64 ? (frow >> 1) & 7 : (frow >> 2) & 3;
+        a_off = (wm * T::WM + frow) * ROWLEN;
+#pragma unroll
+        for (int nf = 0; nf < T::NF; ++nf) {
+            int brow;
+            if (SWIGLU) {
+                constexpr int HALF = T::NF / 2;
+                brow = (nf / HALF) * (T::BN / 2) + wn * (T::WN / 2) + (nf % HALF) * 32;
+            } else {
+                brow = wn * T::WN + nf * 32;
+            }
+            b_off[nf] = T::BM * ROWLEN + (brow + frow) * ROWLEN;
+        }
+    }
+    __device__ __forceinline__ int chunk_off(int ks) const { return ((ks * 2 + kb) ^ swz) << 3; }
+    // all fragments of k-step 0 of the stage at `tile`
+    __device__ __forceinline__ void prime(const bf16_t* tile) {
+        const int coff = chunk_off(0);
+#pragma unroll
+        for (int mf = 0; mf < T::MF; ++mf)
+            a[mf] = *reinterpret_cast<const bf16x8*>(tile + a_off + mf * 32 * ROWLEN + coff);
+#pragma unroll
+        for (int nf = 0; nf < T::NF; ++nf) b[0][nf] = *reinterpret_cast<const bf16x8*>(tile + b_off[nf] + coff);
+    }
+    // MFMAs of k-step `ks` (weight fragment first); behind them, the fragments of k-step `nks`
+    // of the stage at `next` are read: the weight fragments up front into the other buffer, each
+    // activation fragment as soon as its MFMAs are issued
+    __device__ __forceinline__ void step(int ks, f32x16 (&acc)[T::MF][T::NF], const bf16_t* next, int nks) {
+        const int coff = chunk_off(nks), buf = ks & 1;
+#pragma unroll
+        for (int nf = 0; nf < T::NF; ++nf) b[buf ^ 1][nf] = *reinterpret_cast<const bf16x8*>(next + b_off[nf] + coff);
+#pragma unroll
+        for (int mf = 0; mf < T::MF; ++mf) {
+#pragma unroll
+            for (int nf = 0; nf < T::NF; ++nf)
+                acc[mf][nf] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[buf][nf], a[mf], acc[mf][nf], 0, 0, 0);
+            a[mf] = *reinterpret_cast<const bf16x8*>(next + a_off + mf * 32 * ROWLEN + coff);
+        }
+    }
+};
+
 __device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + __expf(-x)); }
 
 template <class T>
@@ -674,20 +731,23 @@ __global__ __launch_bounds__(T::NT, T::WAVES_PER_EU) void rows_gemm_ws_kernel(Ro
             for (int j = 0; j < T::B_INSTR; ++j)
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_b, MTS_LDS_PTR(sb + j * 512), 16, (int)voff_b[j], soff, 0, 0);
         };
+        // Barrier kt tells the consumers that tiles kt and kt+1 have landed (they read the first
+        // fragments of tile kt+1 behind the last MFMAs of tile kt) and tells the producers that
+        // every consumer is done with tile kt-1, whose stage then takes tile kt-1+S.
 #pragma unroll
-        for (int s = 0; s < S - 1; ++s)
+        for (int s = 0; s < S; ++s)
             if (s < nk) issue(s, s);
-        int stage = 0;
+        int stage = S - 1;   // stage of tile kt-1
         for (int kt = 0; kt < nk; ++kt) {
-            const int younger = nk - 1 - kt;
-            if (S >= 4 && younger >= 2) wait_vmcnt<L * (S >= 4 ? 2 : 0)>();
-            else if (younger >= 1) wait_vmcnt<L>();
+            // tiles up to kt+1 must have landed; tile kt+2 (and, before barrier 0, tile 3) may be in flight
+            if (kt == 0 && S >= 4 && nk >= 4) wait_vmcnt<L * (S >= 4 ? 2 : 0)>();
+            else if (S >= 3 && kt + 2 < nk) wait_vmcnt<L>();
             else wait_vmcnt<0>();
-            __builtin_amdgcn_s_barrier();   // tile kt is visible; every consumer is done with tile kt-1
-            if (kt + S - 1 < nk) issue(stage == 0 ? S - 1 : stage - 1, kt + S - 1);
+            __builtin_amdgcn_s_barrier();
+            if (kt >= 1 && kt - 1 + S < nk) issue(stage, kt - 1 + S);
             stage = stage + 1 == S ? 0 : stage + 1;
         }
-        __builtin_amdgcn_s_barrier();       // matches the consumers' barrier before the epilogue
+        __builtin_amdgcn_s_barrier();       // matches the consumers' barrier behind the last tile
         return;
     }
 
@@ -695,14 +755,24 @@ __global__ __launch_bounds__(T::NT, T::WAVES_PER_EU) void rows_gemm_ws_kernel(Ro
     const int wm = wave / T::WAVES_N, wn = wave % T::WAVES_N;
     f32x16 acc[T::MF][T::NF];
     zero_acc<T>(acc);
+    FragPipe<T, SWIGLU, T::BKS> pipe;
+    pipe.init(wm, wn);
+    constexpr int KSTEPS = T::BKS / 16;
+    __builtin_amdgcn_s_barrier();   // tiles 0 and 1 are visible
+    pipe.prime(smem);
     int stage = 0;
     for (int kt = 0; kt < nk; ++kt) {
-        __builtin_amdgcn_s_barrier();
         const bf16_t* cur = smem + stage * T::STAGE;
-        mma_tile<T, SWIGLU, T::BKS>(cur, cur + T::BM * T::BKS, wm, wn, acc);
         stage = stage + 1 == S ? 0 : stage + 1;
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS - 1; ++ks) pipe.step(ks, acc, cur, ks + 1);
+        // behind the last k-step the first fragments of tile kt+1 are read (after the last tile
+        // this reads a stage nobody uses: harmless)
+        pipe.step(KSTEPS - 1, acc, smem + stage * T::STAGE, 0);
+        // tile kt+2 is visible after this barrier and tile kt may be overwritten; behind the last
+        // tile it is the barrier that frees the ring for the epilogue
+        __builtin_amdgcn_s_barrier();
     }
-    __builtin_amdgcn_s_barrier();  // every consumer is done reading the ring before it is reused
     rows_epilogue<T, EPI>(p, acc, smem, row0, rend, n0, wm, wn);
 }
 
@@ -1007,52 +1077,71 @@ __global__ __launch_bounds__(T::NT) void dw_gemm_ws_kernel(DwParams p) {
             }
         };
 
+        // Barrier kt tells the consumers that tiles kt and kt+1 have landed (they read the first
+        // fragments of tile kt+1 behind the last MFMAs of tile kt) and tells the producers that
+        // every consumer is done with tile kt-1, whose stage then takes tile kt-1+S.
 #pragma unroll
-        for (int s = 0; s < S - 1; ++s) {
+        for (int s = 0; s < S; ++s) {
             if (s < nk) {
                 fetch_index(rbeg + s * T::BKS);
                 issue(s, rbeg + s * T::BKS);
             }
         }
-        if (S - 1 < nk) fetch_index(rbeg + (S - 1) * T::BKS);
-        int stage = 0;
+        if (S < nk) fetch_index(rbeg + S * T::BKS);
+        int stage = S - 1;   // stage of tile kt-1
         for (int kt = 0; kt < nk; ++kt) {
-            // tile kt has landed when at most the L loads of each later tile are outstanding
-            const int younger = nk - 1 - kt;
-            if (S >= 4 && younger >= 2) wait_vmcnt<L * (S >= 4 ? 2 : 0)>();
-            else if (younger >= 1) wait_vmcnt<L>();
+            // tiles up to kt+1 must have landed; tile kt+2 (and, before barrier 0, tile 3) may be in flight
+            if (kt == 0 && S >= 4 && nk >= 4) wait_vmcnt<L * (S >= 4 ? 2 : 0)>();
+            else if (kt + 2 < nk) wait_vmcnt<L>();
             else wait_vmcnt<0>();
-            __builtin_amdgcn_s_barrier();   // tile kt is visible; every consumer is done with tile kt-1
-            if (kt + S - 1 < nk) issue(stage == 0 ? S - 1 : stage - 1, rbeg + (kt + S - 1) * T::BKS);
-            if (kt + S < nk) fetch_index(rbeg + (kt + S) * T::BKS);
+            __builtin_amdgcn_s_barrier();
+            if (kt >= 1 && kt - 1 + S < nk) {
+                issue(stage, rbeg + (kt - 1 + S) * T::BKS);
+                if (kt + S < nk) fetch_index(rbeg + (kt + S) * T::BKS);
+            }
             stage = stage + 1 == S ? 0 : stage + 1;
         }
+        __builtin_amdgcn_s_barrier();   // matches the consumers' barrier behind the last tile
         return;
     }
 
     // -------------------------------- consumer --------------------------------
+    // Fragments run one k-step ahead of the MFMAs, across tile boundaries: Q fragments are
+    // double buffered, a P fragment is reloaded right behind the MFMAs that used it.
     const int wm = wave / T::WAVES_N, wn = wave % T::WAVES_N;
     f32x16 acc[T::MF][T::NF];
     zero_acc<T>(acc);
+    constexpr int KSTEPS = T::BKS / 16;
+    static_assert(KSTEPS % 2 == 0, "fragment buffers alternate with the k-step");
+    bf16x8 fa[T::MF], fb[2][T::NF];
+    auto step = [&](int ks, const bf16_t* next, int nks) {
+        const bf16_t* nB = next + T::BKS * T::BM;
+        const int buf = ks & 1;
+#pragma unroll
+        for (int nf = 0; nf < T::NF; ++nf) fb[buf ^ 1][nf] = read_frag_tr<T::BN>(nB, nks * 16, wn * T::WN + nf * 32);
+#pragma unroll
+        for (int mf = 0; mf < T::MF; ++mf) {
+#pragma unroll
+            for (int nf = 0; nf < T::NF; ++nf)
+                acc[mf][nf] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[mf], fb[buf][nf], acc[mf][nf], 0, 0, 0);
+            fa[mf] = read_frag_tr<T::BM>(next, nks * 16, wm * T::WM + mf * 32);
+        }
+    };
+    __builtin_amdgcn_s_barrier();   // tiles 0 and 1 are visible
+#pragma unroll
+    for (int mf = 0; mf < T::MF; ++mf) fa[mf] = read_frag_tr<T::BM>(smem, 0, wm * T::WM + mf * 32);
+#pragma unroll
+    for (int nf = 0; nf < T::NF; ++nf) fb[0][nf] = read_frag_tr<T::BN>(smem + T::BKS * T::BM, 0, wn * T::WN + nf * 32);
     int stage = 0;
     for (int kt = 0; kt < nk; ++kt) {
-        __builtin_amdgcn_s_barrier();
-        const bf16_t* As = smem + stage * T::STAGE;
-        const bf16_t* Bs = As + T::BKS * T::BM;
-#pragma unroll
-        for (int ks = 0; ks < T::BKS / 16; ++ks) {
-            bf16x8 b[T::NF];
-#pragma unroll
-            for (int nf = 0; nf < T::NF; ++nf) b[nf] = read_frag_tr<T::BN>(Bs, ks * 16, wn * T::WN + nf * 32);
-#pragma unroll
-            for (int mf = 0; mf < T::MF; ++mf) {
-                const bf16x8 a = read_frag_tr<T::BM>(As, ks * 16, wm * T::WM + mf * 32);
-#pragma unroll
-                for (int nf = 0; nf < T::NF; ++nf)
-                    acc[mf][nf] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b[nf], acc[mf][nf], 0, 0, 0);
-            }
-        }
+        const bf16_t* cur = smem + stage * T::STAGE;
         stage = stage + 1 == S ? 0 : stage + 1;
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS - 1; ++ks) step(ks, cur, ks + 1);
+        // behind the last k-step the first fragments of tile kt+1 are read (after the last tile
+        // this reads a stage nobody uses: harmless)
+        step(KSTEPS - 1, smem + stage * T::STAGE, 0);
+        __builtin_amdgcn_s_barrier();   // tile kt+2 is visible, tile kt may be overwritten
     }
 
     OutT* C = reinterpret_cast<OutT*>(p.C) + (int64_t)e * p.M * p.N;
@@ -1135,6 +1224,7 @@ int launch_rows_any(int kind, RowsParams p, int64_t TK, hipStream_t s) {
     } else if (choice == 2) {
         const dim3 grid = rows_grid<WsLarge, EPI>(p, TK);
         rows_gemm_ws_kernel<WsLarge, EPI><<<grid, WsLarge::NT, 0, s>>>(p);
+
     } else {
         const dim3 grid = rows_grid<StagedSmall, EPI>(p, TK);
         rows_gemm_kernel<StagedSmall, EPI><<<grid, StagedSmall::NT, 0, s>>>(p);
