@@ -311,6 +311,16 @@ __device__ __forceinline__ void rows_epilogue(const RowsParams& p, f32x16 (&acc)
     const __amdgpu_buffer_rsrc_t rs_c2 = make_rsrc(p.C2, EPI == EPI_PLAIN ? 0 : p.TK * (int64_t)N * 2);
     const __amdgpu_buffer_rsrc_t rs_pre = make_rsrc(p.pre_act, EPI == EPI_DY1 ? p.TK * (int64_t)N * 4 : 0);
 
+    // routing weight of each of the lane's rows (dY1 only): two dependent loads, issued for all
+    // rows up front
+    float srow[T::MF];
+    if (EPI == EPI_DY1) {
+#pragma unroll
+        for (int mf = 0; mf < T::MF; ++mf) {
+            const int row = row0 + wm * T::WM + mf * 32 + ml;
+            srow[mf] = row < rend ? (float)p.route_w[p.s_scatter[row]] : 0.f;
+        }
+    }
 #pragma unroll
     for (int mf = 0; mf < T::MF; ++mf) {
         const int rowg0 = row0 + wm * T::WM + mf * 32;
@@ -346,19 +356,34 @@ __device__ __forceinline__ void rows_epilogue(const RowsParams& p, f32x16 (&acc)
         } else {  // EPI_DY1
             const int row = rowg0 + ml;
             const bool rok = row < rend;
-            float s = 0.f;
-            if (rok) s = (float)p.route_w[p.s_scatter[row]];
+            const float s = srow[mf];
+            // gate and up pre-activations of the wave's 32 x COLS tile: row-contiguous 16-byte
+            // loads, staged in the buffers that take d_gate and d_up afterwards (a lane reads
+            // exactly the positions it overwrites)
+            {
+                constexpr int LPR = COLS / 8, RPI = MTS_WAVE / LPR;
+                const int c = (lane % LPR) * 8;
+#pragma unroll
+                for (int it = 0; it < 32 / RPI; ++it) {
+                    const int r = it * RPI + lane / LPR;
+                    const int grow = rowg0 + r;
+                    const bool ok = grow < rend && ncol0 + c < p.N;
+                    const uint32_t po = ok ? ((uint32_t)grow * 2u * N + (uint32_t)(ncol0 + c)) * 2u : kInvalid;
+                    const u32x4 gv = buf_load16(rs_pre, po);
+                    const u32x4 uv = buf_load16(rs_pre, po == kInvalid ? kInvalid : po + N * 2u);
+                    *reinterpret_cast<u32x4*>(buf1 + r * LDW + c) = gv;
+                    *reinterpret_cast<u32x4*>(buf2 + r * LDW + c) = uv;
+                }
+            }
             float dsp = 0.f;
 #pragma unroll
             for (int nf = 0; nf < T::NF; ++nf)
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const int nl = nf * 32 + 8 * j + nq;   // column inside the wave tile
-                    const int n = ncol0 + nl;
-                    const uint32_t po = (rok && n < p.N) ? ((uint32_t)row * 2u * N + (uint32_t)n) * 2u : kInvalid;
-                    const uint2 gr = __builtin_bit_cast(uint2, __builtin_amdgcn_raw_buffer_load_b64(rs_pre, (int)po, 0, 0));
-                    const uint2 ur = __builtin_bit_cast(
-                        uint2, __builtin_amdgcn_raw_buffer_load_b64(rs_pre, (int)(po == kInvalid ? kInvalid : po + N * 2u), 0, 0));
+                    const int o = ml * LDW + nl;
+                    const uint2 gr = *reinterpret_cast<const uint2*>(buf1 + o);
+                    const uint2 ur = *reinterpret_cast<const uint2*>(buf2 + o);
                     float wa[4], dg[4], du[4];
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
@@ -375,7 +400,6 @@ __device__ __forceinline__ void rows_epilogue(const RowsParams& p, f32x16 (&acc)
                         dg[q] = da * (silu * (1.0f - sig) + sig) * u;
                         du[q] = da * silu;
                     }
-                    const int o = ml * LDW + nl;
                     stage4(buf0 + o, wa[0], wa[1], wa[2], wa[3]);
                     stage4(buf1 + o, dg[0], dg[1], dg[2], dg[3]);
                     stage4(buf2 + o, du[0], du[1], du[2], du[3]);
@@ -671,7 +695,7 @@ struct WsTile {
     static_assert(BKS == 32 || BKS == 64, "LDS rows are 64 or 128 bytes");
     static_assert(WM % 32 == 0 && WN % 64 == 0, "wave tile must hold whole 32x32 fragments");
     static_assert(A_INSTR * RPI * PRODUCERS == BM && B_INSTR * RPI * PRODUCERS == BN, "loader split");
-    static_assert(STAGES >= 3 && STAGES <= 4 && (A_INSTR + B_INSTR) * (STAGES - 2) <= 63, "vmcnt range");
+    static_assert(STAGES == 4 && (A_INSTR + B_INSTR) * 2 <= 63, "the producer waits are written for a 4-stage ring");
     static_assert(LDS_ELEMS * 2 <= 160 * 1024, "LDS capacity");
 };
 
@@ -981,7 +1005,7 @@ struct DwWsTile {
     static constexpr int LDS_ELEMS = STAGES * STAGE;
     static_assert(A_INSTR >= 1 && B_INSTR >= 1 && A_INSTR * RPI_A * PRODUCERS == BKS && B_INSTR * RPI_B * PRODUCERS == BKS,
                   "loader split");
-    static_assert(STAGES >= 3 && STAGES <= 4 && (A_INSTR + B_INSTR) * (STAGES - 2) <= 63, "vmcnt range");
+    static_assert(STAGES == 4 && (A_INSTR + B_INSTR) * 2 <= 63, "the producer waits are written for a 4-stage ring");
     static_assert(LDS_ELEMS * 2 <= 160 * 1024, "LDS capacity");
 };
 
@@ -1224,6 +1248,7 @@ int launch_rows_any(int kind, RowsParams p, int64_t TK, hipStream_t s) {
     } else if (choice == 2) {
         const dim3 grid = rows_grid<WsLarge, EPI>(p, TK);
         rows_gemm_ws_kernel<WsLarge, EPI><<<grid, WsLarge::NT, 0, s>>>(p);
+
 
     } else {
         const dim3 grid = rows_grid<StagedSmall, EPI>(p, TK);
