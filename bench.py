@@ -74,9 +74,16 @@ class Layer:
     def step(self):
         for t in (self.x, self.w_r, self.w1, self.w2):
             t.grad = None
-        logits = F.linear(self.x.float(), self.w_r)
+        fused = getattr(self.ops, "router_logits", None)
+        logits = fused(self.x, self.w_r) if fused is not None else None
+        if logits is None:
+            logits = F.linear(self.x.float(), self.w_r)
         route = self.ops.router_postprocess(logits, self.K, normalize=True)
-        counts = torch.bincount(route.expert_indices.flatten().long(), minlength=self.E)
+        count_routes = getattr(self.ops, "expert_counts", None)
+        if count_routes is not None:
+            counts = count_routes(route.expert_indices, self.E)
+        else:
+            counts = torch.bincount(route.expert_indices.flatten().long(), minlength=self.E)
         aux = self.E * torch.sum(counts.float() / route.expert_indices.numel() * route.probability_per_expert)
         out = self.ops.fused_moe(self.x, self.w1, self.w2, route.expert_indices, route.expert_weights.to(self.x.dtype))
         loss_side = 0.01 * aux + 0.001 * route.z_loss

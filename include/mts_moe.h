@@ -64,6 +64,23 @@ int mts_router_bwd(const float* logits, const float* weights, const int32_t* ind
                    const float* g_weights, const float* g_prob_mean, const float* g_z_loss,
                    int64_t T, int E, int K, int normalize, float* dlogits, void* stream);
 
+/* ---- router projection ----------------------------------------------------
+ * Replaces the fp32 router GEMM of TopKRouter.forward and its autograd backward
+ * (minitrain/model/moe_router.py:64-76: `hidden_states.float()` followed by
+ * `F.linear(router_input, weight.float())`): logits[t,e] = sum_h float(x[t,h]) * w_r[e,h],
+ * fp32 products and sums, x [T,H] read in act_dtype (no fp32 copy), w_r [E,H] f32.
+ * E <= 16, H a multiple of 4.                                                  */
+int mts_router_logits_fwd(const void* x, const float* w_r, int64_t T, int H, int E,
+                          int act_dtype, float* logits, void* stream);
+
+/* dx[t,h] = sum_e dlogits[t,e] * w_r[e,h] (written in act_dtype, the cast the autograd
+ * of `.float()` applies), d_w_r[e,h] = sum_t dlogits[t,e] * float(x[t,h]) (f32; partial
+ * sums per block of rows in the workspace, added in a fixed order).  H <= 1024.   */
+int64_t mts_router_logits_bwd_workspace_bytes(int64_t T, int H, int E);
+int mts_router_logits_bwd(const float* dlogits, const void* x, const float* w_r, int64_t T,
+                          int H, int E, int act_dtype, void* dx, float* d_w_r,
+                          void* workspace, int64_t workspace_bytes, void* stream);
+
 /* ---- routing metadata ---------------------------------------------------
  * Replaces compute_routing_metadata (minitrain/kernels/triton/fused_moe.py:74-154)
  * and its three kernels (fused_moe_kernels.py:25-234): per-expert counts [E],
@@ -71,6 +88,9 @@ int mts_router_bwd(const float* logits, const float* weights, const int32_t* ind
  * entry, s_reverse [TK]: entry -> row, x_gather [TK]: row -> token) and, when
  * tile_row_start/tile_expert/tile_count are not NULL, the list of block_m-row
  * tiles (capacity min(TK, ceil(TK/block_m)+E-1) each, tile_count [1]).
+ * s_scatter, s_reverse and x_gather may all be NULL: then only counts and
+ * expert_start (and the tile list) are written, which is what the router module
+ * needs in place of its torch.bincount (minitrain/model/moe_router.py:82).
  * Returns MTS_ERR_SHAPE if E > MTS_MAX_EXPERTS; indices outside [0,E) are a
  * caller error: they are clamped into range (memory-safe, result undefined).                        */
 int64_t mts_moe_route_workspace_bytes(int64_t T, int K, int E);

@@ -170,9 +170,11 @@ extern "C" int mts_moe_route(const int32_t* top_k_index, int64_t T, int K, int E
                              int32_t* s_reverse, int32_t* x_gather, int32_t* tile_row_start,
                              int32_t* tile_expert, int32_t* tile_count, void* workspace,
                              int64_t workspace_bytes, void* stream) {
-    if (!top_k_index || !counts || !expert_start || !s_scatter || !s_reverse || !x_gather ||
-        !workspace)
-        return MTS_ERR_NULL;
+    // the three permutation arrays are optional as a group: without them only the counts,
+    // the expert offsets and (if asked for) the tile list are produced
+    const bool permute = s_scatter || s_reverse || x_gather;
+    if (!top_k_index || !counts || !expert_start || !workspace) return MTS_ERR_NULL;
+    if (permute && (!s_scatter || !s_reverse || !x_gather)) return MTS_ERR_NULL;
     if (T <= 0 || K < 1 || E < 1 || E > MTS_MAX_EXPERTS || block_m < 1 ||
         T * (int64_t)K > 0x7fffffffLL)
         return MTS_ERR_SHAPE;
@@ -188,6 +190,7 @@ extern "C" int mts_moe_route(const int32_t* top_k_index, int64_t T, int K, int E
     route_scan_kernel<<<1, 1024, 0, s>>>(cnt, n_chunks, E, TK, block_m, counts, expert_start,
                                          tile_row_start, tile_expert, tile_count);
     MTS_CHECK_LAUNCH();
+    if (!permute) return MTS_OK;
     route_scatter_kernel<<<grid, kThreads, lds, s>>>(top_k_index, TK, K, E, cnt, expert_start,
                                                      s_scatter, s_reverse, x_gather);
     MTS_CHECK_LAUNCH();

@@ -6,8 +6,13 @@ that class there is no fallback: an unsupported tensor contract raises.
 """
 
 from minitrain_amd.kernels.dense_ops import DenseTorchOps
-from minitrain_amd.kernels.hip.fused_moe import fused_moe, is_fused_moe_supported
-from minitrain_amd.kernels.hip.router import is_router_postprocess_supported, router_postprocess
+from minitrain_amd.kernels.hip.fused_moe import expert_counts, fused_moe, is_fused_moe_supported
+from minitrain_amd.kernels.hip.router import (
+    is_router_logits_supported,
+    is_router_postprocess_supported,
+    router_logits,
+    router_postprocess,
+)
 
 
 class HipOpsBackend(DenseTorchOps):
@@ -19,11 +24,26 @@ class HipOpsBackend(DenseTorchOps):
     def fused_moe(self, x, gate_up_proj, down_proj, top_k_index, top_k_weights):
         return fused_moe(x, gate_up_proj, down_proj, top_k_index, top_k_weights)
 
+    def expert_counts(self, expert_indices, num_experts):
+        """Extension: routes per expert (int32 ``[E]``) without a host synchronisation."""
+        return expert_counts(expert_indices, num_experts)
+
+    def router_logits(self, hidden_states, weight):
+        """Extension beyond the reference's operator interface: the router projection in fp32
+        straight from the activation dtype.  Returns None when the contract is not supported,
+        and the caller then runs its own ``F.linear``."""
+        if not is_router_logits_supported(hidden_states, weight):
+            return None
+        return router_logits(hidden_states, weight)
+
 
 __all__ = [
     "HipOpsBackend",
+    "expert_counts",
     "fused_moe",
     "is_fused_moe_supported",
+    "is_router_logits_supported",
     "is_router_postprocess_supported",
+    "router_logits",
     "router_postprocess",
 ]

@@ -102,6 +102,31 @@ def compute_routing_metadata(topk_indices: torch.Tensor, E: int, block_m_token: 
     )
 
 
+def expert_counts(topk_indices: torch.Tensor, E: int) -> torch.Tensor:
+    """Routes per expert, int32 ``[E]``: the histogram pass of the routing metadata alone.
+
+    Stands in for ``torch.bincount(expert_indices.flatten().long(), minlength=E)`` of the
+    router module (minitrain/model/moe_router.py:82) without its host synchronisation.
+    """
+    lib = _lib.load()
+    topk_indices = topk_indices.contiguous()
+    if topk_indices.dtype != torch.int32 or topk_indices.ndim != 2 or not topk_indices.is_cuda:
+        raise RuntimeError("hip expert_counts requires a 2D int32 index tensor on the GPU")
+    T, K = topk_indices.shape
+    dev = topk_indices.device
+    out = torch.empty(2 * E + 1, dtype=torch.int32, device=dev)   # counts, then expert_start
+    ws_bytes = lib.mts_moe_route_workspace_bytes(T, K, E)
+    ws = torch.empty(max(ws_bytes, 4), dtype=torch.uint8, device=dev)
+    _lib.check(
+        lib.mts_moe_route(
+            topk_indices.data_ptr(), T, K, E, BLOCK_M_TOKEN, out.data_ptr(), out[E:].data_ptr(), None, None, None,
+            None, None, None, ws.data_ptr(), ws_bytes, _lib.stream_of(topk_indices),
+        ),
+        "mts_moe_route",
+    )
+    return out[:E]
+
+
 def _stage(lib, w: torch.Tensor, transpose: bool, dtype: torch.dtype) -> torch.Tensor:
     """Copy of an expert weight ``[E,R,C]`` in the activation dtype, optionally as ``[E,C,R]``."""
     if not transpose and w.dtype == dtype:

@@ -108,3 +108,75 @@ def router_postprocess(logits: torch.Tensor, top_k: int, *, normalize: bool) -> 
         z_loss=z_loss,
         entropy=entropy,
     )
+
+
+def is_router_logits_supported(hidden_states: torch.Tensor, weight: torch.Tensor) -> bool:
+    return (
+        hidden_states.is_cuda
+        and weight.is_cuda
+        and hidden_states.ndim == 2
+        and weight.ndim == 2
+        and hidden_states.dtype in (torch.bfloat16, torch.float32)
+        and weight.dtype == torch.float32
+        and hidden_states.shape[0] > 0
+        and hidden_states.shape[1] == weight.shape[1]
+        and weight.shape[0] <= 16
+        and hidden_states.shape[1] % 4 == 0
+        and hidden_states.shape[1] <= 1024
+    )
+
+
+class _RouterLogitsFunction(torch.autograd.Function):
+    """logits = float(x) @ W_r^T without the fp32 copy of x; backward gives dx in x.dtype."""
+
+    @staticmethod
+    def forward(ctx, hidden_states: torch.Tensor, weight: torch.Tensor):
+        lib = _lib.load()
+        x = hidden_states.contiguous()
+        w = weight.contiguous()
+        T, H = x.shape
+        E = w.shape[0]
+        logits = torch.empty((T, E), device=x.device, dtype=torch.float32)
+        _lib.check(
+            lib.mts_router_logits_fwd(
+                x.data_ptr(), w.data_ptr(), T, H, E, _lib.dtype_code(x.dtype), logits.data_ptr(), _lib.stream_of(x)
+            ),
+            "mts_router_logits_fwd",
+        )
+        ctx.save_for_backward(x, w)
+        return logits
+
+    @staticmethod
+    def backward(ctx, grad_logits):
+        lib = _lib.load()
+        x, w = ctx.saved_tensors
+        T, H = x.shape
+        E = w.shape[0]
+        g = grad_logits.to(torch.float32).contiguous()
+        dx = torch.empty_like(x)
+        dw = torch.empty_like(w)
+        ws_bytes = lib.mts_router_logits_bwd_workspace_bytes(T, H, E)
+        ws = torch.empty(ws_bytes, device=x.device, dtype=torch.uint8)
+        _lib.check(
+            lib.mts_router_logits_bwd(
+                g.data_ptr(), x.data_ptr(), w.data_ptr(), T, H, E, _lib.dtype_code(x.dtype), dx.data_ptr(),
+                dw.data_ptr(), ws.data_ptr(), ws_bytes, _lib.stream_of(x),
+            ),
+            "mts_router_logits_bwd",
+        )
+        return dx, dw
+
+
+def router_logits(hidden_states: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """fp32 router logits of ``hidden_states`` [T,H] (bf16 or fp32) and ``weight`` [E,H] (fp32).
+
+    Stands in for ``F.linear(hidden_states.float(), weight.float())`` of the reference's
+    TopKRouter.forward (minitrain/model/moe_router.py:64-76).
+    """
+
+    if not is_router_logits_supported(hidden_states, weight):
+        raise RuntimeError(
+            "hip router_logits requires 2D bf16/fp32 activations and a 2D fp32 weight on the GPU with "
+            "at most 16 experts and a hidden size that is a multiple of 4 and at most 1024"
+        )
+    return _RouterLogitsFunction.apply(hidden_states, weight)

@@ -36,20 +36,34 @@ class TopKRouter(nn.Module):
 
     def forward(self, hidden_states: torch.Tensor, ops: OpsBackend) -> RouterOutput:
         cfg = self.cfg
-        router_input = hidden_states.float()
-        if self.training and cfg.router_jitter_noise:
-            noise = torch.empty_like(router_input).uniform_(
-                1.0 - cfg.router_jitter_noise, 1.0 + cfg.router_jitter_noise
-            )
-            router_input = router_input * noise
+        jitter = self.training and cfg.router_jitter_noise
+        # a backend may offer the projection straight from the activation dtype (same fp32
+        # arithmetic, no fp32 copy of the activations); jitter noise needs the fp32 copy
+        fused_logits = None if jitter else getattr(ops, "router_logits", None)
+        logits = None
+        if fused_logits is not None and hidden_states.ndim == 2:
+            with torch.autocast(device_type=hidden_states.device.type, enabled=False):
+                logits = fused_logits(hidden_states, self.weight)
+        if logits is None:
+            router_input = hidden_states.float()
+            if jitter:
+                noise = torch.empty_like(router_input).uniform_(
+                    1.0 - cfg.router_jitter_noise, 1.0 + cfg.router_jitter_noise
+                )
+                router_input = router_input * noise
 
         with torch.autocast(device_type=hidden_states.device.type, enabled=False):
-            logits = F.linear(router_input, self.weight.float())
+            if logits is None:
+                logits = F.linear(router_input, self.weight.float())
             route = ops.router_postprocess(logits, cfg.experts_per_token, normalize=cfg.router_normalize_topk)
             expert_weights = route.expert_weights
             expert_indices = route.expert_indices
 
-            route_counts = torch.bincount(expert_indices.flatten().long(), minlength=cfg.num_experts)
+            count_routes = getattr(ops, "expert_counts", None)
+            if count_routes is not None and expert_indices.is_cuda and expert_indices.dtype == torch.int32:
+                route_counts = count_routes(expert_indices, cfg.num_experts)
+            else:
+                route_counts = torch.bincount(expert_indices.flatten().long(), minlength=cfg.num_experts)
             tokens_per_expert = route_counts.float() / expert_indices.numel()
             # the assignment fraction carries no gradient; it enters through the mean probability
             auxiliary_loss = cfg.num_experts * torch.sum(tokens_per_expert * route.probability_per_expert)

@@ -8,6 +8,7 @@ import pytest
 import torch
 
 from oracle import moe_oracle as O
+from tests.helpers import hip_backend
 
 pytestmark = pytest.mark.gpu
 
@@ -75,3 +76,14 @@ def test_edge_patterns():
     idx = rng.choice(8, size=(24576, 2), p=p).astype(np.int32)
     _compare(idx, 8)
     _compare(idx, 8, block_m=256)
+
+
+@pytest.mark.parametrize("T,K,E", [(1, 1, 3), (257, 2, 8), (24576, 2, 8), (5000, 3, 64)])
+def test_expert_counts_only_mode_matches_bincount(T, K, E):
+    """mts_moe_route without the permutation arrays: the router module's count of routes."""
+    ops = hip_backend()
+    rng = np.random.Generator(np.random.Philox(T + K + E))
+    idx = torch.from_numpy(rng.integers(0, E, size=(T, K), dtype=np.int32))
+    got = ops.expert_counts(idx.cuda(), E)
+    assert got.dtype == torch.int32 and got.shape == (E,)
+    assert torch.equal(got.cpu().long(), torch.bincount(idx.flatten().long(), minlength=E))
