@@ -138,7 +138,12 @@ def stage_breakdown(layer, steps):
     B = _lib.MTS_BF16
     gemm = lambda mult: 2.0 * TK * H * I * mult
     esz = 2
+    w_r = layer.w_r.detach()
+    lws = torch.empty(max(4, lib.mts_router_logits_bwd_workspace_bytes(T, H, E)), dtype=torch.uint8, device=dev)
+    dx_r, dw_r, logits2 = torch.empty(T, H, **bf), torch.empty_like(w_r), torch.empty_like(logits)
     stages = [
+        ("router_logits_fwd", "hbm", T * H * esz + T * E * 4 + E * H * 4,
+         lambda: lib.mts_router_logits_fwd(p(x), p(w_r), T, H, E, B, p(logits2), st)),
         ("router_fwd", "hbm", T * E * 4 + T * K * 8,
          lambda: lib.mts_router_fwd(p(logits), T, E, K, 1, p(r_w), p(r_i), p(r_stats), p(r_stats) + 4 * E, p(r_stats) + 4 * E + 4, p(rw), rw.numel(), st)),
         ("route_metadata", "hbm", TK * 4 * 2 + 3 * TK * 4,
@@ -160,6 +165,8 @@ def stage_breakdown(layer, steps):
         ("bwd_dw1", "mfma", gemm(2), lambda: lib.mts_moe_bwd_dw1(p(dpre), p(x), p(xg), p(es), T, K, E, H, I, B, B, p(dw1), st)),
         ("router_bwd", "hbm", T * E * 4 * 2 + T * K * 12,
          lambda: lib.mts_router_bwd(p(logits), p(r_w), p(r_i), p(gw), p(gp), p(gz), T, E, K, 1, p(dlog), st)),
+        ("router_logits_bwd", "hbm", 2 * T * H * esz + T * E * 4 + 2 * E * H * 4,
+         lambda: lib.mts_router_logits_bwd(p(dlog), p(x), p(w_r), T, H, E, B, p(dx_r), p(dw_r), p(lws), lws.numel(), st)),
     ]
     ev = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in stages] for _ in range(steps)]
     for it in range(2 + steps):

@@ -69,13 +69,13 @@ int mts_router_bwd(const float* logits, const float* weights, const int32_t* ind
  * (minitrain/model/moe_router.py:64-76: `hidden_states.float()` followed by
  * `F.linear(router_input, weight.float())`): logits[t,e] = sum_h float(x[t,h]) * w_r[e,h],
  * fp32 products and sums, x [T,H] read in act_dtype (no fp32 copy), w_r [E,H] f32.
- * E <= 16, H a multiple of 4.                                                  */
+ * E <= 16, H a multiple of 4 and at most 1024.                                 */
 int mts_router_logits_fwd(const void* x, const float* w_r, int64_t T, int H, int E,
                           int act_dtype, float* logits, void* stream);
 
 /* dx[t,h] = sum_e dlogits[t,e] * w_r[e,h] (written in act_dtype, the cast the autograd
  * of `.float()` applies), d_w_r[e,h] = sum_t dlogits[t,e] * float(x[t,h]) (f32; partial
- * sums per block of rows in the workspace, added in a fixed order).  H <= 1024.   */
+ * sums per block of rows in the workspace, added in a fixed order).              */
 int64_t mts_router_logits_bwd_workspace_bytes(int64_t T, int H, int E);
 int mts_router_logits_bwd(const float* dlogits, const void* x, const float* w_r, int64_t T,
                           int H, int E, int act_dtype, void* dx, float* d_w_r,

@@ -8,7 +8,7 @@ namespace {
 
 constexpr int kRows = 4;         // rows per wave in the forward kernel
 constexpr int kFwdThreads = 256;
-constexpr int kSegs = 8;         // segments of the partial sums in the reduction kernel
+constexpr int kSegs = 64;        // segments of the partial sums in the reduction kernel
 
 __device__ __forceinline__ f32x4 load4(const bf16_t* p) {
     const bf16x4 v = *reinterpret_cast<const bf16x4*>(p);
@@ -22,13 +22,41 @@ __device__ __forceinline__ void store4(bf16_t* p, f32x4 v) {
 }
 __device__ __forceinline__ void store4(float* p, f32x4 v) { *reinterpret_cast<f32x4*>(p) = v; }
 
+// Butterfly reduce-scatter over the 64 lanes of a wave: N values are live in v[0..N), the
+// partner is `O` lanes away.  While N > 1 a lane hands one half of its values to the partner
+// and adds the partner's copy of the half it keeps; once one value is left the remaining
+// steps are plain pairwise sums.  The order of the additions is fixed.
+template <int NV, int N, int O>
+__device__ __forceinline__ void reduce_scatter(float (&v)[NV], int lane, int& idx) {
+    if constexpr (O >= 1) {
+        if constexpr (N > 1) {
+            const bool up = (lane & O) != 0;
+#pragma unroll
+            for (int i = 0; i < N / 2; ++i) {
+                const float send = up ? v[i] : v[i + N / 2];
+                const float keep = up ? v[i + N / 2] : v[i];
+                v[i] = keep + __shfl_xor(send, O, MTS_WAVE);
+            }
+            idx += up ? N / 2 : 0;
+            reduce_scatter<NV, N / 2, O / 2>(v, lane, idx);
+        } else {
+            v[0] += __shfl_xor(v[0], O, MTS_WAVE);
+            reduce_scatter<NV, 1, O / 2>(v, lane, idx);
+        }
+    }
+}
+
 // One wave computes kRows rows: a lane owns 4 consecutive columns of every 256-column slab,
-// the weights of a slab are read once per kRows rows (they stay in L1/L2), and the E partial
-// dot products of a row are summed across the wave with a fixed shuffle tree.
-template <typename XT, int EP>
+// the weights sit in LDS (loaded once per block), and the E partial dot products of a row are
+// summed across the wave with a fixed shuffle tree.
+template <typename XT, int EP, int PASSES>
 __global__ __launch_bounds__(kFwdThreads) void router_logits_fwd_kernel(const XT* __restrict__ x,
                                                                          const float* __restrict__ w, int64_t T,
                                                                          int H, int E, float* __restrict__ logits) {
+    extern __shared__ __attribute__((aligned(16))) float w_lds[];   // [E][H]
+    for (int i = threadIdx.x * 4; i < E * H; i += kFwdThreads * 4)
+        *reinterpret_cast<f32x4*>(w_lds + i) = *reinterpret_cast<const f32x4*>(w + i);
+    __syncthreads();
     const int lane = threadIdx.x % MTS_WAVE;
     const int64_t wave0 = (int64_t)blockIdx.x * (kFwdThreads / MTS_WAVE) + threadIdx.x / MTS_WAVE;
     const int64_t nwaves = (int64_t)gridDim.x * (kFwdThreads / MTS_WAVE);
@@ -38,34 +66,47 @@ __global__ __launch_bounds__(kFwdThreads) void router_logits_fwd_kernel(const XT
         for (int r = 0; r < kRows; ++r)
 #pragma unroll
             for (int e = 0; e < EP; ++e) acc[r][e] = 0.f;
-        for (int c = lane * 4; c < H; c += MTS_WAVE * 4) {
-            f32x4 xv[kRows];
+        // every load of the row group is issued before the first use
+        f32x4 xv[PASSES][kRows];
+#pragma unroll
+        for (int ps = 0; ps < PASSES; ++ps) {
+            const int c = lane * 4 + ps * MTS_WAVE * 4;
 #pragma unroll
             for (int r = 0; r < kRows; ++r) {
                 const f32x4 z = {0.f, 0.f, 0.f, 0.f};
-                xv[r] = r0 + r < T ? load4(x + (r0 + r) * H + c) : z;
+                xv[ps][r] = (c < H && r0 + r < T) ? load4(x + (r0 + r) * H + c) : z;
             }
+        }
 #pragma unroll
-            for (int e = 0; e < EP; ++e) {
-                if (e < E) {
-                    const f32x4 wv = *reinterpret_cast<const f32x4*>(w + (int64_t)e * H + c);
+        for (int ps = 0; ps < PASSES; ++ps) {
+            const int c = lane * 4 + ps * MTS_WAVE * 4;
+            if (c < H) {
+#pragma unroll
+                for (int e = 0; e < EP; ++e) {
+                    const f32x4 wv = *reinterpret_cast<const f32x4*>(w_lds + (e < E ? e : 0) * H + c);
 #pragma unroll
                     for (int r = 0; r < kRows; ++r)
-                        acc[r][e] += xv[r][0] * wv[0] + xv[r][1] * wv[1] + xv[r][2] * wv[2] + xv[r][3] * wv[3];
+                        acc[r][e] += xv[ps][r][0] * wv[0] + xv[ps][r][1] * wv[1] + xv[ps][r][2] * wv[2] + xv[ps][r][3] * wv[3];
                 }
             }
         }
-        float mine = 0.f;
+        // Sum over the 64 lanes of kRows*EP values: at every step a lane hands half of its
+        // values to the partner lane and adds the partner's copy of the half it keeps, so the
+        // count halves with the lane distance (fixed order: bit-stable).  With kRows*EP == 32
+        // one value is left after the distance-2 step, shared by a lane pair.
+        static_assert(kRows * EP == 32 || kRows * EP == 64, "reduction layout");
+        constexpr int NV = kRows * EP;
+        float v[NV];
 #pragma unroll
         for (int r = 0; r < kRows; ++r)
 #pragma unroll
-            for (int e = 0; e < EP; ++e) {
-                const float v = wave_sum(acc[r][e]);
-                if (lane == r * EP + e) mine = v;
-            }
-        static_assert(kRows * EP <= MTS_WAVE, "one lane per output of the wave");
-        const int r = lane / EP, e = lane % EP;
-        if (lane < kRows * EP && e < E && r0 + r < T) logits[(r0 + r) * E + e] = mine;
+            for (int e = 0; e < EP; ++e) v[r * EP + e] = acc[r][e];
+        int idx = 0;   // index of the value this lane ends up with, built from its lane bits
+        reduce_scatter<NV, NV, 32>(v, lane, idx);
+        const float mine = v[0];
+        const int r = idx / EP, e = idx % EP;
+        const bool writer = NV == 64 ? true : (lane & 1) == 0;
+        if (writer && e < E && r0 + r < T) logits[(r0 + r) * E + e] = mine;
     }
 }
 
@@ -90,18 +131,29 @@ __global__ __launch_bounds__(256) void router_logits_bwd_kernel(const float* __r
     }
     const int64_t row_beg = (int64_t)blockIdx.x * rows_per_block;
     const int64_t row_end = row_beg + rows_per_block < T ? row_beg + rows_per_block : T;
-    for (int64_t row = row_beg; row < row_end; ++row) {
-        const f32x4 xv = load4(x + row * H + c);
-        f32x4 d = {0.f, 0.f, 0.f, 0.f};
+    constexpr int UN = 4;   // rows in flight per thread
+#pragma unroll 1
+    for (int64_t row = row_beg; row < row_end; row += UN) {
+        f32x4 xv[UN];
 #pragma unroll
-        for (int e = 0; e < EP; ++e) {
-            if (e < E) {
-                const float g = dl[row * E + e];   // the same address for every thread of the block
-                d += g * wv[e];
-                acc[e] += g * xv;
+        for (int u = 0; u < UN; ++u) {
+            const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+            xv[u] = row + u < row_end ? load4(x + (row + u) * H + c) : z;
+        }
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            if (row + u < row_end) {
+                f32x4 d = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int e = 0; e < EP; ++e) {
+                    // the same address for every thread of the block; experts past E have zero weights
+                    const float g = dl[(row + u) * E + (e < E ? e : 0)];
+                    d += g * wv[e];
+                    acc[e] += (e < E ? g : 0.f) * xv[u];
+                }
+                store4(dx + (row + u) * H + c, d);
             }
         }
-        store4(dx + row * H + c, d);
     }
     float* out = part + (int64_t)blockIdx.x * E * H;
 #pragma unroll
@@ -133,11 +185,12 @@ __global__ __launch_bounds__(256) void router_dw_reduce_kernel(const float* __re
 }
 
 constexpr int kMaxE = 16;
-constexpr int kBwdBlocks = 512;
+constexpr int kMaxH = 1024;   // E*H floats of weights fit the 64 KiB of LDS a block may use by default
+constexpr int kBwdBlocks = 1024;
 
 int check(const void* x, const float* w, int64_t T, int H, int E, int act_dtype) {
     if (!x || !w) return MTS_ERR_NULL;
-    if (T <= 0 || E < 1 || E > kMaxE || H < 4 || H % 4) return MTS_ERR_SHAPE;
+    if (T <= 0 || E < 1 || E > kMaxE || H < 4 || H % 4 || H > kMaxH) return MTS_ERR_SHAPE;
     if (act_dtype != MTS_BF16 && act_dtype != MTS_F32) return MTS_ERR_DTYPE;
     if (!mts_aligned16(w) || (reinterpret_cast<uintptr_t>(x) & 15u)) return MTS_ERR_ALIGN;
     return MTS_OK;
@@ -155,15 +208,28 @@ extern "C" int mts_router_logits_fwd(const void* x, const float* w_r, int64_t T,
     hipStream_t s = (hipStream_t)stream;
     const int64_t groups = (T + kRows - 1) / kRows;
     int64_t blocks = (groups + 3) / 4;
-    if (blocks > 256 * 8) blocks = 256 * 8;
+    if (blocks > 256 * 4) blocks = 256 * 4;
     const dim3 grid((unsigned)blocks);
+    const size_t lds = (size_t)E * H * sizeof(float);
+    const int passes = (H + MTS_WAVE * 4 - 1) / (MTS_WAVE * 4);   // 1..4 since H <= 1024
+#define MTS_FWD(XT, EP, PS) \
+    router_logits_fwd_kernel<XT, EP, PS><<<grid, kFwdThreads, lds, s>>>((const XT*)x, w_r, T, H, E, logits)
+#define MTS_FWD_PASSES(XT, EP)                   \
+    do {                                         \
+        if (passes == 1) MTS_FWD(XT, EP, 1);     \
+        else if (passes == 2) MTS_FWD(XT, EP, 2); \
+        else if (passes == 3) MTS_FWD(XT, EP, 3); \
+        else MTS_FWD(XT, EP, 4);                 \
+    } while (0)
     if (act_dtype == MTS_BF16) {
-        if (E <= 8) router_logits_fwd_kernel<bf16_t, 8><<<grid, kFwdThreads, 0, s>>>((const bf16_t*)x, w_r, T, H, E, logits);
-        else router_logits_fwd_kernel<bf16_t, 16><<<grid, kFwdThreads, 0, s>>>((const bf16_t*)x, w_r, T, H, E, logits);
+        if (E <= 8) MTS_FWD_PASSES(bf16_t, 8);
+        else MTS_FWD_PASSES(bf16_t, 16);
     } else {
-        if (E <= 8) router_logits_fwd_kernel<float, 8><<<grid, kFwdThreads, 0, s>>>((const float*)x, w_r, T, H, E, logits);
-        else router_logits_fwd_kernel<float, 16><<<grid, kFwdThreads, 0, s>>>((const float*)x, w_r, T, H, E, logits);
+        if (E <= 8) MTS_FWD_PASSES(float, 8);
+        else MTS_FWD_PASSES(float, 16);
     }
+#undef MTS_FWD_PASSES
+#undef MTS_FWD
     MTS_CHECK_LAUNCH();
     return MTS_OK;
 }
@@ -179,21 +245,23 @@ extern "C" int mts_router_logits_bwd(const float* dlogits, const void* x, const 
     const int rc = check(x, w_r, T, H, E, act_dtype);
     if (rc != MTS_OK) return rc;
     if (!dlogits || !dx || !d_w_r || !workspace) return MTS_ERR_NULL;
-    if (H > 1024) return MTS_ERR_SHAPE;   // one thread per 4 columns, one block per row
     if (workspace_bytes < mts_router_logits_bwd_workspace_bytes(T, H, E)) return MTS_ERR_WORKSPACE;
     if (!mts_aligned16(workspace) || !mts_aligned16(d_w_r) || (reinterpret_cast<uintptr_t>(dx) & 15u)) return MTS_ERR_ALIGN;
     hipStream_t s = (hipStream_t)stream;
     const int nb = bwd_blocks(T);
     const int rows_per_block = (int)((T + nb - 1) / nb);
-    const int threads = ((H / 4 + MTS_WAVE - 1) / MTS_WAVE) * MTS_WAVE;
+    const int threads = ((H / 4 + MTS_WAVE - 1) / MTS_WAVE) * MTS_WAVE;   // one thread per 4 columns
     float* part = (float*)workspace;
+#define MTS_BWD(XT, EP) \
+    router_logits_bwd_kernel<XT, EP><<<nb, threads, 0, s>>>(dlogits, (const XT*)x, w_r, T, H, E, rows_per_block, (XT*)dx, part)
     if (act_dtype == MTS_BF16) {
-        if (E <= 8) router_logits_bwd_kernel<bf16_t, 8><<<nb, threads, 0, s>>>(dlogits, (const bf16_t*)x, w_r, T, H, E, rows_per_block, (bf16_t*)dx, part);
-        else router_logits_bwd_kernel<bf16_t, 16><<<nb, threads, 0, s>>>(dlogits, (const bf16_t*)x, w_r, T, H, E, rows_per_block, (bf16_t*)dx, part);
+        if (E <= 8) MTS_BWD(bf16_t, 8);
+        else MTS_BWD(bf16_t, 16);
     } else {
-        if (E <= 8) router_logits_bwd_kernel<float, 8><<<nb, threads, 0, s>>>(dlogits, (const float*)x, w_r, T, H, E, rows_per_block, (float*)dx, part);
-        else router_logits_bwd_kernel<float, 16><<<nb, threads, 0, s>>>(dlogits, (const float*)x, w_r, T, H, E, rows_per_block, (float*)dx, part);
+        if (E <= 8) MTS_BWD(float, 8);
+        else MTS_BWD(float, 16);
     }
+#undef MTS_BWD
     MTS_CHECK_LAUNCH();
     const int64_t EH = (int64_t)E * H;
     const int per_block = (256 / kSegs) * 4;
