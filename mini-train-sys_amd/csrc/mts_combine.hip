@@ -99,6 +99,36 @@ __global__ __launch_bounds__(kThreads) void stage_weights_kernel(const SrcT* __r
     }
 }
 
+// bf16 -> bf16 transpose with 16-byte global accesses: a block moves a 64x64 tile; a thread
+// reads 8 consecutive source elements of two rows, and writes 8 consecutive elements of two
+// output rows (8 consecutive source rows of one column, gathered from LDS).  The tile rows are
+// padded to 66 elements so that the column gather spreads over the banks.
+__global__ __launch_bounds__(kThreads) void transpose_bf16_kernel(const bf16_t* __restrict__ src,
+                                                                  bf16_t* __restrict__ dst, int R, int C) {
+    __shared__ bf16_t tile[64][66];
+    const int64_t e = blockIdx.z;
+    const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+    const bf16_t* s = src + e * (int64_t)R * C;
+    bf16_t* d = dst + e * (int64_t)R * C;
+    const int v = threadIdx.x % 8, rr = threadIdx.x / 8;   // 8 vectors per tile row, 32 rows per pass
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int r = rr + 32 * h;
+        const bf16x8 x = *reinterpret_cast<const bf16x8*>(s + (int64_t)(r0 + r) * C + c0 + v * 8);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) tile[r][v * 8 + j] = x[j];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int c = rr + 32 * h;   // source column = output row
+        bf16x8 y;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) y[j] = tile[v * 8 + j][c];
+        *reinterpret_cast<bf16x8*>(d + (int64_t)(c0 + c) * R + r0 + v * 8) = y;
+    }
+}
+
 int grid_1d(int64_t total) {
     int64_t b = (total + kThreads - 1) / kThreads;
     const int64_t cap = 256 * 32;
@@ -159,7 +189,10 @@ extern "C" int mts_moe_stage_weights(const void* src, int src_dtype, void* dst, 
     hipStream_t s = (hipStream_t)stream;
     dim3 grid((unsigned)((C + 63) / 64), (unsigned)((R + 63) / 64), (unsigned)E);
     if (grid.y > 65535) return MTS_ERR_SHAPE;
-    if (src_dtype == MTS_F32 && dst_dtype == MTS_BF16) launch_stage<float, bf16_t>(src, dst, grid, R, C, transpose, s);
+    if (src_dtype == MTS_BF16 && dst_dtype == MTS_BF16 && transpose && R % 64 == 0 && C % 64 == 0 &&
+        mts_aligned16(src) && mts_aligned16(dst) && R <= 0x7fffffff && C <= 0x7fffffff)
+        transpose_bf16_kernel<<<grid, kThreads, 0, s>>>((const bf16_t*)src, (bf16_t*)dst, (int)R, (int)C);
+    else if (src_dtype == MTS_F32 && dst_dtype == MTS_BF16) launch_stage<float, bf16_t>(src, dst, grid, R, C, transpose, s);
     else if (src_dtype == MTS_BF16 && dst_dtype == MTS_BF16) launch_stage<bf16_t, bf16_t>(src, dst, grid, R, C, transpose, s);
     else if (src_dtype == MTS_F32 && dst_dtype == MTS_F32) launch_stage<float, float>(src, dst, grid, R, C, transpose, s);
     else if (src_dtype == MTS_BF16 && dst_dtype == MTS_F32) launch_stage<bf16_t, float>(src, dst, grid, R, C, transpose, s);
