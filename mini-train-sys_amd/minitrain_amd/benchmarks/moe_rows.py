@@ -1,0 +1,190 @@
+"""Fused-MoE operator rows in the schema of the reference's operator benchmarks
+(benchmarks/operators/measurement.py:25-38, 485-496 and moe_runner.py:53,176-193):
+``fwd/bwd/full_p50_ms`` and ``_p95_ms``, ``*_peak_mem_mb``, ``*_speedup`` against the PyTorch
+expert loop on the same GPU, and the correctness columns ``max_abs``, ``max_rel``,
+``relative_l2``, ``cosine_similarity`` with the acceptance rule
+``relative_l2 <= 1e-2 and cosine_similarity >= 0.9999``.
+
+    python -m minitrain_amd.benchmarks.moe_rows --profile layer --tokens 24576
+    python -m minitrain_amd.benchmarks.moe_rows --profile mixtral --tokens 4096
+
+prints one JSON row per provider (``hip``, ``torch``).  The ``torch`` provider is the expert loop
+of the reference's PyTorch backend (minitrain/kernels/torch_ops.py:122-150) restated here as the
+baseline of the table; it is not used by the operator.
+"""
+
+import argparse
+import json
+import math
+
+import torch
+import torch.nn.functional as F
+
+PROFILES = {
+    # name: (hidden, expert width, experts, top-k)
+    "layer": (768, 1024, 8, 2),
+    "mixtral": (4096, 14336, 8, 2),
+}
+
+
+def torch_expert_loop(x, gate_up, down, idx, w):
+    out = torch.zeros_like(x)
+    I = gate_up.shape[1] // 2
+    for e in torch.unique(idx).tolist():
+        tok, kpos = torch.where(idx == e)
+        h = F.linear(x[tok], gate_up[e])
+        y = F.linear(F.silu(h[:, :I]) * h[:, I:], down[e]) * w[tok, kpos].unsqueeze(-1)
+        out.index_add_(0, tok, y)
+    return out
+
+
+def make_case(tokens, H, I, E, K, dtype, seed):
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    rn = lambda *s, std=1.0: (torch.randn(*s, generator=g, device="cuda") * std).to(dtype)
+    x, gate_up, down = rn(tokens, H), rn(E, 2 * I, H, std=0.02), rn(E, H, I, std=0.02)
+    logits = torch.randn(tokens, E, generator=g, device="cuda")
+    p, idx = torch.topk(torch.softmax(logits, dim=-1), K, dim=-1)
+    w = (p / p.sum(dim=-1, keepdim=True)).to(dtype)
+    grad = rn(tokens, H)
+    return dict(x=x, gate_up=gate_up, down=down, idx=idx.int(), w=w, grad=grad)
+
+
+def _stats(actual, expected):
+    a, b = actual.double().flatten(), expected.double().flatten()
+    diff = (a - b).abs()
+    na, nb = float(a.norm()), float(b.norm())
+    return {
+        "max_abs": float(diff.max()),
+        "max_rel": float((diff / b.abs().clamp_min(1e-6)).max()),
+        "relative_l2": float((a - b).norm()) / nb if nb > 0 else math.inf,
+        "cosine_similarity": float(torch.dot(a, b)) / (na * nb) if na * nb > 0 else -1.0,
+    }
+
+
+def _quantiles(samples):
+    v = torch.tensor(samples, dtype=torch.float64)
+    p50, p95 = torch.quantile(v, torch.tensor([0.5, 0.95], dtype=torch.float64)).tolist()
+    return p50, p95
+
+
+def _time(fn, iters, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    out = []
+    for _ in range(iters):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        fn()
+        b.record()
+        torch.cuda.synchronize()
+        out.append(a.elapsed_time(b))
+    return _quantiles(out)
+
+
+def _peak_mb(fn):
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+    torch.cuda.reset_peak_memory_stats()
+    base = torch.cuda.memory_allocated()
+    fn()
+    torch.cuda.synchronize()
+    return max(0.0, (torch.cuda.max_memory_allocated() - base) / 2**20)
+
+
+def measure(provider, op, case, iters, warmup):
+    leaves = {n: case[n].detach().clone().requires_grad_(True) for n in ("x", "gate_up", "down", "w")}
+
+    def fwd():
+        with torch.no_grad():
+            op(leaves["x"], leaves["gate_up"], leaves["down"], case["idx"], leaves["w"])
+
+    def full():
+        for t in leaves.values():
+            t.grad = None
+        op(leaves["x"], leaves["gate_up"], leaves["down"], case["idx"], leaves["w"]).backward(case["grad"])
+
+    held = {}
+
+    def bwd_setup():
+        for t in leaves.values():
+            t.grad = None
+        held["out"] = op(leaves["x"], leaves["gate_up"], leaves["down"], case["idx"], leaves["w"])
+
+    def bwd_timed():
+        samples = []
+        for i in range(warmup + iters):
+            bwd_setup()
+            torch.cuda.synchronize()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            held["out"].backward(case["grad"])
+            b.record()
+            torch.cuda.synchronize()
+            if i >= warmup:
+                samples.append(a.elapsed_time(b))
+        return _quantiles(samples)
+
+    row = {"provider": provider}
+    row["fwd_p50_ms"], row["fwd_p95_ms"] = _time(fwd, iters, warmup)
+    row["bwd_p50_ms"], row["bwd_p95_ms"] = bwd_timed()
+    row["full_p50_ms"], row["full_p95_ms"] = _time(full, iters, warmup)
+    row["fwd_peak_mem_mb"] = _peak_mb(fwd)
+    row["full_peak_mem_mb"] = _peak_mb(full)
+    bwd_setup()
+    row["bwd_peak_mem_mb"] = _peak_mb(lambda: held["out"].backward(case["grad"]))
+    held.clear()
+    return row
+
+
+def correctness(op, case):
+    """hip against the expert loop evaluated in fp32 on the same inputs (gradients concatenated)."""
+    def run(fn, dtype):
+        leaves = {n: case[n].detach().to(dtype).requires_grad_(True) for n in ("x", "gate_up", "down", "w")}
+        out = fn(leaves["x"], leaves["gate_up"], leaves["down"], case["idx"], leaves["w"])
+        out.backward(case["grad"].to(dtype))
+        return out.detach(), [leaves[n].grad for n in ("x", "gate_up", "down", "w")]
+
+    out_a, g_a = run(op, case["x"].dtype)
+    out_b, g_b = run(torch_expert_loop, torch.float32)
+    fwd = _stats(out_a, out_b)
+    bwd = _stats(torch.cat([g.flatten().float() for g in g_a]), torch.cat([g.flatten() for g in g_b]))
+    ok = lambda s: s["relative_l2"] <= 1e-2 and s["cosine_similarity"] >= 0.9999
+    row = {f"fwd_{k}": v for k, v in fwd.items()}
+    row.update({f"bwd_{k}": v for k, v in bwd.items()})
+    row["fwd_correct"], row["bwd_correct"] = ok(fwd), ok(bwd)
+    row["acceptance"] = "relative_l2<=1e-2_and_cosine>=0.9999"
+    return row
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--profile", choices=sorted(PROFILES), default="layer")
+    ap.add_argument("--tokens", type=int, default=24576)
+    ap.add_argument("--iters", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--seed", type=int, default=1)
+    ap.add_argument("--no-torch", action="store_true", help="skip the PyTorch expert-loop baseline rows")
+    args = ap.parse_args()
+    from minitrain_amd.model.ops import get_ops_backend
+
+    H, I, E, K = PROFILES[args.profile]
+    ops = get_ops_backend("hip")
+    case = make_case(args.tokens, H, I, E, K, torch.bfloat16, args.seed)
+    common = dict(op="fused_moe", profile=args.profile, size=args.tokens, hidden=H, expert_width=I, experts=E,
+                  top_k=K, dtype="bf16", device=torch.cuda.get_device_name(0), timer="cuda_events")
+    hip = measure("hip", ops.fused_moe, case, args.iters, args.warmup)
+    hip.update(correctness(ops.fused_moe, case))
+    rows = [hip]
+    if not args.no_torch:
+        ref = measure("torch", torch_expert_loop, case, max(3, args.iters // 4), 2)
+        for m in ("fwd", "bwd", "full"):
+            hip[f"{m}_speedup"] = ref[f"{m}_p50_ms"] / hip[f"{m}_p50_ms"]
+            ref[f"{m}_speedup"] = 1.0
+        rows.append(ref)
+    for r in rows:
+        print(json.dumps({**common, **r}))
+
+
+if __name__ == "__main__":
+    main()

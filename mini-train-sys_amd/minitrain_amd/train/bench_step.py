@@ -1,0 +1,117 @@
+"""End-to-end training step of the MoE decoder with the `hip` MoE layer swapped in.
+
+    python -m minitrain_amd.train.bench_step            # 12 layers, 24 x 1024 tokens, bf16 autocast
+    python -m minitrain_amd.train.bench_step --layers 2 --batch 2 --seq 128 --vocab 1000
+
+Model, data and step follow the reference's MoE model configuration
+(configs/synbios_moe/model.yaml:1-20, with seq_len 1024 and dropout 0.0) and
+``Trainer.train_step`` (minitrain/train/trainer.py:85-159): fp32 parameters, bf16 autocast,
+AdamW, global-norm clipping; token ids are uniform on [0, vocab).  Prints one JSON line with
+tokens/s and the MoE share of the step (HIP events around the forward and the backward of every
+MoE feed-forward block, summed, over the step time).
+"""
+
+import argparse
+import json
+import time
+
+import torch
+
+from minitrain_amd.model.config import ModelConfig
+from minitrain_amd.model.decoder import MiniTransformer
+from minitrain_amd.model.ops import get_ops_backend
+from minitrain_amd.train.step import build_optimizer, train_step
+
+
+class MoeRanges:
+    """HIP events around forward and backward of every MoE block.
+
+    Forward: module hooks.  Backward: tensor hooks, from the arrival of the gradient of the
+    block's output to the moment the gradient of its input is complete (router and expert
+    contributions summed).
+    """
+
+    def __init__(self, model):
+        self.pairs, self.open = [], {}
+        for i, block in enumerate(model.blocks):
+            block.ffn.register_forward_pre_hook(lambda m, a, i=i: self._enter(a[0], i))
+            block.ffn.register_forward_hook(lambda m, a, o, i=i: self._leave(o.hidden_states, i))
+
+    def _enter(self, x, i):
+        self._start(("f", i))
+        if x.requires_grad:
+            x.register_hook(lambda g, i=i: self._stop(("b", i)))
+
+    def _leave(self, out, i):
+        self._stop(("f", i))
+        if out.requires_grad:
+            out.register_hook(lambda g, i=i: self._start(("b", i)))
+
+    def _start(self, key):
+        ev = torch.cuda.Event(enable_timing=True)
+        ev.record()
+        self.open[key] = ev
+
+    def _stop(self, key):
+        if key not in self.open:
+            return
+        ev = torch.cuda.Event(enable_timing=True)
+        ev.record()
+        self.pairs.append((self.open.pop(key), ev))
+
+    def total_ms(self):
+        t = sum(a.elapsed_time(b) for a, b in self.pairs)
+        self.pairs.clear()
+        return t
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--layers", type=int, default=12)
+    ap.add_argument("--batch", type=int, default=24)
+    ap.add_argument("--seq", type=int, default=1024)
+    ap.add_argument("--vocab", type=int, default=50257)
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--seed", type=int, default=4)
+    ap.add_argument("--fused-loss", action="store_true")
+    args = ap.parse_args()
+
+    torch.manual_seed(args.seed)
+    cfg = ModelConfig(vocab_size=args.vocab, seq_len=args.seq, n_layers=args.layers, n_heads=12, hidden_size=768,
+                      intermediate_size=1024, dropout=0.0, tie_word_embeddings=True, ffn_type="moe",
+                      num_experts=8, experts_per_token=2)
+    model = MiniTransformer(cfg, get_ops_backend("hip"), activation_dtype=torch.bfloat16).cuda()
+    opt = build_optimizer(model)
+    ranges = MoeRanges(model)
+    g = torch.Generator().manual_seed(args.seed)
+    ids = torch.randint(0, args.vocab, (args.batch, args.seq + 1), generator=g)
+    batch = {"input_ids": ids[:, :-1].contiguous(), "targets": ids[:, 1:].contiguous()}
+    losses = []
+    for _ in range(args.warmup):
+        losses.append(float(train_step(model, opt, batch, use_fused_loss=args.fused_loss)))
+    ranges.total_ms()
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        losses.append(float(train_step(model, opt, batch, use_fused_loss=args.fused_loss)))
+    torch.cuda.synchronize()
+    step_ms = (time.perf_counter() - t0) / args.steps * 1e3
+    moe_ms = ranges.total_ms() / args.steps
+    tokens = args.batch * args.seq
+    print(json.dumps({
+        "metric": "decoder training step tokens/s (hip MoE layer via OpsBackend)",
+        "value": tokens / (step_ms * 1e-3), "unit": "tokens/s", "ms_per_step": step_ms,
+        "moe_ms_per_step": moe_ms, "moe_share_of_step": moe_ms / step_ms,
+        "parameters": sum(p.numel() for p in model.parameters()),
+        "peak_allocated_gib": torch.cuda.max_memory_allocated() / 2**30,
+        "losses": losses,
+        "config": {"layers": args.layers, "batch": args.batch, "seq_len": args.seq, "vocab": args.vocab,
+                   "d_model": 768, "heads": 12, "experts": 8, "top_k": 2, "d_ff": 1024, "dtype": "bf16 autocast, fp32 params",
+                   "optimizer": "AdamW", "data": "synthetic token ids, uniform", "seed": args.seed},
+    }))
+
+
+if __name__ == "__main__":
+    main()

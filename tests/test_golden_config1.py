@@ -49,7 +49,7 @@ def test_hip_fp32_layer_matches_the_vectors():
     c = CONFIG1
     print("config1 fp32 on the GPU", flush=True)
     x, w_r, w1, w2, g = O.make_inputs(c["seed"], c["T"], c["H"], c["E"], c["I"])
-    cfg = ModelConfig(hidden_size=c["H"], intermediate_size=c["I"], num_experts=c["E"], experts_per_token=c["K"])
+    cfg = ModelConfig(hidden_size=c["H"], n_heads=1, intermediate_size=c["I"], num_experts=c["E"], experts_per_token=c["K"])
     block = MoEFeedForward(cfg).cuda()
     with torch.no_grad():
         block.router.weight.copy_(w_r)

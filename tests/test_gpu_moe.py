@@ -136,7 +136,7 @@ def test_moe_block_end_to_end():
     from minitrain_amd.model.config import ModelConfig
 
     T, H, E, I, K = 512, 128, 8, 256, 2
-    cfg = ModelConfig(hidden_size=H, intermediate_size=I, num_experts=E, experts_per_token=K, n_layers=12)
+    cfg = ModelConfig(hidden_size=H, n_heads=1, intermediate_size=I, num_experts=E, experts_per_token=K, n_layers=12)
     x, w_r, w1, w2, g = O.make_inputs(7, T, H, E, I)
     block = MoEFeedForward(cfg).cuda()
     with torch.no_grad():
