@@ -3,10 +3,13 @@
 Counterpart of minitrain/kernels/triton/fused_moe.py:37-449: the support
 predicate, the routing-metadata step, the autograd function and the module-level
 entry point.  Every buffer is a torch tensor on the caller's device; kernels are
-enqueued on the current stream through the C ABI and nothing synchronises.
+enqueued through the C ABI and nothing synchronises with the host.  The backward pass
+forks two side streams from the current stream for kernels that do not depend on one
+another and joins them before it returns.
 """
 
 import functools
+import os
 
 import torch
 
@@ -127,7 +130,20 @@ def expert_counts(topk_indices: torch.Tensor, E: int) -> torch.Tensor:
     return out[:E]
 
 
-def _stage(lib, w: torch.Tensor, transpose: bool, dtype: torch.dtype) -> torch.Tensor:
+# MTS_NO_OVERLAP=1 keeps every kernel of the backward pass on the caller's stream
+_OVERLAP = os.environ.get("MTS_NO_OVERLAP", "0") != "1"
+_SIDE_STREAMS: dict = {}
+
+
+def _side_stream(device: torch.device, index: int) -> torch.cuda.Stream:
+    key = (device.index if device.index is not None else torch.cuda.current_device(), index)
+    s = _SIDE_STREAMS.get(key)
+    if s is None:
+        s = _SIDE_STREAMS[key] = torch.cuda.Stream(device=device)   # default priority
+    return s
+
+
+def _stage(lib, w: torch.Tensor, transpose: bool, dtype: torch.dtype, stream: int | None = None) -> torch.Tensor:
     """Copy of an expert weight ``[E,R,C]`` in the activation dtype, optionally as ``[E,C,R]``."""
     if not transpose and w.dtype == dtype:
         return w
@@ -136,7 +152,7 @@ def _stage(lib, w: torch.Tensor, transpose: bool, dtype: torch.dtype) -> torch.T
     _lib.check(
         lib.mts_moe_stage_weights(
             w.data_ptr(), _lib.dtype_code(w.dtype), out.data_ptr(), _lib.dtype_code(dtype), E, R, C, int(transpose),
-            _lib.stream_of(w),
+            _lib.stream_of(w) if stream is None else stream,
         ),
         "mts_moe_stage_weights",
     )
@@ -213,6 +229,35 @@ class _FusedMoEFunction(torch.autograd.Function):
         stream = _lib.stream_of(dO)
         need_x, need_w1, need_w2, _, need_s = ctx.needs_input_grad
 
+        # Kernels that do not depend on one another run side by side: the transposed copy of W1 (needed
+        # by dX only) next to the dO*W2 GEMM, and then dW2, dW1 and dX, which depend only on what that
+        # GEMM wrote; the two weight-gradient GEMMs have fewer tiles than the chip has CUs.  Two side
+        # streams (default priority) are forked from and joined to the caller's stream with events;
+        # everything they read stays referenced until the join has been enqueued.
+        main = torch.cuda.current_stream(dev)
+        overlap = _OVERLAP
+        side = [_side_stream(dev, 0), _side_stream(dev, 1)] if overlap else [main, main]
+
+        def fork(to):
+            if overlap:
+                ev = torch.cuda.Event()
+                ev.record(main)
+                to.wait_event(ev)
+
+        def join(frm):
+            if overlap:
+                ev = torch.cuda.Event()
+                ev.record(frm)
+                main.wait_event(ev)
+
+        w1t = None
+        if need_x:
+            fork(side[0])
+            w1t = _stage(lib, gate_up_proj, True, x.dtype, side[0].cuda_stream)  # [E, H, 2I]
+            w1t_ready = torch.cuda.Event() if overlap else None
+            if overlap:
+                w1t_ready.record(side[0])
+
         w2t = _stage(lib, down_proj, True, x.dtype)  # [E, I, H]
         d_pre_act = torch.empty(TK, 2 * I, dtype=x.dtype, device=dev)
         weighted_act = torch.empty(TK, I, dtype=x.dtype, device=dev)
@@ -226,7 +271,30 @@ class _FusedMoEFunction(torch.autograd.Function):
             ),
             "mts_moe_bwd_dy1",
         )
-        del w2t
+
+        ddown_proj = None
+        if need_w2:
+            ddown_proj = torch.empty_like(down_proj)
+            fork(side[0])
+            _lib.check(
+                lib.mts_moe_bwd_dw2(
+                    dO.data_ptr(), weighted_act.data_ptr(), x_gather.data_ptr(), expert_start.data_ptr(), T, K, E, H,
+                    I, act, _lib.dtype_code(down_proj.dtype), ddown_proj.data_ptr(), side[0].cuda_stream,
+                ),
+                "mts_moe_bwd_dw2",
+            )
+
+        dgate_up_proj = None
+        if need_w1:
+            dgate_up_proj = torch.empty_like(gate_up_proj)
+            fork(side[1])
+            _lib.check(
+                lib.mts_moe_bwd_dw1(
+                    d_pre_act.data_ptr(), x.data_ptr(), x_gather.data_ptr(), expert_start.data_ptr(), T, K, E, H, I,
+                    act, _lib.dtype_code(gate_up_proj.dtype), dgate_up_proj.data_ptr(), side[1].cuda_stream,
+                ),
+                "mts_moe_bwd_dw1",
+            )
 
         d_weights = None
         if need_s:
@@ -236,21 +304,10 @@ class _FusedMoEFunction(torch.autograd.Function):
                 "mts_moe_bwd_ds",
             )
 
-        ddown_proj = None
-        if need_w2:
-            ddown_proj = torch.empty_like(down_proj)
-            _lib.check(
-                lib.mts_moe_bwd_dw2(
-                    dO.data_ptr(), weighted_act.data_ptr(), x_gather.data_ptr(), expert_start.data_ptr(), T, K, E, H,
-                    I, act, _lib.dtype_code(down_proj.dtype), ddown_proj.data_ptr(), stream,
-                ),
-                "mts_moe_bwd_dw2",
-            )
-        del weighted_act
-
         dx = None
         if need_x:
-            w1t = _stage(lib, gate_up_proj, True, x.dtype)  # [E, H, 2I]
+            if overlap:
+                main.wait_event(w1t_ready)
             dx_expanded = torch.empty(TK, H, dtype=x.dtype, device=dev)
             _lib.check(
                 lib.mts_moe_bwd_dx(
@@ -267,16 +324,10 @@ class _FusedMoEFunction(torch.autograd.Function):
                 "mts_moe_combine",
             )
 
-        dgate_up_proj = None
+        if need_w2 or need_x:
+            join(side[0])
         if need_w1:
-            dgate_up_proj = torch.empty_like(gate_up_proj)
-            _lib.check(
-                lib.mts_moe_bwd_dw1(
-                    d_pre_act.data_ptr(), x.data_ptr(), x_gather.data_ptr(), expert_start.data_ptr(), T, K, E, H, I,
-                    act, _lib.dtype_code(gate_up_proj.dtype), dgate_up_proj.data_ptr(), stream,
-                ),
-                "mts_moe_bwd_dw1",
-            )
+            join(side[1])
 
         return dx, dgate_up_proj, ddown_proj, None, d_weights
 
