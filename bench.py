@@ -79,12 +79,10 @@ class Layer:
         if logits is None:
             logits = F.linear(self.x.float(), self.w_r)
         route = self.ops.router_postprocess(logits, self.K, normalize=True)
-        count_routes = getattr(self.ops, "expert_counts", None)
-        if count_routes is not None:
-            counts = count_routes(route.expert_indices, self.E)
-        else:
+        aux = getattr(route, "load_balance_loss", None)
+        if aux is None:
             counts = torch.bincount(route.expert_indices.flatten().long(), minlength=self.E)
-        aux = self.E * torch.sum(counts.float() / route.expert_indices.numel() * route.probability_per_expert)
+            aux = self.E * torch.sum(counts.float() / route.expert_indices.numel() * route.probability_per_expert)
         out = self.ops.fused_moe(self.x, self.w1, self.w2, route.expert_indices, route.expert_weights.to(self.x.dtype))
         loss_side = 0.01 * aux + 0.001 * route.z_loss
         torch.autograd.backward([out, loss_side], [self.g, torch.ones_like(loss_side)])
@@ -128,7 +126,7 @@ def stage_breakdown(layer, steps):
     rw = torch.empty(lib.mts_router_workspace_bytes(T, E), dtype=torch.uint8, device=dev)
     rws = torch.empty(max(4, lib.mts_moe_route_workspace_bytes(T, K, E)), dtype=torch.uint8, device=dev)
     r_w, r_i = torch.empty(T, K, dtype=torch.float32, device=dev), torch.empty(T, K, dtype=torch.int32, device=dev)
-    r_stats = torch.empty(E + 2, dtype=torch.float32, device=dev)
+    r_stats = torch.empty(E + 3, dtype=torch.float32, device=dev)
     i32 = dict(dtype=torch.int32, device=dev)
     cnt, es2, a1, a2, a3 = torch.empty(E, **i32), torch.empty(E + 1, **i32), torch.empty(TK, **i32), torch.empty(TK, **i32), torch.empty(TK, **i32)
     dlog = torch.empty_like(logits)
@@ -145,7 +143,7 @@ def stage_breakdown(layer, steps):
         ("router_logits_fwd", "hbm", T * H * esz + T * E * 4 + E * H * 4,
          lambda: lib.mts_router_logits_fwd(p(x), p(w_r), T, H, E, B, p(logits2), st)),
         ("router_fwd", "hbm", T * E * 4 + T * K * 8,
-         lambda: lib.mts_router_fwd(p(logits), T, E, K, 1, p(r_w), p(r_i), p(r_stats), p(r_stats) + 4 * E, p(r_stats) + 4 * E + 4, p(rw), rw.numel(), st)),
+         lambda: lib.mts_router_fwd(p(logits), T, E, K, 1, p(r_w), p(r_i), p(r_stats), p(r_stats) + 4 * E, p(r_stats) + 4 * E + 4, p(cnt), p(r_stats) + 4 * E + 8, p(rw), rw.numel(), st)),
         ("route_metadata", "hbm", TK * 4 * 2 + 3 * TK * 4,
          lambda: lib.mts_moe_route(p(idx), T, K, E, 64, p(cnt), p(es2), p(a1), p(a2), p(a3), None, None, None, p(rws), rws.numel(), st)),
         ("fwd_gateup_swiglu", "mfma", gemm(2),
@@ -164,7 +162,7 @@ def stage_breakdown(layer, steps):
          lambda: lib.mts_moe_combine(p(dxe), None, p(sr), T, K, H, B, p(dx), st)),
         ("bwd_dw1", "mfma", gemm(2), lambda: lib.mts_moe_bwd_dw1(p(dpre), p(x), p(xg), p(es), T, K, E, H, I, B, B, p(dw1), st)),
         ("router_bwd", "hbm", T * E * 4 * 2 + T * K * 12,
-         lambda: lib.mts_router_bwd(p(logits), p(r_w), p(r_i), p(gw), p(gp), p(gz), T, E, K, 1, p(dlog), st)),
+         lambda: lib.mts_router_bwd(p(logits), p(r_w), p(r_i), p(gw), p(gp), p(gz), p(gz), p(cnt), T, E, K, 1, p(dlog), st)),
         ("router_logits_bwd", "hbm", 2 * T * H * esz + T * E * 4 + 2 * E * H * 4,
          lambda: lib.mts_router_logits_bwd(p(dlog), p(x), p(w_r), T, H, E, B, p(dx_r), p(dw_r), p(lws), lws.numel(), st)),
     ]

@@ -52,17 +52,26 @@ const char* mts_error_string(int code);
  * and _router_forward_kernel (minitrain/kernels/triton/router.py:62-152).
  * logits [T,E] f32 -> weights [T,K] f32, indices [T,K] i32 (rank order, ties to
  * the lower expert index), prob_mean [E], z_loss [1], entropy [1].
- * The statistics are reduced in a fixed order (no float atomics).            */
+ * The statistics are reduced in a fixed order (no float atomics).
+ * counts [E] i32 and load_balance [1] may be NULL.  They stand in for the router
+ * module's bookkeeping around the operator (minitrain/model/moe_router.py:82-90):
+ * routes per expert (its torch.bincount) and E * sum_e (counts_e / (T*K)) * prob_mean_e
+ * (its auxiliary loss); load_balance needs counts.                              */
 int64_t mts_router_workspace_bytes(int64_t T, int E);
 int mts_router_fwd(const float* logits, int64_t T, int E, int K, int normalize,
                    float* weights, int32_t* indices, float* prob_mean, float* z_loss,
-                   float* entropy, void* workspace, int64_t workspace_bytes, void* stream);
+                   float* entropy, int32_t* counts, float* load_balance, void* workspace,
+                   int64_t workspace_bytes, void* stream);
 
 /* Replaces _router_backward_kernel (minitrain/kernels/triton/router.py:155-259).
- * g_weights [T,K], g_prob_mean [E], g_z_loss [1] -> dlogits [T,E].            */
+ * g_weights [T,K], g_prob_mean [E], g_z_loss [1] -> dlogits [T,E].
+ * g_load_balance [1] (may be NULL) is the gradient of the load-balancing term; it
+ * reaches the logits through prob_mean only (the route fractions counts/(T*K)
+ * carry no gradient) and needs the counts the forward call wrote.              */
 int mts_router_bwd(const float* logits, const float* weights, const int32_t* indices,
                    const float* g_weights, const float* g_prob_mean, const float* g_z_loss,
-                   int64_t T, int E, int K, int normalize, float* dlogits, void* stream);
+                   const float* g_load_balance, const int32_t* counts, int64_t T, int E, int K,
+                   int normalize, float* dlogits, void* stream);
 
 /* ---- router projection ----------------------------------------------------
  * Replaces the fp32 router GEMM of TopKRouter.forward and its autograd backward

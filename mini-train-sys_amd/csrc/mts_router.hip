@@ -75,13 +75,18 @@ __device__ __forceinline__ void load_row(const float* __restrict__ logits, int64
 template <int EP, int G>
 __global__ __launch_bounds__(kThreads) void router_fwd_kernel(
     const float* __restrict__ logits, int64_t T, int E, int K, int normalize,
-    float* __restrict__ weights, int32_t* __restrict__ indices, float* __restrict__ partial) {
+    float* __restrict__ weights, int32_t* __restrict__ indices, float* __restrict__ partial,
+    int32_t* __restrict__ partial_counts) {
     constexpr int ROWS = kThreads / G;
     const int g = threadIdx.x % G;
     const int rl = threadIdx.x / G;
     float psum[EP];
+    int csum[EP];   // routes to the experts this lane owns (slot j is expert j*G + g)
 #pragma unroll
-    for (int j = 0; j < EP; ++j) psum[j] = 0.f;
+    for (int j = 0; j < EP; ++j) {
+        psum[j] = 0.f;
+        csum[j] = 0;
+    }
     float zsum = 0.f, hsum = 0.f;
 
     for (int64_t row0 = (int64_t)blockIdx.x * ROWS; row0 < T; row0 += (int64_t)gridDim.x * ROWS) {
@@ -124,6 +129,8 @@ __global__ __launch_bounds__(kThreads) void router_fwd_kernel(
                     }
                 }
                 if (be % G == g) taken |= 1u << (be / G);
+#pragma unroll
+                for (int j = 0; j < EP; ++j) csum[j] += (live && j * G + g == be) ? 1 : 0;
                 float pk = expf(bv - r.m) / r.s;
                 sel_p[k] = pk;
                 sel_e[k] = be;
@@ -160,12 +167,21 @@ __global__ __launch_bounds__(kThreads) void router_fwd_kernel(
     }
     zsum = wave_sum(zsum);
     hsum = wave_sum(hsum);
+#pragma unroll
+    for (int j = 0; j < EP; ++j) {
+#pragma unroll
+        for (int o = 32; o >= G; o >>= 1) csum[j] += __shfl_xor(csum[j], o, MTS_WAVE);
+    }
 
     __shared__ float red[kThreads / MTS_WAVE][EP * G + 2];
+    __shared__ int32_t cred[kThreads / MTS_WAVE][EP * G];
     const int wave = threadIdx.x / MTS_WAVE, lane = threadIdx.x % MTS_WAVE;
     if (lane < G) {
 #pragma unroll
-        for (int j = 0; j < EP; ++j) red[wave][j * G + lane] = psum[j];
+        for (int j = 0; j < EP; ++j) {
+            red[wave][j * G + lane] = psum[j];
+            cred[wave][j * G + lane] = csum[j];
+        }
     }
     if (lane == 0) {
         red[wave][EP * G] = zsum;
@@ -180,23 +196,54 @@ __global__ __launch_bounds__(kThreads) void router_fwd_kernel(
         for (int w = 0; w < kThreads / MTS_WAVE; ++w) v += red[w][src];
         out[i] = v;
     }
+    int32_t* cout = partial_counts + (int64_t)blockIdx.x * E;
+    for (int i = threadIdx.x; i < E; i += kThreads) {
+        int32_t v = 0;
+#pragma unroll
+        for (int w = 0; w < kThreads / MTS_WAVE; ++w) v += cred[w][i];
+        cout[i] = v;
+    }
 }
 
 // One block: wave w reduces columns w, w+4, ...; lanes stride over the per-block
-// partials and the lane sums meet in a fixed shuffle tree (bit-stable).
+// partials and the lane sums meet in a fixed shuffle tree (bit-stable).  Also the routes per
+// expert and, if asked for, the load-balancing term E * sum_e (routes_e / routes) * mean_prob_e.
 __global__ __launch_bounds__(kThreads) void router_stats_kernel(
-    const float* __restrict__ partial, int nblocks, int E, float inv_t,
-    float* __restrict__ prob_mean, float* __restrict__ z_loss, float* __restrict__ entropy) {
+    const float* __restrict__ partial, const int32_t* __restrict__ partial_counts, int nblocks, int E,
+    float inv_t, float inv_routes, float* __restrict__ prob_mean, float* __restrict__ z_loss,
+    float* __restrict__ entropy, int32_t* __restrict__ counts, float* __restrict__ load_balance) {
+    __shared__ float prod[MTS_MAX_EXPERTS];   // fraction of routes x mean probability, per expert
     const int wave = threadIdx.x / MTS_WAVE, lane = threadIdx.x % MTS_WAVE;
     for (int i = wave; i < E + 2; i += kThreads / MTS_WAVE) {
         float v = 0.f;
         for (int b = lane; b < nblocks; b += MTS_WAVE) v += partial[(int64_t)b * (E + 2) + i];
         v = wave_sum(v) * inv_t;
-        if (lane == 0) {
-            if (i < E) prob_mean[i] = v;
-            else if (i == E) z_loss[0] = v;
-            else entropy[0] = v;
+        int c = 0;
+        if (i < E) {
+            for (int b = lane; b < nblocks; b += MTS_WAVE) c += partial_counts[(int64_t)b * E + i];
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) c += __shfl_xor(c, o, MTS_WAVE);
         }
+        if (lane == 0) {
+            if (i < E) {
+                prob_mean[i] = v;
+                prod[i] = (float)c * inv_routes * v;
+                if (counts) counts[i] = c;
+            } else if (i == E) {
+                z_loss[0] = v;
+            } else {
+                entropy[0] = v;
+            }
+        }
+    }
+    if (!load_balance) return;
+    __syncthreads();
+    // E * sum_e f_e * pbar_e, summed in a fixed order by one wave
+    if (wave == 0) {
+        float v = 0.f;
+        for (int e = lane; e < E; e += MTS_WAVE) v += prod[e];
+        v = wave_sum(v);
+        if (lane == 0) load_balance[0] = (float)E * v;
     }
 }
 
@@ -204,7 +251,8 @@ template <int EP, int G>
 __global__ __launch_bounds__(kThreads) void router_bwd_kernel(
     const float* __restrict__ logits, const float* __restrict__ weights,
     const int32_t* __restrict__ indices, const float* __restrict__ g_w,
-    const float* __restrict__ g_p, const float* __restrict__ g_z, int64_t T, int E, int K,
+    const float* __restrict__ g_p, const float* __restrict__ g_z, const float* __restrict__ g_lb,
+    const int32_t* __restrict__ counts, int64_t T, int E, int K,
     int normalize, float* __restrict__ dlogits) {
     constexpr int ROWS = kThreads / G;
     const int g = threadIdx.x % G;
@@ -216,6 +264,8 @@ __global__ __launch_bounds__(kThreads) void router_bwd_kernel(
     for (int j = 0; j < EP; ++j) {
         int e = j * G + g;
         gp[j] = (e < E) ? g_p[e] * inv_t : 0.f;
+        // load-balancing term: d/d(mean_prob_e) = E * routes_e / routes (the route fractions carry no gradient)
+        if (g_lb && e < E) gp[j] += g_lb[0] * (float)E * ((float)counts[e] / ((float)T * (float)K)) * inv_t;
     }
     for (int64_t row0 = (int64_t)blockIdx.x * ROWS; row0 < T; row0 += (int64_t)gridDim.x * ROWS) {
         int64_t row = row0 + rl;
@@ -309,45 +359,50 @@ int check_router(const void* logits, int64_t T, int E, int K) {
 
 extern "C" int64_t mts_router_workspace_bytes(int64_t T, int E) {
     (void)T;
-    return (int64_t)kMaxBlocks * (E + 2) * (int64_t)sizeof(float);
+    return (int64_t)kMaxBlocks * (2 * E + 2) * (int64_t)sizeof(float);   // float partials, then int32 route counts
 }
 
 extern "C" int mts_router_fwd(const float* logits, int64_t T, int E, int K, int normalize,
                               float* weights, int32_t* indices, float* prob_mean, float* z_loss,
-                              float* entropy, void* workspace, int64_t workspace_bytes,
-                              void* stream) {
+                              float* entropy, int32_t* counts, float* load_balance, void* workspace,
+                              int64_t workspace_bytes, void* stream) {
     int rc = check_router(logits, T, E, K);
     if (rc) return rc;
     if (!weights || !indices || !prob_mean || !z_loss || !entropy || !workspace) return MTS_ERR_NULL;
+    if ((counts || load_balance) && T * (int64_t)K > 0x7fffffffLL) return MTS_ERR_SHAPE;   // int32 route counts
     if (workspace_bytes < mts_router_workspace_bytes(T, E)) return MTS_ERR_WORKSPACE;
     hipStream_t s = (hipStream_t)stream;
     float* partial = (float*)workspace;
+    int32_t* partial_counts = (int32_t*)(partial + (int64_t)kMaxBlocks * (E + 2));
     int G = E > 512 ? 64 : lanes_for(E);
     int grid = grid_for(T, G);
-    MTS_ROUTER_DISPATCH(router_fwd_kernel,
-                        <<<grid, kThreads, 0, s>>>(logits, T, E, K, normalize, weights, indices, partial));
+    MTS_ROUTER_DISPATCH(router_fwd_kernel, <<<grid, kThreads, 0, s>>>(logits, T, E, K, normalize, weights, indices,
+                                                                      partial, partial_counts));
     MTS_CHECK_LAUNCH();
-    router_stats_kernel<<<1, kThreads, 0, s>>>(partial, grid, E, 1.0f / (float)T, prob_mean, z_loss,
-                                               entropy);
+    router_stats_kernel<<<1, kThreads, 0, s>>>(partial, partial_counts, grid, E, 1.0f / (float)T,
+                                               1.0f / ((float)T * (float)K), prob_mean, z_loss, entropy, counts,
+                                               load_balance);
     MTS_CHECK_LAUNCH();
     return MTS_OK;
 }
 
 extern "C" int mts_router_bwd(const float* logits, const float* weights, const int32_t* indices,
                               const float* g_weights, const float* g_prob_mean,
-                              const float* g_z_loss, int64_t T, int E, int K, int normalize,
-                              float* dlogits, void* stream) {
+                              const float* g_z_loss, const float* g_load_balance, const int32_t* counts,
+                              int64_t T, int E, int K, int normalize, float* dlogits, void* stream) {
     int rc = check_router(logits, T, E, K);
     if (rc) return rc;
     if (!weights || !indices || !g_weights || !g_prob_mean || !g_z_loss || !dlogits)
         return MTS_ERR_NULL;
+    if (g_load_balance && !counts) return MTS_ERR_NULL;
     if (E == 8 && !mts_aligned16(dlogits)) return MTS_ERR_ALIGN;
     hipStream_t s = (hipStream_t)stream;
     int G = E > 512 ? 64 : lanes_for(E);
     int grid = grid_for(T, G);
     MTS_ROUTER_DISPATCH(router_bwd_kernel,
                         <<<grid, kThreads, 0, s>>>(logits, weights, indices, g_weights, g_prob_mean,
-                                                   g_z_loss, T, E, K, normalize, dlogits));
+                                                   g_z_loss, g_load_balance, counts, T, E, K, normalize,
+                                                   dlogits));
     MTS_CHECK_LAUNCH();
     return MTS_OK;
 }

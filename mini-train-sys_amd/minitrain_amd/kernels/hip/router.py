@@ -38,29 +38,31 @@ class _RouterPostprocessFunction(torch.autograd.Function):
         dev = logits.device
         weights = torch.empty((T, top_k), device=dev, dtype=torch.float32)
         indices = torch.empty((T, top_k), device=dev, dtype=torch.int32)
-        stats = torch.empty(E + 2, device=dev, dtype=torch.float32)
+        stats = torch.empty(E + 3, device=dev, dtype=torch.float32)
+        counts = torch.empty(E, device=dev, dtype=torch.int32)
         ws_bytes = lib.mts_router_workspace_bytes(T, E)
         ws = torch.empty(ws_bytes, device=dev, dtype=torch.uint8)
-        prob_mean, z_loss, entropy = stats[:E], stats[E], stats[E + 1]
+        prob_mean, z_loss, entropy, load_balance = stats[:E], stats[E], stats[E + 1], stats[E + 2]
         _lib.check(
             lib.mts_router_fwd(
                 logits.data_ptr(), T, E, top_k, int(normalize), weights.data_ptr(), indices.data_ptr(),
-                prob_mean.data_ptr(), z_loss.data_ptr(), entropy.data_ptr(), ws.data_ptr(), ws_bytes,
-                _lib.stream_of(logits),
+                prob_mean.data_ptr(), z_loss.data_ptr(), entropy.data_ptr(), counts.data_ptr(),
+                load_balance.data_ptr(), ws.data_ptr(), ws_bytes, _lib.stream_of(logits),
             ),
             "mts_router_fwd",
         )
-        ctx.save_for_backward(logits, weights, indices)
+        ctx.save_for_backward(logits, weights, indices, counts)
         ctx.top_k = top_k
         ctx.normalize = normalize
-        ctx.mark_non_differentiable(indices, entropy)
-        return weights, indices, prob_mean, z_loss, entropy
+        ctx.mark_non_differentiable(indices, entropy, counts)
+        return weights, indices, prob_mean, z_loss, entropy, counts, load_balance
 
     @staticmethod
     @torch.amp.custom_bwd(device_type="cuda")
-    def backward(ctx, grad_weights, _grad_indices, grad_probability_mean, grad_z_loss, _grad_entropy):
+    def backward(ctx, grad_weights, _grad_indices, grad_probability_mean, grad_z_loss, _grad_entropy, _grad_counts,
+                 grad_load_balance):
         lib = _lib.load()
-        logits, weights, indices = ctx.saved_tensors
+        logits, weights, indices, counts = ctx.saved_tensors
         T, E = logits.shape
         dev = logits.device
 
@@ -72,12 +74,13 @@ class _RouterPostprocessFunction(torch.autograd.Function):
         g_w = dense(grad_weights, (T, ctx.top_k))
         g_p = dense(grad_probability_mean, (E,))
         g_z = dense(grad_z_loss, ())
+        g_lb = None if grad_load_balance is None else grad_load_balance.to(torch.float32).contiguous()
         grad_logits = torch.empty_like(logits)
         _lib.check(
             lib.mts_router_bwd(
                 logits.data_ptr(), weights.data_ptr(), indices.data_ptr(), g_w.data_ptr(), g_p.data_ptr(),
-                g_z.data_ptr(), T, E, ctx.top_k, int(ctx.normalize), grad_logits.data_ptr(),
-                _lib.stream_of(logits),
+                g_z.data_ptr(), _lib.ptr(g_lb), counts.data_ptr(), T, E, ctx.top_k, int(ctx.normalize),
+                grad_logits.data_ptr(), _lib.stream_of(logits),
             ),
             "mts_router_bwd",
         )
@@ -98,7 +101,7 @@ def router_postprocess(logits: torch.Tensor, top_k: int, *, normalize: bool) -> 
             "hip router postprocess requires non-empty 2D fp32 logits on the GPU, "
             f"1 <= top_k <= {_MAX_TOP_K} and at most {_MAX_EXPERTS} experts"
         )
-    weights, indices, probability_mean, z_loss, entropy = _RouterPostprocessFunction.apply(
+    weights, indices, probability_mean, z_loss, entropy, counts, load_balance = _RouterPostprocessFunction.apply(
         logits, top_k, normalize
     )
     return RouterPostprocessOutput(
@@ -107,6 +110,8 @@ def router_postprocess(logits: torch.Tensor, top_k: int, *, normalize: bool) -> 
         probability_per_expert=probability_mean,
         z_loss=z_loss,
         entropy=entropy,
+        expert_counts=counts,
+        load_balance_loss=load_balance,
     )
 
 

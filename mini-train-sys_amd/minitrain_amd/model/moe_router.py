@@ -59,14 +59,18 @@ class TopKRouter(nn.Module):
             expert_weights = route.expert_weights
             expert_indices = route.expert_indices
 
-            count_routes = getattr(ops, "expert_counts", None)
-            if count_routes is not None and expert_indices.is_cuda and expert_indices.dtype == torch.int32:
-                route_counts = count_routes(expert_indices, cfg.num_experts)
-            else:
-                route_counts = torch.bincount(expert_indices.flatten().long(), minlength=cfg.num_experts)
-            tokens_per_expert = route_counts.float() / expert_indices.numel()
-            # the assignment fraction carries no gradient; it enters through the mean probability
-            auxiliary_loss = cfg.num_experts * torch.sum(tokens_per_expert * route.probability_per_expert)
+            route_counts = getattr(route, "expert_counts", None)
+            auxiliary_loss = getattr(route, "load_balance_loss", None)
+            if route_counts is None:
+                count_routes = getattr(ops, "expert_counts", None)
+                if count_routes is not None and expert_indices.is_cuda and expert_indices.dtype == torch.int32:
+                    route_counts = count_routes(expert_indices, cfg.num_experts)
+                else:
+                    route_counts = torch.bincount(expert_indices.flatten().long(), minlength=cfg.num_experts)
+            if auxiliary_loss is None:
+                tokens_per_expert = route_counts.float() / expert_indices.numel()
+                # the assignment fraction carries no gradient; it enters through the mean probability
+                auxiliary_loss = cfg.num_experts * torch.sum(tokens_per_expert * route.probability_per_expert)
 
             accepted = route_counts.float()
             load_fraction = accepted / max(expert_indices.numel(), 1)

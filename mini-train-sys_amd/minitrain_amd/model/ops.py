@@ -20,6 +20,12 @@ class RouterPostprocessOutput:
     probability_per_expert: torch.Tensor
     z_loss: torch.Tensor
     entropy: torch.Tensor
+    # Beyond the reference's record (minitrain/model/ops.py:7-15), filled by backends that
+    # compute them in the same pass: routes per expert (int32 [E], no gradient) and the
+    # load-balancing term E * sum_e (routes_e / routes) * probability_per_expert_e, which is
+    # differentiable through the mean probability.  None means the caller computes them.
+    expert_counts: torch.Tensor | None = None
+    load_balance_loss: torch.Tensor | None = None
 
 
 class OpsBackend(Protocol):

@@ -30,14 +30,24 @@ def _check(logits, K, normalize, *, tied=False):
     torch.testing.assert_close(got.z_loss.cpu(), ref.z_loss, rtol=FWD_TOL, atol=FWD_TOL)
     torch.testing.assert_close(got.entropy.cpu(), ref.entropy, rtol=FWD_TOL, atol=FWD_TOL)
     assert not got.expert_indices.requires_grad and not got.entropy.requires_grad
+    # the bookkeeping of the router module, computed in the same pass: routes per expert (exact)
+    # and the load-balancing term E * sum_e f_e * pbar_e
+    T_, E_ = logits.shape
+    ref_counts = torch.bincount(ref.expert_indices.flatten().long(), minlength=E_)
+    assert got.expert_counts.dtype == torch.int32 and torch.equal(got.expert_counts.cpu().long(), ref_counts)
+    ref_lb = E_ * torch.sum(ref_counts.double() / (T_ * K) * ref.probability_per_expert.double())
+    torch.testing.assert_close(got.load_balance_loss.cpu().double(), ref_lb, rtol=FWD_TOL, atol=FWD_TOL)
     # backward through the combined objective of the reference's parity probe
     T, E = logits.shape
     rng = np.random.Generator(np.random.Philox(99))
     g_w = torch.from_numpy(rng.standard_normal((T, K)).astype(np.float32))
     g_p = torch.from_numpy(rng.standard_normal(E).astype(np.float32))
-    obj = (got.expert_weights * g_w.cuda()).sum() + (got.probability_per_expert * g_p.cuda()).sum() + 0.13 * got.z_loss
+    obj = ((got.expert_weights * g_w.cuda()).sum() + (got.probability_per_expert * g_p.cuda()).sum()
+           + 0.13 * got.z_loss + 0.37 * got.load_balance_loss)
     obj.backward()
-    closed = O.router_backward_closed(logits, ref.expert_indices, ref.expert_weights.double(), g_w, g_p, 0.13,
+    # the load-balancing term reaches the logits through the mean probability only
+    g_p_eff = g_p + (0.37 * E * ref_counts.double() / (T * K)).float()
+    closed = O.router_backward_closed(logits, ref.expert_indices, ref.expert_weights.double(), g_w, g_p_eff, 0.13,
                                       normalize=normalize)
     np.testing.assert_allclose(lg.grad.cpu().numpy(), closed, rtol=BWD_TOL, atol=BWD_TOL)
 
