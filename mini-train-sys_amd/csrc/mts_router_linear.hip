@@ -22,6 +22,24 @@ __device__ __forceinline__ void store4(bf16_t* p, f32x4 v) {
 }
 __device__ __forceinline__ void store4(float* p, f32x4 v) { *reinterpret_cast<f32x4*>(p) = v; }
 
+template <typename XT>
+struct RawVec;
+template <>
+struct RawVec<bf16_t> {
+    typedef bf16x4 type;
+};
+template <>
+struct RawVec<float> {
+    typedef f32x4 type;
+};
+__device__ __forceinline__ bf16x4 load_raw(const bf16_t* p) { return *reinterpret_cast<const bf16x4*>(p); }
+__device__ __forceinline__ f32x4 load_raw(const float* p) { return *reinterpret_cast<const f32x4*>(p); }
+__device__ __forceinline__ f32x4 widen(bf16x4 v) {
+    f32x4 r = {(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
+    return r;
+}
+__device__ __forceinline__ f32x4 widen(f32x4 v) { return v; }
+
 // Butterfly reduce-scatter over the 64 lanes of a wave: N values are live in v[0..N), the
 // partner is `O` lanes away.  While N > 1 a lane hands one half of its values to the partner
 // and adds the partner's copy of the half it keeps; once one value is left the remaining
@@ -54,42 +72,59 @@ __global__ __launch_bounds__(kFwdThreads) void router_logits_fwd_kernel(const XT
                                                                          const float* __restrict__ w, int64_t T,
                                                                          int H, int E, float* __restrict__ logits) {
     extern __shared__ __attribute__((aligned(16))) float w_lds[];   // [E][H]
+#pragma unroll 8
     for (int i = threadIdx.x * 4; i < E * H; i += kFwdThreads * 4)
         *reinterpret_cast<f32x4*>(w_lds + i) = *reinterpret_cast<const f32x4*>(w + i);
-    __syncthreads();
     const int lane = threadIdx.x % MTS_WAVE;
     const int64_t wave0 = (int64_t)blockIdx.x * (kFwdThreads / MTS_WAVE) + threadIdx.x / MTS_WAVE;
-    const int64_t nwaves = (int64_t)gridDim.x * (kFwdThreads / MTS_WAVE);
-    for (int64_t r0 = wave0 * kRows; r0 < T; r0 += nwaves * kRows) {
-        float acc[kRows][EP];
-#pragma unroll
-        for (int r = 0; r < kRows; ++r)
-#pragma unroll
-            for (int e = 0; e < EP; ++e) acc[r][e] = 0.f;
-        // every load of the row group is issued before the first use
-        f32x4 xv[PASSES][kRows];
+    const int64_t stride = (int64_t)gridDim.x * (kFwdThreads / MTS_WAVE) * kRows;
+    typedef typename RawVec<XT>::type raw_t;
+    // the loads of the next row group are issued before the arithmetic of the current one
+    raw_t cur[PASSES][kRows], nxt[PASSES][kRows];
+    auto load_group = [&](raw_t (&dst)[PASSES][kRows], int64_t r0) {
 #pragma unroll
         for (int ps = 0; ps < PASSES; ++ps) {
             const int c = lane * 4 + ps * MTS_WAVE * 4;
 #pragma unroll
             for (int r = 0; r < kRows; ++r) {
-                const f32x4 z = {0.f, 0.f, 0.f, 0.f};
-                xv[ps][r] = (c < H && r0 + r < T) ? load4(x + (r0 + r) * H + c) : z;
+                const bool ok = c < H && r0 + r < T;
+                dst[ps][r] = load_raw(x + (ok ? (r0 + r) * H + c : 0));   // a masked lane reads element 0; its weights are skipped
             }
         }
+    };
+    int64_t r0 = wave0 * kRows;
+    if (r0 < T) load_group(cur, r0);
+    __syncthreads();
+    for (; r0 < T; r0 += stride) {
+        if (r0 + stride < T) load_group(nxt, r0 + stride);
+        float acc[kRows][EP];
+#pragma unroll
+        for (int r = 0; r < kRows; ++r)
+#pragma unroll
+            for (int e = 0; e < EP; ++e) acc[r][e] = 0.f;
 #pragma unroll
         for (int ps = 0; ps < PASSES; ++ps) {
             const int c = lane * 4 + ps * MTS_WAVE * 4;
             if (c < H) {
+                f32x4 xv[kRows];
+#pragma unroll
+                for (int r = 0; r < kRows; ++r) {
+                    const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+                    xv[r] = r0 + r < T ? widen(cur[ps][r]) : z;
+                }
 #pragma unroll
                 for (int e = 0; e < EP; ++e) {
                     const f32x4 wv = *reinterpret_cast<const f32x4*>(w_lds + (e < E ? e : 0) * H + c);
 #pragma unroll
                     for (int r = 0; r < kRows; ++r)
-                        acc[r][e] += xv[ps][r][0] * wv[0] + xv[ps][r][1] * wv[1] + xv[ps][r][2] * wv[2] + xv[ps][r][3] * wv[3];
+                        acc[r][e] += xv[r][0] * wv[0] + xv[r][1] * wv[1] + xv[r][2] * wv[2] + xv[r][3] * wv[3];
                 }
             }
         }
+#pragma unroll
+        for (int ps = 0; ps < PASSES; ++ps)
+#pragma unroll
+            for (int r = 0; r < kRows; ++r) cur[ps][r] = nxt[ps][r];
         // Sum over the 64 lanes of kRows*EP values: at every step a lane hands half of its
         // values to the partner lane and adds the partner's copy of the half it keeps, so the
         // count halves with the lane distance (fixed order: bit-stable).  With kRows*EP == 32
@@ -208,7 +243,7 @@ extern "C" int mts_router_logits_fwd(const void* x, const float* w_r, int64_t T,
     hipStream_t s = (hipStream_t)stream;
     const int64_t groups = (T + kRows - 1) / kRows;
     int64_t blocks = (groups + 3) / 4;
-    if (blocks > 256 * 4) blocks = 256 * 4;
+    if (blocks > 256 * 2) blocks = 256 * 2;
     const dim3 grid((unsigned)blocks);
     const size_t lds = (size_t)E * H * sizeof(float);
     const int passes = (H + MTS_WAVE * 4 - 1) / (MTS_WAVE * 4);   // 1..4 since H <= 1024
