@@ -9,8 +9,54 @@ constexpr int kThreads = 256;
 
 // ---- combine -------------------------------------------------------------
 // One thread produces 8 consecutive columns (16 bytes of bf16) of one token:
-// K row loads of 16 bytes each, fp32 accumulation, one rounding.
+// K row loads of 16 bytes each, fp32 accumulation, one rounding.  A thread works on
+// UN outputs at a time (token t, t + T/UN, ...) and issues all their index, weight
+// and row loads before the first use, to keep enough bytes in flight per CU.
+template <int KK, int UN>
 __global__ __launch_bounds__(kThreads) void combine_bf16_kernel(
+    const bf16_t* __restrict__ y, const bf16_t* __restrict__ w, const int32_t* __restrict__ s_rev,
+    int64_t T, int K, int H, bf16_t* __restrict__ out) {
+    const int vec_per_row = H / 8;
+    const int64_t chunk = (T + UN - 1) / UN;           // tokens per unrolled slice
+    const int64_t total = chunk * (int64_t)vec_per_row;
+    for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total;
+         i += (int64_t)gridDim.x * kThreads) {
+        const int64_t t0 = i / vec_per_row;
+        const int c = (int)(i - t0 * vec_per_row);
+        bf16x8 v[UN][KK];
+        float s[UN][KK];
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const int64_t t = t0 + u * chunk;
+#pragma unroll
+            for (int k = 0; k < KK; ++k) {
+                const bool ok = t < T && k < K;
+                const int64_t row = ok ? s_rev[t * K + k] : 0;
+                s[u][k] = ok ? (w ? (float)w[t * K + k] : 1.0f) : 0.f;
+                v[u][k] = *reinterpret_cast<const bf16x8*>(y + row * H + c * 8);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const int64_t t = t0 + u * chunk;
+            if (t >= T) continue;
+            float acc[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+#pragma unroll
+            for (int k = 0; k < KK; ++k)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) acc[j] += s[u][k] * (float)v[u][k][j];
+            bf16x8 o;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) o[j] = (bf16_t)acc[j];
+            *reinterpret_cast<bf16x8*>(out + t * H + c * 8) = o;
+        }
+    }
+}
+
+// any K: the routes of a token are visited in a loop
+__global__ __launch_bounds__(kThreads) void combine_bf16_anyk_kernel(
     const bf16_t* __restrict__ y, const bf16_t* __restrict__ w, const int32_t* __restrict__ s_rev,
     int64_t T, int K, int H, bf16_t* __restrict__ out) {
     const int vec_per_row = H / 8;
@@ -145,8 +191,17 @@ extern "C" int mts_moe_combine(const void* y, const void* weights, const int32_t
     hipStream_t s = (hipStream_t)stream;
     if (act_dtype == MTS_BF16) {
         if (H % 8) return MTS_ERR_SHAPE;
-        combine_bf16_kernel<<<grid_1d(T * (int64_t)(H / 8)), kThreads, 0, s>>>(
-            (const bf16_t*)y, (const bf16_t*)weights, s_reverse, T, K, H, (bf16_t*)out);
+        constexpr int UN = 2;
+        const int64_t sliced = ((T + UN - 1) / UN) * (int64_t)(H / 8);
+        if (K <= 2)
+            combine_bf16_kernel<2, UN><<<grid_1d(sliced), kThreads, 0, s>>>(
+                (const bf16_t*)y, (const bf16_t*)weights, s_reverse, T, K, H, (bf16_t*)out);
+        else if (K <= 4)
+            combine_bf16_kernel<4, UN><<<grid_1d(sliced), kThreads, 0, s>>>(
+                (const bf16_t*)y, (const bf16_t*)weights, s_reverse, T, K, H, (bf16_t*)out);
+        else
+            combine_bf16_anyk_kernel<<<grid_1d(T * (int64_t)(H / 8)), kThreads, 0, s>>>(
+                (const bf16_t*)y, (const bf16_t*)weights, s_reverse, T, K, H, (bf16_t*)out);
     } else if (act_dtype == MTS_F32) {
         if (H % 4) return MTS_ERR_SHAPE;
         combine_f32_kernel<<<grid_1d(T * (int64_t)(H / 4)), kThreads, 0, s>>>(
