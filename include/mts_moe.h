@@ -100,14 +100,34 @@ int mts_router_logits_bwd(const float* dlogits, const void* x, const float* w_r,
  * s_scatter, s_reverse and x_gather may all be NULL: then only counts and
  * expert_start (and the tile list) are written, which is what the router module
  * needs in place of its torch.bincount (minitrain/model/moe_router.py:82).
- * Returns MTS_ERR_SHAPE if E > MTS_MAX_EXPERTS; indices outside [0,E) are a
- * caller error: they are clamped into range (memory-safe, result undefined).                        */
+ * A negative index marks a dropped route (see mts_moe_capacity_mask): it is not
+ * counted and gets no row, its s_reverse entry is -1, and expert_start[E] is the
+ * number of kept routes; every kernel below works on the kept rows only, combine
+ * and the routing-weight gradient skip the -1 entries.
+ * Returns MTS_ERR_SHAPE if E > MTS_MAX_EXPERTS; indices >= E are a caller error:
+ * they are clamped into range (memory-safe, result undefined).                  */
 int64_t mts_moe_route_workspace_bytes(int64_t T, int K, int E);
 int mts_moe_route(const int32_t* top_k_index, int64_t T, int K, int E, int block_m,
                   int32_t* counts, int32_t* expert_start, int32_t* s_scatter,
                   int32_t* s_reverse, int32_t* x_gather, int32_t* tile_row_start,
                   int32_t* tile_expert, int32_t* tile_count, void* workspace,
                   int64_t workspace_bytes, void* stream);
+
+/* ---- capacity-limited dispatch --------------------------------------------
+ * The selection rule of TopKRouter._capacity_mask (minitrain/model/moe_router.py:
+ * 29-61): per expert, the `capacity` routes with the largest router weight are
+ * kept, equal weights in ascending flat entry (t*K+k) order.  keep [T*K] gets 1/0
+ * per entry; kept_index [T*K] (may be NULL) gets the expert index of a kept route
+ * and -1 for a dropped one, which is the form mts_moe_route takes for a compacted
+ * dispatch (the compaction the reference reserves its expert_capacity_factor for,
+ * minitrain/model/config.py:24-28); accepted_counts [E] = min(count_e, capacity).
+ * top_k_weights are the fp32 router weights.  The caller computes capacity =
+ * max(min_capacity, ceil(factor*T*K/E)) (moe_router.py:38-42).                 */
+int64_t mts_moe_capacity_workspace_bytes(int64_t T, int K, int E);
+int mts_moe_capacity_mask(const int32_t* top_k_index, const float* top_k_weights, int64_t T, int K,
+                          int E, int64_t capacity, uint8_t* keep, int32_t* kept_index,
+                          int32_t* accepted_counts, void* workspace, int64_t workspace_bytes,
+                          void* stream);
 
 /* ---- weight staging -----------------------------------------------------
  * src [E,R,C] of src_dtype -> dst of dst_dtype, [E,R,C] (transpose=0) or [E,C,R]

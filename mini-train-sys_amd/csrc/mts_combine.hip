@@ -12,6 +12,7 @@ constexpr int kThreads = 256;
 // K row loads of 16 bytes each, fp32 accumulation, one rounding.  A thread works on
 // UN outputs at a time (token t, t + T/UN, ...) and issues all their index, weight
 // and row loads before the first use, to keep enough bytes in flight per CU.
+// A negative s_rev entry is a dropped route: it contributes nothing, whatever its weight.
 template <int KK, int UN>
 __global__ __launch_bounds__(kThreads) void combine_bf16_kernel(
     const bf16_t* __restrict__ y, const bf16_t* __restrict__ w, const int32_t* __restrict__ s_rev,
@@ -30,10 +31,14 @@ __global__ __launch_bounds__(kThreads) void combine_bf16_kernel(
             const int64_t t = t0 + u * chunk;
 #pragma unroll
             for (int k = 0; k < KK; ++k) {
-                const bool ok = t < T && k < K;
-                const int64_t row = ok ? s_rev[t * K + k] : 0;
-                s[u][k] = ok ? (w ? (float)w[t * K + k] : 1.0f) : 0.f;
+                const bool in = t < T && k < K;
+                const int32_t r = in ? s_rev[t * K + k] : -1;
+                const bool ok = r >= 0;
+                const int64_t row = ok ? r : 0;
+                const float wt = in ? (w ? (float)w[t * K + k] : 1.0f) : 0.f;
+                s[u][k] = ok ? wt : 0.f;
                 v[u][k] = *reinterpret_cast<const bf16x8*>(y + row * H + c * 8);
+                if (!ok) v[u][k] = bf16x8{};   // row 0 may hold anything
             }
         }
 #pragma unroll
@@ -70,6 +75,7 @@ __global__ __launch_bounds__(kThreads) void combine_bf16_anyk_kernel(
         for (int j = 0; j < 8; ++j) acc[j] = 0.f;
         for (int k = 0; k < K; ++k) {
             const int64_t row = s_rev[t * K + k];
+            if (row < 0) continue;
             const float s = w ? (float)w[t * K + k] : 1.0f;
             const bf16x8 v = *reinterpret_cast<const bf16x8*>(y + row * H + c * 8);
 #pragma unroll
@@ -94,6 +100,7 @@ __global__ __launch_bounds__(kThreads) void combine_f32_kernel(
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
         for (int k = 0; k < K; ++k) {
             const int64_t row = s_rev[t * K + k];
+            if (row < 0) continue;
             const float s = w ? w[t * K + k] : 1.0f;
             const f32x4 v = *reinterpret_cast<const f32x4*>(y + row * H + c * 4);
             acc += s * v;
@@ -110,9 +117,12 @@ __global__ __launch_bounds__(kThreads) void ds_reduce_kernel(const float* __rest
                                                              OutT* __restrict__ d_w) {
     for (int64_t n = (int64_t)blockIdx.x * kThreads + threadIdx.x; n < TK;
          n += (int64_t)gridDim.x * kThreads) {
-        const float* p = part + (int64_t)s_rev[n] * np;
+        const int32_t r = s_rev[n];   // negative: dropped route, no gradient
         float v = 0.f;
-        for (int j = 0; j < np; ++j) v += p[j];
+        if (r >= 0) {
+            const float* p = part + (int64_t)r * np;
+            for (int j = 0; j < np; ++j) v += p[j];
+        }
         d_w[n] = (OutT)v;
     }
 }

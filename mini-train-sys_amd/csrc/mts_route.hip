@@ -9,6 +9,10 @@
 //                  same expert are found with ballots, rank inside the group is a
 //                  popcount of the lower lanes, so entries keep ascending order
 //                  inside every expert (a stable sort by expert).
+//
+// A negative expert id marks a dropped route (capacity-limited dispatch): it is not
+// counted, gets no row, and its s_reverse entry is -1.  expert_start[E] is the number
+// of routes that were kept.
 #include "mts_common.h"
 
 namespace {
@@ -18,9 +22,9 @@ constexpr int kWaves = kThreads / MTS_WAVE;
 constexpr int kChunk = 256;   // entries per wave
 constexpr int kSteps = kChunk / MTS_WAVE;
 
-// Expert ids outside [0,E) are a caller error; they are clamped so that no
-// address derived from them can leave the output arrays.
-__device__ __forceinline__ int clamp_expert(int e, int E) { return e < 0 ? 0 : (e >= E ? E - 1 : e); }
+// Expert ids >= E are a caller error; they are clamped so that no address derived from
+// them can leave the output arrays.  Negative ids (dropped routes) stay negative.
+__device__ __forceinline__ int clamp_expert(int e, int E) { return e >= E ? E - 1 : e; }
 
 __global__ __launch_bounds__(kThreads) void route_hist_kernel(const int32_t* __restrict__ idx,
                                                               int64_t TK, int E,
@@ -34,7 +38,8 @@ __global__ __launch_bounds__(kThreads) void route_hist_kernel(const int32_t* __r
     int32_t* mine = lds + wave * E;
     for (int i = lane; i < kChunk; i += MTS_WAVE) {
         int64_t n = base + i;
-        if (n < TK) atomicAdd(&mine[clamp_expert(idx[n], E)], 1);
+        const int e = n < TK ? clamp_expert(idx[n], E) : -1;
+        if (e >= 0) atomicAdd(&mine[e], 1);
     }
     __syncthreads();
     if (base < TK) {
@@ -99,7 +104,7 @@ __global__ __launch_bounds__(1024) void route_scan_kernel(
         if (lane == 0) {
             start[E] = carry;
             tile_off[E] = tcarry;
-            expert_start[E] = (int32_t)TK;
+            expert_start[E] = carry;
             if (tile_count) tile_count[0] = tcarry;
         }
     }
@@ -136,9 +141,9 @@ __global__ __launch_bounds__(kThreads) void route_scatter_kernel(
 #pragma unroll
     for (int s = 0; s < kSteps; ++s) {
         const int64_t n = base + s * MTS_WAVE + lane;
-        const bool valid = n < TK;
         const int e = ev[s];
-        int pos = 0;
+        const bool valid = e >= 0;
+        int pos = -1;
         uint64_t todo = __ballot(valid);
         while (todo) {
             int leader = __ffsll((unsigned long long)todo) - 1;
@@ -149,8 +154,8 @@ __global__ __launch_bounds__(kThreads) void route_scatter_kernel(
             if (lane == leader) next[el] = first + __popcll(same);
             todo &= ~same;
         }
+        if (n < TK) s_reverse[n] = pos;
         if (valid) {
-            s_reverse[n] = pos;
             s_scatter[pos] = (int32_t)n;
             x_gather[pos] = (int32_t)(n / K);
         }

@@ -6,6 +6,7 @@ that class there is no fallback: an unsupported tensor contract raises.
 """
 
 from minitrain_amd.kernels.dense_ops import DenseTorchOps
+from minitrain_amd.kernels.hip.capacity import capacity_mask, is_capacity_mask_supported
 from minitrain_amd.kernels.hip.fused_moe import expert_counts, fused_moe, is_fused_moe_supported
 from minitrain_amd.kernels.hip.router import (
     is_router_logits_supported,
@@ -17,6 +18,8 @@ from minitrain_amd.kernels.hip.router import (
 
 class HipOpsBackend(DenseTorchOps):
     name = "hip"
+    # fused_moe gives a route whose expert index is negative no row in the expert GEMMs
+    drops_routes = True
 
     def router_postprocess(self, logits, top_k, *, normalize):
         return router_postprocess(logits, top_k, normalize=normalize)
@@ -27,6 +30,13 @@ class HipOpsBackend(DenseTorchOps):
     def expert_counts(self, expert_indices, num_experts):
         """Extension: routes per expert (int32 ``[E]``) without a host synchronisation."""
         return expert_counts(expert_indices, num_experts)
+
+    def capacity_mask(self, expert_indices, expert_weights, num_experts, capacity):
+        """Extension: ``(keep, kept_index, accepted)`` of a capacity-limited dispatch, or None when
+        the contract is not supported (the caller then uses its own sort-based selection)."""
+        if not is_capacity_mask_supported(expert_indices, expert_weights, num_experts):
+            return None
+        return capacity_mask(expert_indices, expert_weights, num_experts, capacity)
 
     def router_logits(self, hidden_states, weight):
         """Extension beyond the reference's operator interface: the router projection in fp32
@@ -39,8 +49,10 @@ class HipOpsBackend(DenseTorchOps):
 
 __all__ = [
     "HipOpsBackend",
+    "capacity_mask",
     "expert_counts",
     "fused_moe",
+    "is_capacity_mask_supported",
     "is_fused_moe_supported",
     "is_router_logits_supported",
     "is_router_postprocess_supported",

@@ -39,9 +39,9 @@ class MoEFeedForward(nn.Module):
         shape = x.shape
         flat_x = x.reshape(-1, shape[-1])
         route = self.router(flat_x, ops)
-        hidden = ops.fused_moe(
-            flat_x, self.gate_up_proj, self.down_proj, route.expert_indices, route.expert_weights
-        ).view(shape)
+        # under a capacity limit the router may hand over a dispatch in which dropped routes carry -1
+        dispatch = route.expert_indices if route.dispatch_indices is None else route.dispatch_indices
+        hidden = ops.fused_moe(flat_x, self.gate_up_proj, self.down_proj, dispatch, route.expert_weights).view(shape)
         return FeedForwardOutput(
             hidden_states=self.dropout(hidden),
             router_aux_loss=route.auxiliary_loss,

@@ -1,5 +1,7 @@
 """Model configuration: the fields, names and defaults of the reference's ``ModelConfig``
-(minitrain/model/config.py:4-27) that the decoder and its MoE blocks read."""
+(minitrain/model/config.py:4-63) that the decoder and its MoE blocks read.  The reference
+reserves ``expert_capacity_factor`` / ``expert_min_capacity`` for a compacted dispatch and
+ignores them (config.py:24-28); here a factor other than None switches that dispatch on."""
 
 from dataclasses import dataclass
 
@@ -23,6 +25,8 @@ class ModelConfig:
     router_z_loss_coef: float = 1e-3
     router_normalize_topk: bool = True
     router_jitter_noise: float = 0.0
+    expert_capacity_factor: float | None = None
+    expert_min_capacity: int = 4
 
     def __post_init__(self) -> None:
         sizes = (self.vocab_size, self.seq_len, self.n_layers, self.n_heads, self.hidden_size, self.intermediate_size)
@@ -44,6 +48,10 @@ class ModelConfig:
             raise ValueError("router loss coefficients must be non-negative")
         if not 0 <= self.router_jitter_noise < 1:
             raise ValueError("router_jitter_noise must be in [0, 1)")
+        if self.expert_capacity_factor is not None and self.expert_capacity_factor <= 0:
+            raise ValueError("expert_capacity_factor must be positive or null")
+        if self.expert_min_capacity <= 0:
+            raise ValueError("expert_min_capacity must be positive")
 
     @property
     def head_dim(self) -> int:

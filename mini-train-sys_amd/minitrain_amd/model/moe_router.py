@@ -5,6 +5,12 @@ Same arithmetic and record as the reference's ``TopKRouter``
 post-process operator, assignment counts, the load-balancing loss
 ``E * sum_e f_e * pbar_e`` and the load metrics; indices are returned as int32 and
 weights in the activation dtype.
+
+With ``cfg.expert_capacity_factor`` set, the capacity limit the reference keeps switched
+off (moe_router.py:29-61 and the commented block at :92-110) is applied: an expert accepts
+its ``capacity`` most confident routes, the weights of dropped routes become zero, the
+remaining weights of a token are renormalised, and ``dispatch_indices`` tells a backend
+that compacts its dispatch (``ops.drops_routes``) which routes to leave out.
 """
 
 import math
@@ -25,6 +31,33 @@ class RouterOutput:
     auxiliary_loss: torch.Tensor
     z_loss: torch.Tensor
     metrics: dict[str, torch.Tensor]
+    # what fused_moe is called with when it differs from expert_indices: -1 marks a dropped route
+    dispatch_indices: torch.Tensor | None = None
+
+
+def _order_key(weights: torch.Tensor) -> torch.Tensor:
+    """int64 key that grows with the fp32 weight (-0 and +0 alike)."""
+    w = torch.where(weights == 0, torch.zeros_like(weights), weights).float().contiguous()
+    bits = w.view(torch.int32).long() & 0xFFFFFFFF
+    return torch.where(bits >= 2**31, 0xFFFFFFFF - bits, bits + 2**31)
+
+
+def capacity_selection(expert_indices: torch.Tensor, expert_weights: torch.Tensor, num_experts: int, capacity: int):
+    """``(keep, kept_index, accepted)``: per expert the ``capacity`` routes with the largest
+    weight, equal weights in ascending flat-entry order (the rule of the reference's
+    ``_capacity_mask``, minitrain/model/moe_router.py:43-61), from one stable sort of a
+    composite (expert, descending weight) key."""
+    flat_experts = expert_indices.flatten().long()
+    composite = flat_experts * 2**32 + (0xFFFFFFFF - _order_key(expert_weights.detach().flatten()))
+    order = torch.sort(composite, stable=True).indices
+    counts = torch.bincount(flat_experts, minlength=num_experts)
+    first_row = counts.cumsum(0) - counts
+    rank = torch.arange(order.numel(), device=order.device) - first_row[flat_experts[order]]
+    keep = torch.empty_like(flat_experts, dtype=torch.bool)
+    keep[order] = rank < capacity
+    keep = keep.view_as(expert_indices)
+    kept_index = torch.where(keep, expert_indices, torch.full_like(expert_indices, -1))
+    return keep, kept_index, counts.clamp(max=capacity)
 
 
 class TopKRouter(nn.Module):
@@ -72,7 +105,33 @@ class TopKRouter(nn.Module):
                 # the assignment fraction carries no gradient; it enters through the mean probability
                 auxiliary_loss = cfg.num_experts * torch.sum(tokens_per_expert * route.probability_per_expert)
 
+            dispatch_indices = None
+            dropped_fraction = expert_weights.new_zeros(())
             accepted = route_counts.float()
+            if cfg.expert_capacity_factor is not None:
+                tokens, top_k = expert_indices.shape
+                capacity = max(
+                    cfg.expert_min_capacity, math.ceil(cfg.expert_capacity_factor * tokens * top_k / cfg.num_experts)
+                )
+                selection = None
+                select = getattr(ops, "capacity_mask", None)
+                if select is not None:
+                    selection = select(expert_indices, expert_weights, cfg.num_experts, capacity)
+                if selection is None:
+                    selection = capacity_selection(expert_indices, expert_weights, cfg.num_experts, capacity)
+                keep, kept_index, accepted_counts = selection
+                expert_weights = expert_weights * keep
+                if cfg.router_normalize_topk:
+                    denominator = expert_weights.sum(dim=-1, keepdim=True)
+                    expert_weights = torch.where(
+                        denominator > 0,
+                        expert_weights / denominator.clamp_min(torch.finfo(expert_weights.dtype).eps),
+                        expert_weights,
+                    )
+                if getattr(ops, "drops_routes", False):
+                    dispatch_indices = kept_index.to(torch.int32)
+                accepted = accepted_counts.float()
+                dropped_fraction = 1.0 - keep.float().mean()
             load_fraction = accepted / max(expert_indices.numel(), 1)
             uniform = 1.0 / cfg.num_experts
             metrics = {
@@ -80,7 +139,7 @@ class TopKRouter(nn.Module):
                 "moe/router_entropy_normalized": (
                     route.entropy / (math.log(cfg.num_experts) if cfg.num_experts > 1 else 1.0)
                 ).detach(),
-                "moe/dropped_route_fraction": expert_weights.new_zeros(()).detach(),
+                "moe/dropped_route_fraction": dropped_fraction.detach(),
                 "moe/max_expert_load": accepted.max().detach(),
                 "moe/min_expert_load": accepted.min().detach(),
                 "moe/expert_load_cv": (load_fraction.std(unbiased=False) / uniform).detach(),
@@ -96,4 +155,5 @@ class TopKRouter(nn.Module):
             auxiliary_loss=auxiliary_loss,
             z_loss=route.z_loss,
             metrics=metrics,
+            dispatch_indices=dispatch_indices,
         )

@@ -19,6 +19,9 @@ Reference lines each function follows (paths relative to the reference root):
                                  567-596 (dS, dgate, dup), 627-672 (dW2),
                                  700-756 (dx), 783-828 (dW1).
 * ``topk_router``             -> minitrain/model/moe_router.py:63-90, 138-144.
+* ``expert_capacity``, ``capacity_mask`` -> minitrain/model/moe_router.py:29-61.
+* ``apply_capacity``          -> the switched-off block at minitrain/model/moe_router.py:
+                                 98-110 (mask the weights, renormalise per token).
 * ``moe_feed_forward``        -> minitrain/model/blocks.py:86-96.
 
 How each function is pinned (see tests/test_oracle_*.py):
@@ -33,6 +36,13 @@ How each function is pinned (see tests/test_oracle_*.py):
 * fused MoE forward: a per-route float64 brute-force loop on tiny shapes.
 * fused MoE backward: float64 finite differences and autograd against the
   closed form.
+* capacity mask: a per-expert Python sort on small cases, the invariants of the
+  rule (kept = min(count, capacity) per expert, no dropped route outweighs a kept
+  one of its expert, ties leave in descending entry order) and the all-ties case
+  K=1 with normalised weights, where the first ``capacity`` tokens of an expert stay.
+* dropped routes in ``fused_moe`` (expert index -1): the same outputs and
+  gradients as the reference's own convention for them, a zero weight
+  (minitrain/kernels/torch_ops.py:135-140).
 
 Two behaviours of the reference's PyTorch path are library-defined and are NOT
 reproduced bit for bit ("parity unpinned" at the bit level, pinned at tolerance
@@ -171,7 +181,7 @@ def router_backward_closed(logits, indices, weights, g_w, g_p, g_z, *, normalize
 @dataclass
 class RoutingMeta:
     counts: np.ndarray            # [E]   routes per expert
-    expert_start: np.ndarray      # [E+1] exclusive prefix sum, last = T*K
+    expert_start: np.ndarray      # [E+1] exclusive prefix sum, last = number of kept routes (T*K without drops)
     s_scatter_idx: np.ndarray     # [TK]  sorted position -> entry (t*K+k)
     s_reverse_scatter_idx: np.ndarray  # [TK] entry -> sorted position
     x_gather_idx: np.ndarray      # [TK]  sorted position -> token
@@ -183,12 +193,14 @@ def routing_metadata(top_k_index, E: int, block_m: int = 64) -> RoutingMeta:
     idx = np.asarray(top_k_index)
     T, K = idx.shape
     flat = idx.reshape(-1).astype(np.int64)
-    counts = np.bincount(flat, minlength=E).astype(np.int32)
+    # a negative index is a dropped route of a capacity-limited dispatch: it gets no row
+    kept = np.flatnonzero(flat >= 0)
+    counts = np.bincount(flat[kept], minlength=E).astype(np.int32)
     expert_start = np.zeros(E + 1, dtype=np.int32)
     expert_start[1:] = np.cumsum(counts)
-    order = np.argsort(flat, kind="stable").astype(np.int32)
-    rev = np.empty(T * K, dtype=np.int32)
-    rev[order] = np.arange(T * K, dtype=np.int32)
+    order = kept[np.argsort(flat[kept], kind="stable")].astype(np.int32)
+    rev = np.full(T * K, -1, dtype=np.int32)
+    rev[order] = np.arange(order.size, dtype=np.int32)
     rows, experts = [], []
     for e in range(E):
         for r in range(int(expert_start[e]), int(expert_start[e + 1]), block_m):
@@ -221,6 +233,8 @@ def fused_moe(x, gate_up_proj, down_proj, top_k_index, top_k_weights, *, compute
         top_k_weights = top_k_weights.to(compute_dtype)
     out = torch.zeros_like(x)
     for e in torch.unique(top_k_index).tolist():
+        if e < 0:   # dropped route of a capacity-limited dispatch: no contribution
+            continue
         tok, kpos = torch.where(top_k_index == e)
         if tok.numel() == 0:
             continue
@@ -246,6 +260,8 @@ def fused_moe_bruteforce(x, gate_up_proj, down_proj, top_k_index, top_k_weights)
     for t in range(T):
         for k in range(idx.shape[1]):
             e = int(idx[t, k])
+            if e < 0:
+                continue
             g = np.array([sum(w1[e, i, h] * x[t, h] for h in range(H)) for i in range(I)])
             u = np.array([sum(w1[e, I + i, h] * x[t, h] for h in range(H)) for i in range(I)])
             a = g / (1.0 + np.exp(-g)) * u
@@ -272,6 +288,8 @@ def fused_moe_backward_closed(x, gate_up_proj, down_proj, top_k_index, top_k_wei
     for t in range(T):
         for k in range(K):
             e = int(idx[t, k])
+            if e < 0:
+                continue
             z = w1[e] @ x[t]
             g, u = z[:I], z[I:]
             sig = 1.0 / (1.0 + np.exp(-g))
@@ -286,6 +304,39 @@ def fused_moe_backward_closed(x, gate_up_proj, down_proj, top_k_index, top_k_wei
             dw1[e] += np.outer(dz, x[t])
             dx[t] += w1[e].T @ dz
     return dx, dw1, dw2, dS
+
+
+# ---------------------------------------------------------------------------
+# Capacity-limited dispatch
+# ---------------------------------------------------------------------------
+
+def expert_capacity(tokens: int, top_k: int, num_experts: int, factor: float, min_capacity: int) -> int:
+    return max(min_capacity, math.ceil(factor * tokens * top_k / num_experts))
+
+
+def capacity_mask(expert_indices, expert_weights, num_experts: int, capacity: int) -> torch.Tensor:
+    """bool ``[T,K]``: routes ordered by descending weight (stable), then grouped by expert
+    (stable); a route stays if its rank inside its expert is below ``capacity``."""
+    e = np.asarray(expert_indices).reshape(-1).astype(np.int64)
+    w = np.asarray(expert_weights.detach().float()).reshape(-1)
+    by_weight = np.argsort(-w, kind="stable")
+    route_order = by_weight[np.argsort(e[by_weight], kind="stable")]
+    counts = np.bincount(e, minlength=num_experts)
+    first = np.cumsum(counts) - counts
+    rank = np.arange(e.size) - np.repeat(first, counts)
+    keep = np.zeros(e.size, dtype=bool)
+    keep[route_order] = rank < capacity
+    return torch.from_numpy(keep.reshape(tuple(expert_indices.shape)))
+
+
+def apply_capacity(expert_weights, keep, *, normalize: bool):
+    """Weights of dropped routes become zero; with ``normalize`` the weights a token has
+    left are rescaled to sum to one (a token that lost every route keeps zeros)."""
+    w = expert_weights * keep
+    if normalize:
+        denominator = w.sum(dim=-1, keepdim=True)
+        w = torch.where(denominator > 0, w / denominator.clamp_min(torch.finfo(w.dtype).eps), w)
+    return w
 
 
 # ---------------------------------------------------------------------------
