@@ -185,16 +185,28 @@ int mts_moe_bwd_dx(const void* d_pre_act, const void* w1t, const int32_t* expert
 
 /* Replaces _moe_bwd_dW2_kernel (fused_moe_kernels.py:602-672):
  * dW2[e] = sum_{r in e} dO[x_gather[r]] (x) weighted_act[r]   -> [E,H,I] grad_dtype.
- * Experts without routes receive zeros.                                      */
+ * Experts without routes receive zeros.
+ *
+ * workspace (both weight-gradient entry points): NULL, or at least
+ * mts_moe_bwd_dw_workspace_bytes(which, E, H, I) bytes (which = 1 for dW1, 2 for dW2).
+ * With a workspace, an expert that holds more than 1.25 times the balanced share of the
+ * routes has its rows cut into chunks that run as separate blocks and are added in a
+ * fixed order by a second kernel, so that skewed routing does not leave the GPU waiting
+ * for the tiles of the fullest expert; results stay run-to-run identical.  Without one,
+ * every tile reduces over all rows of its expert in one block (bf16 activations only;
+ * the fp32 path ignores the workspace).                                        */
+int64_t mts_moe_bwd_dw_workspace_bytes(int which, int E, int H, int I);
 int mts_moe_bwd_dw2(const void* d_out, const void* weighted_act, const int32_t* x_gather,
                     const int32_t* expert_start, int64_t T, int K, int E, int H, int I,
-                    int act_dtype, int grad_dtype, void* d_w2, void* stream);
+                    int act_dtype, int grad_dtype, void* d_w2, void* workspace,
+                    int64_t workspace_bytes, void* stream);
 
 /* Replaces _moe_bwd_dW1_kernel (fused_moe_kernels.py:758-828):
  * dW1[e] = sum_{r in e} [dg;du][r] (x) x[x_gather[r]]        -> [E,2I,H] grad_dtype. */
 int mts_moe_bwd_dw1(const void* d_pre_act, const void* x, const int32_t* x_gather,
                     const int32_t* expert_start, int64_t T, int K, int E, int H, int I,
-                    int act_dtype, int grad_dtype, void* d_w1, void* stream);
+                    int act_dtype, int grad_dtype, void* d_w1, void* workspace,
+                    int64_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus
 }

@@ -816,8 +816,114 @@ struct DwParams {
     int64_t TK;
     const int32_t* expert_start;
     void* C;  // [E][M][N], bf16 or f32
+    float* part;   // fp32 tile partials of experts whose rows are split over several blocks, or null
     int E, n_tiles, tiles_per_expert;  // set by the launcher
 };
+
+// ---------------------------------------------------------------------------
+// Row chunks of over-full experts.  A weight-gradient tile reduces over all rows of its
+// expert, so with skewed routing the tiles of the fullest expert set the kernel's time.
+// When the caller supplies a workspace, an expert with more than 1.25 times the balanced
+// share of rows (share = ceil(kept routes / E), rounded up to 32) is cut into
+// ceil(count / share) chunks of equal length (a multiple of 32 rows).  A (expert, chunk)
+// pair is a unit; the units of an expert that was cut write fp32 tiles to the workspace,
+// slot by slot, and a second kernel adds the chunks of a tile in chunk order, so the result
+// does not depend on the order the blocks ran in.  There are at most 2E units.
+// ---------------------------------------------------------------------------
+struct DwUnit {
+    int e, rbeg, rend;   // expert and the rows of this unit
+    int slot;            // index of the unit's partial tiles in the workspace, -1: writes C itself
+};
+
+__device__ __forceinline__ int dw_share(const DwParams& p) {
+    const int total = p.expert_start[p.E];
+    return ((total + p.E - 1) / p.E + 31) / 32 * 32;
+}
+
+__device__ __forceinline__ int dw_chunks(const DwParams& p, int count, int share) {
+    return (p.part != nullptr && count > share + share / 4) ? (count + share - 1) / share : 1;
+}
+
+// every lane of the calling wave gets the same answer
+__device__ __forceinline__ bool locate_dw_unit(const DwParams& p, int unit, DwUnit& u) {
+    const int lane = threadIdx.x % MTS_WAVE;
+    const int share = dw_share(p);
+    int seen = 0, seen_slots = 0;
+    for (int e0 = 0; e0 < p.E; e0 += MTS_WAVE) {
+        const int le = e0 + lane;
+        const int s0 = le < p.E ? p.expert_start[le] : 0;
+        const int s1 = le < p.E ? p.expert_start[le + 1] : 0;
+        const int nc = le < p.E ? dw_chunks(p, s1 - s0, share) : 0;
+        const int ns = nc > 1 ? nc : 0;
+        int incl = nc, sincl = ns;
+#pragma unroll
+        for (int o = 1; o < MTS_WAVE; o <<= 1) {
+            const int up = __shfl_up(incl, o, MTS_WAVE), sup = __shfl_up(sincl, o, MTS_WAVE);
+            if (lane >= o) {
+                incl += up;
+                sincl += sup;
+            }
+        }
+        const uint64_t hit = __ballot(le < p.E && unit < seen + incl);
+        if (hit) {
+            const int w = __ffsll((unsigned long long)hit) - 1;
+            const int ncw = __shfl(nc, w, MTS_WAVE);
+            const int c = unit - (seen + __shfl(incl, w, MTS_WAVE) - ncw);
+            const int b = __shfl(s0, w, MTS_WAVE), e = __shfl(s1, w, MTS_WAVE);
+            const int per = ((e - b + ncw - 1) / ncw + 31) / 32 * 32;
+            const int r0 = b + c * per;
+            u.e = e0 + w;
+            u.rbeg = r0 < e ? r0 : e;
+            u.rend = r0 + per < e ? r0 + per : e;
+            u.slot = ncw > 1 ? seen_slots + __shfl(sincl, w, MTS_WAVE) - __shfl(ns, w, MTS_WAVE) + c : -1;
+            return true;
+        }
+        seen += __shfl(incl, MTS_WAVE - 1, MTS_WAVE);
+        seen_slots += __shfl(sincl, MTS_WAVE - 1, MTS_WAVE);
+    }
+    return false;
+}
+
+// Adds the chunk partials of the experts that were cut: thread = 4 consecutive columns of a tile row.
+template <int BM, int BN, typename OutT>
+__global__ __launch_bounds__(256) void dw_chunk_sum_kernel(DwParams p) {
+    const int e = blockIdx.y;
+    const int lane = threadIdx.x % MTS_WAVE;
+    const int share = dw_share(p);
+    const int nc = dw_chunks(p, p.expert_start[e + 1] - p.expert_start[e], share);
+    if (nc <= 1) return;
+    int before = 0;   // slots of the experts below e
+    for (int le = lane; le < e; le += MTS_WAVE) {
+        const int c = dw_chunks(p, p.expert_start[le + 1] - p.expert_start[le], share);
+        before += c > 1 ? c : 0;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) before += __shfl_xor(before, o, MTS_WAVE);
+    constexpr int PER_TILE = BM * BN / 4;
+    const int64_t tile_stride = (int64_t)BM * BN;
+    const int64_t items = (int64_t)p.tiles_per_expert * PER_TILE;
+    for (int64_t item = (int64_t)blockIdx.x * 256 + threadIdx.x; item < items; item += (int64_t)gridDim.x * 256) {
+        const int tile = (int)(item / PER_TILE), within = (int)(item % PER_TILE);
+        const int ml = within / (BN / 4), nl = (within % (BN / 4)) * 4;
+        const int m = (tile / p.n_tiles) * BM + ml, n = (tile % p.n_tiles) * BN + nl;
+        if (m >= p.M || n >= p.N) continue;
+        const float* src = p.part + ((int64_t)before * p.tiles_per_expert + tile) * tile_stride + (int64_t)ml * BN + nl;
+        const int64_t chunk_stride = (int64_t)p.tiles_per_expert * tile_stride;
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        for (int c0 = 0; c0 < nc; c0 += 4) {   // four loads in flight, added in chunk order
+            f32x4 v[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                v[j] = c0 + j < nc ? *reinterpret_cast<const f32x4*>(src + (c0 + j) * chunk_stride) : f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc += v[j];
+        }
+        OutT* C = reinterpret_cast<OutT*>(p.C) + ((int64_t)e * p.M + m) * p.N + n;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (n + j < p.N) C[j] = (OutT)acc[j];
+    }
+}
 
 // Stages a [64 k][64 m] block per wave-item: lane = (kgrp = lane%8, mc = lane/8) loads
 // rows k = 8*kgrp+i, columns 8*mc..8*mc+7, transposes the 8x8 block in registers
@@ -1014,12 +1120,15 @@ template <class T, typename OutT>
 __global__ __launch_bounds__(T::NT) void dw_gemm_ws_kernel(DwParams p) {
     __shared__ __attribute__((aligned(1024))) bf16_t smem[T::LDS_ELEMS];
     constexpr int S = T::STAGES, L = T::A_INSTR + T::B_INSTR;
+    // all tiles of a unit (an expert, or a row chunk of an over-full one) run on one XCD
     const int xcd = blockIdx.x % kXcds, jb = blockIdx.x / kXcds;
-    const int e = xcd + kXcds * (jb / p.tiles_per_expert);
-    if (e >= p.E) return;
+    DwUnit unit;
+    if (!locate_dw_unit(p, xcd + kXcds * (jb / p.tiles_per_expert), unit)) return;
+    const int e = __builtin_amdgcn_readfirstlane(unit.e);
+    const int rbeg = __builtin_amdgcn_readfirstlane(unit.rbeg), rend = __builtin_amdgcn_readfirstlane(unit.rend);
+    const int slot = __builtin_amdgcn_readfirstlane(unit.slot);
     const int tile = jb % p.tiles_per_expert;
     const int m0 = (tile / p.n_tiles) * T::BM, n0 = (tile % p.n_tiles) * T::BN;
-    const int rbeg = p.expert_start[e], rend = p.expert_start[e + 1];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / MTS_WAVE), lane = threadIdx.x % MTS_WAVE;
     const int nk = (rend - rbeg + T::BKS - 1) / T::BKS;
 
@@ -1169,8 +1278,21 @@ __global__ __launch_bounds__(T::NT) void dw_gemm_ws_kernel(DwParams p) {
         __builtin_amdgcn_s_barrier();   // tile kt+2 is visible, tile kt may be overwritten
     }
 
-    OutT* C = reinterpret_cast<OutT*>(p.C) + (int64_t)e * p.M * p.N;
     const int fcol = lane % 32, frow4 = (lane / 32) * 4;
+    if (slot >= 0) {   // a row chunk: the whole fp32 tile goes to the unit's slot of the workspace
+        float* part = p.part + ((int64_t)slot * p.tiles_per_expert + tile) * (int64_t)(T::BM * T::BN);
+#pragma unroll
+        for (int mf = 0; mf < T::MF; ++mf)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int ml = wm * T::WM + mf * 32 + 8 * (i / 4) + frow4 + (i % 4);
+#pragma unroll
+                for (int nf = 0; nf < T::NF; ++nf)
+                    part[ml * T::BN + wn * T::WN + nf * 32 + fcol] = acc[mf][nf][i];
+            }
+        return;
+    }
+    OutT* C = reinterpret_cast<OutT*>(p.C) + (int64_t)e * p.M * p.N;
 #pragma unroll
     for (int mf = 0; mf < T::MF; ++mf)
 #pragma unroll
@@ -1260,21 +1382,43 @@ int launch_rows_any(int kind, RowsParams p, int64_t TK, hipStream_t s) {
 }
 
 template <class T>
-dim3 dw_grid(DwParams& p, int E) {
+dim3 dw_grid(DwParams& p, int E, int units) {
     p.E = E;
     p.n_tiles = (p.N + T::BN - 1) / T::BN;
     p.tiles_per_expert = ((p.M + T::BM - 1) / T::BM) * p.n_tiles;
-    return dim3((unsigned)(((E + kXcds - 1) / kXcds) * kXcds * p.tiles_per_expert));
+    return dim3((unsigned)(((units + kXcds - 1) / kXcds) * kXcds * p.tiles_per_expert));
 }
 
-int launch_dw_any(int kind, DwParams p, int E, int grad_dtype, hipStream_t s) {
+// fp32 tile partials of up to 2E row-chunk units (see DwUnit)
+int64_t dw_chunk_workspace_bytes(int E, int M, int N) {
+    typedef DwWsLarge T;
+    const int64_t tiles = (int64_t)((M + T::BM - 1) / T::BM) * ((N + T::BN - 1) / T::BN);
+    return 2 * (int64_t)E * tiles * T::BM * T::BN * (int64_t)sizeof(float);
+}
+
+int launch_dw_any(int kind, DwParams p, int E, int grad_dtype, void* workspace, int64_t workspace_bytes,
+                  hipStream_t s) {
     if (grad_dtype != MTS_BF16 && grad_dtype != MTS_F32) return MTS_ERR_DTYPE;
     if (tile_choice(kind) == 2) {
-        const dim3 grid = dw_grid<DwWsLarge>(p, E);
-        if (grad_dtype == MTS_BF16) dw_gemm_ws_kernel<DwWsLarge, bf16_t><<<grid, DwWsLarge::NT, 0, s>>>(p);
-        else dw_gemm_ws_kernel<DwWsLarge, float><<<grid, DwWsLarge::NT, 0, s>>>(p);
+        typedef DwWsLarge T;
+        if (workspace) {
+            if (workspace_bytes < dw_chunk_workspace_bytes(E, p.M, p.N)) return MTS_ERR_WORKSPACE;
+            if (!mts_aligned16(workspace)) return MTS_ERR_ALIGN;
+            p.part = (float*)workspace;
+        }
+        const dim3 grid = dw_grid<T>(p, E, p.part ? 2 * E : E);
+        if (grad_dtype == MTS_BF16) dw_gemm_ws_kernel<T, bf16_t><<<grid, T::NT, 0, s>>>(p);
+        else dw_gemm_ws_kernel<T, float><<<grid, T::NT, 0, s>>>(p);
+        if (p.part) {
+            MTS_CHECK_LAUNCH();
+            const int64_t items = (int64_t)p.tiles_per_expert * (T::BM * T::BN / 4);
+            const int64_t want = (items + 255) / 256;   // experts that were not cut leave at once
+            const dim3 sum_grid((unsigned)(want < 256 ? want : 256), (unsigned)E);
+            if (grad_dtype == MTS_BF16) dw_chunk_sum_kernel<T::BM, T::BN, bf16_t><<<sum_grid, 256, 0, s>>>(p);
+            else dw_chunk_sum_kernel<T::BM, T::BN, float><<<sum_grid, 256, 0, s>>>(p);
+        }
     } else {
-        const dim3 grid = dw_grid<StagedSmall>(p, E);
+        const dim3 grid = dw_grid<StagedSmall>(p, E, E);
         if (grad_dtype == MTS_BF16) dw_gemm_kernel<StagedSmall, bf16_t><<<grid, StagedSmall::NT, 0, s>>>(p);
         else dw_gemm_kernel<StagedSmall, float><<<grid, StagedSmall::NT, 0, s>>>(p);
     }
@@ -1384,9 +1528,15 @@ extern "C" int mts_moe_bwd_dx(const void* d_pre_act, const void* w1t, const int3
     return launch_rows_any<EPI_PLAIN>(K_DX, p, TK, (hipStream_t)stream);
 }
 
+extern "C" int64_t mts_moe_bwd_dw_workspace_bytes(int which, int E, int H, int I) {
+    if (E < 1 || H < 1 || I < 1 || (which != 1 && which != 2)) return 0;
+    return which == 1 ? dw_chunk_workspace_bytes(E, 2 * I, H) : dw_chunk_workspace_bytes(E, H, I);
+}
+
 extern "C" int mts_moe_bwd_dw2(const void* d_out, const void* weighted_act, const int32_t* x_gather,
                                const int32_t* expert_start, int64_t T, int K, int E, int H, int I,
-                               int act_dtype, int grad_dtype, void* d_w2, void* stream) {
+                               int act_dtype, int grad_dtype, void* d_w2, void* workspace,
+                               int64_t workspace_bytes, void* stream) {
     if (!d_out || !weighted_act || !x_gather || !expert_start || !d_w2) return MTS_ERR_NULL;
     if (T <= 0 || K < 1) return MTS_ERR_SHAPE;
     if (act_dtype == MTS_F32) {
@@ -1402,12 +1552,13 @@ extern "C" int mts_moe_bwd_dw2(const void* d_out, const void* weighted_act, cons
     p.P = (const bf16_t*)d_out; p.p_rows = T; p.p_gather = x_gather;
     p.Q = (const bf16_t*)weighted_act; p.q_rows = T * K; p.q_gather = nullptr;
     p.M = H; p.N = I; p.TK = T * K; p.expert_start = expert_start; p.C = d_w2;
-    return launch_dw_any(K_DW2, p, E, grad_dtype, (hipStream_t)stream);
+    return launch_dw_any(K_DW2, p, E, grad_dtype, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
 extern "C" int mts_moe_bwd_dw1(const void* d_pre_act, const void* x, const int32_t* x_gather,
                                const int32_t* expert_start, int64_t T, int K, int E, int H, int I,
-                               int act_dtype, int grad_dtype, void* d_w1, void* stream) {
+                               int act_dtype, int grad_dtype, void* d_w1, void* workspace,
+                               int64_t workspace_bytes, void* stream) {
     if (!d_pre_act || !x || !x_gather || !expert_start || !d_w1) return MTS_ERR_NULL;
     if (T <= 0 || K < 1) return MTS_ERR_SHAPE;
     if (act_dtype == MTS_F32) {
@@ -1423,5 +1574,5 @@ extern "C" int mts_moe_bwd_dw1(const void* d_pre_act, const void* x, const int32
     p.P = (const bf16_t*)d_pre_act; p.p_rows = T * K; p.p_gather = nullptr;
     p.Q = (const bf16_t*)x; p.q_rows = T; p.q_gather = x_gather;
     p.M = 2 * I; p.N = H; p.TK = T * K; p.expert_start = expert_start; p.C = d_w1;
-    return launch_dw_any(K_DW1, p, E, grad_dtype, (hipStream_t)stream);
+    return launch_dw_any(K_DW1, p, E, grad_dtype, workspace, workspace_bytes, (hipStream_t)stream);
 }

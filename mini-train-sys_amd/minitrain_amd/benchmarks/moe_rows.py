@@ -8,7 +8,14 @@ expert loop on the same GPU, and the correctness columns ``max_abs``, ``max_rel`
     python -m minitrain_amd.benchmarks.moe_rows --profile layer --tokens 24576
     python -m minitrain_amd.benchmarks.moe_rows --profile mixtral --tokens 4096
 
-prints one JSON row per provider (``hip``, ``torch``).  The ``torch`` provider is the expert loop
+    python -m minitrain_amd.benchmarks.moe_rows --tokens 24576 --zipf --capacity-factor 1.0
+
+prints one JSON row per provider (``hip``, ``torch``).  ``--zipf`` skews the routing towards the
+low expert ids (probability ~ rank^-1.2); with ``--capacity-factor`` every expert accepts at most
+``ceil(factor*T*K/E)`` routes (minitrain/model/moe_router.py:38-42), the ``hip`` row runs the compacted
+dispatch (dropped routes carry index -1), a ``hip_zero_weight`` row runs the same weights with every
+route still dispatched, which is what masking the weights alone amounts to, and the selection kernel
+is timed by itself (``capacity_mask_p50_ms``).  The ``torch`` provider is the expert loop
 of the reference's PyTorch backend (minitrain/kernels/torch_ops.py:122-150) restated here as the
 baseline of the table; it is not used by the operator.
 """
@@ -38,15 +45,32 @@ def torch_expert_loop(x, gate_up, down, idx, w):
     return out
 
 
-def make_case(tokens, H, I, E, K, dtype, seed):
+def make_case(tokens, H, I, E, K, dtype, seed, zipf=False):
     g = torch.Generator(device="cuda").manual_seed(seed)
     rn = lambda *s, std=1.0: (torch.randn(*s, generator=g, device="cuda") * std).to(dtype)
     x, gate_up, down = rn(tokens, H), rn(E, 2 * I, H, std=0.02), rn(E, H, I, std=0.02)
     logits = torch.randn(tokens, E, generator=g, device="cuda")
+    if zipf:
+        rank = torch.arange(1, E + 1, device="cuda", dtype=torch.float32)
+        logits = logits + torch.log(rank ** -1.2 / (rank ** -1.2).sum())
     p, idx = torch.topk(torch.softmax(logits, dim=-1), K, dim=-1)
-    w = (p / p.sum(dim=-1, keepdim=True)).to(dtype)
+    w32 = p / p.sum(dim=-1, keepdim=True)
     grad = rn(tokens, H)
-    return dict(x=x, gate_up=gate_up, down=down, idx=idx.int(), w=w, grad=grad)
+    idx = idx.int()
+    return dict(x=x, gate_up=gate_up, down=down, idx=idx, idx_all=idx, w=w32.to(dtype), w32=w32, grad=grad)
+
+
+def limit_capacity(case, ops, E, factor, min_capacity=4):
+    """Applies the capacity limit to a case: masked and renormalised weights, and the dispatch with
+    -1 on the dropped routes under ``idx`` (``idx_all`` keeps every route)."""
+    tokens, K = case["idx_all"].shape
+    capacity = max(min_capacity, math.ceil(factor * tokens * K / E))
+    keep, kept_index, accepted = ops.capacity_mask(case["idx_all"], case["w32"], E, capacity)
+    w = case["w32"] * keep
+    denom = w.sum(dim=-1, keepdim=True)
+    w = torch.where(denom > 0, w / denom.clamp_min(torch.finfo(w.dtype).eps), w)
+    case.update(idx=kept_index, w=w.to(case["x"].dtype))
+    return capacity, float(1.0 - keep.float().mean()), accepted.tolist()
 
 
 def _stats(actual, expected):
@@ -92,7 +116,8 @@ def _peak_mb(fn):
     return max(0.0, (torch.cuda.max_memory_allocated() - base) / 2**20)
 
 
-def measure(provider, op, case, iters, warmup):
+def measure(provider, op, case, iters, warmup, idx_key="idx"):
+    case = {**case, "idx": case[idx_key]}
     leaves = {n: case[n].detach().clone().requires_grad_(True) for n in ("x", "gate_up", "down", "w")}
 
     def fwd():
@@ -146,7 +171,12 @@ def correctness(op, case):
         return out.detach(), [leaves[n].grad for n in ("x", "gate_up", "down", "w")]
 
     out_a, g_a = run(op, case["x"].dtype)
+    case = {**case, "idx": case["idx_all"]}     # the expert loop dispatches every route; dropped ones weigh zero
     out_b, g_b = run(torch_expert_loop, torch.float32)
+    # the gradient of a dropped route's weight is defined while it is dispatched and zero once it is not
+    dropped = case["w"] == 0
+    g_a[3] = torch.where(dropped, torch.zeros_like(g_a[3]), g_a[3])
+    g_b[3] = torch.where(dropped, torch.zeros_like(g_b[3]), g_b[3])
     fwd = _stats(out_a, out_b)
     bwd = _stats(torch.cat([g.flatten().float() for g in g_a]), torch.cat([g.flatten() for g in g_b]))
     ok = lambda s: s["relative_l2"] <= 1e-2 and s["cosine_similarity"] >= 0.9999
@@ -165,19 +195,29 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--seed", type=int, default=1)
     ap.add_argument("--no-torch", action="store_true", help="skip the PyTorch expert-loop baseline rows")
+    ap.add_argument("--zipf", action="store_true", help="routing skewed towards the low expert ids")
+    ap.add_argument("--capacity-factor", type=float, default=None)
     args = ap.parse_args()
     from minitrain_amd.model.ops import get_ops_backend
 
     H, I, E, K = PROFILES[args.profile]
     ops = get_ops_backend("hip")
-    case = make_case(args.tokens, H, I, E, K, torch.bfloat16, args.seed)
+    case = make_case(args.tokens, H, I, E, K, torch.bfloat16, args.seed, zipf=args.zipf)
     common = dict(op="fused_moe", profile=args.profile, size=args.tokens, hidden=H, expert_width=I, experts=E,
-                  top_k=K, dtype="bf16", device=torch.cuda.get_device_name(0), timer="cuda_events")
+                  top_k=K, dtype="bf16", device=torch.cuda.get_device_name(0), timer="cuda_events",
+                  routing="zipf" if args.zipf else "uniform")
+    extra_rows = []
+    if args.capacity_factor is not None:
+        capacity, dropped, accepted = limit_capacity(case, ops, E, args.capacity_factor)
+        p50, p95 = _time(lambda: ops.capacity_mask(case["idx_all"], case["w32"], E, capacity), args.iters, args.warmup)
+        common.update(capacity_factor=args.capacity_factor, capacity=capacity, dropped_route_fraction=dropped,
+                      accepted_per_expert=accepted, capacity_mask_p50_ms=p50, capacity_mask_p95_ms=p95)
+        extra_rows.append(measure("hip_zero_weight", ops.fused_moe, case, args.iters, args.warmup, idx_key="idx_all"))
     hip = measure("hip", ops.fused_moe, case, args.iters, args.warmup)
     hip.update(correctness(ops.fused_moe, case))
-    rows = [hip]
+    rows = [hip] + extra_rows
     if not args.no_torch:
-        ref = measure("torch", torch_expert_loop, case, max(3, args.iters // 4), 2)
+        ref = measure("torch", torch_expert_loop, case, max(3, args.iters // 4), 2, idx_key="idx_all")
         for m in ("fwd", "bwd", "full"):
             hip[f"{m}_speedup"] = ref[f"{m}_p50_ms"] / hip[f"{m}_p50_ms"]
             ref[f"{m}_speedup"] = 1.0

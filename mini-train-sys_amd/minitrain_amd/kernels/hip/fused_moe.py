@@ -143,6 +143,19 @@ def _side_stream(device: torch.device, index: int) -> torch.cuda.Stream:
     return s
 
 
+# The weight-gradient GEMMs cut the rows of an over-full expert into chunks when they are given a
+# workspace for the chunk partials (skewed routing); beyond this size they run without one.
+_DW_WORKSPACE_LIMIT = 512 * 2**20
+
+
+def _dw_workspace(lib, which: int, E: int, H: int, I: int, dtype: torch.dtype, device):
+    nbytes = lib.mts_moe_bwd_dw_workspace_bytes(which, E, H, I) if dtype == torch.bfloat16 else 0
+    if nbytes <= 0 or nbytes > _DW_WORKSPACE_LIMIT:
+        return None, 0, 0
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    return ws, ws.data_ptr(), nbytes
+
+
 def _stage(lib, w: torch.Tensor, transpose: bool, dtype: torch.dtype, stream: int | None = None) -> torch.Tensor:
     """Copy of an expert weight ``[E,R,C]`` in the activation dtype, optionally as ``[E,C,R]``."""
     if not transpose and w.dtype == dtype:
@@ -275,11 +288,13 @@ class _FusedMoEFunction(torch.autograd.Function):
         ddown_proj = None
         if need_w2:
             ddown_proj = torch.empty_like(down_proj)
+            ws2, ws2_ptr, ws2_bytes = _dw_workspace(lib, 2, E, H, I, x.dtype, dev)
             fork(side[0])
             _lib.check(
                 lib.mts_moe_bwd_dw2(
                     dO.data_ptr(), weighted_act.data_ptr(), x_gather.data_ptr(), expert_start.data_ptr(), T, K, E, H,
-                    I, act, _lib.dtype_code(down_proj.dtype), ddown_proj.data_ptr(), side[0].cuda_stream,
+                    I, act, _lib.dtype_code(down_proj.dtype), ddown_proj.data_ptr(), ws2_ptr, ws2_bytes,
+                    side[0].cuda_stream,
                 ),
                 "mts_moe_bwd_dw2",
             )
@@ -287,11 +302,13 @@ class _FusedMoEFunction(torch.autograd.Function):
         dgate_up_proj = None
         if need_w1:
             dgate_up_proj = torch.empty_like(gate_up_proj)
+            ws1, ws1_ptr, ws1_bytes = _dw_workspace(lib, 1, E, H, I, x.dtype, dev)
             fork(side[1])
             _lib.check(
                 lib.mts_moe_bwd_dw1(
                     d_pre_act.data_ptr(), x.data_ptr(), x_gather.data_ptr(), expert_start.data_ptr(), T, K, E, H, I,
-                    act, _lib.dtype_code(gate_up_proj.dtype), dgate_up_proj.data_ptr(), side[1].cuda_stream,
+                    act, _lib.dtype_code(gate_up_proj.dtype), dgate_up_proj.data_ptr(), ws1_ptr, ws1_bytes,
+                    side[1].cuda_stream,
                 ),
                 "mts_moe_bwd_dw1",
             )

@@ -96,6 +96,35 @@ def test_run_to_run_determinism():
         assert torch.equal(u, v)
 
 
+@pytest.mark.parametrize("T,H,E,I,skew", [(3000, 256, 8, 256, 0.7), (1500, 128, 4, 192, 0.55), (2000, 72, 16, 40, 0.4),
+                                          (700, 256, 64, 256, 0.5)])
+def test_weight_gradients_with_row_chunks(T, H, E, I, skew, monkeypatch):
+    """Skewed routing: the weight-gradient GEMMs cut the rows of the over-full experts into chunks
+    (workspace given) and must agree with the oracle and with the uncut reduction (no workspace)."""
+    print(f"moe row chunks T={T} H={H} E={E} I={I} skew={skew}", flush=True)
+    import importlib
+
+    F = importlib.import_module("minitrain_amd.kernels.hip.fused_moe")
+    K = 2
+    case = routed_case(50 + T, T, H, E, I, K)
+    rng = np.random.Generator(np.random.Philox(T))
+    idx = case["idx"].clone()
+    heavy = torch.from_numpy(rng.random(T) < skew)
+    idx[heavy, 0] = 1                                   # expert 1 takes most first choices
+    idx[heavy & (idx[:, 1] == 1), 1] = 0
+    case.update(idx=idx)
+    counts = np.bincount(idx.flatten().numpy(), minlength=E)
+    share = (-(-T * K // E) + 31) // 32 * 32
+    assert counts.max() > 1.25 * share
+    _compare(case)
+    cut = hip_moe_grads(case["x"], case["w1"], case["w2"], idx, case["w"], case["g"])
+    monkeypatch.setattr(F, "_DW_WORKSPACE_LIMIT", 0)
+    uncut = hip_moe_grads(case["x"], case["w1"], case["w2"], idx, case["w"], case["g"])
+    for name, a, b in zip(NAMES, cut[1], uncut[1]):
+        assert_close_scaled(a, b, 4e-3, name + " cut vs uncut")   # one bf16 rounding of fp32 sums in either order
+    assert torch.equal(cut[1][0], uncut[1][0]) and torch.equal(cut[1][3], uncut[1][3])   # dx and dS do not change
+
+
 def test_layer_shape_subset_of_tokens():
     """293M-class layer dims at 2048 tokens: the whole oracle still runs on the CPU in seconds."""
     print("moe 2048x768x1024", flush=True)
