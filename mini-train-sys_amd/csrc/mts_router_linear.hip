@@ -149,7 +149,11 @@ __global__ __launch_bounds__(kFwdThreads) void router_logits_fwd_kernel(const XT
 // dtype) from the row's E logit gradients and its weight columns, and adds the row's
 // contribution to its E x 4 block of dW_r; every block writes its partial dW_r to the
 // workspace, and the reduction kernel sums the partials in block order.
-template <typename XT, int EP>
+// The row loop works on groups of UN rows without a bounds test (the raw loads of the next
+// group are issued before the arithmetic of the current one); the rows left over are done one
+// by one.  EXACT: E == EP, so a row's logit gradients are EP consecutive floats at an address
+// every thread of the block shares, which the compiler turns into scalar loads.
+template <typename XT, int EP, bool EXACT>
 __global__ __launch_bounds__(256) void router_logits_bwd_kernel(const float* __restrict__ dl,
                                                                  const XT* __restrict__ x,
                                                                  const float* __restrict__ w, int64_t T, int H,
@@ -157,6 +161,7 @@ __global__ __launch_bounds__(256) void router_logits_bwd_kernel(const float* __r
                                                                  float* __restrict__ part) {
     const int c = threadIdx.x * 4;
     if (c >= H) return;
+    typedef typename RawVec<XT>::type raw_t;
     f32x4 wv[EP], acc[EP];
 #pragma unroll
     for (int e = 0; e < EP; ++e) {
@@ -166,30 +171,54 @@ __global__ __launch_bounds__(256) void router_logits_bwd_kernel(const float* __r
     }
     const int64_t row_beg = (int64_t)blockIdx.x * rows_per_block;
     const int64_t row_end = row_beg + rows_per_block < T ? row_beg + rows_per_block : T;
-    constexpr int UN = 4;   // rows in flight per thread
-#pragma unroll 1
-    for (int64_t row = row_beg; row < row_end; row += UN) {
-        f32x4 xv[UN];
+    auto one_row = [&](int64_t row, raw_t raw) {
+        const f32x4 xv = widen(raw);
+        float g[EP];
+        if constexpr (EXACT) {
 #pragma unroll
-        for (int u = 0; u < UN; ++u) {
-            const f32x4 z = {0.f, 0.f, 0.f, 0.f};
-            xv[u] = row + u < row_end ? load4(x + (row + u) * H + c) : z;
-        }
-#pragma unroll
-        for (int u = 0; u < UN; ++u) {
-            if (row + u < row_end) {
-                f32x4 d = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int e = 0; e < EP; ++e) {
-                    // the same address for every thread of the block; experts past E have zero weights
-                    const float g = dl[(row + u) * E + (e < E ? e : 0)];
-                    d += g * wv[e];
-                    acc[e] += (e < E ? g : 0.f) * xv[u];
-                }
-                store4(dx + (row + u) * H + c, d);
+            for (int q = 0; q < EP / 4; ++q) {
+                const f32x4 v = *reinterpret_cast<const f32x4*>(dl + row * EP + q * 4);
+                g[q * 4] = v[0], g[q * 4 + 1] = v[1], g[q * 4 + 2] = v[2], g[q * 4 + 3] = v[3];
             }
+        } else {
+#pragma unroll
+            for (int e = 0; e < EP; ++e) g[e] = e < E ? dl[row * E + e] : 0.f;   // experts past E have zero weights
         }
+        f32x4 d = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int e = 0; e < EP; ++e) {
+            d += g[e] * wv[e];
+            acc[e] += g[e] * xv;
+        }
+        store4(dx + row * H + c, d);
+    };
+    constexpr int UN = 4;   // rows per group; two groups are in flight, in two register sets that swap roles
+    int64_t row = row_beg;
+    raw_t ga[UN], gb[UN];
+    auto load_group = [&](raw_t (&dst)[UN], int64_t r0) {
+#pragma unroll
+        for (int u = 0; u < UN; ++u) dst[u] = load_raw(x + (r0 + u) * H + c);
+    };
+    auto do_group = [&](raw_t (&src)[UN], int64_t r0) {
+#pragma unroll
+        for (int u = 0; u < UN; ++u) one_row(r0 + u, src[u]);
+    };
+    bool have_a = row + UN <= row_end;   // every condition here is block-uniform
+    if (have_a) load_group(ga, row);
+#pragma unroll 1
+    while (have_a) {
+        const bool have_b = row + 2 * UN <= row_end;
+        if (have_b) load_group(gb, row + UN);
+        do_group(ga, row);
+        row += UN;
+        if (!have_b) break;
+        have_a = row + 2 * UN <= row_end;
+        if (have_a) load_group(ga, row + UN);
+        do_group(gb, row);
+        row += UN;
     }
+#pragma unroll 1
+    for (; row < row_end; ++row) one_row(row, load_raw(x + row * H + c));
     float* out = part + (int64_t)blockIdx.x * E * H;
 #pragma unroll
     for (int e = 0; e < EP; ++e)
@@ -287,8 +316,16 @@ extern "C" int mts_router_logits_bwd(const float* dlogits, const void* x, const 
     const int rows_per_block = (int)((T + nb - 1) / nb);
     const int threads = ((H / 4 + MTS_WAVE - 1) / MTS_WAVE) * MTS_WAVE;   // one thread per 4 columns
     float* part = (float*)workspace;
-#define MTS_BWD(XT, EP) \
-    router_logits_bwd_kernel<XT, EP><<<nb, threads, 0, s>>>(dlogits, (const XT*)x, w_r, T, H, E, rows_per_block, (XT*)dx, part)
+    const bool vec_dl = mts_aligned16(dlogits);
+#define MTS_BWD(XT, EP)                                                                                    \
+    do {                                                                                                   \
+        if (E == EP && vec_dl)                                                                             \
+            router_logits_bwd_kernel<XT, EP, true><<<nb, threads, 0, s>>>(dlogits, (const XT*)x, w_r, T, H, E, \
+                                                                          rows_per_block, (XT*)dx, part);  \
+        else                                                                                               \
+            router_logits_bwd_kernel<XT, EP, false><<<nb, threads, 0, s>>>(dlogits, (const XT*)x, w_r, T, H, E, \
+                                                                           rows_per_block, (XT*)dx, part); \
+    } while (0)
     if (act_dtype == MTS_BF16) {
         if (E <= 8) MTS_BWD(bf16_t, 8);
         else MTS_BWD(bf16_t, 16);
