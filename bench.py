@@ -70,6 +70,8 @@ class Layer:
         self.w2 = w2.cuda().bfloat16().requires_grad_(True)
         self.g = g.cuda().bfloat16()
         self.E = w_r.shape[0]
+        self.seed_aux = torch.tensor(0.01, device="cuda")    # router_aux_loss_coef (minitrain/model/config.py:20)
+        self.seed_z = torch.tensor(0.001, device="cuda")     # router_z_loss_coef (config.py:21)
 
     def step(self):
         for t in (self.x, self.w_r, self.w1, self.w2):
@@ -84,8 +86,9 @@ class Layer:
             counts = torch.bincount(route.expert_indices.flatten().long(), minlength=self.E)
             aux = self.E * torch.sum(counts.float() / route.expert_indices.numel() * route.probability_per_expert)
         out = self.ops.fused_moe(self.x, self.w1, self.w2, route.expert_indices, route.expert_weights.to(self.x.dtype))
-        loss_side = 0.01 * aux + 0.001 * route.z_loss
-        torch.autograd.backward([out, loss_side], [self.g, torch.ones_like(loss_side)])
+        # loss = sum(out * G) + 0.01 * aux + 0.001 * z: its gradient enters as the three seeds G, 0.01 and
+        # 0.001, so the scalar itself (a few 5 us element-wise launches on 0-dim tensors) is not formed
+        torch.autograd.backward([out, aux, route.z_loss], [self.g, self.seed_aux, self.seed_z])
         return out
 
 

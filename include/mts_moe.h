@@ -64,8 +64,9 @@ int mts_router_fwd(const float* logits, int64_t T, int E, int K, int normalize,
                    int64_t workspace_bytes, void* stream);
 
 /* Replaces _router_backward_kernel (minitrain/kernels/triton/router.py:155-259).
- * g_weights [T,K], g_prob_mean [E], g_z_loss [1] -> dlogits [T,E].
- * g_load_balance [1] (may be NULL) is the gradient of the load-balancing term; it
+ * g_weights [T,K], g_prob_mean [E], g_z_loss [1] -> dlogits [T,E]; each of the
+ * gradient inputs may be NULL, which stands for zeros (an output that took no part in
+ * the loss).  g_load_balance [1] is the gradient of the load-balancing term; it
  * reaches the logits through prob_mean only (the route fractions counts/(T*K)
  * carry no gradient) and needs the counts the forward call wrote.              */
 int mts_router_bwd(const float* logits, const float* weights, const int32_t* indices,

@@ -836,7 +836,7 @@ struct DwUnit {
 };
 
 __device__ __forceinline__ int dw_share(const DwParams& p) {
-    const int total = p.expert_start[p.E];
+    const int total = p.expert_start[p.E] - p.expert_start[0];   // the caller may pass a sub-range of the experts
     return ((total + p.E - 1) / p.E + 31) / 32 * 32;
 }
 

@@ -258,12 +258,12 @@ __global__ __launch_bounds__(kThreads) void router_bwd_kernel(
     const int g = threadIdx.x % G;
     const int rl = threadIdx.x / G;
     const float inv_t = 1.0f / (float)T;
-    const float gz = g_z[0] * 2.0f * inv_t;
+    const float gz = g_z ? g_z[0] * 2.0f * inv_t : 0.f;   // every gradient input may be absent (null = zeros)
     float gp[EP];
 #pragma unroll
     for (int j = 0; j < EP; ++j) {
         int e = j * G + g;
-        gp[j] = (e < E) ? g_p[e] * inv_t : 0.f;
+        gp[j] = (g_p && e < E) ? g_p[e] * inv_t : 0.f;
         // load-balancing term: d/d(mean_prob_e) = E * routes_e / routes (the route fractions carry no gradient)
         if (g_lb && e < E) gp[j] += g_lb[0] * (float)E * ((float)counts[e] / ((float)T * (float)K)) * inv_t;
     }
@@ -281,11 +281,11 @@ __global__ __launch_bounds__(kThreads) void router_bwd_kernel(
         }
         float wdot = 0.f;
         if (normalize) {
-            for (int k = 0; k < K; ++k) wdot += weights[rr * K + k] * g_w[rr * K + k];
+            for (int k = 0; k < K; ++k) wdot += weights[rr * K + k] * (g_w ? g_w[rr * K + k] : 0.f);
         }
         for (int k = 0; k < K; ++k) {
             int e = indices[rr * K + k];
-            float gw = g_w[rr * K + k];
+            float gw = g_w ? g_w[rr * K + k] : 0.f;
             float w = weights[rr * K + k];
 #pragma unroll
             for (int j = 0; j < EP; ++j) {
@@ -392,8 +392,7 @@ extern "C" int mts_router_bwd(const float* logits, const float* weights, const i
                               int64_t T, int E, int K, int normalize, float* dlogits, void* stream) {
     int rc = check_router(logits, T, E, K);
     if (rc) return rc;
-    if (!weights || !indices || !g_weights || !g_prob_mean || !g_z_loss || !dlogits)
-        return MTS_ERR_NULL;
+    if (!weights || !indices || !dlogits) return MTS_ERR_NULL;
     if (g_load_balance && !counts) return MTS_ERR_NULL;
     if (E == 8 && !mts_aligned16(dlogits)) return MTS_ERR_ALIGN;
     hipStream_t s = (hipStream_t)stream;

@@ -251,11 +251,13 @@ class _FusedMoEFunction(torch.autograd.Function):
         overlap = _OVERLAP
         side = [_side_stream(dev, 0), _side_stream(dev, 1)] if overlap else [main, main]
 
-        def fork(to):
+        def fork(*to):
+            # one marker on the caller's stream, however many side streams wait for it
             if overlap:
                 ev = torch.cuda.Event()
                 ev.record(main)
-                to.wait_event(ev)
+                for s in to:
+                    s.wait_event(ev)
 
         def join(frm):
             if overlap:
@@ -286,10 +288,16 @@ class _FusedMoEFunction(torch.autograd.Function):
         )
 
         ddown_proj = None
+        ws1, ws1_ptr, ws1_bytes = _dw_workspace(lib, 1, E, H, I, x.dtype, dev) if need_w1 else (None, 0, 0)
+        ws2, ws2_ptr, ws2_bytes = _dw_workspace(lib, 2, E, H, I, x.dtype, dev) if need_w2 else (None, 0, 0)
+        if need_w1 and need_w2:
+            fork(side[0], side[1])
+        elif need_w2:
+            fork(side[0])
+        elif need_w1:
+            fork(side[1])
         if need_w2:
             ddown_proj = torch.empty_like(down_proj)
-            ws2, ws2_ptr, ws2_bytes = _dw_workspace(lib, 2, E, H, I, x.dtype, dev)
-            fork(side[0])
             _lib.check(
                 lib.mts_moe_bwd_dw2(
                     dO.data_ptr(), weighted_act.data_ptr(), x_gather.data_ptr(), expert_start.data_ptr(), T, K, E, H,
@@ -302,8 +310,6 @@ class _FusedMoEFunction(torch.autograd.Function):
         dgate_up_proj = None
         if need_w1:
             dgate_up_proj = torch.empty_like(gate_up_proj)
-            ws1, ws1_ptr, ws1_bytes = _dw_workspace(lib, 1, E, H, I, x.dtype, dev)
-            fork(side[1])
             _lib.check(
                 lib.mts_moe_bwd_dw1(
                     d_pre_act.data_ptr(), x.data_ptr(), x_gather.data_ptr(), expert_start.data_ptr(), T, K, E, H, I,

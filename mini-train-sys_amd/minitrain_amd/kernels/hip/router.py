@@ -55,6 +55,7 @@ class _RouterPostprocessFunction(torch.autograd.Function):
         ctx.top_k = top_k
         ctx.normalize = normalize
         ctx.mark_non_differentiable(indices, entropy, counts)
+        ctx.set_materialize_grads(False)   # no zero tensors for the outputs that took no part in the loss
         return weights, indices, prob_mean, z_loss, entropy, counts, load_balance
 
     @staticmethod
@@ -66,20 +67,18 @@ class _RouterPostprocessFunction(torch.autograd.Function):
         T, E = logits.shape
         dev = logits.device
 
-        def dense(g, shape):
-            if g is None:
-                return torch.zeros(shape, device=dev, dtype=torch.float32)
-            return g.to(torch.float32).contiguous()
+        def dense(g):   # an output that took no part in the loss comes as None and goes down as a null pointer
+            return None if g is None else g.to(torch.float32).contiguous()
 
-        g_w = dense(grad_weights, (T, ctx.top_k))
-        g_p = dense(grad_probability_mean, (E,))
-        g_z = dense(grad_z_loss, ())
-        g_lb = None if grad_load_balance is None else grad_load_balance.to(torch.float32).contiguous()
+        g_w = dense(grad_weights)
+        g_p = dense(grad_probability_mean)
+        g_z = dense(grad_z_loss)
+        g_lb = dense(grad_load_balance)
         grad_logits = torch.empty_like(logits)
         _lib.check(
             lib.mts_router_bwd(
-                logits.data_ptr(), weights.data_ptr(), indices.data_ptr(), g_w.data_ptr(), g_p.data_ptr(),
-                g_z.data_ptr(), _lib.ptr(g_lb), counts.data_ptr(), T, E, ctx.top_k, int(ctx.normalize),
+                logits.data_ptr(), weights.data_ptr(), indices.data_ptr(), _lib.ptr(g_w), _lib.ptr(g_p),
+                _lib.ptr(g_z), _lib.ptr(g_lb), counts.data_ptr(), T, E, ctx.top_k, int(ctx.normalize),
                 grad_logits.data_ptr(), _lib.stream_of(logits),
             ),
             "mts_router_bwd",
