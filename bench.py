@@ -124,7 +124,6 @@ def stage_breakdown(layer, steps):
     npart = lib.mts_moe_ds_partials(I)
     dsp = torch.empty(TK, npart, dtype=torch.float32, device=dev)
     dwts = torch.empty(T, K, **bf)
-    w2t, w1t = torch.empty(E, I, H, **bf), torch.empty(E, H, 2 * I, **bf)
     dw1, dw2 = torch.empty_like(w1), torch.empty_like(w2)
     # chunk partials of the weight-gradient GEMMs, as the operator passes them
     dws1 = torch.empty(lib.mts_moe_bwd_dw_workspace_bytes(1, E, H, I), dtype=torch.uint8, device=dev)
@@ -157,13 +156,11 @@ def stage_breakdown(layer, steps):
         ("fwd_down", "mfma", gemm(1), lambda: lib.mts_moe_fwd_down(p(post), p(w2), p(es), TK, E, H, I, B, p(y), st)),
         ("combine", "hbm", TK * H * esz + T * H * esz + TK * 4 + TK * esz,
          lambda: lib.mts_moe_combine(p(y), p(wts), p(sr), T, K, H, B, p(out), st)),
-        ("stage_w2_transposed", "hbm", 2 * E * H * I * esz, lambda: lib.mts_moe_stage_weights(p(w2), B, p(w2t), B, E, H, I, 1, st)),
         ("bwd_dy1", "mfma", gemm(1),
-         lambda: lib.mts_moe_bwd_dy1(p(g), p(w2t), p(pre), p(wts), p(xg), p(ss), p(es), T, K, E, H, I, B, p(dpre), p(wact), p(dsp), st)),
+         lambda: lib.mts_moe_bwd_dy1(p(g), p(w2), 1, p(pre), p(wts), p(xg), p(ss), p(es), T, K, E, H, I, B, p(dpre), p(wact), p(dsp), st)),
         ("bwd_ds", "hbm", TK * npart * 4 + TK * 4 + TK * esz, lambda: lib.mts_moe_bwd_ds(p(dsp), p(sr), TK, I, B, p(dwts), st)),
         ("bwd_dw2", "mfma", gemm(1), lambda: lib.mts_moe_bwd_dw2(p(g), p(wact), p(xg), p(es), T, K, E, H, I, B, B, p(dw2), p(dws2), dws2.numel(), st)),
-        ("stage_w1_transposed", "hbm", 2 * E * 2 * I * H * esz, lambda: lib.mts_moe_stage_weights(p(w1), B, p(w1t), B, E, 2 * I, H, 1, st)),
-        ("bwd_dx", "mfma", gemm(2), lambda: lib.mts_moe_bwd_dx(p(dpre), p(w1t), p(es), TK, E, H, I, B, p(dxe), st)),
+        ("bwd_dx", "mfma", gemm(2), lambda: lib.mts_moe_bwd_dx(p(dpre), p(w1), 1, p(es), TK, E, H, I, B, p(dxe), st)),
         ("dx_combine", "hbm", TK * H * esz + T * H * esz + TK * 4,
          lambda: lib.mts_moe_combine(p(dxe), None, p(sr), T, K, H, B, p(dx), st)),
         ("bwd_dw1", "mfma", gemm(2), lambda: lib.mts_moe_bwd_dw1(p(dpre), p(x), p(xg), p(es), T, K, E, H, I, B, B, p(dw1), p(dws1), dws1.numel(), st)),

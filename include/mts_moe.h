@@ -163,10 +163,16 @@ int mts_moe_combine(const void* y, const void* weights, const int32_t* s_reverse
 /* ---- backward -----------------------------------------------------------
  * Replaces _moe_bwd_down_proj_kernel (fused_moe_kernels.py:500-600):
  * A = W2[e]^T dO[t];  dS = <A,a>;  weighted_act = s*a;  [dg;du] = d(s*A)/d[g;u].
- * w2t is W2 staged as [E,I,H].  ds_partial is [TK, mts_moe_ds_partials(I)]
- * f32 scratch reduced by mts_moe_bwd_ds (fixed order, no atomics).            */
+ * The weight operand comes in one of two layouts: w2_as_stored = 1, w2 is W2 itself
+ * [E,H,I] in the activation dtype, or w2_as_stored = 0, it is the transposed copy [E,I,H]
+ * made by mts_moe_stage_weights.  mts_moe_bwd_weights_as_stored(act_dtype, H, I) says
+ * whether this entry point and mts_moe_bwd_dx take the stored layout (bf16, H and 2I
+ * multiples of 64); otherwise they return MTS_ERR_SHAPE for it.  ds_partial is
+ * [TK, mts_moe_ds_partials(I)] f32 scratch reduced by mts_moe_bwd_ds (fixed order, no
+ * atomics).                                                                    */
 int mts_moe_ds_partials(int I);
-int mts_moe_bwd_dy1(const void* d_out, const void* w2t, const void* pre_act,
+int mts_moe_bwd_weights_as_stored(int act_dtype, int H, int I);
+int mts_moe_bwd_dy1(const void* d_out, const void* w2, int w2_as_stored, const void* pre_act,
                     const void* weights, const int32_t* x_gather, const int32_t* s_scatter,
                     const int32_t* expert_start, int64_t T, int K, int E, int H, int I,
                     int act_dtype, void* d_pre_act, void* weighted_act, float* ds_partial,
@@ -178,11 +184,12 @@ int mts_moe_bwd_ds(const float* ds_partial, const int32_t* s_reverse, int64_t TK
                    int act_dtype, void* d_weights, void* stream);
 
 /* Replaces _moe_bwd_dX_expanded_kernel (fused_moe_kernels.py:674-756):
- * dx_expanded[r] = W1[e]^T [dg;du][r];  w1t is W1 staged as [E,H,2I].
+ * dx_expanded[r] = W1[e]^T [dg;du][r];  w1 is W1 itself [E,2I,H] (w1_as_stored = 1) or
+ * its transposed copy [E,H,2I] (w1_as_stored = 0), see mts_moe_bwd_dy1.
  * The per-token sum is mts_moe_combine with weights == NULL.                 */
-int mts_moe_bwd_dx(const void* d_pre_act, const void* w1t, const int32_t* expert_start,
-                   int64_t TK, int E, int H, int I, int act_dtype, void* dx_expanded,
-                   void* stream);
+int mts_moe_bwd_dx(const void* d_pre_act, const void* w1, int w1_as_stored,
+                   const int32_t* expert_start, int64_t TK, int E, int H, int I, int act_dtype,
+                   void* dx_expanded, void* stream);
 
 /* Replaces _moe_bwd_dW2_kernel (fused_moe_kernels.py:602-672):
  * dW2[e] = sum_{r in e} dO[x_gather[r]] (x) weighted_act[r]   -> [E,H,I] grad_dtype.

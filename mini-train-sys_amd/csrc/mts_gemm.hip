@@ -133,6 +133,29 @@ struct KMajorLoader {
 
 // one MFMA sweep over a staged k-tile
 // (ROWLEN = k extent of the LDS rows: 64 with swizzle (row>>1)&7, 32 with (row>>2)&3)
+// 32 x 16 MFMA fragments out of LDS tiles that hold one k per row ("k-major": the operand's
+// memory rows are k) are read with the transposing LDS load; the layout is described at the
+// weight-gradient GEMMs below.
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+
+// 32 (m) x 16 (k) MFMA fragment out of a k-major LDS tile with row length ROWLEN
+template <int ROWLEN>
+__device__ __forceinline__ bf16x8 read_frag_tr(const bf16_t* tile, int krow0, int col0) {
+    const int lane = threadIdx.x % MTS_WAVE;
+    const int col = col0 + 16 * ((lane / 16) % 2) + 4 * (lane % 4);
+    const int chunk = col / 8, within = col % 8;
+    s16x4 h[2];
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+        const int row = krow0 + 8 * (lane / 32) + 4 * q + (lane % 16) / 4;
+        const bf16_t* src = tile + row * ROWLEN + ((chunk ^ ((row & 3) << 2)) << 3) + within;
+        h[q] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(src));
+    }
+    typedef __attribute__((ext_vector_type(8))) short s16x8;
+    s16x8 v = {h[0][0], h[0][1], h[0][2], h[0][3], h[1][0], h[1][1], h[1][2], h[1][3]};
+    return __builtin_bit_cast(bf16x8, v);
+}
+
 struct NoHook {
     __device__ __forceinline__ void operator()(int) const {}
 };
@@ -140,7 +163,8 @@ struct NoHook {
 // `hook(ks)` runs once per 16-wide k-step, between the fragment reads and the MFMAs.
 // Fragments are double buffered: the LDS reads of k-step ks+1 are issued before the
 // MFMAs of k-step ks, so that their latency is covered by the matrix pipe.
-template <class T, bool SWIGLU, int ROWLEN = BK, bool WEIGHT_FIRST = true, class Hook = NoHook>
+// BKM: the B tile is k-major, [ROWLEN k][T::BN] (weights in their stored layout).
+template <class T, bool SWIGLU, int ROWLEN = BK, bool WEIGHT_FIRST = true, bool BKM = false, class Hook = NoHook>
 __device__ __forceinline__ void mma_tile(const bf16_t* As, const bf16_t* Bs, int wm, int wn,
                                          f32x16 (&acc)[T::MF][T::NF], Hook hook = Hook()) {
     const int lane = threadIdx.x % MTS_WAVE;
@@ -165,7 +189,8 @@ __device__ __forceinline__ void mma_tile(const bf16_t* As, const bf16_t* Bs, int
             } else {
                 brow = wn * T::WN + nf * 32;
             }
-            b[buf][nf] = *reinterpret_cast<const bf16x8*>(b_base + brow * ROWLEN + coff);
+            if constexpr (BKM) b[buf][nf] = read_frag_tr<T::BN>(Bs, ks * 16, brow);
+            else b[buf][nf] = *reinterpret_cast<const bf16x8*>(b_base + brow * ROWLEN + coff);
         }
     };
 
@@ -190,7 +215,7 @@ __device__ __forceinline__ void mma_tile(const bf16_t* As, const bf16_t* Bs, int
 // current step are issued, so the matrix pipe does not idle at the start of a k-tile.
 // Weight fragments are double buffered; an activation fragment is reloaded for the next
 // k-step right behind the MFMAs that used it.
-template <class T, bool SWIGLU, int ROWLEN>
+template <class T, bool SWIGLU, int ROWLEN, bool BKM = false>
 struct FragPipe {
     static constexpr int KSTEPS = ROWLEN / 16;
     static_assert(KSTEPS % 2 == 0, "weight fragment buffers alternate with the k-step");
@@ -212,8 +237,13 @@ struct FragPipe {
             } else {
                 brow = wn * T::WN + nf * 32;
             }
-            b_off[nf] = T::BM * ROWLEN + (brow + frow) * ROWLEN;
+            // k-major B: b_off is the fragment's first column; the tile starts behind the A tile
+            b_off[nf] = BKM ? brow : T::BM * ROWLEN + (brow + frow) * ROWLEN;
         }
+    }
+    __device__ __forceinline__ bf16x8 read_b(const bf16_t* tile, int nf, int ks, int coff) const {
+        if constexpr (BKM) return read_frag_tr<T::BN>(tile + T::BM * ROWLEN, ks * 16, b_off[nf]);
+        else return *reinterpret_cast<const bf16x8*>(tile + b_off[nf] + coff);
     }
     __device__ __forceinline__ int chunk_off(int ks) const { return ((ks * 2 + kb) ^ swz) << 3; }
     // all fragments of k-step 0 of the stage at `tile`
@@ -223,7 +253,7 @@ struct FragPipe {
         for (int mf = 0; mf < T::MF; ++mf)
             a[mf] = *reinterpret_cast<const bf16x8*>(tile + a_off + mf * 32 * ROWLEN + coff);
 #pragma unroll
-        for (int nf = 0; nf < T::NF; ++nf) b[0][nf] = *reinterpret_cast<const bf16x8*>(tile + b_off[nf] + coff);
+        for (int nf = 0; nf < T::NF; ++nf) b[0][nf] = read_b(tile, nf, 0, coff);
     }
     // MFMAs of k-step `ks` (weight fragment first); behind them, the fragments of k-step `nks`
     // of the stage at `next` are read: the weight fragments up front into the other buffer, each
@@ -231,7 +261,7 @@ struct FragPipe {
     __device__ __forceinline__ void step(int ks, f32x16 (&acc)[T::MF][T::NF], const bf16_t* next, int nks) {
         const int coff = chunk_off(nks), buf = ks & 1;
 #pragma unroll
-        for (int nf = 0; nf < T::NF; ++nf) b[buf ^ 1][nf] = *reinterpret_cast<const bf16x8*>(next + b_off[nf] + coff);
+        for (int nf = 0; nf < T::NF; ++nf) b[buf ^ 1][nf] = read_b(next, nf, nks, coff);
 #pragma unroll
         for (int mf = 0; mf < T::MF; ++mf) {
 #pragma unroll
@@ -581,7 +611,10 @@ __device__ __forceinline__ void wait_vmcnt() {
     __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | 0x0F70);
 }
 
-template <class T, int EPI>
+// BKM: B is read in the weights' stored layout [E][Kdim][N] (a row is one k) instead of the
+// transposed copy [E][N][Kdim]; its tiles land in LDS as [BKS k][BN] like the operands of the
+// weight-gradient GEMMs.
+template <class T, int EPI, bool BKM = false>
 __global__ __launch_bounds__(T::NT, T::WAVES_PER_EU) void rows_gemm_ring_kernel(RowsParams p) {
     constexpr int LDS_ELEMS = T::LDS_ELEMS > EpiShape<T, EPI>::ELEMS ? T::LDS_ELEMS : EpiShape<T, EPI>::ELEMS;
     static_assert(LDS_ELEMS * 2 <= 160 * 1024, "LDS capacity");
@@ -595,6 +628,8 @@ __global__ __launch_bounds__(T::NT, T::WAVES_PER_EU) void rows_gemm_ring_kernel(
     const int wave = threadIdx.x / MTS_WAVE, lane = threadIdx.x % MTS_WAVE;
     const int wm = wave / T::WAVES_N, wn = wave % T::WAVES_N;
 
+    constexpr int CPR_B = T::BN / 8, RPI_B = MTS_WAVE / CPR_B;   // k-major B: chunks per tile row, rows per instruction
+    static_assert(!BKM || (EPI != EPI_SWIGLU && T::BKS / RPI_B / T::NWAVES == T::B_INSTR), "k-major B loader split");
     const __amdgpu_buffer_rsrc_t rs_a = make_rsrc(p.A, p.a_rows * p.lda * 2);
     const __amdgpu_buffer_rsrc_t rs_b =
         make_rsrc(p.B + (int64_t)e * p.b_rows * p.Kdim, (int64_t)p.b_rows * p.Kdim * 2);
@@ -612,17 +647,23 @@ __global__ __launch_bounds__(T::NT, T::WAVES_PER_EU) void rows_gemm_ring_kernel(
         }
 #pragma unroll
         for (int j = 0; j < T::B_INSTR; ++j) {
-            const int br = (wave * T::B_INSTR + j) * T::RPI + rin;   // row inside the B tile
-            const int chunk = slot ^ (T::CHUNKS == 8 ? (br >> 1) & 7 : (br >> 2) & 3);
-            int n, grow;
-            if (SWIGLU) {
-                n = n0 + br % (T::BN / 2);
-                grow = (br / (T::BN / 2)) * p.N + n;
+            if constexpr (BKM) {
+                const int tr = (wave * T::B_INSTR + j) * RPI_B + lane / CPR_B;   // k row inside the B tile
+                const int c = n0 + (((lane % CPR_B) ^ ((tr & 3) << 2)) << 3);
+                voff_b[j] = c < p.N ? ((uint32_t)tr * (uint32_t)p.N + (uint32_t)c) * 2u : kInvalid;
             } else {
-                n = n0 + br;
-                grow = n;
+                const int br = (wave * T::B_INSTR + j) * T::RPI + rin;   // row inside the B tile
+                const int chunk = slot ^ (T::CHUNKS == 8 ? (br >> 1) & 7 : (br >> 2) & 3);
+                int n, grow;
+                if (SWIGLU) {
+                    n = n0 + br % (T::BN / 2);
+                    grow = (br / (T::BN / 2)) * p.N + n;
+                } else {
+                    n = n0 + br;
+                    grow = n;
+                }
+                voff_b[j] = (n < p.N) ? ((uint32_t)grow * (uint32_t)p.Kdim + chunk * 8) * 2u : kInvalid;
             }
-            voff_b[j] = (n < p.N) ? ((uint32_t)grow * (uint32_t)p.Kdim + chunk * 8) * 2u : kInvalid;
         }
     }
 
@@ -632,6 +673,7 @@ __global__ __launch_bounds__(T::NT, T::WAVES_PER_EU) void rows_gemm_ring_kernel(
         bf16_t* sa = smem + stage * T::STAGE + wave * T::A_INSTR * 512;
         bf16_t* sb = smem + stage * T::STAGE + T::BM * T::BKS + wave * T::B_INSTR * 512;
         const int soff = kt * T::BKS * 2;
+        const int soff_b = BKM ? kt * T::BKS * p.N * 2 : soff;   // a k-tile of k-major B is BKS memory rows further
 #pragma unroll
         for (int j = 0; j < T::A_INSTR; ++j)
             if (j % parts == part)
@@ -639,7 +681,7 @@ __global__ __launch_bounds__(T::NT, T::WAVES_PER_EU) void rows_gemm_ring_kernel(
 #pragma unroll
         for (int j = 0; j < T::B_INSTR; ++j)
             if ((j + T::A_INSTR) % parts == part)
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_b, MTS_LDS_PTR(sb + j * 512), 16, (int)voff_b[j], soff, 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_b, MTS_LDS_PTR(sb + j * 512), 16, (int)voff_b[j], soff_b, 0, 0);
     };
 
     f32x16 acc[T::MF][T::NF];
@@ -662,7 +704,7 @@ __global__ __launch_bounds__(T::NT, T::WAVES_PER_EU) void rows_gemm_ring_kernel(
         const int rstage = stage == 0 ? S - 1 : stage - 1;
         const bf16_t* cur = smem + stage * T::STAGE;
         constexpr int KSTEPS = T::BKS / 16;
-        mma_tile<T, SWIGLU, T::BKS>(cur, cur + T::BM * T::BKS, wm, wn, acc, [&](int ks) {
+        mma_tile<T, SWIGLU, T::BKS, true, BKM>(cur, cur + T::BM * T::BKS, wm, wn, acc, [&](int ks) {
             if (refill && (T::NWAVES < 8 ? true : ks == (wave / 4) % KSTEPS)) {
                 if (T::NWAVES < 8) issue(rstage, kt + S - 1, ks, KSTEPS);
                 else issue(rstage, kt + S - 1, 0, 1);  // waves w and w+4 share a SIMD and take turns
@@ -701,7 +743,7 @@ struct WsTile {
     static_assert(LDS_ELEMS * 2 <= 160 * 1024, "LDS capacity");
 };
 
-template <class T, int EPI>
+template <class T, int EPI, bool BKM = false>
 __global__ __launch_bounds__(T::NT, T::WAVES_PER_EU) void rows_gemm_ws_kernel(RowsParams p) {
     constexpr int LDS_ELEMS = T::LDS_ELEMS > EpiShape<T, EPI>::ELEMS ? T::LDS_ELEMS : EpiShape<T, EPI>::ELEMS;
     static_assert(LDS_ELEMS * 2 <= 160 * 1024, "LDS capacity");
@@ -723,6 +765,8 @@ __global__ __launch_bounds__(T::NT, T::WAVES_PER_EU) void rows_gemm_ws_kernel(Ro
             make_rsrc(p.B + (int64_t)e * p.b_rows * p.Kdim, (int64_t)p.b_rows * p.Kdim * 2);
         uint32_t voff_a[T::A_INSTR], voff_b[T::B_INSTR];
         const int slot = lane % T::CHUNKS, rin = lane / T::CHUNKS;
+        constexpr int CPR_B = T::BN / 8, RPI_B = MTS_WAVE / CPR_B;   // k-major B: chunks per tile row, rows per instruction
+        static_assert(!BKM || (EPI != EPI_SWIGLU && T::BKS / RPI_B / T::PRODUCERS == T::B_INSTR), "k-major B loader split");
 #pragma unroll
         for (int j = 0; j < T::A_INSTR; ++j) {
             const int tr = (pw * T::A_INSTR + j) * T::RPI + rin;
@@ -734,28 +778,35 @@ __global__ __launch_bounds__(T::NT, T::WAVES_PER_EU) void rows_gemm_ws_kernel(Ro
         }
 #pragma unroll
         for (int j = 0; j < T::B_INSTR; ++j) {
-            const int br = (pw * T::B_INSTR + j) * T::RPI + rin;
-            const int chunk = slot ^ (T::CHUNKS == 8 ? (br >> 1) & 7 : (br >> 2) & 3);
-            int n, grow;
-            if (SWIGLU) {
-                n = n0 + br % (T::BN / 2);
-                grow = (br / (T::BN / 2)) * p.N + n;
+            if constexpr (BKM) {
+                const int tr = (pw * T::B_INSTR + j) * RPI_B + lane / CPR_B;   // k row inside the B tile
+                const int c = n0 + (((lane % CPR_B) ^ ((tr & 3) << 2)) << 3);
+                voff_b[j] = c < p.N ? ((uint32_t)tr * (uint32_t)p.N + (uint32_t)c) * 2u : kInvalid;
             } else {
-                n = n0 + br;
-                grow = n;
+                const int br = (pw * T::B_INSTR + j) * T::RPI + rin;
+                const int chunk = slot ^ (T::CHUNKS == 8 ? (br >> 1) & 7 : (br >> 2) & 3);
+                int n, grow;
+                if (SWIGLU) {
+                    n = n0 + br % (T::BN / 2);
+                    grow = (br / (T::BN / 2)) * p.N + n;
+                } else {
+                    n = n0 + br;
+                    grow = n;
+                }
+                voff_b[j] = (n < p.N) ? ((uint32_t)grow * (uint32_t)p.Kdim + chunk * 8) * 2u : kInvalid;
             }
-            voff_b[j] = (n < p.N) ? ((uint32_t)grow * (uint32_t)p.Kdim + chunk * 8) * 2u : kInvalid;
         }
         auto issue = [&](int stage, int kt) {
             bf16_t* sa = smem + stage * T::STAGE + pw * T::A_INSTR * 512;
             bf16_t* sb = smem + stage * T::STAGE + T::BM * T::BKS + pw * T::B_INSTR * 512;
             const int soff = kt * T::BKS * 2;
+            const int soff_b = BKM ? kt * T::BKS * p.N * 2 : soff;   // a k-tile of k-major B is BKS memory rows further
 #pragma unroll
             for (int j = 0; j < T::A_INSTR; ++j)
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, MTS_LDS_PTR(sa + j * 512), 16, (int)voff_a[j], soff, 0, 0);
 #pragma unroll
             for (int j = 0; j < T::B_INSTR; ++j)
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_b, MTS_LDS_PTR(sb + j * 512), 16, (int)voff_b[j], soff, 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_b, MTS_LDS_PTR(sb + j * 512), 16, (int)voff_b[j], soff_b, 0, 0);
         };
         // Barrier kt tells the consumers that tiles kt and kt+1 have landed (they read the first
         // fragments of tile kt+1 behind the last MFMAs of tile kt) and tells the producers that
@@ -781,7 +832,7 @@ __global__ __launch_bounds__(T::NT, T::WAVES_PER_EU) void rows_gemm_ws_kernel(Ro
     const int wm = wave / T::WAVES_N, wn = wave % T::WAVES_N;
     f32x16 acc[T::MF][T::NF];
     zero_acc<T>(acc);
-    FragPipe<T, SWIGLU, T::BKS> pipe;
+    FragPipe<T, SWIGLU, T::BKS, BKM> pipe;
     pipe.init(wm, wn);
     constexpr int KSTEPS = T::BKS / 16;
     __builtin_amdgcn_s_barrier();   // tiles 0 and 1 are visible
@@ -1077,26 +1128,6 @@ __global__ __launch_bounds__(T::NT) void dw_gemm_kernel(DwParams p) {
 // arrive once tiles kt and kt+1 have landed, consumers once they are done reading
 // tile kt-1.
 // ---------------------------------------------------------------------------
-typedef __attribute__((ext_vector_type(4))) short s16x4;
-
-// 32 (m) x 16 (k) MFMA fragment out of a k-major LDS tile with row length ROWLEN
-template <int ROWLEN>
-__device__ __forceinline__ bf16x8 read_frag_tr(const bf16_t* tile, int krow0, int col0) {
-    const int lane = threadIdx.x % MTS_WAVE;
-    const int col = col0 + 16 * ((lane / 16) % 2) + 4 * (lane % 4);
-    const int chunk = col / 8, within = col % 8;
-    s16x4 h[2];
-#pragma unroll
-    for (int q = 0; q < 2; ++q) {
-        const int row = krow0 + 8 * (lane / 32) + 4 * q + (lane % 16) / 4;
-        const bf16_t* src = tile + row * ROWLEN + ((chunk ^ ((row & 3) << 2)) << 3) + within;
-        h[q] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(src));
-    }
-    typedef __attribute__((ext_vector_type(8))) short s16x8;
-    s16x8 v = {h[0][0], h[0][1], h[0][2], h[0][3], h[1][0], h[1][1], h[1][2], h[1][3]};
-    return __builtin_bit_cast(bf16x8, v);
-}
-
 template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int BKS_, int STAGES_, int PRODUCERS_>
 struct DwWsTile {
     static constexpr int BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
@@ -1360,19 +1391,33 @@ dim3 rows_grid(RowsParams& p, int64_t TK) {
     return dim3((unsigned)(m_groups * kXcds * p.n_tiles));
 }
 
+// does launch_rows_any take B in the weights' stored layout for this kind and reduction length?
+bool rows_kmajor_ok(int kind, int Kdim) { return tile_choice(kind) >= 1 && Kdim % 64 == 0; }
+
+// b_kmajor: B is [E][Kdim][N] (the weights as stored) instead of the transposed copy [E][N][Kdim];
+// only the ring and specialised kernels read it that way
 template <int EPI>
-int launch_rows_any(int kind, RowsParams p, int64_t TK, hipStream_t s) {
+int launch_rows_any(int kind, RowsParams p, int64_t TK, hipStream_t s, bool b_kmajor = false) {
     int choice = tile_choice(kind);
     // the ring kernels need whole k-tiles; other shapes use the staged kernel
     if (choice >= 1 && p.Kdim % 64 != 0) choice = 0;
+    if (b_kmajor && (choice == 0 || EPI == EPI_SWIGLU)) return MTS_ERR_SHAPE;
     if (choice == 1) {
         const dim3 grid = rows_grid<RingTwoPerCu, EPI>(p, TK);
-        rows_gemm_ring_kernel<RingTwoPerCu, EPI><<<grid, RingTwoPerCu::NT, 0, s>>>(p);
+        if constexpr (EPI != EPI_SWIGLU) {
+            if (b_kmajor) rows_gemm_ring_kernel<RingTwoPerCu, EPI, true><<<grid, RingTwoPerCu::NT, 0, s>>>(p);
+            else rows_gemm_ring_kernel<RingTwoPerCu, EPI><<<grid, RingTwoPerCu::NT, 0, s>>>(p);
+        } else {
+            rows_gemm_ring_kernel<RingTwoPerCu, EPI><<<grid, RingTwoPerCu::NT, 0, s>>>(p);
+        }
     } else if (choice == 2) {
         const dim3 grid = rows_grid<WsLarge, EPI>(p, TK);
-        rows_gemm_ws_kernel<WsLarge, EPI><<<grid, WsLarge::NT, 0, s>>>(p);
-
-
+        if constexpr (EPI != EPI_SWIGLU) {
+            if (b_kmajor) rows_gemm_ws_kernel<WsLarge, EPI, true><<<grid, WsLarge::NT, 0, s>>>(p);
+            else rows_gemm_ws_kernel<WsLarge, EPI><<<grid, WsLarge::NT, 0, s>>>(p);
+        } else {
+            rows_gemm_ws_kernel<WsLarge, EPI><<<grid, WsLarge::NT, 0, s>>>(p);
+        }
     } else {
         const dim3 grid = rows_grid<StagedSmall, EPI>(p, TK);
         rows_gemm_kernel<StagedSmall, EPI><<<grid, StagedSmall::NT, 0, s>>>(p);
@@ -1477,7 +1522,11 @@ extern "C" int mts_moe_fwd_down(const void* post_act, const void* w2, const int3
     return launch_rows_any<EPI_PLAIN>(K_DOWN, p, TK, (hipStream_t)stream);
 }
 
-extern "C" int mts_moe_bwd_dy1(const void* d_out, const void* w2t, const void* pre_act,
+extern "C" int mts_moe_bwd_weights_as_stored(int act_dtype, int H, int I) {
+    return act_dtype == MTS_BF16 && rows_kmajor_ok(K_DY1, H) && rows_kmajor_ok(K_DX, 2 * I) ? 1 : 0;
+}
+
+extern "C" int mts_moe_bwd_dy1(const void* d_out, const void* w2t, int w2_as_stored, const void* pre_act,
                                const void* weights, const int32_t* x_gather,
                                const int32_t* s_scatter, const int32_t* expert_start, int64_t T,
                                int K, int E, int H, int I, int act_dtype, void* d_pre_act,
@@ -1487,7 +1536,7 @@ extern "C" int mts_moe_bwd_dy1(const void* d_out, const void* w2t, const void* p
         return MTS_ERR_NULL;
     if (T <= 0 || K < 1) return MTS_ERR_SHAPE;
     if (act_dtype == MTS_F32) {
-        if (E < 1 || E > MTS_MAX_EXPERTS || H < 1 || I < 1 || T * K > 0x7fffffffLL) return MTS_ERR_SHAPE;
+        if (E < 1 || E > MTS_MAX_EXPERTS || H < 1 || I < 1 || T * K > 0x7fffffffLL || w2_as_stored) return MTS_ERR_SHAPE;
         return mts_f32_rows(2, (const float*)d_out, H, x_gather, (const float*)w2t, I, I, H, expert_start, E, T * K,
                             (float*)d_pre_act, (float*)weighted_act, (const float*)pre_act, (const float*)weights,
                             s_scatter, ds_partial, mts_moe_ds_partials(I), (hipStream_t)stream);
@@ -1503,15 +1552,15 @@ extern "C" int mts_moe_bwd_dy1(const void* d_out, const void* w2t, const void* p
     p.C = (bf16_t*)d_pre_act; p.C2 = (bf16_t*)weighted_act;
     p.pre_act = (const bf16_t*)pre_act; p.route_w = (const bf16_t*)weights;
     p.s_scatter = s_scatter; p.ds_part = ds_partial; p.np = mts_moe_ds_partials(I); p.TK = T * K;
-    return launch_rows_any<EPI_DY1>(K_DY1, p, T * K, (hipStream_t)stream);
+    return launch_rows_any<EPI_DY1>(K_DY1, p, T * K, (hipStream_t)stream, w2_as_stored != 0);
 }
 
-extern "C" int mts_moe_bwd_dx(const void* d_pre_act, const void* w1t, const int32_t* expert_start,
-                              int64_t TK, int E, int H, int I, int act_dtype, void* dx_expanded,
-                              void* stream) {
+extern "C" int mts_moe_bwd_dx(const void* d_pre_act, const void* w1t, int w1_as_stored,
+                              const int32_t* expert_start, int64_t TK, int E, int H, int I, int act_dtype,
+                              void* dx_expanded, void* stream) {
     if (!d_pre_act || !w1t || !expert_start || !dx_expanded) return MTS_ERR_NULL;
     if (act_dtype == MTS_F32) {
-        if (TK <= 0 || TK > 0x7fffffffLL || E < 1 || E > MTS_MAX_EXPERTS || H < 1 || I < 1) return MTS_ERR_SHAPE;
+        if (TK <= 0 || TK > 0x7fffffffLL || E < 1 || E > MTS_MAX_EXPERTS || H < 1 || I < 1 || w1_as_stored) return MTS_ERR_SHAPE;
         return mts_f32_rows(0, (const float*)d_pre_act, 2 * I, nullptr, (const float*)w1t, H, H, 2 * I, expert_start, E,
                             TK, (float*)dx_expanded, nullptr, nullptr, nullptr, nullptr, nullptr, 0,
                             (hipStream_t)stream);
@@ -1525,7 +1574,7 @@ extern "C" int mts_moe_bwd_dx(const void* d_pre_act, const void* w1t, const int3
     p.B = (const bf16_t*)w1t; p.b_rows = H;
     p.N = H; p.Kdim = 2 * I; p.expert_start = expert_start; p.E = E;
     p.C = (bf16_t*)dx_expanded; p.TK = TK;
-    return launch_rows_any<EPI_PLAIN>(K_DX, p, TK, (hipStream_t)stream);
+    return launch_rows_any<EPI_PLAIN>(K_DX, p, TK, (hipStream_t)stream, w1_as_stored != 0);
 }
 
 extern "C" int64_t mts_moe_bwd_dw_workspace_bytes(int which, int E, int H, int I) {

@@ -43,9 +43,10 @@ SIGNATURES = {
     "mts_moe_fwd_down": (_i, [_p, _p, _p, _l, _i, _i, _i, _i, _p, _p]),
     "mts_moe_combine": (_i, [_p, _p, _p, _l, _i, _i, _i, _p, _p]),
     "mts_moe_ds_partials": (_i, [_i]),
-    "mts_moe_bwd_dy1": (_i, [_p, _p, _p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p, _p, _p, _p]),
+    "mts_moe_bwd_weights_as_stored": (_i, [_i, _i, _i]),
+    "mts_moe_bwd_dy1": (_i, [_p, _p, _i, _p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p, _p, _p, _p]),
     "mts_moe_bwd_ds": (_i, [_p, _p, _l, _i, _i, _p, _p]),
-    "mts_moe_bwd_dx": (_i, [_p, _p, _p, _l, _i, _i, _i, _i, _p, _p]),
+    "mts_moe_bwd_dx": (_i, [_p, _p, _i, _p, _l, _i, _i, _i, _i, _p, _p]),
     "mts_moe_bwd_dw_workspace_bytes": (_l, [_i, _i, _i, _i]),
     "mts_moe_bwd_dw2": (_i, [_p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _i, _p, _p, _l, _p]),
     "mts_moe_bwd_dw1": (_i, [_p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _i, _p, _p, _l, _p]),

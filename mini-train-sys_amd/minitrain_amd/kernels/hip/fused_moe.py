@@ -265,22 +265,29 @@ class _FusedMoEFunction(torch.autograd.Function):
                 ev.record(frm)
                 main.wait_event(ev)
 
-        w1t = None
+        # The ring kernels read the weights in their stored layout (bf16, whole 64-wide k-tiles);
+        # other contracts get transposed copies, W1's made on a side stream next to the dO*W2 GEMM.
+        as_stored = bool(lib.mts_moe_bwd_weights_as_stored(act, H, I))
+        w1_bwd = None
         if need_x:
-            fork(side[0])
-            w1t = _stage(lib, gate_up_proj, True, x.dtype, side[0].cuda_stream)  # [E, H, 2I]
-            w1t_ready = torch.cuda.Event() if overlap else None
-            if overlap:
-                w1t_ready.record(side[0])
+            if as_stored:
+                w1_bwd = _stage(lib, gate_up_proj, False, x.dtype)  # [E, 2I, H], a cast only for fp32 parameters
+            else:
+                fork(side[0])
+                w1_bwd = _stage(lib, gate_up_proj, True, x.dtype, side[0].cuda_stream)  # [E, H, 2I]
+                w1t_ready = torch.cuda.Event() if overlap else None
+                if overlap:
+                    w1t_ready.record(side[0])
 
-        w2t = _stage(lib, down_proj, True, x.dtype)  # [E, I, H]
+        w2_bwd = _stage(lib, down_proj, not as_stored, x.dtype)  # [E, H, I] as stored, else [E, I, H]
         d_pre_act = torch.empty(TK, 2 * I, dtype=x.dtype, device=dev)
         weighted_act = torch.empty(TK, I, dtype=x.dtype, device=dev)
         n_part = lib.mts_moe_ds_partials(I)
         ds_part = torch.empty(TK, n_part, dtype=torch.float32, device=dev)
         _lib.check(
             lib.mts_moe_bwd_dy1(
-                dO.data_ptr(), w2t.data_ptr(), pre_act.data_ptr(), weights_flat.data_ptr(), x_gather.data_ptr(),
+                dO.data_ptr(), w2_bwd.data_ptr(), int(as_stored), pre_act.data_ptr(), weights_flat.data_ptr(),
+                x_gather.data_ptr(),
                 s_scatter.data_ptr(), expert_start.data_ptr(), T, K, E, H, I, act, d_pre_act.data_ptr(),
                 weighted_act.data_ptr(), ds_part.data_ptr(), stream,
             ),
@@ -329,13 +336,13 @@ class _FusedMoEFunction(torch.autograd.Function):
 
         dx = None
         if need_x:
-            if overlap:
+            if overlap and not as_stored:
                 main.wait_event(w1t_ready)
             dx_expanded = torch.empty(TK, H, dtype=x.dtype, device=dev)
             _lib.check(
                 lib.mts_moe_bwd_dx(
-                    d_pre_act.data_ptr(), w1t.data_ptr(), expert_start.data_ptr(), TK, E, H, I, act,
-                    dx_expanded.data_ptr(), stream,
+                    d_pre_act.data_ptr(), w1_bwd.data_ptr(), int(as_stored), expert_start.data_ptr(), TK, E, H, I,
+                    act, dx_expanded.data_ptr(), stream,
                 ),
                 "mts_moe_bwd_dx",
             )
