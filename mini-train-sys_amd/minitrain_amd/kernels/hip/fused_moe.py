@@ -303,6 +303,19 @@ class _FusedMoEFunction(torch.autograd.Function):
             fork(side[0])
         elif need_w1:
             fork(side[1])
+        # the routing-weight gradient is needed after the join only: it leads one of the side streams
+        # (when there is one) so that dX follows the dO*W2 GEMM directly on the caller's stream
+        d_weights = None
+        if need_s:
+            ds_stream = side[0].cuda_stream if need_w2 else (side[1].cuda_stream if need_w1 else stream)
+            d_weights = torch.empty(T, K, dtype=weights_flat.dtype, device=dev)
+            _lib.check(
+                lib.mts_moe_bwd_ds(
+                    ds_part.data_ptr(), s_reverse.data_ptr(), TK, I, act, d_weights.data_ptr(), ds_stream
+                ),
+                "mts_moe_bwd_ds",
+            )
+
         if need_w2:
             ddown_proj = torch.empty_like(down_proj)
             _lib.check(
@@ -324,14 +337,6 @@ class _FusedMoEFunction(torch.autograd.Function):
                     side[1].cuda_stream,
                 ),
                 "mts_moe_bwd_dw1",
-            )
-
-        d_weights = None
-        if need_s:
-            d_weights = torch.empty(T, K, dtype=weights_flat.dtype, device=dev)
-            _lib.check(
-                lib.mts_moe_bwd_ds(ds_part.data_ptr(), s_reverse.data_ptr(), TK, I, act, d_weights.data_ptr(), stream),
-                "mts_moe_bwd_ds",
             )
 
         dx = None
