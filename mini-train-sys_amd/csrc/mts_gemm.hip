@@ -327,7 +327,9 @@ __device__ __forceinline__ void flush_tile(const bf16_t* buf, __amdgpu_buffer_rs
     }
 }
 
-template <class T, int EPI>
+// PREFETCH (dY1): the pre-activations of slab mf+1 are loaded into registers before the
+// arithmetic of slab mf (32 more registers: for the kernels that have them to spare).
+template <class T, int EPI, bool PREFETCH = false>
 __device__ __forceinline__ void rows_epilogue(const RowsParams& p, f32x16 (&acc)[T::MF][T::NF], bf16_t* smem,
                                               int row0, int rend, int n0, int wm, int wn) {
     typedef EpiShape<T, EPI> ES;
@@ -346,12 +348,29 @@ __device__ __forceinline__ void rows_epilogue(const RowsParams& p, f32x16 (&acc)
     // routing weight of each of the lane's rows (dY1 only): two dependent loads, issued for all
     // rows up front
     float srow[T::MF];
+    // dY1: gate and up pre-activations of one 32 x COLS slab of the wave's tile, row-contiguous
+    // 16-byte loads held in registers; the loads of slab mf+1 are issued before the arithmetic of
+    // slab mf so that their latency is covered
+    constexpr int PRE_LPR = COLS / 8, PRE_RPI = MTS_WAVE / PRE_LPR, PRE_IT = 32 / PRE_RPI;
+    u32x4 gv[EPI == EPI_DY1 ? PRE_IT : 1], uv[EPI == EPI_DY1 ? PRE_IT : 1];
+    auto load_pre = [&](int mf) {
+        const int c = (lane % PRE_LPR) * 8;
+#pragma unroll
+        for (int it = 0; it < PRE_IT; ++it) {
+            const int grow = row0 + wm * T::WM + mf * 32 + it * PRE_RPI + lane / PRE_LPR;
+            const bool ok = grow < rend && ncol0 + c < p.N;
+            const uint32_t po = ok ? ((uint32_t)grow * 2u * N + (uint32_t)(ncol0 + c)) * 2u : kInvalid;
+            gv[it] = buf_load16(rs_pre, po);
+            uv[it] = buf_load16(rs_pre, po == kInvalid ? kInvalid : po + N * 2u);
+        }
+    };
     if (EPI == EPI_DY1) {
 #pragma unroll
         for (int mf = 0; mf < T::MF; ++mf) {
             const int row = row0 + wm * T::WM + mf * 32 + ml;
             srow[mf] = row < rend ? (float)p.route_w[p.s_scatter[row]] : 0.f;
         }
+        if (PREFETCH) load_pre(0);
     }
 #pragma unroll
     for (int mf = 0; mf < T::MF; ++mf) {
@@ -389,23 +408,27 @@ __device__ __forceinline__ void rows_epilogue(const RowsParams& p, f32x16 (&acc)
             const int row = rowg0 + ml;
             const bool rok = row < rend;
             const float s = srow[mf];
-            // gate and up pre-activations of the wave's 32 x COLS tile: row-contiguous 16-byte
-            // loads, staged in the buffers that take d_gate and d_up afterwards (a lane reads
-            // exactly the positions it overwrites)
+            // the slab's pre-activations go to the buffers that take d_gate and d_up afterwards (a
+            // lane reads exactly the positions it overwrites), then the next slab's loads start
             {
-                constexpr int LPR = COLS / 8, RPI = MTS_WAVE / LPR;
-                const int c = (lane % LPR) * 8;
+                const int c = (lane % PRE_LPR) * 8;
 #pragma unroll
-                for (int it = 0; it < 32 / RPI; ++it) {
-                    const int r = it * RPI + lane / LPR;
-                    const int grow = rowg0 + r;
-                    const bool ok = grow < rend && ncol0 + c < p.N;
-                    const uint32_t po = ok ? ((uint32_t)grow * 2u * N + (uint32_t)(ncol0 + c)) * 2u : kInvalid;
-                    const u32x4 gv = buf_load16(rs_pre, po);
-                    const u32x4 uv = buf_load16(rs_pre, po == kInvalid ? kInvalid : po + N * 2u);
-                    *reinterpret_cast<u32x4*>(buf1 + r * LDW + c) = gv;
-                    *reinterpret_cast<u32x4*>(buf2 + r * LDW + c) = uv;
+                for (int it = 0; it < PRE_IT; ++it) {
+                    const int r = it * PRE_RPI + lane / PRE_LPR;
+                    if (PREFETCH) {
+                        *reinterpret_cast<u32x4*>(buf1 + r * LDW + c) = gv[it];
+                        *reinterpret_cast<u32x4*>(buf2 + r * LDW + c) = uv[it];
+                    } else {   // load and hand over one row group at a time: few registers live
+                        const int grow = rowg0 + r;
+                        const bool ok = grow < rend && ncol0 + c < p.N;
+                        const uint32_t po = ok ? ((uint32_t)grow * 2u * N + (uint32_t)(ncol0 + c)) * 2u : kInvalid;
+                        const u32x4 g16 = buf_load16(rs_pre, po);
+                        const u32x4 u16 = buf_load16(rs_pre, po == kInvalid ? kInvalid : po + N * 2u);
+                        *reinterpret_cast<u32x4*>(buf1 + r * LDW + c) = g16;
+                        *reinterpret_cast<u32x4*>(buf2 + r * LDW + c) = u16;
+                    }
                 }
+                if (PREFETCH && mf + 1 < T::MF) load_pre(mf + 1);
             }
             float dsp = 0.f;
 #pragma unroll
@@ -713,7 +736,7 @@ __global__ __launch_bounds__(T::NT, T::WAVES_PER_EU) void rows_gemm_ring_kernel(
         stage = stage + 1 == S ? 0 : stage + 1;
     }
     __builtin_amdgcn_s_barrier();  // every wave is done reading the ring before it is reused
-    rows_epilogue<T, EPI>(p, acc, smem, row0, rend, n0, wm, wn);
+    rows_epilogue<T, EPI, true>(p, acc, smem, row0, rend, n0, wm, wn);
 }
 
 // ---------------------------------------------------------------------------
