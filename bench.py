@@ -41,8 +41,8 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # two rocprofv3 counter runs summarised in profiles/moe_layer_24x1024_hbm_traffic.txt (FETCH_SIZE
 # scaled by 2.0, WRITE_SIZE by 1.0 against a plain copy kernel of known size).  Not measured live.
 MEASURED_TRAFFIC_BYTES = {
-    "fwd_gateup_swiglu": 788.3e6, "fwd_down": 303.8e6, "bwd_dx": 531.2e6, "bwd_dy1": 722.4e6,
-    "bwd_dw2": 189.4e6, "bwd_dw1": 302.7e6, "combine": 115.2e6, "dx_combine": 114.4e6,
+    "fwd_gateup_swiglu": 776.5e6, "fwd_down": 303.4e6, "bwd_dx": 533.9e6, "bwd_dy1": 708.7e6,
+    "bwd_dw2": 189.5e6, "bwd_dw1": 302.7e6, "combine": 115.2e6, "dx_combine": 114.4e6,
 }
 
 WORKLOAD = dict(name="moe_layer_24x1024_d768_e8_top2_ff1024_bf16", seed=1, T=24576, H=768, E=8, K=2, I=1024)
