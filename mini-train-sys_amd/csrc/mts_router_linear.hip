@@ -153,24 +153,35 @@ __global__ __launch_bounds__(kFwdThreads) void router_logits_fwd_kernel(const XT
 // group are issued before the arithmetic of the current one); the rows left over are done one
 // by one.  EXACT: E == EP, so a row's logit gradients are EP consecutive floats at an address
 // every thread of the block shares, which the compiler turns into scalar loads.
+// A block holds `groups` sets of column threads; each set takes a contiguous share of the block's
+// rows, and the sets' dW_r sums are added through LDS in set order before the block writes its
+// one partial: a quarter of the partials for the same number of waves in flight.
+constexpr int bwd_max_threads(int EP) { return EP <= 8 ? 768 : 384; }   // 16 experts need twice the registers
+
 template <typename XT, int EP, bool EXACT>
-__global__ __launch_bounds__(256) void router_logits_bwd_kernel(const float* __restrict__ dl,
+__global__ __launch_bounds__(bwd_max_threads(EP)) void router_logits_bwd_kernel(const float* __restrict__ dl,
                                                                  const XT* __restrict__ x,
                                                                  const float* __restrict__ w, int64_t T, int H,
-                                                                 int E, int rows_per_block, XT* __restrict__ dx,
-                                                                 float* __restrict__ part) {
-    const int c = threadIdx.x * 4;
-    if (c >= H) return;
+                                                                 int E, int rows_per_block, int groups,
+                                                                 XT* __restrict__ dx, float* __restrict__ part) {
+    extern __shared__ __attribute__((aligned(16))) float set_sum[];   // [E][H]
+    const int col_threads = blockDim.x / groups;
+    const int grp = threadIdx.x / col_threads;
+    const int c = (threadIdx.x % col_threads) * 4;
+    const bool active = c < H;
     typedef typename RawVec<XT>::type raw_t;
     f32x4 wv[EP], acc[EP];
 #pragma unroll
     for (int e = 0; e < EP; ++e) {
         const f32x4 z = {0.f, 0.f, 0.f, 0.f};
-        wv[e] = e < E ? *reinterpret_cast<const f32x4*>(w + (int64_t)e * H + c) : z;
+        wv[e] = (active && e < E) ? *reinterpret_cast<const f32x4*>(w + (int64_t)e * H + c) : z;
         acc[e] = z;
     }
-    const int64_t row_beg = (int64_t)blockIdx.x * rows_per_block;
-    const int64_t row_end = row_beg + rows_per_block < T ? row_beg + rows_per_block : T;
+    const int64_t block_beg = (int64_t)blockIdx.x * rows_per_block;
+    const int64_t block_end = block_beg + rows_per_block < T ? block_beg + rows_per_block : T;
+    const int64_t per_set = (block_end - block_beg + groups - 1) / groups;
+    const int64_t row_beg = block_beg + grp * per_set < block_end ? block_beg + grp * per_set : block_end;
+    const int64_t row_end = !active ? row_beg : (row_beg + per_set < block_end ? row_beg + per_set : block_end);
     auto one_row = [&](int64_t row, raw_t raw) {
         const f32x4 xv = widen(raw);
         float g[EP];
@@ -219,6 +230,21 @@ __global__ __launch_bounds__(256) void router_logits_bwd_kernel(const float* __r
     }
 #pragma unroll 1
     for (; row < row_end; ++row) one_row(row, load_raw(x + row * H + c));
+    for (int r = 1; r < groups; ++r) {   // set 0 collects the others in set order
+        if (grp == r && active) {
+#pragma unroll
+            for (int e = 0; e < EP; ++e)
+                if (e < E) *reinterpret_cast<f32x4*>(set_sum + e * H + c) = acc[e];
+        }
+        __syncthreads();
+        if (grp == 0 && active) {
+#pragma unroll
+            for (int e = 0; e < EP; ++e)
+                if (e < E) acc[e] += *reinterpret_cast<const f32x4*>(set_sum + e * H + c);
+        }
+        __syncthreads();
+    }
+    if (grp != 0 || !active) return;
     float* out = part + (int64_t)blockIdx.x * E * H;
 #pragma unroll
     for (int e = 0; e < EP; ++e)
@@ -312,19 +338,24 @@ extern "C" int mts_router_logits_bwd(const float* dlogits, const void* x, const 
     if (workspace_bytes < mts_router_logits_bwd_workspace_bytes(T, H, E)) return MTS_ERR_WORKSPACE;
     if (!mts_aligned16(workspace) || !mts_aligned16(d_w_r) || (reinterpret_cast<uintptr_t>(dx) & 15u)) return MTS_ERR_ALIGN;
     hipStream_t s = (hipStream_t)stream;
-    const int nb = bwd_blocks(T);
+    const int col_threads = ((H / 4 + MTS_WAVE - 1) / MTS_WAVE) * MTS_WAVE;   // one thread per 4 columns
+    const int max_threads = bwd_max_threads(E <= 8 ? 8 : 16);
+    const int groups = max_threads / col_threads < 4 ? (max_threads / col_threads < 1 ? 1 : max_threads / col_threads) : 4;   // row sets per block
+    const int threads = groups * col_threads;
+    int nb = (bwd_blocks(T) + groups - 1) / groups;
     const int rows_per_block = (int)((T + nb - 1) / nb);
-    const int threads = ((H / 4 + MTS_WAVE - 1) / MTS_WAVE) * MTS_WAVE;   // one thread per 4 columns
+    nb = (int)((T + rows_per_block - 1) / rows_per_block);   // every block has at least one row
+    const size_t lds = (size_t)E * H * sizeof(float);
     float* part = (float*)workspace;
     const bool vec_dl = mts_aligned16(dlogits);
 #define MTS_BWD(XT, EP)                                                                                    \
     do {                                                                                                   \
         if (E == EP && vec_dl)                                                                             \
-            router_logits_bwd_kernel<XT, EP, true><<<nb, threads, 0, s>>>(dlogits, (const XT*)x, w_r, T, H, E, \
-                                                                          rows_per_block, (XT*)dx, part);  \
+            router_logits_bwd_kernel<XT, EP, true><<<nb, threads, lds, s>>>(dlogits, (const XT*)x, w_r, T, H, E, \
+                                                                            rows_per_block, groups, (XT*)dx, part); \
         else                                                                                               \
-            router_logits_bwd_kernel<XT, EP, false><<<nb, threads, 0, s>>>(dlogits, (const XT*)x, w_r, T, H, E, \
-                                                                           rows_per_block, (XT*)dx, part); \
+            router_logits_bwd_kernel<XT, EP, false><<<nb, threads, lds, s>>>(dlogits, (const XT*)x, w_r, T, H, E, \
+                                                                             rows_per_block, groups, (XT*)dx, part); \
     } while (0)
     if (act_dtype == MTS_BF16) {
         if (E <= 8) MTS_BWD(bf16_t, 8);
