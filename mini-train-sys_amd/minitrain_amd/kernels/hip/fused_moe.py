@@ -220,6 +220,10 @@ class _FusedMoEFunction(torch.autograd.Function):
             x, gate_up_proj, down_proj, pre_act, weights_flat, expert_start, x_gather, s_scatter, s_reverse
         )
         ctx.dims = (T, K, E, H, I)
+        # fp32 parameters under a bf16 activation dtype: the backward GEMMs that read the weights as
+        # stored reuse the casts made here (38 MB a layer at the 768/1024 shape) instead of repeating them
+        keep = bool(lib.mts_moe_bwd_weights_as_stored(act, H, I))
+        ctx.staged = (w1 if keep and w1 is not gate_up_proj else None, w2 if keep and w2 is not down_proj else None)
         ctx.mark_non_differentiable(top_k_index)
         ctx.set_materialize_grads(False)
         return out
@@ -271,7 +275,8 @@ class _FusedMoEFunction(torch.autograd.Function):
         w1_bwd = None
         if need_x:
             if as_stored:
-                w1_bwd = _stage(lib, gate_up_proj, False, x.dtype)  # [E, 2I, H], a cast only for fp32 parameters
+                # [E, 2I, H]: the parameter itself, or the forward pass's cast of an fp32 parameter
+                w1_bwd = ctx.staged[0] if ctx.staged[0] is not None else _stage(lib, gate_up_proj, False, x.dtype)
             else:
                 fork(side[0])
                 w1_bwd = _stage(lib, gate_up_proj, True, x.dtype, side[0].cuda_stream)  # [E, H, 2I]
@@ -279,7 +284,10 @@ class _FusedMoEFunction(torch.autograd.Function):
                 if overlap:
                     w1t_ready.record(side[0])
 
-        w2_bwd = _stage(lib, down_proj, not as_stored, x.dtype)  # [E, H, I] as stored, else [E, I, H]
+        if as_stored and ctx.staged[1] is not None:
+            w2_bwd = ctx.staged[1]
+        else:
+            w2_bwd = _stage(lib, down_proj, not as_stored, x.dtype)  # [E, H, I] as stored, else [E, I, H]
         d_pre_act = torch.empty(TK, 2 * I, dtype=x.dtype, device=dev)
         weighted_act = torch.empty(TK, I, dtype=x.dtype, device=dev)
         n_part = lib.mts_moe_ds_partials(I)
