@@ -25,25 +25,29 @@ class FeedForwardOutput:
 
 
 class MoEFeedForward(nn.Module):
+    """Owner of the expert parameters; calls the router and ``ops.fused_moe`` on flattened tokens."""
+
     def __init__(self, cfg: ModelConfig) -> None:
         super().__init__()
+        E, H, I = cfg.num_experts, cfg.hidden_size, cfg.intermediate_size
         self.cfg = cfg
         self.router = TopKRouter(cfg)
-        self.gate_up_proj = nn.Parameter(torch.empty(cfg.num_experts, 2 * cfg.intermediate_size, cfg.hidden_size))
-        self.down_proj = nn.Parameter(torch.empty(cfg.num_experts, cfg.hidden_size, cfg.intermediate_size))
+        # rows 0..I-1 of an expert's gate_up_proj are the gate, rows I..2I-1 the up projection
+        self.gate_up_proj = nn.Parameter(torch.empty(E, 2 * I, H))
+        self.down_proj = nn.Parameter(torch.empty(E, H, I))
         self.dropout = nn.Dropout(cfg.dropout)
-        nn.init.normal_(self.gate_up_proj, mean=0.0, std=0.02)
-        nn.init.normal_(self.down_proj, mean=0.0, std=0.02 / math.sqrt(2 * cfg.n_layers))
+        with torch.no_grad():
+            self.gate_up_proj.normal_(0.0, 0.02)
+            self.down_proj.normal_(0.0, 0.02 / math.sqrt(2 * cfg.n_layers))   # residual-branch scaling
 
     def forward(self, x: torch.Tensor, ops: OpsBackend) -> FeedForwardOutput:
-        shape = x.shape
-        flat_x = x.reshape(-1, shape[-1])
-        route = self.router(flat_x, ops)
+        tokens = x.reshape(-1, x.shape[-1])
+        route = self.router(tokens, ops)
         # under a capacity limit the router may hand over a dispatch in which dropped routes carry -1
         dispatch = route.expert_indices if route.dispatch_indices is None else route.dispatch_indices
-        hidden = ops.fused_moe(flat_x, self.gate_up_proj, self.down_proj, dispatch, route.expert_weights).view(shape)
+        mixed = ops.fused_moe(tokens, self.gate_up_proj, self.down_proj, dispatch, route.expert_weights)
         return FeedForwardOutput(
-            hidden_states=self.dropout(hidden),
+            hidden_states=self.dropout(mixed.view(x.shape)),
             router_aux_loss=route.auxiliary_loss,
             router_z_loss=route.z_loss,
             router_metrics=route.metrics,

@@ -1,13 +1,18 @@
-"""Model configuration: the fields, names and defaults of the reference's ``ModelConfig``
-(minitrain/model/config.py:4-63) that the decoder and its MoE blocks read.  The reference
-reserves ``expert_capacity_factor`` / ``expert_min_capacity`` for a compacted dispatch and
-ignores them (config.py:24-28); here a factor other than None switches that dispatch on."""
+"""Model configuration.
 
-from dataclasses import dataclass
+Field names and defaults are those of the reference's ``ModelConfig``
+(minitrain/model/config.py:4-63), since configs written for it must load here; the checks raise
+``ValueError`` for the same conditions.  One deliberate difference: the reference reserves
+``expert_capacity_factor`` / ``expert_min_capacity`` for a compacted dispatch and ignores them
+(config.py:24-28); here a factor other than None switches that dispatch on.
+"""
+
+from dataclasses import dataclass, fields
 
 
 @dataclass(frozen=True)
 class ModelConfig:
+    # decoder geometry
     vocab_size: int = 32000
     seq_len: int = 2048
     n_layers: int = 12
@@ -18,6 +23,7 @@ class ModelConfig:
     rope_theta: float = 10000.0
     dropout: float = 0.0
     tie_word_embeddings: bool = False
+    # feed-forward flavour and router
     ffn_type: str = "moe"
     num_experts: int = 8
     experts_per_token: int = 2
@@ -29,29 +35,35 @@ class ModelConfig:
     expert_min_capacity: int = 4
 
     def __post_init__(self) -> None:
-        sizes = (self.vocab_size, self.seq_len, self.n_layers, self.n_heads, self.hidden_size, self.intermediate_size)
-        if min(sizes) <= 0:
-            raise ValueError("all model dimensions must be positive")
-        if not 0 <= self.dropout < 1:
-            raise ValueError("dropout must be in [0, 1)")
-        if self.norm_eps <= 0 or self.rope_theta <= 0:
-            raise ValueError("norm_eps and rope_theta must be positive")
-        if self.ffn_type not in {"dense", "moe"}:
-            raise ValueError("ffn_type must be either 'dense' or 'moe'")
-        if self.hidden_size % self.n_heads != 0:
-            raise ValueError("hidden_size must be divisible by n_heads")
-        if self.num_experts <= 0:
-            raise ValueError("num_experts must be positive")
-        if not 0 < self.experts_per_token <= self.num_experts:
-            raise ValueError("experts_per_token must be in [1, num_experts]")
-        if self.router_aux_loss_coef < 0 or self.router_z_loss_coef < 0:
-            raise ValueError("router loss coefficients must be non-negative")
-        if not 0 <= self.router_jitter_noise < 1:
-            raise ValueError("router_jitter_noise must be in [0, 1)")
+        problem = self._first_problem()
+        if problem:
+            raise ValueError(problem)
+
+    def _first_problem(self) -> str | None:
+        sizes = ("vocab_size", "seq_len", "n_layers", "n_heads", "hidden_size", "intermediate_size", "num_experts",
+                 "expert_min_capacity")
+        for name in sizes:
+            if getattr(self, name) <= 0:
+                return f"{name} must be positive"
+        unit_interval = ("dropout", "router_jitter_noise")
+        for name in unit_interval:
+            if not 0 <= getattr(self, name) < 1:
+                return f"{name} must be in [0, 1)"
+        for name in ("norm_eps", "rope_theta"):
+            if getattr(self, name) <= 0:
+                return f"{name} must be positive"
+        for name in ("router_aux_loss_coef", "router_z_loss_coef"):
+            if getattr(self, name) < 0:
+                return f"{name} must be non-negative"
+        if self.ffn_type not in ("dense", "moe"):
+            return "ffn_type must be either 'dense' or 'moe'"
+        if self.hidden_size % self.n_heads:
+            return "hidden_size must be divisible by n_heads"
+        if not 1 <= self.experts_per_token <= self.num_experts:
+            return "experts_per_token must be in [1, num_experts]"
         if self.expert_capacity_factor is not None and self.expert_capacity_factor <= 0:
-            raise ValueError("expert_capacity_factor must be positive or null")
-        if self.expert_min_capacity <= 0:
-            raise ValueError("expert_min_capacity must be positive")
+            return "expert_capacity_factor must be positive or null"
+        return None
 
     @property
     def head_dim(self) -> int:
@@ -60,3 +72,7 @@ class ModelConfig:
     @property
     def is_moe(self) -> bool:
         return self.ffn_type == "moe"
+
+    @classmethod
+    def field_names(cls) -> tuple[str, ...]:
+        return tuple(f.name for f in fields(cls))

@@ -60,37 +60,79 @@ def capacity_selection(expert_indices: torch.Tensor, expert_weights: torch.Tenso
     return keep, kept_index, counts.clamp(max=capacity)
 
 
+def load_metrics(route, accepted: torch.Tensor, routes: int, dropped_fraction: torch.Tensor, num_experts: int):
+    """The router's monitoring record, keys as in the reference (minitrain/model/moe_router.py:113-135);
+    ``accepted`` = routes each expert takes, as floats."""
+    share = accepted / max(routes, 1)
+    scale = float(num_experts)                      # 1 / (uniform share)
+    log_e = math.log(num_experts) if num_experts > 1 else 1.0
+    record = {
+        "moe/router_entropy": route.entropy,
+        "moe/router_entropy_normalized": route.entropy / log_e,
+        "moe/dropped_route_fraction": dropped_fraction,
+        "moe/max_expert_load": accepted.max(),
+        "moe/min_expert_load": accepted.min(),
+        "moe/expert_load_cv": share.std(unbiased=False) * scale,
+        "moe/max_to_mean_load": share.max() * scale,
+        "moe/dead_expert_count": (accepted == 0).sum(),
+        "moe/expert_load_fraction": share,           # per expert: stacked by layer for heat maps
+        "moe/expert_probability": route.probability_per_expert,
+    }
+    return {k: (v if k == "moe/router_entropy" else v.detach()) for k, v in record.items()}
+
+
 class TopKRouter(nn.Module):
     def __init__(self, cfg: ModelConfig) -> None:
         super().__init__()
         self.cfg = cfg
         self.weight = nn.Parameter(torch.empty(cfg.num_experts, cfg.hidden_size))
-        nn.init.normal_(self.weight, mean=0.0, std=0.02)
+        with torch.no_grad():
+            self.weight.normal_(0.0, 0.02)
+
+    def _logits(self, hidden_states: torch.Tensor, ops: OpsBackend) -> torch.Tensor:
+        """fp32 router projection with autocast off (minitrain/model/moe_router.py:64-76)."""
+        cfg = self.cfg
+        jitter = self.training and cfg.router_jitter_noise
+        device_type = hidden_states.device.type
+        # a backend may offer the projection straight from the activation dtype (same fp32
+        # arithmetic, no fp32 copy of the activations); jitter noise needs the fp32 copy
+        fused = None if jitter else getattr(ops, "router_logits", None)
+        if fused is not None and hidden_states.ndim == 2:
+            with torch.autocast(device_type=device_type, enabled=False):
+                logits = fused(hidden_states, self.weight)
+            if logits is not None:
+                return logits
+        wide = hidden_states.float()
+        if jitter:
+            low, high = 1.0 - cfg.router_jitter_noise, 1.0 + cfg.router_jitter_noise
+            wide = wide * torch.empty_like(wide).uniform_(low, high)
+        with torch.autocast(device_type=device_type, enabled=False):
+            return F.linear(wide, self.weight.float())
+
+    def _limit_capacity(self, ops: OpsBackend, expert_indices: torch.Tensor, expert_weights: torch.Tensor):
+        """Masked and renormalised weights, dispatch indices (or None), accepted counts, dropped fraction."""
+        cfg = self.cfg
+        tokens, top_k = expert_indices.shape
+        capacity = max(cfg.expert_min_capacity, math.ceil(cfg.expert_capacity_factor * tokens * top_k / cfg.num_experts))
+        select = getattr(ops, "capacity_mask", None)
+        selection = select(expert_indices, expert_weights, cfg.num_experts, capacity) if select is not None else None
+        if selection is None:
+            selection = capacity_selection(expert_indices, expert_weights, cfg.num_experts, capacity)
+        keep, kept_index, accepted_counts = selection
+        weights = expert_weights * keep
+        if cfg.router_normalize_topk:
+            total = weights.sum(dim=-1, keepdim=True)
+            smallest = torch.finfo(weights.dtype).eps
+            weights = torch.where(total > 0, weights / total.clamp_min(smallest), weights)   # a token may lose every route
+        dispatch = kept_index.to(torch.int32) if getattr(ops, "drops_routes", False) else None
+        return weights, dispatch, accepted_counts.float(), 1.0 - keep.float().mean()
 
     def forward(self, hidden_states: torch.Tensor, ops: OpsBackend) -> RouterOutput:
         cfg = self.cfg
-        jitter = self.training and cfg.router_jitter_noise
-        # a backend may offer the projection straight from the activation dtype (same fp32
-        # arithmetic, no fp32 copy of the activations); jitter noise needs the fp32 copy
-        fused_logits = None if jitter else getattr(ops, "router_logits", None)
-        logits = None
-        if fused_logits is not None and hidden_states.ndim == 2:
-            with torch.autocast(device_type=hidden_states.device.type, enabled=False):
-                logits = fused_logits(hidden_states, self.weight)
-        if logits is None:
-            router_input = hidden_states.float()
-            if jitter:
-                noise = torch.empty_like(router_input).uniform_(
-                    1.0 - cfg.router_jitter_noise, 1.0 + cfg.router_jitter_noise
-                )
-                router_input = router_input * noise
-
+        logits = self._logits(hidden_states, ops)
         with torch.autocast(device_type=hidden_states.device.type, enabled=False):
-            if logits is None:
-                logits = F.linear(router_input, self.weight.float())
             route = ops.router_postprocess(logits, cfg.experts_per_token, normalize=cfg.router_normalize_topk)
-            expert_weights = route.expert_weights
-            expert_indices = route.expert_indices
+            expert_weights, expert_indices = route.expert_weights, route.expert_indices
 
             route_counts = getattr(route, "expert_counts", None)
             auxiliary_loss = getattr(route, "load_balance_loss", None)
@@ -101,53 +143,18 @@ class TopKRouter(nn.Module):
                 else:
                     route_counts = torch.bincount(expert_indices.flatten().long(), minlength=cfg.num_experts)
             if auxiliary_loss is None:
-                tokens_per_expert = route_counts.float() / expert_indices.numel()
-                # the assignment fraction carries no gradient; it enters through the mean probability
-                auxiliary_loss = cfg.num_experts * torch.sum(tokens_per_expert * route.probability_per_expert)
+                # E * sum_e f_e * pbar_e; the route fractions f carry no gradient, the mean probability does
+                route_fraction = route_counts.float() / expert_indices.numel()
+                auxiliary_loss = cfg.num_experts * torch.sum(route_fraction * route.probability_per_expert)
 
             dispatch_indices = None
             dropped_fraction = expert_weights.new_zeros(())
             accepted = route_counts.float()
             if cfg.expert_capacity_factor is not None:
-                tokens, top_k = expert_indices.shape
-                capacity = max(
-                    cfg.expert_min_capacity, math.ceil(cfg.expert_capacity_factor * tokens * top_k / cfg.num_experts)
+                expert_weights, dispatch_indices, accepted, dropped_fraction = self._limit_capacity(
+                    ops, expert_indices, expert_weights
                 )
-                selection = None
-                select = getattr(ops, "capacity_mask", None)
-                if select is not None:
-                    selection = select(expert_indices, expert_weights, cfg.num_experts, capacity)
-                if selection is None:
-                    selection = capacity_selection(expert_indices, expert_weights, cfg.num_experts, capacity)
-                keep, kept_index, accepted_counts = selection
-                expert_weights = expert_weights * keep
-                if cfg.router_normalize_topk:
-                    denominator = expert_weights.sum(dim=-1, keepdim=True)
-                    expert_weights = torch.where(
-                        denominator > 0,
-                        expert_weights / denominator.clamp_min(torch.finfo(expert_weights.dtype).eps),
-                        expert_weights,
-                    )
-                if getattr(ops, "drops_routes", False):
-                    dispatch_indices = kept_index.to(torch.int32)
-                accepted = accepted_counts.float()
-                dropped_fraction = 1.0 - keep.float().mean()
-            load_fraction = accepted / max(expert_indices.numel(), 1)
-            uniform = 1.0 / cfg.num_experts
-            metrics = {
-                "moe/router_entropy": route.entropy,
-                "moe/router_entropy_normalized": (
-                    route.entropy / (math.log(cfg.num_experts) if cfg.num_experts > 1 else 1.0)
-                ).detach(),
-                "moe/dropped_route_fraction": dropped_fraction.detach(),
-                "moe/max_expert_load": accepted.max().detach(),
-                "moe/min_expert_load": accepted.min().detach(),
-                "moe/expert_load_cv": (load_fraction.std(unbiased=False) / uniform).detach(),
-                "moe/max_to_mean_load": (load_fraction.max() / uniform).detach(),
-                "moe/dead_expert_count": (accepted == 0).sum().detach(),
-                "moe/expert_load_fraction": load_fraction.detach(),
-                "moe/expert_probability": route.probability_per_expert.detach(),
-            }
+            metrics = load_metrics(route, accepted, expert_indices.numel(), dropped_fraction, cfg.num_experts)
 
         return RouterOutput(
             expert_indices=expert_indices.to(torch.int32),

@@ -1,8 +1,9 @@
-"""Operator boundary between the MoE block and kernel backends.
+"""Operator boundary between the model code and the kernel backends.
 
-Mirror of the reference's ``minitrain/model/ops.py:7-112``: the same record type,
-the same protocol (eight methods) and the same factory function, plus the
-``hip`` branch a maintainer would add there.
+The interface is the reference's (minitrain/model/ops.py:7-112): a result record for the router
+post-process, a structural protocol with eight operators, and a factory that builds a backend
+from its name.  Only the names, arguments and return types are shared with it; this package
+ships one backend, ``hip``.
 """
 
 from dataclasses import dataclass
@@ -10,62 +11,61 @@ from typing import Protocol
 
 import torch
 
+Tensor = torch.Tensor
+
 
 @dataclass
 class RouterPostprocessOutput:
-    """Backend-neutral result of processing fp32 router logits."""
+    """What ``router_postprocess`` hands back, whichever backend computed it."""
 
-    expert_weights: torch.Tensor
-    expert_indices: torch.Tensor
-    probability_per_expert: torch.Tensor
-    z_loss: torch.Tensor
-    entropy: torch.Tensor
-    # Beyond the reference's record (minitrain/model/ops.py:7-15), filled by backends that
-    # compute them in the same pass: routes per expert (int32 [E], no gradient) and the
-    # load-balancing term E * sum_e (routes_e / routes) * probability_per_expert_e, which is
-    # differentiable through the mean probability.  None means the caller computes them.
-    expert_counts: torch.Tensor | None = None
-    load_balance_loss: torch.Tensor | None = None
+    expert_weights: Tensor           # [T, K] fp32, weight of each selected expert
+    expert_indices: Tensor           # [T, K] expert ids, rank 0 first
+    probability_per_expert: Tensor   # [E] mean softmax probability over the tokens
+    z_loss: Tensor                   # [] mean squared log-partition
+    entropy: Tensor                  # [] mean routing entropy, detached
+    # Not in the reference's record (minitrain/model/ops.py:7-15); a backend that has them from the
+    # same pass fills them in, None leaves the computation to the caller: routes per expert (int32
+    # [E], no gradient) and E * sum_e (routes_e / routes) * probability_per_expert_e, which carries a
+    # gradient through the mean probability.
+    expert_counts: Tensor | None = None
+    load_balance_loss: Tensor | None = None
 
 
 class OpsBackend(Protocol):
+    """The eight operators a backend provides; the model only ever sees this protocol."""
+
     name: str
 
-    def rmsnorm(self, x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor: ...
+    # dense operators: stay on stock PyTorch-ROCm in the ``hip`` backend
+    def rmsnorm(self, x: Tensor, weight: Tensor, eps: float) -> Tensor: ...
 
-    def rope(self, q, k, cos, sin) -> tuple[torch.Tensor, torch.Tensor]: ...
+    def rope(self, q: Tensor, k: Tensor, cos: Tensor, sin: Tensor) -> tuple[Tensor, Tensor]: ...
 
-    def swiglu(self, gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor: ...
+    def swiglu(self, gate: Tensor, up: Tensor) -> Tensor: ...
 
-    def attention(self, q, k, v, *, is_causal: bool, dropout_p: float) -> torch.Tensor: ...
+    def attention(self, q: Tensor, k: Tensor, v: Tensor, *, is_causal: bool, dropout_p: float) -> Tensor: ...
 
-    def cross_entropy(self, logits: torch.Tensor, targets: torch.Tensor) -> torch.Tensor: ...
+    def cross_entropy(self, logits: Tensor, targets: Tensor) -> Tensor: ...
 
-    def fused_linear_cross_entropy(self, x, weight, targets) -> torch.Tensor: ...
+    def fused_linear_cross_entropy(self, x: Tensor, weight: Tensor, targets: Tensor) -> Tensor: ...
 
-    def router_postprocess(
-        self, logits: torch.Tensor, top_k: int, *, normalize: bool
-    ) -> RouterPostprocessOutput:
-        """Process fp32 router logits and return differentiable routing statistics."""
+    # the two MoE operators
+    def router_postprocess(self, logits: Tensor, top_k: int, *, normalize: bool) -> RouterPostprocessOutput:
+        """fp32 logits ``[T, E]`` -> top-k weights and indices plus the routing statistics; differentiable
+        through the weights, the mean probability and the z-loss."""
         ...
 
     def fused_moe(
-        self,
-        x: torch.Tensor,
-        gate_up_proj: torch.Tensor,
-        down_proj: torch.Tensor,
-        top_k_index: torch.Tensor,
-        top_k_weights: torch.Tensor,
-    ) -> torch.Tensor:
-        """Apply routed SwiGLU experts and aggregate the selected outputs."""
+        self, x: Tensor, gate_up_proj: Tensor, down_proj: Tensor, top_k_index: Tensor, top_k_weights: Tensor
+    ) -> Tensor:
+        """``out[t] = sum_k w[t,k] * W2[e] (silu(g) * u)`` with ``[g; u] = W1[e] x[t]``, ``e = index[t,k]``."""
         ...
 
 
 def get_ops_backend(name: str) -> OpsBackend:
-    """Construct an operator backend by name (only ``hip`` lives in this package)."""
+    """Backend instance for ``name``; unknown names raise ``ValueError`` as in the reference."""
+    if name != "hip":
+        raise ValueError(f"Unknown ops backend: {name}")
+    from minitrain_amd.kernels.hip import HipOpsBackend
 
-    if name == "hip":
-        from minitrain_amd.kernels.hip import HipOpsBackend
-
-        return HipOpsBackend()
-    raise ValueError(f"Unknown ops backend: {name}")
+    return HipOpsBackend()
