@@ -33,6 +33,7 @@ extern "C" {
 /* element types of activations / weights / weight gradients */
 #define MTS_BF16 0
 #define MTS_F32 1
+#define MTS_F16 2
 
 #define MTS_OK 0
 #define MTS_ERR_NULL (-1)        /* a required pointer is NULL                      */
@@ -143,7 +144,7 @@ int mts_moe_stage_weights(const void* src, int src_dtype, void* dst, int dst_dty
  * Replaces _fused_up_proj_swiglu_kernel (fused_moe_kernels.py:264-367):
  * for every row r (token x_gather[r], expert e): [g;u] = W1[e] x ; a = silu(g)*u.
  * x [T,H], w1 [E,2I,H], pre_act [TK,2I], post_act [TK,I], all of act_dtype
- * (MTS_BF16: MFMA kernels, H and I multiples of 8; MTS_F32: plain fp32 kernels). */
+ * (MTS_BF16, MTS_F16: MFMA kernels, H and I multiples of 8; MTS_F32: plain fp32 kernels). */
 int mts_moe_fwd_gateup_swiglu(const void* x, const void* w1, const int32_t* x_gather,
                               const int32_t* expert_start, int64_t T, int K, int E, int H,
                               int I, int act_dtype, void* pre_act, void* post_act,

@@ -13,10 +13,23 @@ constexpr int kThreads = 256;
 // UN outputs at a time (token t, t + T/UN, ...) and issues all their index, weight
 // and row loads before the first use, to keep enough bytes in flight per CU.
 // A negative s_rev entry is a dropped route: it contributes nothing, whatever its weight.
-template <int KK, int UN>
+// ET is the 16-bit element type (bf16 or fp16).
+template <typename ET>
+struct Vec8;
+template <>
+struct Vec8<bf16_t> {
+    typedef bf16x8 type;
+};
+template <>
+struct Vec8<mts_f16_t> {
+    typedef mts_f16x8 type;
+};
+
+template <typename ET, int KK, int UN>
 __global__ __launch_bounds__(kThreads) void combine_bf16_kernel(
-    const bf16_t* __restrict__ y, const bf16_t* __restrict__ w, const int32_t* __restrict__ s_rev,
-    int64_t T, int K, int H, bf16_t* __restrict__ out) {
+    const ET* __restrict__ y, const ET* __restrict__ w, const int32_t* __restrict__ s_rev,
+    int64_t T, int K, int H, ET* __restrict__ out) {
+    typedef typename Vec8<ET>::type bf16x8;   // the build's 8-element vector
     const int vec_per_row = H / 8;
     const int64_t chunk = (T + UN - 1) / UN;           // tokens per unrolled slice
     const int64_t total = chunk * (int64_t)vec_per_row;
@@ -54,16 +67,18 @@ __global__ __launch_bounds__(kThreads) void combine_bf16_kernel(
                 for (int j = 0; j < 8; ++j) acc[j] += s[u][k] * (float)v[u][k][j];
             bf16x8 o;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) o[j] = (bf16_t)acc[j];
+            for (int j = 0; j < 8; ++j) o[j] = (ET)acc[j];
             *reinterpret_cast<bf16x8*>(out + t * H + c * 8) = o;
         }
     }
 }
 
 // any K: the routes of a token are visited in a loop
+template <typename ET>
 __global__ __launch_bounds__(kThreads) void combine_bf16_anyk_kernel(
-    const bf16_t* __restrict__ y, const bf16_t* __restrict__ w, const int32_t* __restrict__ s_rev,
-    int64_t T, int K, int H, bf16_t* __restrict__ out) {
+    const ET* __restrict__ y, const ET* __restrict__ w, const int32_t* __restrict__ s_rev,
+    int64_t T, int K, int H, ET* __restrict__ out) {
+    typedef typename Vec8<ET>::type bf16x8;
     const int vec_per_row = H / 8;
     const int64_t total = T * (int64_t)vec_per_row;
     for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total;
@@ -83,7 +98,7 @@ __global__ __launch_bounds__(kThreads) void combine_bf16_anyk_kernel(
         }
         bf16x8 o;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) o[j] = (bf16_t)acc[j];
+        for (int j = 0; j < 8; ++j) o[j] = (ET)acc[j];
         *reinterpret_cast<bf16x8*>(out + t * H + c * 8) = o;
     }
 }
@@ -199,19 +214,25 @@ extern "C" int mts_moe_combine(const void* y, const void* weights, const int32_t
     if (T <= 0 || K < 1 || H < 1) return MTS_ERR_SHAPE;
     if (!mts_aligned16(y) || !mts_aligned16(out)) return MTS_ERR_ALIGN;
     hipStream_t s = (hipStream_t)stream;
-    if (act_dtype == MTS_BF16) {
+    if (act_dtype == MTS_BF16 || act_dtype == MTS_F16) {
         if (H % 8) return MTS_ERR_SHAPE;
         constexpr int UN = 2;
         const int64_t sliced = ((T + UN - 1) / UN) * (int64_t)(H / 8);
-        if (K <= 2)
-            combine_bf16_kernel<2, UN><<<grid_1d(sliced), kThreads, 0, s>>>(
-                (const bf16_t*)y, (const bf16_t*)weights, s_reverse, T, K, H, (bf16_t*)out);
-        else if (K <= 4)
-            combine_bf16_kernel<4, UN><<<grid_1d(sliced), kThreads, 0, s>>>(
-                (const bf16_t*)y, (const bf16_t*)weights, s_reverse, T, K, H, (bf16_t*)out);
-        else
-            combine_bf16_anyk_kernel<<<grid_1d(T * (int64_t)(H / 8)), kThreads, 0, s>>>(
-                (const bf16_t*)y, (const bf16_t*)weights, s_reverse, T, K, H, (bf16_t*)out);
+#define MTS_COMBINE16(ET)                                                                                     \
+    do {                                                                                                      \
+        if (K <= 2)                                                                                           \
+            combine_bf16_kernel<ET, 2, UN><<<grid_1d(sliced), kThreads, 0, s>>>(                              \
+                (const ET*)y, (const ET*)weights, s_reverse, T, K, H, (ET*)out);                              \
+        else if (K <= 4)                                                                                      \
+            combine_bf16_kernel<ET, 4, UN><<<grid_1d(sliced), kThreads, 0, s>>>(                              \
+                (const ET*)y, (const ET*)weights, s_reverse, T, K, H, (ET*)out);                              \
+        else                                                                                                  \
+            combine_bf16_anyk_kernel<ET><<<grid_1d(T * (int64_t)(H / 8)), kThreads, 0, s>>>(                  \
+                (const ET*)y, (const ET*)weights, s_reverse, T, K, H, (ET*)out);                              \
+    } while (0)
+        if (act_dtype == MTS_BF16) MTS_COMBINE16(bf16_t);
+        else MTS_COMBINE16(mts_f16_t);
+#undef MTS_COMBINE16
     } else if (act_dtype == MTS_F32) {
         if (H % 4) return MTS_ERR_SHAPE;
         combine_f32_kernel<<<grid_1d(T * (int64_t)(H / 4)), kThreads, 0, s>>>(
@@ -232,6 +253,9 @@ extern "C" int mts_moe_bwd_ds(const float* ds_partial, const int32_t* s_reverse,
     if (act_dtype == MTS_BF16)
         ds_reduce_kernel<bf16_t><<<grid_1d(TK), kThreads, 0, s>>>(ds_partial, s_reverse, TK, np,
                                                                   (bf16_t*)d_weights);
+    else if (act_dtype == MTS_F16)
+        ds_reduce_kernel<mts_f16_t><<<grid_1d(TK), kThreads, 0, s>>>(ds_partial, s_reverse, TK, np,
+                                                                     (mts_f16_t*)d_weights);
     else if (act_dtype == MTS_F32)
         ds_reduce_kernel<float><<<grid_1d(TK), kThreads, 0, s>>>(ds_partial, s_reverse, TK, np,
                                                                  (float*)d_weights);
@@ -254,13 +278,16 @@ extern "C" int mts_moe_stage_weights(const void* src, int src_dtype, void* dst, 
     hipStream_t s = (hipStream_t)stream;
     dim3 grid((unsigned)((C + 63) / 64), (unsigned)((R + 63) / 64), (unsigned)E);
     if (grid.y > 65535) return MTS_ERR_SHAPE;
-    if (src_dtype == MTS_BF16 && dst_dtype == MTS_BF16 && transpose && R % 64 == 0 && C % 64 == 0 &&
+    if (src_dtype == dst_dtype && (src_dtype == MTS_BF16 || src_dtype == MTS_F16) && transpose && R % 64 == 0 && C % 64 == 0 &&
         mts_aligned16(src) && mts_aligned16(dst) && R <= 0x7fffffff && C <= 0x7fffffff)
         transpose_bf16_kernel<<<grid, kThreads, 0, s>>>((const bf16_t*)src, (bf16_t*)dst, (int)R, (int)C);
     else if (src_dtype == MTS_F32 && dst_dtype == MTS_BF16) launch_stage<float, bf16_t>(src, dst, grid, R, C, transpose, s);
     else if (src_dtype == MTS_BF16 && dst_dtype == MTS_BF16) launch_stage<bf16_t, bf16_t>(src, dst, grid, R, C, transpose, s);
     else if (src_dtype == MTS_F32 && dst_dtype == MTS_F32) launch_stage<float, float>(src, dst, grid, R, C, transpose, s);
     else if (src_dtype == MTS_BF16 && dst_dtype == MTS_F32) launch_stage<bf16_t, float>(src, dst, grid, R, C, transpose, s);
+    else if (src_dtype == MTS_F32 && dst_dtype == MTS_F16) launch_stage<float, mts_f16_t>(src, dst, grid, R, C, transpose, s);
+    else if (src_dtype == MTS_F16 && dst_dtype == MTS_F16) launch_stage<mts_f16_t, mts_f16_t>(src, dst, grid, R, C, transpose, s);
+    else if (src_dtype == MTS_F16 && dst_dtype == MTS_F32) launch_stage<mts_f16_t, float>(src, dst, grid, R, C, transpose, s);
     else return MTS_ERR_DTYPE;
     MTS_CHECK_LAUNCH();
     return MTS_OK;

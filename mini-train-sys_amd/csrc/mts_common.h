@@ -10,6 +10,9 @@ typedef __bf16 bf16_t;
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef _Float16 mts_f16_t;
+typedef __attribute__((ext_vector_type(8))) _Float16 mts_f16x8;
+typedef __attribute__((ext_vector_type(4))) _Float16 mts_f16x4;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
@@ -37,6 +40,27 @@ __device__ __forceinline__ uint64_t lanemask_lt() {
 }
 
 static inline bool mts_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// fp16 instantiation of the grouped GEMMs (mts_gemm_f16.hip); the public entry points forward to it
+extern "C" {
+int mts_moe_fwd_gateup_swiglu_f16(const void* x, const void* w1, const int32_t* x_gather, const int32_t* expert_start,
+                                  int64_t T, int K, int E, int H, int I, int act_dtype, void* pre_act, void* post_act,
+                                  void* stream);
+int mts_moe_fwd_down_f16(const void* post_act, const void* w2, const int32_t* expert_start, int64_t TK, int E, int H,
+                         int I, int act_dtype, void* y, void* stream);
+int mts_moe_bwd_dy1_f16(const void* d_out, const void* w2, int w2_as_stored, const void* pre_act, const void* weights,
+                        const int32_t* x_gather, const int32_t* s_scatter, const int32_t* expert_start, int64_t T,
+                        int K, int E, int H, int I, int act_dtype, void* d_pre_act, void* weighted_act,
+                        float* ds_partial, void* stream);
+int mts_moe_bwd_dx_f16(const void* d_pre_act, const void* w1, int w1_as_stored, const int32_t* expert_start,
+                       int64_t TK, int E, int H, int I, int act_dtype, void* dx_expanded, void* stream);
+int mts_moe_bwd_dw2_f16(const void* d_out, const void* weighted_act, const int32_t* x_gather,
+                        const int32_t* expert_start, int64_t T, int K, int E, int H, int I, int act_dtype,
+                        int grad_dtype, void* d_w2, void* workspace, int64_t workspace_bytes, void* stream);
+int mts_moe_bwd_dw1_f16(const void* d_pre_act, const void* x, const int32_t* x_gather, const int32_t* expert_start,
+                        int64_t T, int K, int E, int H, int I, int act_dtype, int grad_dtype, void* d_w1,
+                        void* workspace, int64_t workspace_bytes, void* stream);
+}
 
 // fp32 GEMM launchers (mts_gemm_f32.hip); epi: 0 plain, 1 SwiGLU, 2 dO*W2 with SwiGLU backward
 int mts_f32_rows(int epi, const float* A, int lda, const int32_t* a_gather, const float* B, int b_rows,

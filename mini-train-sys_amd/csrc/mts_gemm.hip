@@ -29,7 +29,33 @@
 
 #include <stdlib.h>
 
+// This source is compiled twice: as it stands for bf16, and from mts_gemm_f16.hip with
+// MTS_GEMM_F16 defined for fp16 (same tiles and pipelines, the fp16 MFMA, entry points with an
+// _f16 suffix that the bf16 build's entry points forward to).  Below, bf16_t / bf16x8 / bf16x4 are
+// the 16-bit element type of the build.
+#ifdef MTS_GEMM_F16
+#define bf16_t mts_f16_t
+#define bf16x8 mts_f16x8
+#define bf16x4 mts_f16x4
+#define MTS_GEMM_ENTRY(name) name##_f16
+#define MTS_GEMM_DTYPE MTS_F16
+#define MTS_MFMA_32x32x16 __builtin_amdgcn_mfma_f32_32x32x16_f16
+#else
+#define MTS_GEMM_ENTRY(name) name
+#define MTS_GEMM_DTYPE MTS_BF16
+#define MTS_MFMA_32x32x16 __builtin_amdgcn_mfma_f32_32x32x16_bf16
+#endif
+
 namespace {
+
+// fp32 value of a 16-bit element given as the low bits of a word
+__device__ __forceinline__ float elem_bits_to_f32(uint32_t bits16) {
+#ifdef MTS_GEMM_F16
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)bits16);
+#else
+    return bf16_bits_to_f32(bits16);
+#endif
+}
 
 constexpr int BK = 64;                       // k extent of an LDS tile (8 chunks of 8 bf16)
 constexpr uint32_t kInvalid = 0x80000000u;   // buffer offset that is out of range for every operand
@@ -205,8 +231,8 @@ __device__ __forceinline__ void mma_tile(const bf16_t* As, const bf16_t* Bs, int
 #pragma unroll
             for (int nf = 0; nf < T::NF; ++nf)
                 acc[mf][nf] = WEIGHT_FIRST
-                                  ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[cur][nf], a[cur][mf], acc[mf][nf], 0, 0, 0)
-                                  : __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[cur][mf], b[cur][nf], acc[mf][nf], 0, 0, 0);
+                                  ? MTS_MFMA_32x32x16(b[cur][nf], a[cur][mf], acc[mf][nf], 0, 0, 0)
+                                  : MTS_MFMA_32x32x16(a[cur][mf], b[cur][nf], acc[mf][nf], 0, 0, 0);
     }
 }
 
@@ -266,7 +292,7 @@ struct FragPipe {
         for (int mf = 0; mf < T::MF; ++mf) {
 #pragma unroll
             for (int nf = 0; nf < T::NF; ++nf)
-                acc[mf][nf] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[buf][nf], a[mf], acc[mf][nf], 0, 0, 0);
+                acc[mf][nf] = MTS_MFMA_32x32x16(b[buf][nf], a[mf], acc[mf][nf], 0, 0, 0);
             a[mf] = *reinterpret_cast<const bf16x8*>(next + a_off + mf * 32 * ROWLEN + coff);
         }
     }
@@ -443,8 +469,8 @@ __device__ __forceinline__ void rows_epilogue(const RowsParams& p, f32x16 (&acc)
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
                         const uint32_t gw = q < 2 ? gr.x : gr.y, uw = q < 2 ? ur.x : ur.y;
-                        const float g = bf16_bits_to_f32((q & 1) ? gw >> 16 : gw & 0xffffu);
-                        const float u = bf16_bits_to_f32((q & 1) ? uw >> 16 : uw & 0xffffu);
+                        const float g = elem_bits_to_f32((q & 1) ? gw >> 16 : gw & 0xffffu);
+                        const float u = elem_bits_to_f32((q & 1) ? uw >> 16 : uw & 0xffffu);
                         const float a = acc[mf][nf][4 * j + q];
                         const float sig = sigmoidf_(g);
                         const float silu = g * sig;
@@ -1311,7 +1337,7 @@ __global__ __launch_bounds__(T::NT) void dw_gemm_ws_kernel(DwParams p) {
         for (int mf = 0; mf < T::MF; ++mf) {
 #pragma unroll
             for (int nf = 0; nf < T::NF; ++nf)
-                acc[mf][nf] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[mf], fb[buf][nf], acc[mf][nf], 0, 0, 0);
+                acc[mf][nf] = MTS_MFMA_32x32x16(fa[mf], fb[buf][nf], acc[mf][nf], 0, 0, 0);
             fa[mf] = read_frag_tr<T::BM>(next, nks * 16, wm * T::WM + mf * 32);
         }
     };
@@ -1466,7 +1492,7 @@ int64_t dw_chunk_workspace_bytes(int E, int M, int N) {
 
 int launch_dw_any(int kind, DwParams p, int E, int grad_dtype, void* workspace, int64_t workspace_bytes,
                   hipStream_t s) {
-    if (grad_dtype != MTS_BF16 && grad_dtype != MTS_F32) return MTS_ERR_DTYPE;
+    if (grad_dtype != MTS_GEMM_DTYPE && grad_dtype != MTS_F32) return MTS_ERR_DTYPE;
     if (tile_choice(kind) == 2) {
         typedef DwWsLarge T;
         if (workspace) {
@@ -1475,19 +1501,19 @@ int launch_dw_any(int kind, DwParams p, int E, int grad_dtype, void* workspace, 
             p.part = (float*)workspace;
         }
         const dim3 grid = dw_grid<T>(p, E, p.part ? 2 * E : E);
-        if (grad_dtype == MTS_BF16) dw_gemm_ws_kernel<T, bf16_t><<<grid, T::NT, 0, s>>>(p);
+        if (grad_dtype == MTS_GEMM_DTYPE) dw_gemm_ws_kernel<T, bf16_t><<<grid, T::NT, 0, s>>>(p);
         else dw_gemm_ws_kernel<T, float><<<grid, T::NT, 0, s>>>(p);
         if (p.part) {
             MTS_CHECK_LAUNCH();
             const int64_t items = (int64_t)p.tiles_per_expert * (T::BM * T::BN / 4);
             const int64_t want = (items + 255) / 256;   // experts that were not cut leave at once
             const dim3 sum_grid((unsigned)(want < 256 ? want : 256), (unsigned)E);
-            if (grad_dtype == MTS_BF16) dw_chunk_sum_kernel<T::BM, T::BN, bf16_t><<<sum_grid, 256, 0, s>>>(p);
+            if (grad_dtype == MTS_GEMM_DTYPE) dw_chunk_sum_kernel<T::BM, T::BN, bf16_t><<<sum_grid, 256, 0, s>>>(p);
             else dw_chunk_sum_kernel<T::BM, T::BN, float><<<sum_grid, 256, 0, s>>>(p);
         }
     } else {
         const dim3 grid = dw_grid<StagedSmall>(p, E, E);
-        if (grad_dtype == MTS_BF16) dw_gemm_kernel<StagedSmall, bf16_t><<<grid, StagedSmall::NT, 0, s>>>(p);
+        if (grad_dtype == MTS_GEMM_DTYPE) dw_gemm_kernel<StagedSmall, bf16_t><<<grid, StagedSmall::NT, 0, s>>>(p);
         else dw_gemm_kernel<StagedSmall, float><<<grid, StagedSmall::NT, 0, s>>>(p);
     }
     MTS_CHECK_LAUNCH();
@@ -1498,12 +1524,17 @@ int dy1_partials(int I) { return (I + 63) / 64; }
 
 }  // namespace
 
+#ifndef MTS_GEMM_F16
 extern "C" int mts_moe_ds_partials(int I) { return dy1_partials(I); }
+#endif
 
-extern "C" int mts_moe_fwd_gateup_swiglu(const void* x, const void* w1, const int32_t* x_gather,
+extern "C" int MTS_GEMM_ENTRY(mts_moe_fwd_gateup_swiglu)(const void* x, const void* w1, const int32_t* x_gather,
                                          const int32_t* expert_start, int64_t T, int K, int E,
                                          int H, int I, int act_dtype, void* pre_act,
                                          void* post_act, void* stream) {
+#ifndef MTS_GEMM_F16
+    if (act_dtype == MTS_F16) return mts_moe_fwd_gateup_swiglu_f16(x, w1, x_gather, expert_start, T, K, E, H, I, act_dtype, pre_act, post_act, stream);
+#endif
     if (!x || !w1 || !x_gather || !expert_start || !pre_act || !post_act) return MTS_ERR_NULL;
     if (T <= 0 || K < 1) return MTS_ERR_SHAPE;
     if (act_dtype == MTS_F32) {
@@ -1512,7 +1543,7 @@ extern "C" int mts_moe_fwd_gateup_swiglu(const void* x, const void* w1, const in
                             (float*)pre_act, (float*)post_act, nullptr, nullptr, nullptr, nullptr, 0,
                             (hipStream_t)stream);
     }
-    if (act_dtype != MTS_BF16) return MTS_ERR_DTYPE;
+    if (act_dtype != MTS_GEMM_DTYPE) return MTS_ERR_DTYPE;
     int rc = check_common(T * K, E, H, I);
     if (rc) return rc;
     if (!mts_aligned16(x) || !mts_aligned16(w1)) return MTS_ERR_ALIGN;
@@ -1524,16 +1555,19 @@ extern "C" int mts_moe_fwd_gateup_swiglu(const void* x, const void* w1, const in
     return launch_rows_any<EPI_SWIGLU>(K_GATEUP, p, T * K, (hipStream_t)stream);
 }
 
-extern "C" int mts_moe_fwd_down(const void* post_act, const void* w2, const int32_t* expert_start,
+extern "C" int MTS_GEMM_ENTRY(mts_moe_fwd_down)(const void* post_act, const void* w2, const int32_t* expert_start,
                                 int64_t TK, int E, int H, int I, int act_dtype, void* y,
                                 void* stream) {
+#ifndef MTS_GEMM_F16
+    if (act_dtype == MTS_F16) return mts_moe_fwd_down_f16(post_act, w2, expert_start, TK, E, H, I, act_dtype, y, stream);
+#endif
     if (!post_act || !w2 || !expert_start || !y) return MTS_ERR_NULL;
     if (act_dtype == MTS_F32) {
         if (TK <= 0 || TK > 0x7fffffffLL || E < 1 || E > MTS_MAX_EXPERTS || H < 1 || I < 1) return MTS_ERR_SHAPE;
         return mts_f32_rows(0, (const float*)post_act, I, nullptr, (const float*)w2, H, H, I, expert_start, E, TK,
                             (float*)y, nullptr, nullptr, nullptr, nullptr, nullptr, 0, (hipStream_t)stream);
     }
-    if (act_dtype != MTS_BF16) return MTS_ERR_DTYPE;
+    if (act_dtype != MTS_GEMM_DTYPE) return MTS_ERR_DTYPE;
     int rc = check_common(TK, E, H, I);
     if (rc) return rc;
     if (!mts_aligned16(post_act) || !mts_aligned16(w2)) return MTS_ERR_ALIGN;
@@ -1545,15 +1579,20 @@ extern "C" int mts_moe_fwd_down(const void* post_act, const void* w2, const int3
     return launch_rows_any<EPI_PLAIN>(K_DOWN, p, TK, (hipStream_t)stream);
 }
 
+#ifndef MTS_GEMM_F16
 extern "C" int mts_moe_bwd_weights_as_stored(int act_dtype, int H, int I) {
-    return act_dtype == MTS_BF16 && rows_kmajor_ok(K_DY1, H) && rows_kmajor_ok(K_DX, 2 * I) ? 1 : 0;
+    return (act_dtype == MTS_BF16 || act_dtype == MTS_F16) && rows_kmajor_ok(K_DY1, H) && rows_kmajor_ok(K_DX, 2 * I) ? 1 : 0;
 }
+#endif
 
-extern "C" int mts_moe_bwd_dy1(const void* d_out, const void* w2t, int w2_as_stored, const void* pre_act,
+extern "C" int MTS_GEMM_ENTRY(mts_moe_bwd_dy1)(const void* d_out, const void* w2t, int w2_as_stored, const void* pre_act,
                                const void* weights, const int32_t* x_gather,
                                const int32_t* s_scatter, const int32_t* expert_start, int64_t T,
                                int K, int E, int H, int I, int act_dtype, void* d_pre_act,
                                void* weighted_act, float* ds_partial, void* stream) {
+#ifndef MTS_GEMM_F16
+    if (act_dtype == MTS_F16) return mts_moe_bwd_dy1_f16(d_out, w2t, w2_as_stored, pre_act, weights, x_gather, s_scatter, expert_start, T, K, E, H, I, act_dtype, d_pre_act, weighted_act, ds_partial, stream);
+#endif
     if (!d_out || !w2t || !pre_act || !weights || !x_gather || !s_scatter || !expert_start ||
         !d_pre_act || !weighted_act || !ds_partial)
         return MTS_ERR_NULL;
@@ -1564,7 +1603,7 @@ extern "C" int mts_moe_bwd_dy1(const void* d_out, const void* w2t, int w2_as_sto
                             (float*)d_pre_act, (float*)weighted_act, (const float*)pre_act, (const float*)weights,
                             s_scatter, ds_partial, mts_moe_ds_partials(I), (hipStream_t)stream);
     }
-    if (act_dtype != MTS_BF16) return MTS_ERR_DTYPE;
+    if (act_dtype != MTS_GEMM_DTYPE) return MTS_ERR_DTYPE;
     int rc = check_common(T * K, E, H, I);
     if (rc) return rc;
     if (!mts_aligned16(d_out) || !mts_aligned16(w2t)) return MTS_ERR_ALIGN;
@@ -1578,9 +1617,12 @@ extern "C" int mts_moe_bwd_dy1(const void* d_out, const void* w2t, int w2_as_sto
     return launch_rows_any<EPI_DY1>(K_DY1, p, T * K, (hipStream_t)stream, w2_as_stored != 0);
 }
 
-extern "C" int mts_moe_bwd_dx(const void* d_pre_act, const void* w1t, int w1_as_stored,
+extern "C" int MTS_GEMM_ENTRY(mts_moe_bwd_dx)(const void* d_pre_act, const void* w1t, int w1_as_stored,
                               const int32_t* expert_start, int64_t TK, int E, int H, int I, int act_dtype,
                               void* dx_expanded, void* stream) {
+#ifndef MTS_GEMM_F16
+    if (act_dtype == MTS_F16) return mts_moe_bwd_dx_f16(d_pre_act, w1t, w1_as_stored, expert_start, TK, E, H, I, act_dtype, dx_expanded, stream);
+#endif
     if (!d_pre_act || !w1t || !expert_start || !dx_expanded) return MTS_ERR_NULL;
     if (act_dtype == MTS_F32) {
         if (TK <= 0 || TK > 0x7fffffffLL || E < 1 || E > MTS_MAX_EXPERTS || H < 1 || I < 1 || w1_as_stored) return MTS_ERR_SHAPE;
@@ -1588,7 +1630,7 @@ extern "C" int mts_moe_bwd_dx(const void* d_pre_act, const void* w1t, int w1_as_
                             TK, (float*)dx_expanded, nullptr, nullptr, nullptr, nullptr, nullptr, 0,
                             (hipStream_t)stream);
     }
-    if (act_dtype != MTS_BF16) return MTS_ERR_DTYPE;
+    if (act_dtype != MTS_GEMM_DTYPE) return MTS_ERR_DTYPE;
     int rc = check_common(TK, E, H, I);
     if (rc) return rc;
     if (!mts_aligned16(d_pre_act) || !mts_aligned16(w1t)) return MTS_ERR_ALIGN;
@@ -1600,15 +1642,20 @@ extern "C" int mts_moe_bwd_dx(const void* d_pre_act, const void* w1t, int w1_as_
     return launch_rows_any<EPI_PLAIN>(K_DX, p, TK, (hipStream_t)stream, w1_as_stored != 0);
 }
 
+#ifndef MTS_GEMM_F16
 extern "C" int64_t mts_moe_bwd_dw_workspace_bytes(int which, int E, int H, int I) {
     if (E < 1 || H < 1 || I < 1 || (which != 1 && which != 2)) return 0;
     return which == 1 ? dw_chunk_workspace_bytes(E, 2 * I, H) : dw_chunk_workspace_bytes(E, H, I);
 }
+#endif
 
-extern "C" int mts_moe_bwd_dw2(const void* d_out, const void* weighted_act, const int32_t* x_gather,
+extern "C" int MTS_GEMM_ENTRY(mts_moe_bwd_dw2)(const void* d_out, const void* weighted_act, const int32_t* x_gather,
                                const int32_t* expert_start, int64_t T, int K, int E, int H, int I,
                                int act_dtype, int grad_dtype, void* d_w2, void* workspace,
                                int64_t workspace_bytes, void* stream) {
+#ifndef MTS_GEMM_F16
+    if (act_dtype == MTS_F16) return mts_moe_bwd_dw2_f16(d_out, weighted_act, x_gather, expert_start, T, K, E, H, I, act_dtype, grad_dtype, d_w2, workspace, workspace_bytes, stream);
+#endif
     if (!d_out || !weighted_act || !x_gather || !expert_start || !d_w2) return MTS_ERR_NULL;
     if (T <= 0 || K < 1) return MTS_ERR_SHAPE;
     if (act_dtype == MTS_F32) {
@@ -1616,7 +1663,7 @@ extern "C" int mts_moe_bwd_dw2(const void* d_out, const void* weighted_act, cons
         return mts_f32_dw((const float*)d_out, x_gather, (const float*)weighted_act, nullptr, H, I, expert_start, E,
                           grad_dtype, d_w2, (hipStream_t)stream);
     }
-    if (act_dtype != MTS_BF16) return MTS_ERR_DTYPE;
+    if (act_dtype != MTS_GEMM_DTYPE) return MTS_ERR_DTYPE;
     int rc = check_common(T * K, E, H, I);
     if (rc) return rc;
     if (!mts_aligned16(d_out) || !mts_aligned16(weighted_act)) return MTS_ERR_ALIGN;
@@ -1627,10 +1674,13 @@ extern "C" int mts_moe_bwd_dw2(const void* d_out, const void* weighted_act, cons
     return launch_dw_any(K_DW2, p, E, grad_dtype, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
-extern "C" int mts_moe_bwd_dw1(const void* d_pre_act, const void* x, const int32_t* x_gather,
+extern "C" int MTS_GEMM_ENTRY(mts_moe_bwd_dw1)(const void* d_pre_act, const void* x, const int32_t* x_gather,
                                const int32_t* expert_start, int64_t T, int K, int E, int H, int I,
                                int act_dtype, int grad_dtype, void* d_w1, void* workspace,
                                int64_t workspace_bytes, void* stream) {
+#ifndef MTS_GEMM_F16
+    if (act_dtype == MTS_F16) return mts_moe_bwd_dw1_f16(d_pre_act, x, x_gather, expert_start, T, K, E, H, I, act_dtype, grad_dtype, d_w1, workspace, workspace_bytes, stream);
+#endif
     if (!d_pre_act || !x || !x_gather || !expert_start || !d_w1) return MTS_ERR_NULL;
     if (T <= 0 || K < 1) return MTS_ERR_SHAPE;
     if (act_dtype == MTS_F32) {
@@ -1638,7 +1688,7 @@ extern "C" int mts_moe_bwd_dw1(const void* d_pre_act, const void* x, const int32
         return mts_f32_dw((const float*)d_pre_act, nullptr, (const float*)x, x_gather, 2 * I, H, expert_start, E,
                           grad_dtype, d_w1, (hipStream_t)stream);
     }
-    if (act_dtype != MTS_BF16) return MTS_ERR_DTYPE;
+    if (act_dtype != MTS_GEMM_DTYPE) return MTS_ERR_DTYPE;
     int rc = check_common(T * K, E, H, I);
     if (rc) return rc;
     if (!mts_aligned16(d_pre_act) || !mts_aligned16(x)) return MTS_ERR_ALIGN;

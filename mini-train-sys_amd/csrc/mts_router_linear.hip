@@ -15,10 +15,19 @@ __device__ __forceinline__ f32x4 load4(const bf16_t* p) {
     f32x4 r = {(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
     return r;
 }
+__device__ __forceinline__ f32x4 load4(const mts_f16_t* p) {
+    const mts_f16x4 v = *reinterpret_cast<const mts_f16x4*>(p);
+    f32x4 r = {(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
+    return r;
+}
 __device__ __forceinline__ f32x4 load4(const float* p) { return *reinterpret_cast<const f32x4*>(p); }
 __device__ __forceinline__ void store4(bf16_t* p, f32x4 v) {
     bf16x4 o = {(bf16_t)v[0], (bf16_t)v[1], (bf16_t)v[2], (bf16_t)v[3]};
     *reinterpret_cast<bf16x4*>(p) = o;
+}
+__device__ __forceinline__ void store4(mts_f16_t* p, f32x4 v) {
+    mts_f16x4 o = {(mts_f16_t)v[0], (mts_f16_t)v[1], (mts_f16_t)v[2], (mts_f16_t)v[3]};
+    *reinterpret_cast<mts_f16x4*>(p) = o;
 }
 __device__ __forceinline__ void store4(float* p, f32x4 v) { *reinterpret_cast<f32x4*>(p) = v; }
 
@@ -29,12 +38,21 @@ struct RawVec<bf16_t> {
     typedef bf16x4 type;
 };
 template <>
+struct RawVec<mts_f16_t> {
+    typedef mts_f16x4 type;
+};
+template <>
 struct RawVec<float> {
     typedef f32x4 type;
 };
 __device__ __forceinline__ bf16x4 load_raw(const bf16_t* p) { return *reinterpret_cast<const bf16x4*>(p); }
+__device__ __forceinline__ mts_f16x4 load_raw(const mts_f16_t* p) { return *reinterpret_cast<const mts_f16x4*>(p); }
 __device__ __forceinline__ f32x4 load_raw(const float* p) { return *reinterpret_cast<const f32x4*>(p); }
 __device__ __forceinline__ f32x4 widen(bf16x4 v) {
+    f32x4 r = {(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
+    return r;
+}
+__device__ __forceinline__ f32x4 widen(mts_f16x4 v) {
     f32x4 r = {(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
     return r;
 }
@@ -281,7 +299,7 @@ constexpr int kBwdBlocks = 1024;
 int check(const void* x, const float* w, int64_t T, int H, int E, int act_dtype) {
     if (!x || !w) return MTS_ERR_NULL;
     if (T <= 0 || E < 1 || E > kMaxE || H < 4 || H % 4 || H > kMaxH) return MTS_ERR_SHAPE;
-    if (act_dtype != MTS_BF16 && act_dtype != MTS_F32) return MTS_ERR_DTYPE;
+    if (act_dtype != MTS_BF16 && act_dtype != MTS_F16 && act_dtype != MTS_F32) return MTS_ERR_DTYPE;
     if (!mts_aligned16(w) || (reinterpret_cast<uintptr_t>(x) & 15u)) return MTS_ERR_ALIGN;
     return MTS_OK;
 }
@@ -314,6 +332,9 @@ extern "C" int mts_router_logits_fwd(const void* x, const float* w_r, int64_t T,
     if (act_dtype == MTS_BF16) {
         if (E <= 8) MTS_FWD_PASSES(bf16_t, 8);
         else MTS_FWD_PASSES(bf16_t, 16);
+    } else if (act_dtype == MTS_F16) {
+        if (E <= 8) MTS_FWD_PASSES(mts_f16_t, 8);
+        else MTS_FWD_PASSES(mts_f16_t, 16);
     } else {
         if (E <= 8) MTS_FWD_PASSES(float, 8);
         else MTS_FWD_PASSES(float, 16);
@@ -360,6 +381,9 @@ extern "C" int mts_router_logits_bwd(const float* dlogits, const void* x, const 
     if (act_dtype == MTS_BF16) {
         if (E <= 8) MTS_BWD(bf16_t, 8);
         else MTS_BWD(bf16_t, 16);
+    } else if (act_dtype == MTS_F16) {
+        if (E <= 8) MTS_BWD(mts_f16_t, 8);
+        else MTS_BWD(mts_f16_t, 16);
     } else {
         if (E <= 8) MTS_BWD(float, 8);
         else MTS_BWD(float, 16);

@@ -18,6 +18,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libmts_moe.so")
 
 MTS_BF16 = 0
 MTS_F32 = 1
+MTS_F16 = 2
 
 _c = ctypes
 _p = _c.c_void_p
@@ -100,4 +101,6 @@ def dtype_code(dt) -> int:
         return MTS_BF16
     if dt == torch.float32:
         return MTS_F32
+    if dt == torch.float16:
+        return MTS_F16
     raise MtsError(f"unsupported dtype {dt}")

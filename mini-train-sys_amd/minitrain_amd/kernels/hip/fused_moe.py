@@ -41,7 +41,9 @@ def is_fused_moe_supported(x, gate_up_proj, down_proj, top_k_index, top_k_weight
     tokens, hidden = x.shape
     experts, twice_intermediate, weight_hidden = gate_up_proj.shape
     intermediate = twice_intermediate // 2
-    weight_dtypes = (torch.bfloat16, torch.float32)
+    # expert parameters come in the activation dtype or as fp32 master weights; fp32 activations
+    # take 16-bit parameters as well (widened once per call)
+    weight_dtypes = (x.dtype, torch.float32) if x.dtype != torch.float32 else (torch.float32, torch.bfloat16, torch.float16)
     return (
         tokens > 0
         and 0 < experts <= _MAX_EXPERTS
@@ -53,10 +55,10 @@ def is_fused_moe_supported(x, gate_up_proj, down_proj, top_k_index, top_k_weight
         and tokens * top_k_index.shape[1] < 2**31
         and top_k_index.dtype == torch.int32
         and top_k_weights.dtype == x.dtype
-        and x.dtype in (torch.bfloat16, torch.float32)
+        and x.dtype in (torch.bfloat16, torch.float16, torch.float32)
         and gate_up_proj.dtype in weight_dtypes
         and down_proj.dtype in weight_dtypes
-        and hidden % (8 if x.dtype == torch.bfloat16 else 4) == 0
+        and hidden % (4 if x.dtype == torch.float32 else 8) == 0
         and (intermediate % 8 == 0 or x.dtype == torch.float32)
     )
 
@@ -149,7 +151,7 @@ _DW_WORKSPACE_LIMIT = 512 * 2**20
 
 
 def _dw_workspace(lib, which: int, E: int, H: int, I: int, dtype: torch.dtype, device):
-    nbytes = lib.mts_moe_bwd_dw_workspace_bytes(which, E, H, I) if dtype == torch.bfloat16 else 0
+    nbytes = lib.mts_moe_bwd_dw_workspace_bytes(which, E, H, I) if dtype != torch.float32 else 0
     if nbytes <= 0 or nbytes > _DW_WORKSPACE_LIMIT:
         return None, 0, 0
     ws = torch.empty(nbytes, dtype=torch.uint8, device=device)

@@ -120,7 +120,7 @@ def is_router_logits_supported(hidden_states: torch.Tensor, weight: torch.Tensor
         and weight.is_cuda
         and hidden_states.ndim == 2
         and weight.ndim == 2
-        and hidden_states.dtype in (torch.bfloat16, torch.float32)
+        and hidden_states.dtype in (torch.bfloat16, torch.float16, torch.float32)
         and weight.dtype == torch.float32
         and hidden_states.shape[0] > 0
         and hidden_states.shape[1] == weight.shape[1]

@@ -34,6 +34,21 @@ def test_small_shapes(T, H, E, I, K):
     _compare(routed_case(10 + T, T, H, E, I, K))
 
 
+@pytest.mark.parametrize("T,H,E,I,K", [(256, 64, 4, 128, 2), (700, 72, 3, 40, 2), (2048, 768, 8, 1024, 2)])
+def test_fp16_activations(T, H, E, I, K):
+    """fp16 is the third activation dtype of the reference's contract (fused_moe.py:37-71)."""
+    print(f"moe fp16 T={T} H={H} E={E} I={I} K={K}", flush=True)
+    _compare(routed_case(60 + T, T, H, E, I, K, dtype=torch.float16))
+
+
+def test_fp16_activations_fp32_master_weights():
+    print("moe fp16 with fp32 weights", flush=True)
+    case = routed_case(61, 300, 128, 4, 192, 2, dtype=torch.float16)
+    _, w_r, w1, w2, _ = O.make_inputs(61, 300, 128, 4, 192)
+    case.update(w1=w1, w2=w2)
+    _compare(case)
+
+
 def test_reference_edge_probe():
     """T=33, K=3, only experts {0,1} of 8 used, repeated experts inside a token and
     zero weights on [::2, -1]; zero-weight routes must still receive a gradient."""
