@@ -40,6 +40,35 @@ def test_library_exports_every_declared_symbol():
     assert lib.mts_moe_ds_partials(1024) > 0
 
 
+def test_contract_violations_are_reported_before_any_launch():
+    """Argument checks of the newer entry points run on the host: every call here returns a negative
+    MTS_ERR_* code without touching a GPU."""
+    from minitrain_amd import _lib
+
+    lib = _lib.load()
+    NULL, SHAPE, WORKSPACE = -1, -2, -4
+    fake = 4096   # any non-null, 16-byte aligned value: nothing is dereferenced before the checks fail
+    # capacity mask: required pointers, expert limit, workspace size
+    assert lib.mts_moe_capacity_mask(None, fake, 8, 2, 4, 3, fake, None, fake, fake, 1 << 20, None) == NULL
+    assert lib.mts_moe_capacity_mask(fake, fake, 8, 2, 4096, 3, fake, None, fake, fake, 1 << 20, None) == SHAPE
+    assert lib.mts_moe_capacity_mask(fake, fake, 8, 2, 4, 3, fake, None, fake, fake, 16, None) == WORKSPACE
+    assert lib.mts_moe_capacity_workspace_bytes(24576, 2, 8) >= 4 * 49152 * 4
+    # weight layout of the backward GEMMs
+    assert lib.mts_moe_bwd_weights_as_stored(_lib.MTS_BF16, 768, 1024) == 1
+    assert lib.mts_moe_bwd_weights_as_stored(_lib.MTS_F16, 768, 1024) == 1
+    assert lib.mts_moe_bwd_weights_as_stored(_lib.MTS_F32, 768, 1024) == 0      # fp32 path reads transposed copies
+    assert lib.mts_moe_bwd_weights_as_stored(_lib.MTS_BF16, 72, 40) == 0        # no whole 64-wide k-tiles
+    assert lib.mts_moe_bwd_dx(fake, fake, 1, fake, 512, 4, 64, 128, _lib.MTS_F32, fake, None) == SHAPE
+    assert lib.mts_moe_bwd_dx(fake, fake, 1, fake, 512, 4, 72, 40, _lib.MTS_BF16, fake, None) == SHAPE
+    # row-chunk workspace of the weight-gradient GEMMs: 2E slots of 256x256 fp32 tiles
+    assert lib.mts_moe_bwd_dw_workspace_bytes(1, 8, 768, 1024) == 2 * 8 * (8 * 3) * 256 * 256 * 4
+    assert lib.mts_moe_bwd_dw_workspace_bytes(2, 8, 768, 1024) == 2 * 8 * (3 * 4) * 256 * 256 * 4
+    assert lib.mts_moe_bwd_dw1(fake, fake, fake, fake, 256, 2, 4, 64, 128, _lib.MTS_BF16, _lib.MTS_BF16, fake, fake, 16,
+                               None) == WORKSPACE
+    # unknown element type
+    assert lib.mts_moe_combine(fake, None, fake, 8, 2, 64, 7, fake, None) == -3
+
+
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     from minitrain_amd import _lib
 

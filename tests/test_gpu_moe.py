@@ -49,6 +49,30 @@ def test_fp16_activations_fp32_master_weights():
     _compare(case)
 
 
+def _drawn_shapes(n, seed):
+    rng = np.random.Generator(np.random.Philox(seed))
+    out = []
+    for i in range(n):
+        E = int(rng.integers(1, 17))
+        K = int(rng.integers(1, min(E, 4) + 1))
+        # every other draw has whole 64-wide k-tiles (ring / specialised kernels, weights read as stored),
+        # the others take the staged kernels with transposed copies
+        step = 64 if i % 2 == 0 else 8
+        H = int(rng.integers(1, 5)) * step if step == 64 else int(rng.integers(2, 33)) * 8
+        I = int(rng.integers(1, 5)) * (32 if step == 64 else 8)
+        T = int(rng.integers(1, 700))
+        dtype = (torch.bfloat16, torch.float16)[int(rng.integers(0, 2))]
+        out.append((T, H, E, I, K, dtype))
+    return out
+
+
+@pytest.mark.parametrize("T,H,E,I,K,dtype", _drawn_shapes(14, seed=2024))
+def test_drawn_shapes(T, H, E, I, K, dtype):
+    """Seeded draws over token counts, widths, expert counts and top-k, in both 16-bit dtypes."""
+    print(f"moe drawn T={T} H={H} E={E} I={I} K={K} {dtype}", flush=True)
+    _compare(routed_case(T + H + E, T, H, E, I, K, dtype=dtype))
+
+
 def test_reference_edge_probe():
     """T=33, K=3, only experts {0,1} of 8 used, repeated experts inside a token and
     zero weights on [::2, -1]; zero-weight routes must still receive a gradient."""
