@@ -41,8 +41,8 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # two rocprofv3 counter runs summarised in profiles/moe_layer_24x1024_hbm_traffic.txt (FETCH_SIZE
 # scaled by 2.0, WRITE_SIZE by 1.0 against a plain copy kernel of known size).  Not measured live.
 MEASURED_TRAFFIC_BYTES = {
-    "fwd_gateup_swiglu": 776.5e6, "fwd_down": 303.4e6, "bwd_dx": 533.9e6, "bwd_dy1": 708.7e6,
-    "bwd_dw2": 189.5e6, "bwd_dw1": 302.7e6, "combine": 115.2e6, "dx_combine": 114.4e6,
+    "fwd_gateup_swiglu": 781.3e6, "fwd_down": 303.4e6, "bwd_dy1": 708.7e6, "bwd_joint": 1115.7e6,
+    "combine": 115.2e6, "dx_combine": 114.4e6,
 }
 
 WORKLOAD = dict(name="moe_layer_24x1024_d768_e8_top2_ff1024_bf16", seed=1, T=24576, H=768, E=8, K=2, I=1024)
@@ -158,12 +158,12 @@ def stage_breakdown(layer, steps):
          lambda: lib.mts_moe_combine(p(y), p(wts), p(sr), T, K, H, B, p(out), st)),
         ("bwd_dy1", "mfma", gemm(1),
          lambda: lib.mts_moe_bwd_dy1(p(g), p(w2), 1, p(pre), p(wts), p(xg), p(ss), p(es), T, K, E, H, I, B, p(dpre), p(wact), p(dsp), st)),
-        ("bwd_ds", "hbm", TK * npart * 4 + TK * 4 + TK * esz, lambda: lib.mts_moe_bwd_ds(p(dsp), p(sr), TK, I, B, p(dwts), st)),
-        ("bwd_dw2", "mfma", gemm(1), lambda: lib.mts_moe_bwd_dw2(p(g), p(wact), p(xg), p(es), T, K, E, H, I, B, B, p(dw2), p(dws2), dws2.numel(), st)),
-        ("bwd_dx", "mfma", gemm(2), lambda: lib.mts_moe_bwd_dx(p(dpre), p(w1), 1, p(es), TK, E, H, I, B, p(dxe), st)),
+        # dW1, dW2, dX and the dS reduction: one launch (plus the chunk sum), as the operator issues them
+        ("bwd_joint", "mfma", gemm(5),
+         lambda: lib.mts_moe_bwd_joint(p(g), p(wact), p(dpre), p(x), p(w1), p(xg), p(es), p(sr), p(dsp), T, K, E, H, I, B, B,
+                                       p(dxe), p(dw1), p(dw2), p(dwts), p(dws1), dws1.numel(), p(dws2), dws2.numel(), st)),
         ("dx_combine", "hbm", TK * H * esz + T * H * esz + TK * 4,
          lambda: lib.mts_moe_combine(p(dxe), None, p(sr), T, K, H, B, p(dx), st)),
-        ("bwd_dw1", "mfma", gemm(2), lambda: lib.mts_moe_bwd_dw1(p(dpre), p(x), p(xg), p(es), T, K, E, H, I, B, B, p(dw1), p(dws1), dws1.numel(), st)),
         ("router_bwd", "hbm", T * E * 4 * 2 + T * K * 12,
          lambda: lib.mts_router_bwd(p(logits), p(r_w), p(r_i), p(gw), p(gp), p(gz), p(gz), p(cnt), T, E, K, 1, p(dlog), st)),
         ("router_logits_bwd", "hbm", 2 * T * H * esz + T * E * 4 + 2 * E * H * 4,
@@ -227,8 +227,8 @@ def cpu_baseline(budget_s=20.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-breakdown", action="store_true")
     ap.add_argument("--copy-probe", action="store_true",

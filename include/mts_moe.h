@@ -217,6 +217,25 @@ int mts_moe_bwd_dw1(const void* d_pre_act, const void* x, const int32_t* x_gathe
                     int act_dtype, int grad_dtype, void* d_w1, void* workspace,
                     int64_t workspace_bytes, void* stream);
 
+/* Replaces the three launches that follow _moe_bwd_down_proj_kernel in
+ * _FusedMoEFunction.backward (fused_moe.py:351-443: _moe_bwd_dW2_kernel,
+ * _moe_bwd_dX_expanded_kernel, _moe_bwd_dW1_kernel) and the dS reduction with ONE launch
+ * plus the chunk sum: the same arithmetic, block for block, as mts_moe_bwd_dw1,
+ * mts_moe_bwd_dw2, mts_moe_bwd_dx (w1 as stored, [E,2I,H]) and mts_moe_bwd_ds, so the
+ * results are bit-identical to those calls.  The block index orders the work: the
+ * weight-gradient tiles, which are the long ones, start first and the dX tiles fill the
+ * CUs as they come free.  mts_moe_bwd_joint_supported() says whether the shapes allow it
+ * (16-bit activations, 2I a multiple of 64); both weight gradients have grad_dtype.
+ * workspace1 / workspace2: as for mts_moe_bwd_dw1 / mts_moe_bwd_dw2 (may be NULL).     */
+int mts_moe_bwd_joint_supported(int act_dtype, int H, int I);
+int mts_moe_bwd_joint(const void* d_out, const void* weighted_act, const void* d_pre_act,
+                      const void* x, const void* w1, const int32_t* x_gather,
+                      const int32_t* expert_start, const int32_t* s_reverse,
+                      const float* ds_partial, int64_t T, int K, int E, int H, int I,
+                      int act_dtype, int grad_dtype, void* dx_expanded, void* d_w1, void* d_w2,
+                      void* d_weights, void* workspace1, int64_t workspace1_bytes,
+                      void* workspace2, int64_t workspace2_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

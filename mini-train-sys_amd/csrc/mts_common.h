@@ -60,6 +60,12 @@ int mts_moe_bwd_dw2_f16(const void* d_out, const void* weighted_act, const int32
 int mts_moe_bwd_dw1_f16(const void* d_pre_act, const void* x, const int32_t* x_gather, const int32_t* expert_start,
                         int64_t T, int K, int E, int H, int I, int act_dtype, int grad_dtype, void* d_w1,
                         void* workspace, int64_t workspace_bytes, void* stream);
+int mts_moe_bwd_joint_f16(const void* d_out, const void* weighted_act, const void* d_pre_act, const void* x,
+                          const void* w1, const int32_t* x_gather, const int32_t* expert_start,
+                          const int32_t* s_reverse, const float* ds_partial, int64_t T, int K, int E, int H, int I,
+                          int act_dtype, int grad_dtype, void* dx_expanded, void* d_w1, void* d_w2, void* d_weights,
+                          void* workspace1, int64_t workspace1_bytes, void* workspace2, int64_t workspace2_bytes,
+                          void* stream);
 }
 
 // fp32 GEMM launchers (mts_gemm_f32.hip); epi: 0 plain, 1 SwiGLU, 2 dO*W2 with SwiGLU backward

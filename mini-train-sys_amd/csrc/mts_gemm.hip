@@ -516,8 +516,7 @@ constexpr int kXcds = 8;
 // ballot picks the first expert whose offset range contains the tile (63 experts per
 // round; more experts take more rounds).
 template <int BM>
-__device__ __forceinline__ bool locate_rows_tile(const RowsParams& p, int& e, int& row0, int& rend, int& ntile) {
-    const int b = blockIdx.x;
+__device__ __forceinline__ bool locate_rows_tile(const RowsParams& p, int b, int& e, int& row0, int& rend, int& ntile) {
     const int xcd = b % kXcds, j = b / kXcds;
     const int tile = xcd + kXcds * (j / p.n_tiles);
     ntile = j % p.n_tiles;
@@ -559,7 +558,7 @@ __global__ __launch_bounds__(T::NT) void rows_gemm_kernel(RowsParams p) {
     constexpr bool SWIGLU = (EPI == EPI_SWIGLU);
 
     int e, row0, rend, ntile;
-    if (!locate_rows_tile<T::BM>(p, e, row0, rend, ntile)) return;
+    if (!locate_rows_tile<T::BM>(p, blockIdx.x, e, row0, rend, ntile)) return;
     const int n0 = ntile * (SWIGLU ? T::BN / 2 : T::BN);  // first output column of this block
 
     KMajorLoader<T::BM, T::NT> la;
@@ -672,7 +671,7 @@ __global__ __launch_bounds__(T::NT, T::WAVES_PER_EU) void rows_gemm_ring_kernel(
     constexpr int S = T::STAGES, L = T::A_INSTR + T::B_INSTR;
 
     int e, row0, rend, ntile;
-    if (!locate_rows_tile<T::BM>(p, e, row0, rend, ntile)) return;
+    if (!locate_rows_tile<T::BM>(p, blockIdx.x, e, row0, rend, ntile)) return;
     const int n0 = ntile * (SWIGLU ? T::BN / 2 : T::BN);
     const int wave = threadIdx.x / MTS_WAVE, lane = threadIdx.x % MTS_WAVE;
     const int wm = wave / T::WAVES_N, wn = wave % T::WAVES_N;
@@ -792,16 +791,19 @@ struct WsTile {
     static_assert(LDS_ELEMS * 2 <= 160 * 1024, "LDS capacity");
 };
 
-template <class T, int EPI, bool BKM = false>
-__global__ __launch_bounds__(T::NT, T::WAVES_PER_EU) void rows_gemm_ws_kernel(RowsParams p) {
-    constexpr int LDS_ELEMS = T::LDS_ELEMS > EpiShape<T, EPI>::ELEMS ? T::LDS_ELEMS : EpiShape<T, EPI>::ELEMS;
-    static_assert(LDS_ELEMS * 2 <= 160 * 1024, "LDS capacity");
-    __shared__ __attribute__((aligned(1024))) bf16_t smem[LDS_ELEMS];
+template <class T, int EPI>
+constexpr int ws_lds_elems() {
+    return T::LDS_ELEMS > EpiShape<T, EPI>::ELEMS ? T::LDS_ELEMS : EpiShape<T, EPI>::ELEMS;
+}
+
+// the work of block `block` of a launch; `smem` holds ws_lds_elems<T, EPI>() elements, 1 KiB aligned
+template <class T, int EPI, bool BKM>
+__device__ __forceinline__ void rows_gemm_ws_block(const RowsParams& p, bf16_t* smem, int block) {
     constexpr bool SWIGLU = (EPI == EPI_SWIGLU);
     constexpr int S = T::STAGES, L = T::A_INSTR + T::B_INSTR;
 
     int e, row0, rend, ntile;
-    if (!locate_rows_tile<T::BM>(p, e, row0, rend, ntile)) return;
+    if (!locate_rows_tile<T::BM>(p, block, e, row0, rend, ntile)) return;
     const int n0 = ntile * (SWIGLU ? T::BN / 2 : T::BN);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / MTS_WAVE), lane = threadIdx.x % MTS_WAVE;
     const int nk = p.Kdim / T::BKS;
@@ -902,6 +904,13 @@ __global__ __launch_bounds__(T::NT, T::WAVES_PER_EU) void rows_gemm_ws_kernel(Ro
     rows_epilogue<T, EPI>(p, acc, smem, row0, rend, n0, wm, wn);
 }
 
+template <class T, int EPI, bool BKM = false>
+__global__ __launch_bounds__(T::NT, T::WAVES_PER_EU) void rows_gemm_ws_kernel(RowsParams p) {
+    static_assert(ws_lds_elems<T, EPI>() * 2 <= 160 * 1024, "LDS capacity");
+    __shared__ __attribute__((aligned(1024))) bf16_t smem[ws_lds_elems<T, EPI>()];
+    rows_gemm_ws_block<T, EPI, BKM>(p, smem, blockIdx.x);
+}
+
 // ---------------------------------------------------------------------------
 // dw_gemm
 // ---------------------------------------------------------------------------
@@ -986,8 +995,7 @@ __device__ __forceinline__ bool locate_dw_unit(const DwParams& p, int unit, DwUn
 
 // Adds the chunk partials of the experts that were cut: thread = 4 consecutive columns of a tile row.
 template <int BM, int BN, typename OutT>
-__global__ __launch_bounds__(256) void dw_chunk_sum_kernel(DwParams p) {
-    const int e = blockIdx.y;
+__device__ __forceinline__ void dw_chunk_sum_expert(const DwParams& p, int e) {
     const int lane = threadIdx.x % MTS_WAVE;
     const int share = dw_share(p);
     const int nc = dw_chunks(p, p.expert_start[e + 1] - p.expert_start[e], share);
@@ -1023,6 +1031,19 @@ __global__ __launch_bounds__(256) void dw_chunk_sum_kernel(DwParams p) {
         for (int j = 0; j < 4; ++j)
             if (n + j < p.N) C[j] = (OutT)acc[j];
     }
+}
+
+template <int BM, int BN, typename OutT>
+__global__ __launch_bounds__(256) void dw_chunk_sum_kernel(DwParams p) {
+    dw_chunk_sum_expert<BM, BN, OutT>(p, blockIdx.y);
+}
+
+// the same for two GEMMs over the same experts in one launch: blockIdx.y < E is the first's expert
+template <int BM, int BN, typename OutT>
+__global__ __launch_bounds__(256) void dw_chunk_sum_pair_kernel(DwParams a, DwParams b) {
+    const int e = blockIdx.y;
+    if (e < a.E) dw_chunk_sum_expert<BM, BN, OutT>(a, e);
+    else dw_chunk_sum_expert<BM, BN, OutT>(b, e - a.E);
 }
 
 // Stages a [64 k][64 m] block per wave-item: lane = (kgrp = lane%8, mc = lane/8) loads
@@ -1196,12 +1217,12 @@ struct DwWsTile {
     static_assert(LDS_ELEMS * 2 <= 160 * 1024, "LDS capacity");
 };
 
+// the work of block `block` of a launch; `smem` holds T::LDS_ELEMS elements, 1 KiB aligned
 template <class T, typename OutT>
-__global__ __launch_bounds__(T::NT) void dw_gemm_ws_kernel(DwParams p) {
-    __shared__ __attribute__((aligned(1024))) bf16_t smem[T::LDS_ELEMS];
+__device__ __forceinline__ void dw_gemm_ws_block(const DwParams& p, bf16_t* smem, int block) {
     constexpr int S = T::STAGES, L = T::A_INSTR + T::B_INSTR;
     // all tiles of a unit (an expert, or a row chunk of an over-full one) run on one XCD
-    const int xcd = blockIdx.x % kXcds, jb = blockIdx.x / kXcds;
+    const int xcd = block % kXcds, jb = block / kXcds;
     DwUnit unit;
     if (!locate_dw_unit(p, xcd + kXcds * (jb / p.tiles_per_expert), unit)) return;
     const int e = __builtin_amdgcn_readfirstlane(unit.e);
@@ -1386,13 +1407,77 @@ __global__ __launch_bounds__(T::NT) void dw_gemm_ws_kernel(DwParams p) {
         }
 }
 
-// ---------------------------------------------------------------------------
-// host side
-// ---------------------------------------------------------------------------
+template <class T, typename OutT>
+__global__ __launch_bounds__(T::NT) void dw_gemm_ws_kernel(DwParams p) {
+    __shared__ __attribute__((aligned(1024))) bf16_t smem[T::LDS_ELEMS];
+    dw_gemm_ws_block<T, OutT>(p, smem, blockIdx.x);
+}
+
+// the compiled tile shapes
 typedef Tile<128, 128, 2, 2> StagedSmall;                 // 4 waves of 64x64, any K that is a multiple of 8
 typedef RingTile<256, 128, 2, 2, 32, 3, 2> RingTwoPerCu;  // 4 waves of 128x64, 3 x 24 KiB stages, two blocks per CU
 typedef WsTile<256, 256, 2, 4, 32, 4, 4, 3> WsLarge;      // 8 consumer waves of 128x64 + 4 producers, 4 x 32 KiB stages
 typedef DwWsTile<256, 256, 2, 4, 32, 4, 4> DwWsLarge;     // same shape for the weight-gradient GEMMs
+
+// ---------------------------------------------------------------------------
+// dW1, dW2, dX and the reduction of the dS partials as one launch.  All four depend on dY1
+// only.  As separate launches on separate streams they share the CUs in whatever order the
+// hardware queues interleave them, and the long weight-gradient tiles (one tile reduces
+// over all rows of an expert) tend to start last and finish last.  Here the block index
+// fixes the order: the dW1 tiles first, then dW2, then the dX tiles, which are a third as
+// long and fill the CUs as they come free, then a few blocks that add up dS.
+// Every part starts at a multiple of the XCD count, so block % 8 is still the part's own
+// XCD index.
+// ---------------------------------------------------------------------------
+struct BwdJointParams {
+    DwParams dw1, dw2;
+    RowsParams dx;
+    int n_dw1, n_dw2, n_dx;        // blocks per part, in launch order
+    const float* ds_part;          // [entries rows][np]
+    const int32_t* s_reverse;      // entry -> row, negative for a dropped route
+    bf16_t* d_weights;             // [entries]
+    int np;
+    int64_t entries;
+};
+
+template <typename OutT>
+__global__ __launch_bounds__(WsLarge::NT, WsLarge::WAVES_PER_EU) void bwd_joint_kernel(BwdJointParams q) {
+    static_assert(WsLarge::NT == DwWsLarge::NT, "one block shape");
+    constexpr int ROWS_LDS = ws_lds_elems<WsLarge, EPI_PLAIN>();
+    constexpr int LDS_ELEMS = ROWS_LDS > DwWsLarge::LDS_ELEMS ? ROWS_LDS : DwWsLarge::LDS_ELEMS;
+    static_assert(LDS_ELEMS * 2 <= 160 * 1024, "LDS capacity");
+    __shared__ __attribute__((aligned(1024))) bf16_t smem[LDS_ELEMS];
+    int b = blockIdx.x;
+    if (b < q.n_dw1) {
+        dw_gemm_ws_block<DwWsLarge, OutT>(q.dw1, smem, b);
+        return;
+    }
+    b -= q.n_dw1;
+    if (b < q.n_dw2) {
+        dw_gemm_ws_block<DwWsLarge, OutT>(q.dw2, smem, b);
+        return;
+    }
+    b -= q.n_dw2;
+    if (b < q.n_dx) {
+        rows_gemm_ws_block<WsLarge, EPI_PLAIN, true>(q.dx, smem, b);   // W1 as stored: [E][2I][H]
+        return;
+    }
+    b -= q.n_dx;
+    const int nb = (int)gridDim.x - q.n_dw1 - q.n_dw2 - q.n_dx;
+    for (int64_t n = (int64_t)b * WsLarge::NT + threadIdx.x; n < q.entries; n += (int64_t)nb * WsLarge::NT) {
+        const int32_t r = q.s_reverse[n];
+        float v = 0.f;
+        if (r >= 0) {
+            const float* part = q.ds_part + (int64_t)r * q.np;
+            for (int j = 0; j < q.np; ++j) v += part[j];
+        }
+        q.d_weights[n] = (bf16_t)v;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
 
 enum Kind { K_GATEUP = 0, K_DOWN, K_DY1, K_DX, K_DW2, K_DW1, K_COUNT };
 const char* const kKindEnv[K_COUNT] = {"MTS_TILE_GATEUP", "MTS_TILE_DOWN", "MTS_TILE_DY1",
@@ -1490,6 +1575,16 @@ int64_t dw_chunk_workspace_bytes(int E, int M, int N) {
     return 2 * (int64_t)E * tiles * T::BM * T::BN * (int64_t)sizeof(float);
 }
 
+// adds the row-chunk partials of the experts that dw_gemm_ws cut (p.part set, grid values filled in)
+void launch_dw_chunk_sum(const DwParams& p, int E, int grad_dtype, hipStream_t s) {
+    typedef DwWsLarge T;
+    const int64_t items = (int64_t)p.tiles_per_expert * (T::BM * T::BN / 4);
+    const int64_t want = (items + 255) / 256;   // experts that were not cut leave at once
+    const dim3 sum_grid((unsigned)(want < 256 ? want : 256), (unsigned)E);
+    if (grad_dtype == MTS_GEMM_DTYPE) dw_chunk_sum_kernel<T::BM, T::BN, bf16_t><<<sum_grid, 256, 0, s>>>(p);
+    else dw_chunk_sum_kernel<T::BM, T::BN, float><<<sum_grid, 256, 0, s>>>(p);
+}
+
 int launch_dw_any(int kind, DwParams p, int E, int grad_dtype, void* workspace, int64_t workspace_bytes,
                   hipStream_t s) {
     if (grad_dtype != MTS_GEMM_DTYPE && grad_dtype != MTS_F32) return MTS_ERR_DTYPE;
@@ -1505,11 +1600,7 @@ int launch_dw_any(int kind, DwParams p, int E, int grad_dtype, void* workspace, 
         else dw_gemm_ws_kernel<T, float><<<grid, T::NT, 0, s>>>(p);
         if (p.part) {
             MTS_CHECK_LAUNCH();
-            const int64_t items = (int64_t)p.tiles_per_expert * (T::BM * T::BN / 4);
-            const int64_t want = (items + 255) / 256;   // experts that were not cut leave at once
-            const dim3 sum_grid((unsigned)(want < 256 ? want : 256), (unsigned)E);
-            if (grad_dtype == MTS_GEMM_DTYPE) dw_chunk_sum_kernel<T::BM, T::BN, bf16_t><<<sum_grid, 256, 0, s>>>(p);
-            else dw_chunk_sum_kernel<T::BM, T::BN, float><<<sum_grid, 256, 0, s>>>(p);
+            launch_dw_chunk_sum(p, E, grad_dtype, s);
         }
     } else {
         const dim3 grid = dw_grid<StagedSmall>(p, E, E);
@@ -1521,6 +1612,50 @@ int launch_dw_any(int kind, DwParams p, int E, int grad_dtype, void* workspace, 
 }
 
 int dy1_partials(int I) { return (I + 63) / 64; }
+
+// can dW1, dW2, dX and the dS reduction go out as one launch for these shapes?
+bool bwd_joint_ok(int H, int I) {
+    return tile_choice(K_DX) == 2 && tile_choice(K_DW1) == 2 && tile_choice(K_DW2) == 2 && rows_kmajor_ok(K_DX, 2 * I) &&
+           H % 8 == 0;
+}
+
+int launch_bwd_joint(BwdJointParams q, int E, int grad_dtype, void* ws1, int64_t ws1_bytes, void* ws2, int64_t ws2_bytes,
+                     hipStream_t s) {
+    typedef DwWsLarge T;
+    if (grad_dtype != MTS_GEMM_DTYPE && grad_dtype != MTS_F32) return MTS_ERR_DTYPE;
+    if (ws1) {
+        if (ws1_bytes < dw_chunk_workspace_bytes(E, q.dw1.M, q.dw1.N)) return MTS_ERR_WORKSPACE;
+        if (!mts_aligned16(ws1)) return MTS_ERR_ALIGN;
+        q.dw1.part = (float*)ws1;
+    }
+    if (ws2) {
+        if (ws2_bytes < dw_chunk_workspace_bytes(E, q.dw2.M, q.dw2.N)) return MTS_ERR_WORKSPACE;
+        if (!mts_aligned16(ws2)) return MTS_ERR_ALIGN;
+        q.dw2.part = (float*)ws2;
+    }
+    q.n_dw1 = (int)dw_grid<T>(q.dw1, E, q.dw1.part ? 2 * E : E).x;
+    q.n_dw2 = (int)dw_grid<T>(q.dw2, E, q.dw2.part ? 2 * E : E).x;
+    q.n_dx = (int)rows_grid<WsLarge, EPI_PLAIN>(q.dx, q.dx.TK).x;
+    const int64_t want = (q.entries + WsLarge::NT * 4 - 1) / (WsLarge::NT * 4);
+    const int n_ds = (int)(want < 64 ? want : 64);
+    const dim3 grid((unsigned)(q.n_dw1 + q.n_dw2 + q.n_dx + n_ds));
+    if (grad_dtype == MTS_GEMM_DTYPE) bwd_joint_kernel<bf16_t><<<grid, WsLarge::NT, 0, s>>>(q);
+    else bwd_joint_kernel<float><<<grid, WsLarge::NT, 0, s>>>(q);
+    MTS_CHECK_LAUNCH();
+    if (q.dw1.part && q.dw2.part) {
+        const int t = q.dw1.tiles_per_expert > q.dw2.tiles_per_expert ? q.dw1.tiles_per_expert : q.dw2.tiles_per_expert;
+        const int64_t want = ((int64_t)t * (T::BM * T::BN / 4) + 255) / 256;
+        const dim3 sum_grid((unsigned)(want < 256 ? want : 256), (unsigned)(2 * E));
+        if (grad_dtype == MTS_GEMM_DTYPE) dw_chunk_sum_pair_kernel<T::BM, T::BN, bf16_t><<<sum_grid, 256, 0, s>>>(q.dw1, q.dw2);
+        else dw_chunk_sum_pair_kernel<T::BM, T::BN, float><<<sum_grid, 256, 0, s>>>(q.dw1, q.dw2);
+    } else if (q.dw1.part) {
+        launch_dw_chunk_sum(q.dw1, E, grad_dtype, s);
+    } else if (q.dw2.part) {
+        launch_dw_chunk_sum(q.dw2, E, grad_dtype, s);
+    }
+    MTS_CHECK_LAUNCH();
+    return MTS_OK;
+}
 
 }  // namespace
 
@@ -1697,4 +1832,50 @@ extern "C" int MTS_GEMM_ENTRY(mts_moe_bwd_dw1)(const void* d_pre_act, const void
     p.Q = (const bf16_t*)x; p.q_rows = T; p.q_gather = x_gather;
     p.M = 2 * I; p.N = H; p.TK = T * K; p.expert_start = expert_start; p.C = d_w1;
     return launch_dw_any(K_DW1, p, E, grad_dtype, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+#ifndef MTS_GEMM_F16
+extern "C" int mts_moe_bwd_joint_supported(int act_dtype, int H, int I) {
+    return (act_dtype == MTS_BF16 || act_dtype == MTS_F16) && bwd_joint_ok(H, I) ? 1 : 0;
+}
+#endif
+
+extern "C" int MTS_GEMM_ENTRY(mts_moe_bwd_joint)(const void* d_out, const void* weighted_act, const void* d_pre_act,
+                                                 const void* x, const void* w1, const int32_t* x_gather,
+                                                 const int32_t* expert_start, const int32_t* s_reverse,
+                                                 const float* ds_partial, int64_t T, int K, int E, int H, int I,
+                                                 int act_dtype, int grad_dtype, void* dx_expanded, void* d_w1, void* d_w2,
+                                                 void* d_weights, void* workspace1, int64_t workspace1_bytes,
+                                                 void* workspace2, int64_t workspace2_bytes, void* stream) {
+#ifndef MTS_GEMM_F16
+    if (act_dtype == MTS_F16)
+        return mts_moe_bwd_joint_f16(d_out, weighted_act, d_pre_act, x, w1, x_gather, expert_start, s_reverse,
+                                     ds_partial, T, K, E, H, I, act_dtype, grad_dtype, dx_expanded, d_w1, d_w2, d_weights,
+                                     workspace1, workspace1_bytes, workspace2, workspace2_bytes, stream);
+#endif
+    if (!d_out || !weighted_act || !d_pre_act || !x || !w1 || !x_gather || !expert_start || !s_reverse || !ds_partial ||
+        !dx_expanded || !d_w1 || !d_w2 || !d_weights)
+        return MTS_ERR_NULL;
+    if (act_dtype != MTS_GEMM_DTYPE) return MTS_ERR_DTYPE;
+    if (T <= 0 || K < 1) return MTS_ERR_SHAPE;
+    const int64_t TK = T * K;
+    int rc = check_common(TK, E, H, I);
+    if (rc) return rc;
+    if (!bwd_joint_ok(H, I)) return MTS_ERR_SHAPE;
+    if (!mts_aligned16(d_out) || !mts_aligned16(weighted_act) || !mts_aligned16(d_pre_act) || !mts_aligned16(x) ||
+        !mts_aligned16(w1))
+        return MTS_ERR_ALIGN;
+    BwdJointParams q = {};
+    q.dw1.P = (const bf16_t*)d_pre_act; q.dw1.p_rows = TK; q.dw1.p_gather = nullptr;
+    q.dw1.Q = (const bf16_t*)x; q.dw1.q_rows = T; q.dw1.q_gather = x_gather;
+    q.dw1.M = 2 * I; q.dw1.N = H; q.dw1.TK = TK; q.dw1.expert_start = expert_start; q.dw1.C = d_w1;
+    q.dw2.P = (const bf16_t*)d_out; q.dw2.p_rows = T; q.dw2.p_gather = x_gather;
+    q.dw2.Q = (const bf16_t*)weighted_act; q.dw2.q_rows = TK; q.dw2.q_gather = nullptr;
+    q.dw2.M = H; q.dw2.N = I; q.dw2.TK = TK; q.dw2.expert_start = expert_start; q.dw2.C = d_w2;
+    q.dx.A = (const bf16_t*)d_pre_act; q.dx.a_rows = TK; q.dx.lda = 2 * I; q.dx.a_gather = nullptr;
+    q.dx.B = (const bf16_t*)w1; q.dx.b_rows = H;
+    q.dx.N = H; q.dx.Kdim = 2 * I; q.dx.expert_start = expert_start; q.dx.E = E;
+    q.dx.C = (bf16_t*)dx_expanded; q.dx.TK = TK;
+    q.ds_part = ds_partial; q.s_reverse = s_reverse; q.d_weights = (bf16_t*)d_weights; q.np = dy1_partials(I); q.entries = TK;
+    return launch_bwd_joint(q, E, grad_dtype, workspace1, workspace1_bytes, workspace2, workspace2_bytes, (hipStream_t)stream);
 }

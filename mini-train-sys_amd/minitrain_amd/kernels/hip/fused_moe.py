@@ -134,6 +134,8 @@ def expert_counts(topk_indices: torch.Tensor, E: int) -> torch.Tensor:
 
 # MTS_NO_OVERLAP=1 keeps every kernel of the backward pass on the caller's stream
 _OVERLAP = os.environ.get("MTS_NO_OVERLAP", "0") != "1"
+# MTS_NO_JOINT_BWD=1 launches dW2, dW1 and dX separately (on the side streams) even where one launch could hold them
+_JOINT = os.environ.get("MTS_NO_JOINT_BWD", "0") != "1"
 _SIDE_STREAMS: dict = {}
 
 
@@ -307,6 +309,32 @@ class _FusedMoEFunction(torch.autograd.Function):
         ddown_proj = None
         ws1, ws1_ptr, ws1_bytes = _dw_workspace(lib, 1, E, H, I, x.dtype, dev) if need_w1 else (None, 0, 0)
         ws2, ws2_ptr, ws2_bytes = _dw_workspace(lib, 2, E, H, I, x.dtype, dev) if need_w2 else (None, 0, 0)
+
+        # When every gradient is wanted, dW1, dW2, dX and the dS reduction go out as ONE launch whose block
+        # order starts the long weight-gradient tiles first; no side stream is involved.
+        if (
+            _JOINT and need_x and need_w1 and need_w2 and need_s and as_stored
+            and gate_up_proj.dtype == down_proj.dtype and lib.mts_moe_bwd_joint_supported(act, H, I)
+        ):
+            dgate_up_proj, ddown_proj = torch.empty_like(gate_up_proj), torch.empty_like(down_proj)
+            d_weights = torch.empty(T, K, dtype=weights_flat.dtype, device=dev)
+            dx_expanded = torch.empty(TK, H, dtype=x.dtype, device=dev)
+            _lib.check(
+                lib.mts_moe_bwd_joint(
+                    dO.data_ptr(), weighted_act.data_ptr(), d_pre_act.data_ptr(), x.data_ptr(), w1_bwd.data_ptr(),
+                    x_gather.data_ptr(), expert_start.data_ptr(), s_reverse.data_ptr(), ds_part.data_ptr(), T, K, E, H, I,
+                    act, _lib.dtype_code(gate_up_proj.dtype), dx_expanded.data_ptr(), dgate_up_proj.data_ptr(),
+                    ddown_proj.data_ptr(), d_weights.data_ptr(), ws1_ptr, ws1_bytes, ws2_ptr, ws2_bytes, stream,
+                ),
+                "mts_moe_bwd_joint",
+            )
+            dx = torch.empty(T, H, dtype=x.dtype, device=dev)
+            _lib.check(
+                lib.mts_moe_combine(dx_expanded.data_ptr(), None, s_reverse.data_ptr(), T, K, H, act, dx.data_ptr(), stream),
+                "mts_moe_combine",
+            )
+            return dx, dgate_up_proj, ddown_proj, None, d_weights
+
         if need_w1 and need_w2:
             fork(side[0], side[1])
         elif need_w2:

@@ -19,7 +19,8 @@ def _declared():
 def test_header_declares_the_expected_entry_points():
     names = _declared()
     for must in ("mts_router_fwd", "mts_router_bwd", "mts_moe_route", "mts_moe_fwd_gateup_swiglu", "mts_moe_fwd_down",
-                 "mts_moe_combine", "mts_moe_bwd_dy1", "mts_moe_bwd_dx", "mts_moe_bwd_dw1", "mts_moe_bwd_dw2"):
+                 "mts_moe_combine", "mts_moe_bwd_dy1", "mts_moe_bwd_dx", "mts_moe_bwd_dw1", "mts_moe_bwd_dw2",
+                 "mts_moe_bwd_joint"):
         assert must in names
 
 
@@ -65,6 +66,17 @@ def test_contract_violations_are_reported_before_any_launch():
     assert lib.mts_moe_bwd_dw_workspace_bytes(2, 8, 768, 1024) == 2 * 8 * (3 * 4) * 256 * 256 * 4
     assert lib.mts_moe_bwd_dw1(fake, fake, fake, fake, 256, 2, 4, 64, 128, _lib.MTS_BF16, _lib.MTS_BF16, fake, fake, 16,
                                None) == WORKSPACE
+    # dW1 + dW2 + dX + dS as one launch: 16-bit activations with whole 64-wide k-tiles of 2I only
+    assert lib.mts_moe_bwd_joint_supported(_lib.MTS_BF16, 768, 1024) == 1
+    assert lib.mts_moe_bwd_joint_supported(_lib.MTS_F16, 64, 128) == 1
+    assert lib.mts_moe_bwd_joint_supported(_lib.MTS_F32, 768, 1024) == 0
+    assert lib.mts_moe_bwd_joint_supported(_lib.MTS_BF16, 72, 40) == 0
+    joint = lambda *a: lib.mts_moe_bwd_joint(*a)
+    ok_args = [fake] * 9 + [256, 2, 4, 64, 128, _lib.MTS_BF16, _lib.MTS_BF16, fake, fake, fake, fake, None, 0, None, 0, None]
+    assert joint(*([None] + ok_args[1:])) == NULL
+    assert joint(*(ok_args[:14] + [_lib.MTS_F32] + ok_args[15:])) == -3                      # activations must be 16-bit
+    assert joint(*(ok_args[:12] + [72, 40] + ok_args[14:])) == SHAPE                          # 2I = 80 has no whole k-tile
+    assert joint(*(ok_args[:20] + [fake, 16] + ok_args[22:])) == WORKSPACE
     # unknown element type
     assert lib.mts_moe_combine(fake, None, fake, 8, 2, 64, 7, fake, None) == -3
 

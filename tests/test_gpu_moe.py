@@ -164,6 +164,43 @@ def test_weight_gradients_with_row_chunks(T, H, E, I, skew, monkeypatch):
     assert torch.equal(cut[1][0], uncut[1][0]) and torch.equal(cut[1][3], uncut[1][3])   # dx and dS do not change
 
 
+@pytest.mark.parametrize("T,H,E,I,dtype,fp32_weights,skew", [
+    (1000, 128, 8, 256, torch.bfloat16, False, 0.0), (257, 192, 8, 320, torch.bfloat16, False, 0.0),
+    (3000, 256, 8, 256, torch.bfloat16, False, 0.7), (300, 128, 4, 192, torch.bfloat16, True, 0.0),
+    (2048, 768, 8, 1024, torch.float16, False, 0.0), (1, 64, 4, 64, torch.bfloat16, False, 0.0),
+    (700, 256, 64, 256, torch.float16, True, 0.5)])
+def test_joint_backward_launch_equals_separate_launches(T, H, E, I, dtype, fp32_weights, skew, monkeypatch):
+    """dW1, dW2, dX and the dS reduction as one launch run the same blocks as the four separate
+    launches on side streams: every gradient is bit-identical, with and without row chunks."""
+    print(f"moe joint backward T={T} H={H} E={E} I={I} {dtype} fp32_weights={fp32_weights} skew={skew}", flush=True)
+    import importlib
+
+    from minitrain_amd import _lib
+
+    F = importlib.import_module("minitrain_amd.kernels.hip.fused_moe")
+    assert _lib.load().mts_moe_bwd_joint_supported(_lib.dtype_code(dtype), H, I) == 1
+    K = 2 if E > 1 else 1
+    case = routed_case(70 + T, T, H, E, I, K, dtype=dtype)
+    if fp32_weights:
+        _, _, w1, w2, _ = O.make_inputs(70 + T, T, H, E, I)
+        case.update(w1=w1, w2=w2)
+    if skew:
+        rng = np.random.Generator(np.random.Philox(T))
+        idx = case["idx"].clone()
+        heavy = torch.from_numpy(rng.random(T) < skew)
+        idx[heavy, 0] = 1
+        idx[heavy & (idx[:, 1] == 1), 1] = 0
+        case.update(idx=idx)
+    args = (case["x"], case["w1"], case["w2"], case["idx"], case["w"], case["g"])
+    assert F._JOINT
+    joint = hip_moe_grads(*args)
+    monkeypatch.setattr(F, "_JOINT", False)
+    separate = hip_moe_grads(*args)
+    for name, a, b in zip(NAMES, joint[1], separate[1]):
+        assert a.dtype == b.dtype and torch.equal(a, b), name
+    _compare(case)   # and the separate launches against the oracle (the default path is compared everywhere else)
+
+
 def test_layer_shape_subset_of_tokens():
     """293M-class layer dims at 2048 tokens: the whole oracle still runs on the CPU in seconds."""
     print("moe 2048x768x1024", flush=True)
