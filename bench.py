@@ -131,7 +131,7 @@ def stage_breakdown(layer, steps):
     rw = torch.empty(lib.mts_router_workspace_bytes(T, E), dtype=torch.uint8, device=dev)
     rws = torch.empty(max(4, lib.mts_moe_route_workspace_bytes(T, K, E)), dtype=torch.uint8, device=dev)
     r_w, r_i = torch.empty(T, K, dtype=torch.float32, device=dev), torch.empty(T, K, dtype=torch.int32, device=dev)
-    r_stats = torch.empty(E + 3, dtype=torch.float32, device=dev)
+    r_stats = torch.empty(2 * E + 10, dtype=torch.float32, device=dev)
     i32 = dict(dtype=torch.int32, device=dev)
     cnt, es2, a1, a2, a3 = torch.empty(E, **i32), torch.empty(E + 1, **i32), torch.empty(TK, **i32), torch.empty(TK, **i32), torch.empty(TK, **i32)
     dlog = torch.empty_like(logits)
@@ -148,7 +148,7 @@ def stage_breakdown(layer, steps):
         ("router_logits_fwd", "hbm", T * H * esz + T * E * 4 + E * H * 4,
          lambda: lib.mts_router_logits_fwd(p(x), p(w_r), T, H, E, B, p(logits2), st)),
         ("router_fwd", "hbm", T * E * 4 + T * K * 8,
-         lambda: lib.mts_router_fwd(p(logits), T, E, K, 1, p(r_w), p(r_i), p(r_stats), p(r_stats) + 4 * E, p(r_stats) + 4 * E + 4, p(cnt), p(r_stats) + 4 * E + 8, p(rw), rw.numel(), st)),
+         lambda: lib.mts_router_fwd(p(logits), T, E, K, 1, p(r_w), p(r_i), p(r_stats), p(r_stats) + 4 * E, p(r_stats) + 4 * E + 4, p(cnt), p(r_stats) + 4 * E + 8, p(r_stats) + 4 * E + 12, p(rw), rw.numel(), st)),
         ("route_metadata", "hbm", TK * 4 * 2 + 3 * TK * 4,
          lambda: lib.mts_moe_route(p(idx), T, K, E, 64, p(cnt), p(es2), p(a1), p(a2), p(a3), None, None, None, p(rws), rws.numel(), st)),
         ("fwd_gateup_swiglu", "mfma", gemm(2),

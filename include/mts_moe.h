@@ -57,12 +57,18 @@ const char* mts_error_string(int code);
  * counts [E] i32 and load_balance [1] may be NULL.  They stand in for the router
  * module's bookkeeping around the operator (minitrain/model/moe_router.py:82-90):
  * routes per expert (its torch.bincount) and E * sum_e (counts_e / (T*K)) * prob_mean_e
- * (its auxiliary loss); load_balance needs counts.                              */
+ * (its auxiliary loss).
+ * load_stats [E+7] f32 may be NULL; it holds the module's load metrics
+ * (moe_router.py:113-135) for dropless routing: [0,E) the fraction of the routes each
+ * expert takes, [E] the largest and [E+1] the smallest route count, [E+2] the
+ * population standard deviation of the fractions times E, [E+3] the largest fraction
+ * times E, [E+4] the number of experts without a route, [E+5] 0 (no route dropped),
+ * [E+6] entropy / log E (entropy itself for E = 1).                                   */
 int64_t mts_router_workspace_bytes(int64_t T, int E);
 int mts_router_fwd(const float* logits, int64_t T, int E, int K, int normalize,
                    float* weights, int32_t* indices, float* prob_mean, float* z_loss,
-                   float* entropy, int32_t* counts, float* load_balance, void* workspace,
-                   int64_t workspace_bytes, void* stream);
+                   float* entropy, int32_t* counts, float* load_balance, float* load_stats,
+                   void* workspace, int64_t workspace_bytes, void* stream);
 
 /* Replaces _router_backward_kernel (minitrain/kernels/triton/router.py:155-259).
  * g_weights [T,K], g_prob_mean [E], g_z_loss [1] -> dlogits [T,E]; each of the

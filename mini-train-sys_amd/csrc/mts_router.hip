@@ -211,8 +211,12 @@ __global__ __launch_bounds__(kThreads) void router_fwd_kernel(
 __global__ __launch_bounds__(kThreads) void router_stats_kernel(
     const float* __restrict__ partial, const int32_t* __restrict__ partial_counts, int nblocks, int E,
     float inv_t, float inv_routes, float* __restrict__ prob_mean, float* __restrict__ z_loss,
-    float* __restrict__ entropy, int32_t* __restrict__ counts, float* __restrict__ load_balance) {
+    float* __restrict__ entropy, int32_t* __restrict__ counts, float* __restrict__ load_balance,
+    float* __restrict__ load_stats) {
     __shared__ float prod[MTS_MAX_EXPERTS];   // fraction of routes x mean probability, per expert
+    __shared__ float share[MTS_MAX_EXPERTS];  // fraction of routes, per expert
+    __shared__ int routes_of[MTS_MAX_EXPERTS];
+    __shared__ float entropy_s;
     const int wave = threadIdx.x / MTS_WAVE, lane = threadIdx.x % MTS_WAVE;
     for (int i = wave; i < E + 2; i += kThreads / MTS_WAVE) {
         float v = 0.f;
@@ -228,22 +232,67 @@ __global__ __launch_bounds__(kThreads) void router_stats_kernel(
             if (i < E) {
                 prob_mean[i] = v;
                 prod[i] = (float)c * inv_routes * v;
+                share[i] = (float)c * inv_routes;
+                routes_of[i] = c;
                 if (counts) counts[i] = c;
             } else if (i == E) {
                 z_loss[0] = v;
             } else {
                 entropy[0] = v;
+                entropy_s = v;
             }
         }
     }
-    if (!load_balance) return;
+    if (!load_balance && !load_stats) return;
     __syncthreads();
     // E * sum_e f_e * pbar_e, summed in a fixed order by one wave
-    if (wave == 0) {
+    if (wave == 0 && load_balance) {
         float v = 0.f;
         for (int e = lane; e < E; e += MTS_WAVE) v += prod[e];
         v = wave_sum(v);
         if (lane == 0) load_balance[0] = (float)E * v;
+    }
+    // load statistics of the router module (minitrain/model/moe_router.py:113-135) from the route
+    // fractions: [0,E) the fractions, then the largest and smallest route count, the coefficient
+    // of variation (population standard deviation x E), largest fraction x E, the number of
+    // experts without a route, a zero (the dropped-route fraction of dropless routing) and the
+    // entropy over log E
+    if (wave == 1 % (kThreads / MTS_WAVE) && load_stats) {
+        float sum = 0.f, hi = 0.f, dead = 0.f;
+        int most = 0, fewest = 0x7fffffff;
+        for (int e = lane; e < E; e += MTS_WAVE) {
+            const float f = share[e];
+            load_stats[e] = f;
+            sum += f;
+            hi = fmaxf(hi, f);
+            most = max(most, routes_of[e]);
+            fewest = min(fewest, routes_of[e]);
+            dead += routes_of[e] == 0 ? 1.f : 0.f;
+        }
+        sum = wave_sum(sum);
+        dead = wave_sum(dead);
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            hi = fmaxf(hi, __shfl_xor(hi, o, MTS_WAVE));
+            most = max(most, __shfl_xor(most, o, MTS_WAVE));
+            fewest = min(fewest, __shfl_xor(fewest, o, MTS_WAVE));
+        }
+        const float mean = sum / (float)E;
+        float var = 0.f;
+        for (int e = lane; e < E; e += MTS_WAVE) {
+            const float d = share[e] - mean;
+            var += d * d;
+        }
+        var = wave_sum(var) / (float)E;
+        if (lane == 0) {
+            load_stats[E] = (float)most;
+            load_stats[E + 1] = (float)fewest;
+            load_stats[E + 2] = sqrtf(var) * (float)E;
+            load_stats[E + 3] = hi * (float)E;
+            load_stats[E + 4] = dead;
+            load_stats[E + 5] = 0.f;
+            load_stats[E + 6] = entropy_s / (E > 1 ? logf((float)E) : 1.0f);
+        }
     }
 }
 
@@ -364,12 +413,12 @@ extern "C" int64_t mts_router_workspace_bytes(int64_t T, int E) {
 
 extern "C" int mts_router_fwd(const float* logits, int64_t T, int E, int K, int normalize,
                               float* weights, int32_t* indices, float* prob_mean, float* z_loss,
-                              float* entropy, int32_t* counts, float* load_balance, void* workspace,
-                              int64_t workspace_bytes, void* stream) {
+                              float* entropy, int32_t* counts, float* load_balance, float* load_stats,
+                              void* workspace, int64_t workspace_bytes, void* stream) {
     int rc = check_router(logits, T, E, K);
     if (rc) return rc;
     if (!weights || !indices || !prob_mean || !z_loss || !entropy || !workspace) return MTS_ERR_NULL;
-    if ((counts || load_balance) && T * (int64_t)K > 0x7fffffffLL) return MTS_ERR_SHAPE;   // int32 route counts
+    if ((counts || load_balance || load_stats) && T * (int64_t)K > 0x7fffffffLL) return MTS_ERR_SHAPE;   // int32 route counts
     if (workspace_bytes < mts_router_workspace_bytes(T, E)) return MTS_ERR_WORKSPACE;
     hipStream_t s = (hipStream_t)stream;
     float* partial = (float*)workspace;
@@ -381,7 +430,7 @@ extern "C" int mts_router_fwd(const float* logits, int64_t T, int E, int K, int 
     MTS_CHECK_LAUNCH();
     router_stats_kernel<<<1, kThreads, 0, s>>>(partial, partial_counts, grid, E, 1.0f / (float)T,
                                                1.0f / ((float)T * (float)K), prob_mean, z_loss, entropy, counts,
-                                               load_balance);
+                                               load_balance, load_stats);
     MTS_CHECK_LAUNCH();
     return MTS_OK;
 }

@@ -38,30 +38,31 @@ class _RouterPostprocessFunction(torch.autograd.Function):
         dev = logits.device
         weights = torch.empty((T, top_k), device=dev, dtype=torch.float32)
         indices = torch.empty((T, top_k), device=dev, dtype=torch.int32)
-        stats = torch.empty(E + 3, device=dev, dtype=torch.float32)
+        stats = torch.empty(2 * E + 10, device=dev, dtype=torch.float32)   # E + 3 statistics, E + 7 load statistics
         counts = torch.empty(E, device=dev, dtype=torch.int32)
         ws_bytes = lib.mts_router_workspace_bytes(T, E)
         ws = torch.empty(ws_bytes, device=dev, dtype=torch.uint8)
         prob_mean, z_loss, entropy, load_balance = stats[:E], stats[E], stats[E + 1], stats[E + 2]
+        load_stats = stats[E + 3:]
         _lib.check(
             lib.mts_router_fwd(
                 logits.data_ptr(), T, E, top_k, int(normalize), weights.data_ptr(), indices.data_ptr(),
                 prob_mean.data_ptr(), z_loss.data_ptr(), entropy.data_ptr(), counts.data_ptr(),
-                load_balance.data_ptr(), ws.data_ptr(), ws_bytes, _lib.stream_of(logits),
+                load_balance.data_ptr(), load_stats.data_ptr(), ws.data_ptr(), ws_bytes, _lib.stream_of(logits),
             ),
             "mts_router_fwd",
         )
         ctx.save_for_backward(logits, weights, indices, counts)
         ctx.top_k = top_k
         ctx.normalize = normalize
-        ctx.mark_non_differentiable(indices, entropy, counts)
+        ctx.mark_non_differentiable(indices, entropy, counts, load_stats)
         ctx.set_materialize_grads(False)   # no zero tensors for the outputs that took no part in the loss
-        return weights, indices, prob_mean, z_loss, entropy, counts, load_balance
+        return weights, indices, prob_mean, z_loss, entropy, counts, load_balance, load_stats
 
     @staticmethod
     @torch.amp.custom_bwd(device_type="cuda")
     def backward(ctx, grad_weights, _grad_indices, grad_probability_mean, grad_z_loss, _grad_entropy, _grad_counts,
-                 grad_load_balance):
+                 grad_load_balance, _grad_load_stats):
         lib = _lib.load()
         logits, weights, indices, counts = ctx.saved_tensors
         T, E = logits.shape
@@ -100,8 +101,8 @@ def router_postprocess(logits: torch.Tensor, top_k: int, *, normalize: bool) -> 
             "hip router postprocess requires non-empty 2D fp32 logits on the GPU, "
             f"1 <= top_k <= {_MAX_TOP_K} and at most {_MAX_EXPERTS} experts"
         )
-    weights, indices, probability_mean, z_loss, entropy, counts, load_balance = _RouterPostprocessFunction.apply(
-        logits, top_k, normalize
+    weights, indices, probability_mean, z_loss, entropy, counts, load_balance, load_stats = (
+        _RouterPostprocessFunction.apply(logits, top_k, normalize)
     )
     return RouterPostprocessOutput(
         expert_weights=weights,
@@ -111,6 +112,7 @@ def router_postprocess(logits: torch.Tensor, top_k: int, *, normalize: bool) -> 
         entropy=entropy,
         expert_counts=counts,
         load_balance_loss=load_balance,
+        load_stats=load_stats,
     )
 
 

@@ -60,6 +60,24 @@ def capacity_selection(expert_indices: torch.Tensor, expert_weights: torch.Tenso
     return keep, kept_index, counts.clamp(max=capacity)
 
 
+def load_metrics_from_stats(route, num_experts: int):
+    """The same record from a backend's ``load_stats`` (dropless routing): views of one tensor, no launches."""
+    stats, E = route.load_stats, num_experts
+    record = {
+        "moe/router_entropy": route.entropy,
+        "moe/router_entropy_normalized": stats[E + 6],
+        "moe/dropped_route_fraction": stats[E + 5],
+        "moe/max_expert_load": stats[E],
+        "moe/min_expert_load": stats[E + 1],
+        "moe/expert_load_cv": stats[E + 2],
+        "moe/max_to_mean_load": stats[E + 3],
+        "moe/dead_expert_count": stats[E + 4],
+        "moe/expert_load_fraction": stats[:E],
+        "moe/expert_probability": route.probability_per_expert,
+    }
+    return {k: (v if k == "moe/router_entropy" else v.detach()) for k, v in record.items()}
+
+
 def load_metrics(route, accepted: torch.Tensor, routes: int, dropped_fraction: torch.Tensor, num_experts: int):
     """The router's monitoring record, keys as in the reference (minitrain/model/moe_router.py:113-135);
     ``accepted`` = routes each expert takes, as floats."""
@@ -148,13 +166,17 @@ class TopKRouter(nn.Module):
                 auxiliary_loss = cfg.num_experts * torch.sum(route_fraction * route.probability_per_expert)
 
             dispatch_indices = None
-            dropped_fraction = expert_weights.new_zeros(())
-            accepted = route_counts.float()
             if cfg.expert_capacity_factor is not None:
                 expert_weights, dispatch_indices, accepted, dropped_fraction = self._limit_capacity(
                     ops, expert_indices, expert_weights
                 )
-            metrics = load_metrics(route, accepted, expert_indices.numel(), dropped_fraction, cfg.num_experts)
+                metrics = load_metrics(route, accepted, expert_indices.numel(), dropped_fraction, cfg.num_experts)
+            elif getattr(route, "load_stats", None) is not None:
+                metrics = load_metrics_from_stats(route, cfg.num_experts)
+            else:
+                metrics = load_metrics(
+                    route, route_counts.float(), expert_indices.numel(), expert_weights.new_zeros(()), cfg.num_experts
+                )
 
         return RouterOutput(
             expert_indices=expert_indices.to(torch.int32),

@@ -25,10 +25,15 @@ class RouterPostprocessOutput:
     entropy: Tensor                  # [] mean routing entropy, detached
     # Not in the reference's record (minitrain/model/ops.py:7-15); a backend that has them from the
     # same pass fills them in, None leaves the computation to the caller: routes per expert (int32
-    # [E], no gradient) and E * sum_e (routes_e / routes) * probability_per_expert_e, which carries a
-    # gradient through the mean probability.
+    # [E], no gradient), E * sum_e (routes_e / routes) * probability_per_expert_e, which carries a
+    # gradient through the mean probability, and the load statistics below.
     expert_counts: Tensor | None = None
     load_balance_loss: Tensor | None = None
+    # fp32 [E + 7], no gradient: what the router module's load metrics need when no route is dropped --
+    # the fraction of the routes per expert, then the largest and the smallest route count, the
+    # population standard deviation of the fractions x E, the largest fraction x E, the number of
+    # experts without a route, 0 (the dropped-route fraction) and entropy / log E
+    load_stats: Tensor | None = None
 
 
 class OpsBackend(Protocol):

@@ -37,6 +37,15 @@ def _check(logits, K, normalize, *, tied=False):
     assert got.expert_counts.dtype == torch.int32 and torch.equal(got.expert_counts.cpu().long(), ref_counts)
     ref_lb = E_ * torch.sum(ref_counts.double() / (T_ * K) * ref.probability_per_expert.double())
     torch.testing.assert_close(got.load_balance_loss.cpu().double(), ref_lb, rtol=FWD_TOL, atol=FWD_TOL)
+    # the module's load metrics (minitrain/model/moe_router.py:113-135) from the same pass, against numpy in fp64
+    frac = ref_counts.double().numpy() / (T_ * K)
+    want = np.concatenate([frac, [ref_counts.max().item(), ref_counts.min().item(), frac.std() * E_, frac.max() * E_,
+                                  float((ref_counts == 0).sum()), 0.0,
+                                  float(ref.entropy) / (np.log(E_) if E_ > 1 else 1.0)]])
+    stats = got.load_stats.cpu().double().numpy()
+    assert got.load_stats.dtype == torch.float32 and stats.shape == (E_ + 7,) and not got.load_stats.requires_grad
+    np.testing.assert_allclose(stats, want, rtol=2e-5, atol=2e-6)
+    assert stats[E_] == want[E_] and stats[E_ + 1] == want[E_ + 1] and stats[E_ + 4] == want[E_ + 4]   # counts are exact
     # backward through the combined objective of the reference's parity probe
     T, E = logits.shape
     rng = np.random.Generator(np.random.Philox(99))

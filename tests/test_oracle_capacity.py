@@ -134,3 +134,31 @@ def test_routing_metadata_skips_dropped_routes():
     assert np.all(m.s_reverse_scatter_idx[flat < 0] == -1)
     assert np.array_equal(m.s_reverse_scatter_idx[m.s_scatter_idx], np.arange(kept.size))
     assert np.all(np.diff(flat[m.s_scatter_idx]) >= 0)
+
+
+def test_router_metric_record_from_fused_statistics_matches_the_torch_path():
+    """Host logic of the router module: the monitoring record taken as views of a backend's
+    load statistics carries the same keys and values as the one computed with torch ops
+    (keys and formulas of minitrain/model/moe_router.py:113-135)."""
+    import math
+    import sys
+    from pathlib import Path
+    from types import SimpleNamespace
+
+    sys.path.insert(0, str(Path(__file__).resolve().parents[1] / "mini-train-sys_amd"))
+    from minitrain_amd.model.moe_router import load_metrics, load_metrics_from_stats
+
+    E, routes = 8, 4096
+    counts = torch.tensor([900, 0, 300, 512, 512, 1000, 72, 800])
+    assert int(counts.sum()) == routes
+    frac = counts.double() / routes
+    entropy = torch.tensor(1.234)
+    stats = torch.cat([frac, torch.tensor([counts.max(), counts.min(), frac.std(unbiased=False) * E, frac.max() * E,
+                                           (counts == 0).sum(), 0.0, 1.234 / math.log(E)], dtype=torch.float64)]).float()
+    route = SimpleNamespace(entropy=entropy, probability_per_expert=torch.full((E,), 1.0 / E), load_stats=stats)
+    fused = load_metrics_from_stats(route, E)
+    plain = load_metrics(route, counts.float(), routes, torch.zeros(()), E)
+    assert set(fused) == set(plain)
+    for key in plain:
+        torch.testing.assert_close(fused[key].float(), plain[key].float(), rtol=1e-6, atol=1e-7, msg=key)
+        assert fused[key].shape == plain[key].shape, key
