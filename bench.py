@@ -80,12 +80,17 @@ class Layer:
         logits = fused(self.x, self.w_r) if fused is not None else None
         if logits is None:
             logits = F.linear(self.x.float(), self.w_r)
-        route = self.ops.router_postprocess(logits, self.K, normalize=True)
+        # as the router module does: the backend may hand back the weights in the activation dtype itself
+        extra = {"weights_dtype": self.x.dtype} if getattr(self.ops, "casts_router_weights", False) else {}
+        route = self.ops.router_postprocess(logits, self.K, normalize=True, **extra)
         aux = getattr(route, "load_balance_loss", None)
         if aux is None:
             counts = torch.bincount(route.expert_indices.flatten().long(), minlength=self.E)
             aux = self.E * torch.sum(counts.float() / route.expert_indices.numel() * route.probability_per_expert)
-        out = self.ops.fused_moe(self.x, self.w1, self.w2, route.expert_indices, route.expert_weights.to(self.x.dtype))
+        weights = getattr(route, "expert_weights_cast", None)
+        if weights is None:
+            weights = route.expert_weights.to(self.x.dtype)
+        out = self.ops.fused_moe(self.x, self.w1, self.w2, route.expert_indices, weights)
         # loss = sum(out * G) + 0.01 * aux + 0.001 * z: its gradient enters as the three seeds G, 0.01 and
         # 0.001, so the scalar itself (a few 5 us element-wise launches on 0-dim tensors) is not formed
         torch.autograd.backward([out, aux, route.z_loss], [self.g, self.seed_aux, self.seed_z])
@@ -131,6 +136,7 @@ def stage_breakdown(layer, steps):
     rw = torch.empty(lib.mts_router_workspace_bytes(T, E), dtype=torch.uint8, device=dev)
     rws = torch.empty(max(4, lib.mts_moe_route_workspace_bytes(T, K, E)), dtype=torch.uint8, device=dev)
     r_w, r_i = torch.empty(T, K, dtype=torch.float32, device=dev), torch.empty(T, K, dtype=torch.int32, device=dev)
+    r_wa = torch.empty(T, K, **bf)
     r_stats = torch.empty(2 * E + 10, dtype=torch.float32, device=dev)
     i32 = dict(dtype=torch.int32, device=dev)
     cnt, es2, a1, a2, a3 = torch.empty(E, **i32), torch.empty(E + 1, **i32), torch.empty(TK, **i32), torch.empty(TK, **i32), torch.empty(TK, **i32)
@@ -147,8 +153,8 @@ def stage_breakdown(layer, steps):
     stages = [
         ("router_logits_fwd", "hbm", T * H * esz + T * E * 4 + E * H * 4,
          lambda: lib.mts_router_logits_fwd(p(x), p(w_r), T, H, E, B, p(logits2), st)),
-        ("router_fwd", "hbm", T * E * 4 + T * K * 8,
-         lambda: lib.mts_router_fwd(p(logits), T, E, K, 1, p(r_w), p(r_i), p(r_stats), p(r_stats) + 4 * E, p(r_stats) + 4 * E + 4, p(cnt), p(r_stats) + 4 * E + 8, p(r_stats) + 4 * E + 12, p(rw), rw.numel(), st)),
+        ("router_fwd", "hbm", T * E * 4 + T * K * 8 + T * K * esz,
+         lambda: lib.mts_router_fwd(p(logits), T, E, K, 1, p(r_w), p(r_i), p(r_stats), p(r_stats) + 4 * E, p(r_stats) + 4 * E + 4, p(cnt), p(r_stats) + 4 * E + 8, p(r_stats) + 4 * E + 12, p(r_wa), B, p(rw), rw.numel(), st)),
         ("route_metadata", "hbm", TK * 4 * 2 + 3 * TK * 4,
          lambda: lib.mts_moe_route(p(idx), T, K, E, 64, p(cnt), p(es2), p(a1), p(a2), p(a3), None, None, None, p(rws), rws.numel(), st)),
         ("fwd_gateup_swiglu", "mfma", gemm(2),
@@ -164,8 +170,8 @@ def stage_breakdown(layer, steps):
                                        p(dxe), p(dw1), p(dw2), p(dwts), p(dws1), dws1.numel(), p(dws2), dws2.numel(), st)),
         ("dx_combine", "hbm", TK * H * esz + T * H * esz + TK * 4,
          lambda: lib.mts_moe_combine(p(dxe), None, p(sr), T, K, H, B, p(dx), st)),
-        ("router_bwd", "hbm", T * E * 4 * 2 + T * K * 12,
-         lambda: lib.mts_router_bwd(p(logits), p(r_w), p(r_i), p(gw), p(gp), p(gz), p(gz), p(cnt), T, E, K, 1, p(dlog), st)),
+        ("router_bwd", "hbm", T * E * 4 * 2 + T * K * 8 + T * K * esz,
+         lambda: lib.mts_router_bwd(p(logits), p(r_w), p(r_i), None, p(dwts), B, p(gp), p(gz), p(gz), p(cnt), T, E, K, 1, p(dlog), st)),
         ("router_logits_bwd", "hbm", 2 * T * H * esz + T * E * 4 + 2 * E * H * 4,
          lambda: lib.mts_router_logits_bwd(p(dlog), p(x), p(w_r), T, H, E, B, p(dx_r), p(dw_r), p(lws), lws.numel(), st)),
     ]

@@ -63,21 +63,28 @@ const char* mts_error_string(int code);
  * expert takes, [E] the largest and [E+1] the smallest route count, [E+2] the
  * population standard deviation of the fractions times E, [E+3] the largest fraction
  * times E, [E+4] the number of experts without a route, [E+5] 0 (no route dropped),
- * [E+6] entropy / log E (entropy itself for E = 1).                                   */
+ * [E+6] entropy / log E (entropy itself for E = 1).
+ * weights_act [T,K] in act_dtype (MTS_BF16 or MTS_F16) may be NULL; it is the copy of
+ * `weights` the router module makes for the MoE block (`expert_weights.to(
+ * hidden_states.dtype)`, moe_router.py:139-140), rounded to nearest even.             */
 int64_t mts_router_workspace_bytes(int64_t T, int E);
 int mts_router_fwd(const float* logits, int64_t T, int E, int K, int normalize,
                    float* weights, int32_t* indices, float* prob_mean, float* z_loss,
                    float* entropy, int32_t* counts, float* load_balance, float* load_stats,
-                   void* workspace, int64_t workspace_bytes, void* stream);
+                   void* weights_act, int act_dtype, void* workspace, int64_t workspace_bytes,
+                   void* stream);
 
 /* Replaces _router_backward_kernel (minitrain/kernels/triton/router.py:155-259).
  * g_weights [T,K], g_prob_mean [E], g_z_loss [1] -> dlogits [T,E]; each of the
  * gradient inputs may be NULL, which stands for zeros (an output that took no part in
  * the loss).  g_load_balance [1] is the gradient of the load-balancing term; it
  * reaches the logits through prob_mean only (the route fractions counts/(T*K)
- * carry no gradient) and needs the counts the forward call wrote.              */
+ * carry no gradient) and needs the counts the forward call wrote.
+ * g_weights_act [T,K] in act_dtype is the gradient that arrived at the activation-dtype
+ * copy of the weights; it is widened and added to g_weights (either may be NULL).     */
 int mts_router_bwd(const float* logits, const float* weights, const int32_t* indices,
-                   const float* g_weights, const float* g_prob_mean, const float* g_z_loss,
+                   const float* g_weights, const void* g_weights_act, int act_dtype,
+                   const float* g_prob_mean, const float* g_z_loss,
                    const float* g_load_balance, const int32_t* counts, int64_t T, int E, int K,
                    int normalize, float* dlogits, void* stream);
 

@@ -76,7 +76,7 @@ template <int EP, int G>
 __global__ __launch_bounds__(kThreads) void router_fwd_kernel(
     const float* __restrict__ logits, int64_t T, int E, int K, int normalize,
     float* __restrict__ weights, int32_t* __restrict__ indices, float* __restrict__ partial,
-    int32_t* __restrict__ partial_counts) {
+    int32_t* __restrict__ partial_counts, void* __restrict__ weights_act, int act_dtype) {
     constexpr int ROWS = kThreads / G;
     const int g = threadIdx.x % G;
     const int rl = threadIdx.x / G;
@@ -142,8 +142,14 @@ __global__ __launch_bounds__(kThreads) void router_fwd_kernel(
 #pragma unroll
             for (int k = 0; k < MTS_MAX_TOP_K; ++k) {
                 if (k < K) {
-                    weights[row * K + k] = sel_p[k] * inv;
+                    const float wk = sel_p[k] * inv;
+                    weights[row * K + k] = wk;
                     indices[row * K + k] = sel_e[k];
+                    // the copy the MoE block hands to fused_moe: rounded once, as tensor.to() rounds
+                    if (weights_act) {
+                        if (act_dtype == MTS_BF16) reinterpret_cast<bf16_t*>(weights_act)[row * K + k] = (bf16_t)wk;
+                        else reinterpret_cast<mts_f16_t*>(weights_act)[row * K + k] = (mts_f16_t)wk;
+                    }
                 }
             }
         }
@@ -299,10 +305,18 @@ __global__ __launch_bounds__(kThreads) void router_stats_kernel(
 template <int EP, int G>
 __global__ __launch_bounds__(kThreads) void router_bwd_kernel(
     const float* __restrict__ logits, const float* __restrict__ weights,
-    const int32_t* __restrict__ indices, const float* __restrict__ g_w,
+    const int32_t* __restrict__ indices, const float* __restrict__ g_w, const void* __restrict__ g_w_act, int act_dtype,
     const float* __restrict__ g_p, const float* __restrict__ g_z, const float* __restrict__ g_lb,
     const int32_t* __restrict__ counts, int64_t T, int E, int K,
     int normalize, float* __restrict__ dlogits) {
+    // gradient of the routing weights: the fp32 output's and the activation-dtype copy's, either may be absent
+    auto grad_w = [&](int64_t i) {
+        float v = g_w ? g_w[i] : 0.f;
+        if (g_w_act)
+            v += act_dtype == MTS_BF16 ? (float)reinterpret_cast<const bf16_t*>(g_w_act)[i]
+                                       : (float)reinterpret_cast<const mts_f16_t*>(g_w_act)[i];
+        return v;
+    };
     constexpr int ROWS = kThreads / G;
     const int g = threadIdx.x % G;
     const int rl = threadIdx.x / G;
@@ -330,11 +344,11 @@ __global__ __launch_bounds__(kThreads) void router_bwd_kernel(
         }
         float wdot = 0.f;
         if (normalize) {
-            for (int k = 0; k < K; ++k) wdot += weights[rr * K + k] * (g_w ? g_w[rr * K + k] : 0.f);
+            for (int k = 0; k < K; ++k) wdot += weights[rr * K + k] * grad_w(rr * K + k);
         }
         for (int k = 0; k < K; ++k) {
             int e = indices[rr * K + k];
-            float gw = g_w ? g_w[rr * K + k] : 0.f;
+            float gw = grad_w(rr * K + k);
             float w = weights[rr * K + k];
 #pragma unroll
             for (int j = 0; j < EP; ++j) {
@@ -414,9 +428,11 @@ extern "C" int64_t mts_router_workspace_bytes(int64_t T, int E) {
 extern "C" int mts_router_fwd(const float* logits, int64_t T, int E, int K, int normalize,
                               float* weights, int32_t* indices, float* prob_mean, float* z_loss,
                               float* entropy, int32_t* counts, float* load_balance, float* load_stats,
-                              void* workspace, int64_t workspace_bytes, void* stream) {
+                              void* weights_act, int act_dtype, void* workspace, int64_t workspace_bytes,
+                              void* stream) {
     int rc = check_router(logits, T, E, K);
     if (rc) return rc;
+    if (weights_act && act_dtype != MTS_BF16 && act_dtype != MTS_F16) return MTS_ERR_DTYPE;
     if (!weights || !indices || !prob_mean || !z_loss || !entropy || !workspace) return MTS_ERR_NULL;
     if ((counts || load_balance || load_stats) && T * (int64_t)K > 0x7fffffffLL) return MTS_ERR_SHAPE;   // int32 route counts
     if (workspace_bytes < mts_router_workspace_bytes(T, E)) return MTS_ERR_WORKSPACE;
@@ -426,7 +442,7 @@ extern "C" int mts_router_fwd(const float* logits, int64_t T, int E, int K, int 
     int G = E > 512 ? 64 : lanes_for(E);
     int grid = grid_for(T, G);
     MTS_ROUTER_DISPATCH(router_fwd_kernel, <<<grid, kThreads, 0, s>>>(logits, T, E, K, normalize, weights, indices,
-                                                                      partial, partial_counts));
+                                                                      partial, partial_counts, weights_act, act_dtype));
     MTS_CHECK_LAUNCH();
     router_stats_kernel<<<1, kThreads, 0, s>>>(partial, partial_counts, grid, E, 1.0f / (float)T,
                                                1.0f / ((float)T * (float)K), prob_mean, z_loss, entropy, counts,
@@ -436,19 +452,20 @@ extern "C" int mts_router_fwd(const float* logits, int64_t T, int E, int K, int 
 }
 
 extern "C" int mts_router_bwd(const float* logits, const float* weights, const int32_t* indices,
-                              const float* g_weights, const float* g_prob_mean,
+                              const float* g_weights, const void* g_weights_act, int act_dtype, const float* g_prob_mean,
                               const float* g_z_loss, const float* g_load_balance, const int32_t* counts,
                               int64_t T, int E, int K, int normalize, float* dlogits, void* stream) {
     int rc = check_router(logits, T, E, K);
     if (rc) return rc;
     if (!weights || !indices || !dlogits) return MTS_ERR_NULL;
     if (g_load_balance && !counts) return MTS_ERR_NULL;
+    if (g_weights_act && act_dtype != MTS_BF16 && act_dtype != MTS_F16) return MTS_ERR_DTYPE;
     if (E == 8 && !mts_aligned16(dlogits)) return MTS_ERR_ALIGN;
     hipStream_t s = (hipStream_t)stream;
     int G = E > 512 ? 64 : lanes_for(E);
     int grid = grid_for(T, G);
     MTS_ROUTER_DISPATCH(router_bwd_kernel,
-                        <<<grid, kThreads, 0, s>>>(logits, weights, indices, g_weights, g_prob_mean,
+                        <<<grid, kThreads, 0, s>>>(logits, weights, indices, g_weights, g_weights_act, act_dtype, g_prob_mean,
                                                    g_z_loss, g_load_balance, counts, T, E, K, normalize,
                                                    dlogits));
     MTS_CHECK_LAUNCH();

@@ -30,8 +30,8 @@ SIGNATURES = {
     "mts_version": (_i, []),
     "mts_error_string": (_c.c_char_p, [_i]),
     "mts_router_workspace_bytes": (_l, [_l, _i]),
-    "mts_router_fwd": (_i, [_p, _l, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p, _p, _l, _p]),
-    "mts_router_bwd": (_i, [_p, _p, _p, _p, _p, _p, _p, _p, _l, _i, _i, _i, _p, _p]),
+    "mts_router_fwd": (_i, [_p, _l, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _p, _l, _p]),
+    "mts_router_bwd": (_i, [_p, _p, _p, _p, _p, _i, _p, _p, _p, _p, _l, _i, _i, _i, _p, _p]),
     "mts_router_logits_fwd": (_i, [_p, _p, _l, _i, _i, _i, _p, _p]),
     "mts_router_logits_bwd_workspace_bytes": (_l, [_l, _i, _i]),
     "mts_router_logits_bwd": (_i, [_p, _p, _p, _l, _i, _i, _i, _p, _p, _p, _l, _p]),

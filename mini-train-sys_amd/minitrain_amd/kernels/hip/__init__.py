@@ -5,6 +5,8 @@ Counterpart of the reference's ``TritonOpsBackend``
 that class there is no fallback: an unsupported tensor contract raises.
 """
 
+import os
+
 from minitrain_amd.kernels.dense_ops import DenseTorchOps
 from minitrain_amd.kernels.hip.capacity import capacity_mask, is_capacity_mask_supported
 from minitrain_amd.kernels.hip.fused_moe import expert_counts, fused_moe, is_fused_moe_supported
@@ -21,8 +23,12 @@ class HipOpsBackend(DenseTorchOps):
     # fused_moe gives a route whose expert index is negative no row in the expert GEMMs
     drops_routes = True
 
-    def router_postprocess(self, logits, top_k, *, normalize):
-        return router_postprocess(logits, top_k, normalize=normalize)
+    # router_postprocess takes ``weights_dtype`` and then also returns the weights rounded to it
+    # (MTS_NO_ROUTER_CAST=1 leaves the cast to the caller, for comparisons)
+    casts_router_weights = os.environ.get("MTS_NO_ROUTER_CAST", "0") != "1"
+
+    def router_postprocess(self, logits, top_k, *, normalize, weights_dtype=None):
+        return router_postprocess(logits, top_k, normalize=normalize, weights_dtype=weights_dtype)
 
     def fused_moe(self, x, gate_up_proj, down_proj, top_k_index, top_k_weights):
         return fused_moe(x, gate_up_proj, down_proj, top_k_index, top_k_weights)

@@ -31,7 +31,7 @@ def is_router_postprocess_supported(logits: torch.Tensor, top_k: int, normalize:
 class _RouterPostprocessFunction(torch.autograd.Function):
     @staticmethod
     @torch.amp.custom_fwd(device_type="cuda")
-    def forward(ctx, logits: torch.Tensor, top_k: int, normalize: bool):
+    def forward(ctx, logits: torch.Tensor, top_k: int, normalize: bool, weights_dtype):
         lib = _lib.load()
         logits = logits.contiguous()
         T, E = logits.shape
@@ -44,25 +44,31 @@ class _RouterPostprocessFunction(torch.autograd.Function):
         ws = torch.empty(ws_bytes, device=dev, dtype=torch.uint8)
         prob_mean, z_loss, entropy, load_balance = stats[:E], stats[E], stats[E + 1], stats[E + 2]
         load_stats = stats[E + 3:]
+        # the copy of the weights in the activation dtype, written by the same kernel (what the router
+        # module otherwise makes with tensor.to(): one launch forward, one backward)
+        weights_act = torch.empty((T, top_k), device=dev, dtype=weights_dtype) if weights_dtype is not None else None
+        act_code = _lib.dtype_code(weights_dtype) if weights_dtype is not None else 0
         _lib.check(
             lib.mts_router_fwd(
                 logits.data_ptr(), T, E, top_k, int(normalize), weights.data_ptr(), indices.data_ptr(),
                 prob_mean.data_ptr(), z_loss.data_ptr(), entropy.data_ptr(), counts.data_ptr(),
-                load_balance.data_ptr(), load_stats.data_ptr(), ws.data_ptr(), ws_bytes, _lib.stream_of(logits),
+                load_balance.data_ptr(), load_stats.data_ptr(), _lib.ptr(weights_act), act_code, ws.data_ptr(), ws_bytes,
+                _lib.stream_of(logits),
             ),
             "mts_router_fwd",
         )
         ctx.save_for_backward(logits, weights, indices, counts)
         ctx.top_k = top_k
         ctx.normalize = normalize
+        ctx.act_code = act_code
         ctx.mark_non_differentiable(indices, entropy, counts, load_stats)
         ctx.set_materialize_grads(False)   # no zero tensors for the outputs that took no part in the loss
-        return weights, indices, prob_mean, z_loss, entropy, counts, load_balance, load_stats
+        return weights, indices, prob_mean, z_loss, entropy, counts, load_balance, load_stats, weights_act
 
     @staticmethod
     @torch.amp.custom_bwd(device_type="cuda")
     def backward(ctx, grad_weights, _grad_indices, grad_probability_mean, grad_z_loss, _grad_entropy, _grad_counts,
-                 grad_load_balance, _grad_load_stats):
+                 grad_load_balance, _grad_load_stats, grad_weights_act):
         lib = _lib.load()
         logits, weights, indices, counts = ctx.saved_tensors
         T, E = logits.shape
@@ -75,20 +81,24 @@ class _RouterPostprocessFunction(torch.autograd.Function):
         g_p = dense(grad_probability_mean)
         g_z = dense(grad_z_loss)
         g_lb = dense(grad_load_balance)
+        g_w_act = None if grad_weights_act is None else grad_weights_act.contiguous()   # stays in the activation dtype
         grad_logits = torch.empty_like(logits)
         _lib.check(
             lib.mts_router_bwd(
-                logits.data_ptr(), weights.data_ptr(), indices.data_ptr(), _lib.ptr(g_w), _lib.ptr(g_p),
-                _lib.ptr(g_z), _lib.ptr(g_lb), counts.data_ptr(), T, E, ctx.top_k, int(ctx.normalize),
+                logits.data_ptr(), weights.data_ptr(), indices.data_ptr(), _lib.ptr(g_w), _lib.ptr(g_w_act), ctx.act_code,
+                _lib.ptr(g_p), _lib.ptr(g_z), _lib.ptr(g_lb), counts.data_ptr(), T, E, ctx.top_k, int(ctx.normalize),
                 grad_logits.data_ptr(), _lib.stream_of(logits),
             ),
             "mts_router_bwd",
         )
-        return grad_logits, None, None
+        return grad_logits, None, None, None
 
 
-def router_postprocess(logits: torch.Tensor, top_k: int, *, normalize: bool) -> RouterPostprocessOutput:
-    """Process router logits without materialising the full probability matrix."""
+def router_postprocess(logits: torch.Tensor, top_k: int, *, normalize: bool, weights_dtype=None) -> RouterPostprocessOutput:
+    """Process router logits without materialising the full probability matrix.
+
+    ``weights_dtype`` (bf16 or fp16, an extension of the reference's signature) also asks for
+    ``expert_weights_cast``, the differentiable copy of the weights in that dtype."""
 
     if logits.ndim != 2 or logits.dtype != torch.float32:
         raise ValueError("router logits must be a 2D fp32 tensor")
@@ -101,8 +111,10 @@ def router_postprocess(logits: torch.Tensor, top_k: int, *, normalize: bool) -> 
             "hip router postprocess requires non-empty 2D fp32 logits on the GPU, "
             f"1 <= top_k <= {_MAX_TOP_K} and at most {_MAX_EXPERTS} experts"
         )
-    weights, indices, probability_mean, z_loss, entropy, counts, load_balance, load_stats = (
-        _RouterPostprocessFunction.apply(logits, top_k, normalize)
+    if weights_dtype not in (None, torch.bfloat16, torch.float16):
+        raise ValueError("weights_dtype must be bfloat16 or float16")
+    weights, indices, probability_mean, z_loss, entropy, counts, load_balance, load_stats, weights_cast = (
+        _RouterPostprocessFunction.apply(logits, top_k, normalize, weights_dtype)
     )
     return RouterPostprocessOutput(
         expert_weights=weights,
@@ -113,6 +125,7 @@ def router_postprocess(logits: torch.Tensor, top_k: int, *, normalize: bool) -> 
         expert_counts=counts,
         load_balance_loss=load_balance,
         load_stats=load_stats,
+        expert_weights_cast=weights_cast,
     )
 
 

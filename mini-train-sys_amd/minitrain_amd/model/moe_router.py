@@ -149,7 +149,14 @@ class TopKRouter(nn.Module):
         cfg = self.cfg
         logits = self._logits(hidden_states, ops)
         with torch.autocast(device_type=hidden_states.device.type, enabled=False):
-            route = ops.router_postprocess(logits, cfg.experts_per_token, normalize=cfg.router_normalize_topk)
+            # a backend may write the copy of the weights in the activation dtype in the same pass
+            want_cast = (
+                getattr(ops, "casts_router_weights", False)
+                and cfg.expert_capacity_factor is None
+                and hidden_states.dtype in (torch.bfloat16, torch.float16)
+            )
+            extra = {"weights_dtype": hidden_states.dtype} if want_cast else {}
+            route = ops.router_postprocess(logits, cfg.experts_per_token, normalize=cfg.router_normalize_topk, **extra)
             expert_weights, expert_indices = route.expert_weights, route.expert_indices
 
             route_counts = getattr(route, "expert_counts", None)
@@ -178,9 +185,10 @@ class TopKRouter(nn.Module):
                     route, route_counts.float(), expert_indices.numel(), expert_weights.new_zeros(()), cfg.num_experts
                 )
 
+        cast = getattr(route, "expert_weights_cast", None) if want_cast else None
         return RouterOutput(
             expert_indices=expert_indices.to(torch.int32),
-            expert_weights=expert_weights.to(hidden_states.dtype),
+            expert_weights=cast if cast is not None else expert_weights.to(hidden_states.dtype),
             auxiliary_loss=auxiliary_loss,
             z_loss=route.z_loss,
             metrics=metrics,

@@ -34,6 +34,9 @@ class RouterPostprocessOutput:
     # population standard deviation of the fractions x E, the largest fraction x E, the number of
     # experts without a route, 0 (the dropped-route fraction) and entropy / log E
     load_stats: Tensor | None = None
+    # [T, K] in the dtype asked for with ``weights_dtype``: expert_weights rounded to it, differentiable
+    # (what the router module hands to fused_moe); None when not asked for or not offered
+    expert_weights_cast: Tensor | None = None
 
 
 class OpsBackend(Protocol):

@@ -36,7 +36,7 @@ def test_library_exports_every_declared_symbol():
     assert lib.mts_version() == 1
     assert lib.mts_error_string(0) == b"ok"
     # argument checks run on the host before any launch: safe without a GPU
-    assert lib.mts_router_fwd(None, 4, 8, 2, 1, None, None, None, None, None, None, None, None, None, 0, None) == -1
+    assert lib.mts_router_fwd(None, 4, 8, 2, 1, None, None, None, None, None, None, None, None, None, 0, None, 0, None) == -1
     assert lib.mts_moe_route_workspace_bytes(24576, 2, 8) == 192 * 8 * 4
     assert lib.mts_moe_ds_partials(1024) > 0
 

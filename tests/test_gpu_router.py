@@ -102,6 +102,33 @@ def test_router_config2_and_config4_shapes():
     assert share.max() > 0.25          # the load really is imbalanced
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("normalize", [True, False])
+def test_router_weights_in_the_activation_dtype(dtype, normalize):
+    """``weights_dtype`` adds the copy of the weights the router module makes for the MoE block
+    (minitrain/model/moe_router.py:139-140): bit-identical to ``expert_weights.to(dtype)``, and a
+    gradient that arrives at it gives the logits gradient the cast's own backward would give."""
+    print(f"router weights cast {dtype} normalize={normalize}", flush=True)
+    ops = hip_backend()
+    assert ops.casts_router_weights
+    T, E, K = 1000, 8, 2
+    logits = _logits(T, E, 17)
+    g = torch.from_numpy(np.random.Generator(np.random.Philox(5)).standard_normal((T, K)).astype(np.float32)).cuda()
+    a = logits.cuda().requires_grad_(True)
+    got = ops.router_postprocess(a, K, normalize=normalize, weights_dtype=dtype)
+    assert got.expert_weights_cast.dtype == dtype and got.expert_weights.dtype == torch.float32
+    assert torch.equal(got.expert_weights_cast, got.expert_weights.to(dtype))
+    ((got.expert_weights_cast.float() * g).sum() + 0.5 * got.expert_weights.sum()).backward()
+    b = logits.cuda().requires_grad_(True)
+    plain = ops.router_postprocess(b, K, normalize=normalize)
+    assert plain.expert_weights_cast is None
+    ((plain.expert_weights.to(dtype).float() * g).sum() + 0.5 * plain.expert_weights.sum()).backward()
+    # the same numbers enter the same kernel, once as a 16-bit tensor and once widened by torch
+    assert torch.equal(a.grad, b.grad)
+    with pytest.raises(ValueError):
+        ops.router_postprocess(a, K, normalize=normalize, weights_dtype=torch.float64)
+
+
 def test_router_errors_and_determinism():
     ops = hip_backend()
     with pytest.raises(ValueError):
