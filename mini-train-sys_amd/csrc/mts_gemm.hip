@@ -298,7 +298,9 @@ struct FragPipe {
     }
 };
 
-__device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + __expf(-x)); }
+// v_rcp_f32 (1 ulp) instead of the IEEE division sequence, which costs nine more instructions per
+// value; the results are rounded to 16 bits
+__device__ __forceinline__ float sigmoidf_(float x) { return __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }
 
 template <class T>
 __device__ __forceinline__ void zero_acc(f32x16 (&acc)[T::MF][T::NF]) {
@@ -478,7 +480,8 @@ __device__ __forceinline__ void rows_epilogue(const RowsParams& p, f32x16 (&acc)
                         dsp += a * y1;
                         wa[q] = s * y1;
                         const float da = a * s;
-                        dg[q] = da * (silu * (1.0f - sig) + sig) * u;
+                        // d silu/dg * u = (sig + silu (1 - sig)) u = y1 + sig (u - y1)
+                        dg[q] = da * __builtin_fmaf(sig, u - y1, y1);
                         du[q] = da * silu;
                     }
                     stage4(buf0 + o, wa[0], wa[1], wa[2], wa[3]);
