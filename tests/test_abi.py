@@ -104,3 +104,21 @@ def test_cpu_tensors_are_rejected_not_served_by_a_fallback():
                       torch.zeros(4, 1, dtype=torch.bfloat16))
     with pytest.raises(ValueError):
         get_ops_backend("triton")
+
+
+def test_bench_refuses_more_than_one_gpu_and_a_missing_gpu():
+    """bench.py measures one GPU: `--gpus 2` (or a multi-rank launch) exits with a message, and without
+    a GPU it exits instead of timing a CPU path."""
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    bench = str(Path(__file__).resolve().parents[1] / "bench.py")
+    two = subprocess.run([sys.executable, bench, "--gpus", "2"], capture_output=True, text=True, timeout=300)
+    assert two.returncode == 2 and "one GPU" in two.stderr and two.stdout.strip() == ""
+    import torch
+
+    if not torch.cuda.is_available():
+        one = subprocess.run([sys.executable, bench, "--steps", "1", "--warmup", "0"], capture_output=True, text=True,
+                             timeout=300)
+        assert one.returncode == 2 and "needs a GPU" in one.stderr and one.stdout.strip() == ""
