@@ -41,7 +41,7 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # two rocprofv3 counter runs summarised in profiles/moe_layer_24x1024_hbm_traffic.txt (FETCH_SIZE
 # scaled by 2.0, WRITE_SIZE by 1.0 against a plain copy kernel of known size).  Not measured live.
 MEASURED_TRAFFIC_BYTES = {
-    "fwd_gateup_swiglu": 786.8e6, "fwd_down": 303.4e6, "bwd_dy1": 710.5e6, "bwd_joint": 1115.7e6,
+    "fwd_gateup_swiglu": 694.8e6, "fwd_down": 303.4e6, "bwd_dy1": 710.5e6, "bwd_joint": 1115.7e6,
     "combine": 115.2e6, "dx_combine": 114.4e6,
 }
 
