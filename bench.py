@@ -125,7 +125,7 @@ def stage_breakdown(layer, steps):
     idx, wts = route.expert_indices, route.expert_weights.bfloat16().flatten().contiguous()
     (_, es, xg, ss, sr, _, _, _) = compute_routing_metadata(idx, E)
     pre, post, y, out = torch.empty(TK, 2 * I, **bf), torch.empty(TK, I, **bf), torch.empty(TK, H, **bf), torch.empty(T, H, **bf)
-    dpre, wact, dxe, dx = torch.empty(TK, 2 * I, **bf), torch.empty(TK, I, **bf), torch.empty(TK, H, **bf), torch.empty(T, H, **bf)
+    dpre, dxe, dx = torch.empty(TK, 2 * I, **bf), torch.empty(TK, H, **bf), torch.empty(T, H, **bf)
     npart = lib.mts_moe_ds_partials(I)
     dsp = torch.empty(TK, npart, dtype=torch.float32, device=dev)
     dwts = torch.empty(T, K, **bf)
@@ -158,15 +158,15 @@ def stage_breakdown(layer, steps):
         ("route_metadata", "hbm", TK * 4 * 2 + 3 * TK * 4,
          lambda: lib.mts_moe_route(p(idx), T, K, E, 64, p(cnt), p(es2), p(a1), p(a2), p(a3), None, None, None, p(rws), rws.numel(), st)),
         ("fwd_gateup_swiglu", "mfma", gemm(2),
-         lambda: lib.mts_moe_fwd_gateup_swiglu(p(x), p(w1), p(xg), p(es), T, K, E, H, I, B, p(pre), p(post), st)),
+         lambda: lib.mts_moe_fwd_gateup_swiglu(p(x), p(w1), p(xg), p(es), p(wts), p(ss), T, K, E, H, I, B, p(pre), p(post), st)),
         ("fwd_down", "mfma", gemm(1), lambda: lib.mts_moe_fwd_down(p(post), p(w2), p(es), TK, E, H, I, B, p(y), st)),
-        ("combine", "hbm", TK * H * esz + T * H * esz + TK * 4 + TK * esz,
-         lambda: lib.mts_moe_combine(p(y), p(wts), p(sr), T, K, H, B, p(out), st)),
+        ("combine", "hbm", TK * H * esz + T * H * esz + TK * 4,
+         lambda: lib.mts_moe_combine(p(y), None, p(sr), T, K, H, B, p(out), st)),
         ("bwd_dy1", "mfma", gemm(1),
-         lambda: lib.mts_moe_bwd_dy1(p(g), p(w2), 1, p(pre), p(wts), p(xg), p(ss), p(es), T, K, E, H, I, B, p(dpre), p(wact), p(dsp), st)),
+         lambda: lib.mts_moe_bwd_dy1(p(g), p(w2), 1, p(pre), p(wts), p(xg), p(ss), p(es), T, K, E, H, I, B, p(dpre), None, p(dsp), st)),
         # dW1, dW2, dX and the dS reduction: one launch (plus the chunk sum), as the operator issues them
         ("bwd_joint", "mfma", gemm(5),
-         lambda: lib.mts_moe_bwd_joint(p(g), p(wact), p(dpre), p(x), p(w1), p(xg), p(es), p(sr), p(dsp), T, K, E, H, I, B, B,
+         lambda: lib.mts_moe_bwd_joint(p(g), p(post), p(dpre), p(x), p(w1), p(xg), p(es), p(sr), p(dsp), T, K, E, H, I, B, B,
                                        p(dxe), p(dw1), p(dw2), p(dwts), p(dws1), dws1.numel(), p(dws2), dws2.numel(), st)),
         ("dx_combine", "hbm", TK * H * esz + T * H * esz + TK * 4,
          lambda: lib.mts_moe_combine(p(dxe), None, p(sr), T, K, H, B, p(dx), st)),

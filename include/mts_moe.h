@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define MTS_VERSION 1
+#define MTS_VERSION 2
 
 /* element types of activations / weights / weight gradients */
 #define MTS_BF16 0
@@ -157,9 +157,16 @@ int mts_moe_stage_weights(const void* src, int src_dtype, void* dst, int dst_dty
  * Replaces _fused_up_proj_swiglu_kernel (fused_moe_kernels.py:264-367):
  * for every row r (token x_gather[r], expert e): [g;u] = W1[e] x ; a = silu(g)*u.
  * x [T,H], w1 [E,2I,H], pre_act [TK,2I], post_act [TK,I], all of act_dtype
- * (MTS_BF16, MTS_F16: MFMA kernels, H and I multiples of 8; MTS_F32: plain fp32 kernels). */
+ * (MTS_BF16, MTS_F16: MFMA kernels, H and I multiples of 8; MTS_F32: plain fp32 kernels).
+ * weights (flat [T*K], act_dtype) and s_scatter (row -> entry) are optional as a pair.  With
+ * them post_act[r] = s_r * silu(g) * u, s_r = weights[s_scatter[r]] (fp32 product, one
+ * rounding): the down projection then yields s_r * y[r], the combine is the unweighted sum
+ * (mts_moe_combine with weights == NULL), and the same buffer is the `weighted_act` operand of
+ * the dW2 GEMM (the reference recomputes it in the backward kernel, fused_moe_kernels.py:587-588), so
+ * mts_moe_bwd_dy1 need not write it again.                                         */
 int mts_moe_fwd_gateup_swiglu(const void* x, const void* w1, const int32_t* x_gather,
-                              const int32_t* expert_start, int64_t T, int K, int E, int H,
+                              const int32_t* expert_start, const void* weights,
+                              const int32_t* s_scatter, int64_t T, int K, int E, int H,
                               int I, int act_dtype, void* pre_act, void* post_act,
                               void* stream);
 
@@ -183,7 +190,8 @@ int mts_moe_combine(const void* y, const void* weights, const int32_t* s_reverse
  * whether this entry point and mts_moe_bwd_dx take the stored layout (bf16, H and 2I
  * multiples of 64); otherwise they return MTS_ERR_SHAPE for it.  ds_partial is
  * [TK, mts_moe_ds_partials(I)] f32 scratch reduced by mts_moe_bwd_ds (fixed order, no
- * atomics).                                                                    */
+ * atomics).  weighted_act may be NULL: it is then not written (the caller holds s*a already,
+ * see mts_moe_fwd_gateup_swiglu).                                              */
 int mts_moe_ds_partials(int I);
 int mts_moe_bwd_weights_as_stored(int act_dtype, int H, int I);
 int mts_moe_bwd_dy1(const void* d_out, const void* w2, int w2_as_stored, const void* pre_act,

@@ -44,7 +44,7 @@ static inline bool mts_aligned16(const void* p) { return (reinterpret_cast<uintp
 // fp16 instantiation of the grouped GEMMs (mts_gemm_f16.hip); the public entry points forward to it
 extern "C" {
 int mts_moe_fwd_gateup_swiglu_f16(const void* x, const void* w1, const int32_t* x_gather, const int32_t* expert_start,
-                                  int64_t T, int K, int E, int H, int I, int act_dtype, void* pre_act, void* post_act,
+                                  const void* weights, const int32_t* s_scatter, int64_t T, int K, int E, int H, int I, int act_dtype, void* pre_act, void* post_act,
                                   void* stream);
 int mts_moe_fwd_down_f16(const void* post_act, const void* w2, const int32_t* expert_start, int64_t TK, int E, int H,
                          int I, int act_dtype, void* y, void* stream);

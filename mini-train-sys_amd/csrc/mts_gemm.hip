@@ -108,7 +108,10 @@ struct Tile {
     static_assert((BM * 8) % NT == 0 && (BN * 8) % NT == 0, "loader split");
 };
 
-enum Epilogue { EPI_PLAIN = 0, EPI_SWIGLU = 1, EPI_DY1 = 2 };
+// EPI_DY1N: the dO*W2 epilogue without the weighted_act output (the caller kept the forward
+// pass's post_act, which already carries the routing weight)
+enum Epilogue { EPI_PLAIN = 0, EPI_SWIGLU = 1, EPI_DY1 = 2, EPI_DY1N = 3 };
+constexpr bool epi_is_dy1(int epi) { return epi == EPI_DY1 || epi == EPI_DY1N; }
 
 struct RowsParams {
     const bf16_t* A;           // activations, row-major, leading dimension lda
@@ -124,12 +127,13 @@ struct RowsParams {
     bf16_t* C;                 // plain: [TK,N]; SwiGLU: pre_act [TK,2N]; DY1: d_pre_act [TK,2N]
     bf16_t* C2;                // SwiGLU: post_act [TK,N]; DY1: weighted_act [TK,N]
     const bf16_t* pre_act;     // DY1: saved [g;u]
-    const bf16_t* route_w;     // DY1: routing weights, flat [T*K]
-    const int32_t* s_scatter;  // DY1: row -> entry
+    const bf16_t* route_w;     // DY1: routing weights, flat [T*K]; SwiGLU: the same, or NULL (post_act unscaled)
+    const int32_t* s_scatter;  // DY1, SwiGLU with route_w: row -> entry
     float* ds_part;            // DY1: [TK][np]
     int np;
     int64_t TK;                // rows of every output
     int n_tiles;               // column tiles per m-tile (set by the launcher)
+    int xcd_ranges;            // block -> tile mapping: 1 = every XCD takes a contiguous range of m-tiles
 };
 
 // ---------------------------------------------------------------------------
@@ -327,7 +331,7 @@ __device__ __forceinline__ void zero_acc(f32x16 (&acc)[T::MF][T::NF]) {
 template <class T, int EPI>
 struct EpiShape {
     static constexpr int COLS = (EPI == EPI_SWIGLU) ? T::WN / 2 : T::WN;  // contiguous columns per staged tile
-    static constexpr int NBUF = (EPI == EPI_PLAIN) ? 1 : 3;
+    static constexpr int NBUF = (EPI == EPI_PLAIN) ? 1 : (EPI == EPI_DY1N ? 2 : 3);
     static constexpr int LDW = COLS + 8;
     static constexpr int ELEMS = T::NWAVES * NBUF * 32 * LDW;
 };
@@ -362,25 +366,29 @@ __device__ __forceinline__ void rows_epilogue(const RowsParams& p, f32x16 (&acc)
                                               int row0, int rend, int n0, int wm, int wn) {
     typedef EpiShape<T, EPI> ES;
     constexpr int COLS = ES::COLS, LDW = ES::LDW;
+    constexpr bool DY1 = epi_is_dy1(EPI), WACT = (EPI == EPI_DY1);
     const int wave = threadIdx.x / MTS_WAVE, lane = threadIdx.x % MTS_WAVE;
     const int ml = lane % 32, nq = (lane / 32) * 4;
     bf16_t* buf0 = smem + wave * ES::NBUF * 32 * LDW;
     bf16_t* buf1 = buf0 + 32 * LDW;
     bf16_t* buf2 = buf1 + 32 * LDW;
+    // dY1: staging tiles of the gate and up halves, and of weighted_act where it is written
+    bf16_t* bufg = WACT ? buf1 : buf0;
+    bf16_t* bufu = WACT ? buf2 : buf1;
     const int ncol0 = n0 + wn * COLS;  // first output column of this wave
     const uint32_t N = (uint32_t)p.N;
     const __amdgpu_buffer_rsrc_t rs_c = make_rsrc(p.C, p.TK * (int64_t)(EPI == EPI_PLAIN ? N : 2 * N) * 2);
-    const __amdgpu_buffer_rsrc_t rs_c2 = make_rsrc(p.C2, EPI == EPI_PLAIN ? 0 : p.TK * (int64_t)N * 2);
-    const __amdgpu_buffer_rsrc_t rs_pre = make_rsrc(p.pre_act, EPI == EPI_DY1 ? p.TK * (int64_t)N * 4 : 0);
+    const __amdgpu_buffer_rsrc_t rs_c2 = make_rsrc(p.C2, (EPI == EPI_PLAIN || EPI == EPI_DY1N) ? 0 : p.TK * (int64_t)N * 2);
+    const __amdgpu_buffer_rsrc_t rs_pre = make_rsrc(p.pre_act, DY1 ? p.TK * (int64_t)N * 4 : 0);
 
-    // routing weight of each of the lane's rows (dY1 only): two dependent loads, issued for all
-    // rows up front
+    // routing weight of each of the lane's rows (dY1; SwiGLU when post_act carries the weight): two
+    // dependent loads, issued for all rows up front
     float srow[T::MF];
     // dY1: gate and up pre-activations of one 32 x COLS slab of the wave's tile, row-contiguous
     // 16-byte loads held in registers; the loads of slab mf+1 are issued before the arithmetic of
     // slab mf so that their latency is covered
     constexpr int PRE_LPR = COLS / 8, PRE_RPI = MTS_WAVE / PRE_LPR, PRE_IT = 32 / PRE_RPI;
-    u32x4 gv[EPI == EPI_DY1 ? PRE_IT : 1], uv[EPI == EPI_DY1 ? PRE_IT : 1];
+    u32x4 gv[DY1 ? PRE_IT : 1], uv[DY1 ? PRE_IT : 1];
     auto load_pre = [&](int mf) {
         const int c = (lane % PRE_LPR) * 8;
 #pragma unroll
@@ -392,13 +400,14 @@ __device__ __forceinline__ void rows_epilogue(const RowsParams& p, f32x16 (&acc)
             uv[it] = buf_load16(rs_pre, po == kInvalid ? kInvalid : po + N * 2u);
         }
     };
-    if (EPI == EPI_DY1) {
+    if (DY1 || EPI == EPI_SWIGLU) {
+        const bool weighted = DY1 || p.route_w != nullptr;
 #pragma unroll
         for (int mf = 0; mf < T::MF; ++mf) {
             const int row = row0 + wm * T::WM + mf * 32 + ml;
-            srow[mf] = row < rend ? (float)p.route_w[p.s_scatter[row]] : 0.f;
+            srow[mf] = !weighted ? 1.f : (row < rend ? (float)p.route_w[p.s_scatter[row]] : 0.f);
         }
-        if (PREFETCH) load_pre(0);
+        if (DY1 && PREFETCH) load_pre(0);
     }
 #pragma unroll
     for (int mf = 0; mf < T::MF; ++mf) {
@@ -413,6 +422,7 @@ __device__ __forceinline__ void rows_epilogue(const RowsParams& p, f32x16 (&acc)
             flush_tile<COLS>(buf0, rs_c, N, ncol0, rowg0, rend, ncol0, p.N);
         } else if (EPI == EPI_SWIGLU) {
             constexpr int HALF = T::NF / 2;
+            const float s = srow[mf];
 #pragma unroll
             for (int f = 0; f < HALF; ++f)
 #pragma unroll
@@ -422,7 +432,7 @@ __device__ __forceinline__ void rows_epilogue(const RowsParams& p, f32x16 (&acc)
                     for (int q = 0; q < 4; ++q) {
                         g[q] = acc[mf][f][4 * j + q];
                         u[q] = acc[mf][f + HALF][4 * j + q];
-                        a[q] = g[q] * sigmoidf_(g[q]) * u[q];
+                        a[q] = g[q] * sigmoidf_(g[q]) * u[q] * s;
                     }
                     const int o = ml * LDW + f * 32 + 8 * j + nq;
                     stage4(buf0 + o, g[0], g[1], g[2], g[3]);
@@ -432,7 +442,7 @@ __device__ __forceinline__ void rows_epilogue(const RowsParams& p, f32x16 (&acc)
             flush_tile<COLS>(buf0, rs_c, 2 * N, ncol0, rowg0, rend, ncol0, p.N);
             flush_tile<COLS>(buf1, rs_c, 2 * N, N + ncol0, rowg0, rend, ncol0, p.N);
             flush_tile<COLS>(buf2, rs_c2, N, ncol0, rowg0, rend, ncol0, p.N);
-        } else {  // EPI_DY1
+        } else {  // dY1
             const int row = rowg0 + ml;
             const bool rok = row < rend;
             const float s = srow[mf];
@@ -444,16 +454,16 @@ __device__ __forceinline__ void rows_epilogue(const RowsParams& p, f32x16 (&acc)
                 for (int it = 0; it < PRE_IT; ++it) {
                     const int r = it * PRE_RPI + lane / PRE_LPR;
                     if (PREFETCH) {
-                        *reinterpret_cast<u32x4*>(buf1 + r * LDW + c) = gv[it];
-                        *reinterpret_cast<u32x4*>(buf2 + r * LDW + c) = uv[it];
+                        *reinterpret_cast<u32x4*>(bufg + r * LDW + c) = gv[it];
+                        *reinterpret_cast<u32x4*>(bufu + r * LDW + c) = uv[it];
                     } else {   // load and hand over one row group at a time: few registers live
                         const int grow = rowg0 + r;
                         const bool ok = grow < rend && ncol0 + c < p.N;
                         const uint32_t po = ok ? ((uint32_t)grow * 2u * N + (uint32_t)(ncol0 + c)) * 2u : kInvalid;
                         const u32x4 g16 = buf_load16(rs_pre, po);
                         const u32x4 u16 = buf_load16(rs_pre, po == kInvalid ? kInvalid : po + N * 2u);
-                        *reinterpret_cast<u32x4*>(buf1 + r * LDW + c) = g16;
-                        *reinterpret_cast<u32x4*>(buf2 + r * LDW + c) = u16;
+                        *reinterpret_cast<u32x4*>(bufg + r * LDW + c) = g16;
+                        *reinterpret_cast<u32x4*>(bufu + r * LDW + c) = u16;
                     }
                 }
                 if (PREFETCH && mf + 1 < T::MF) load_pre(mf + 1);
@@ -465,8 +475,8 @@ __device__ __forceinline__ void rows_epilogue(const RowsParams& p, f32x16 (&acc)
                 for (int j = 0; j < 4; ++j) {
                     const int nl = nf * 32 + 8 * j + nq;   // column inside the wave tile
                     const int o = ml * LDW + nl;
-                    const uint2 gr = *reinterpret_cast<const uint2*>(buf1 + o);
-                    const uint2 ur = *reinterpret_cast<const uint2*>(buf2 + o);
+                    const uint2 gr = *reinterpret_cast<const uint2*>(bufg + o);
+                    const uint2 ur = *reinterpret_cast<const uint2*>(bufu + o);
                     float wa[4], dg[4], du[4];
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
@@ -484,9 +494,9 @@ __device__ __forceinline__ void rows_epilogue(const RowsParams& p, f32x16 (&acc)
                         dg[q] = da * __builtin_fmaf(sig, u - y1, y1);
                         du[q] = da * silu;
                     }
-                    stage4(buf0 + o, wa[0], wa[1], wa[2], wa[3]);
-                    stage4(buf1 + o, dg[0], dg[1], dg[2], dg[3]);
-                    stage4(buf2 + o, du[0], du[1], du[2], du[3]);
+                    if (WACT) stage4(buf0 + o, wa[0], wa[1], wa[2], wa[3]);
+                    stage4(bufg + o, dg[0], dg[1], dg[2], dg[3]);
+                    stage4(bufu + o, du[0], du[1], du[2], du[3]);
                 }
             dsp += __shfl_xor(dsp, 32, MTS_WAVE);
             // one partial per 64 output columns, whatever the tile shape: a wave that
@@ -497,20 +507,24 @@ __device__ __forceinline__ void rows_epilogue(const RowsParams& p, f32x16 (&acc)
                 for (int q = 0; q < T::WN / 64; ++q)
                     if (slot + q < p.np) p.ds_part[(int64_t)row * p.np + slot + q] = q == 0 ? dsp : 0.f;
             }
-            flush_tile<COLS>(buf0, rs_c2, N, ncol0, rowg0, rend, ncol0, p.N);
-            flush_tile<COLS>(buf1, rs_c, 2 * N, ncol0, rowg0, rend, ncol0, p.N);
-            flush_tile<COLS>(buf2, rs_c, 2 * N, N + ncol0, rowg0, rend, ncol0, p.N);
+            if (WACT) flush_tile<COLS>(buf0, rs_c2, N, ncol0, rowg0, rend, ncol0, p.N);
+            flush_tile<COLS>(bufg, rs_c, 2 * N, ncol0, rowg0, rend, ncol0, p.N);
+            flush_tile<COLS>(bufu, rs_c, 2 * N, N + ncol0, rowg0, rend, ncol0, p.N);
         }
     }
 }
 
 // ---------------------------------------------------------------------------
 // block -> tile mapping.  Workgroups are handed to the 8 XCDs round-robin
-// (block b runs on XCD b % 8) and every XCD has its own L2, so the blocks that
-// share operand panels are given to one XCD back to back: the j-th block of XCD x
-// computes m-tile x + 8*(j / n_tiles), n-tile j % n_tiles, i.e. all n-tiles of an
-// m-tile (same activation rows) and a few m-tiles of the same expert (same
-// weights) are in flight on one XCD at the same time.
+// (block b runs on XCD b % 8) and every XCD has its own L2.  The m-tiles are in
+// expert order, so every XCD is given a contiguous range of them (xcd_ranges = 1):
+// it works its way through one expert after the other, the expert's weights are
+// fetched into that L2 once and every m-tile of the range finds them there, and the
+// j-th block of an XCD computes n-tile j % n_tiles of the range's m-tile j / n_tiles,
+// so all column tiles of an m-tile (same activation rows) run side by side.  The
+// older mapping (xcd_ranges = 0) deals the m-tiles round-robin, m-tile
+// xcd + 8*(j / n_tiles): all eight L2s then stream the same expert's weights at the
+// same time and each of them again for every group of m-tiles.
 // ---------------------------------------------------------------------------
 constexpr int kXcds = 8;
 
@@ -521,9 +535,20 @@ constexpr int kXcds = 8;
 template <int BM>
 __device__ __forceinline__ bool locate_rows_tile(const RowsParams& p, int b, int& e, int& row0, int& rend, int& ntile) {
     const int xcd = b % kXcds, j = b / kXcds;
-    const int tile = xcd + kXcds * (j / p.n_tiles);
-    ntile = j % p.n_tiles;
     const int lane = threadIdx.x % MTS_WAVE;
+    int tile = xcd + kXcds * (j / p.n_tiles);
+    ntile = j % p.n_tiles;
+    if (p.xcd_ranges) {
+        // m-tiles of the launch: the first (total % 8) XCDs take one more than the others
+        int mine = 0;
+        for (int le = lane; le < p.E; le += MTS_WAVE) mine += (p.expert_start[le + 1] - p.expert_start[le] + BM - 1) / BM;
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) mine += __shfl_xor(mine, o, MTS_WAVE);
+        const int per = mine / kXcds, rem = mine % kXcds;
+        const int k = j / p.n_tiles;
+        if (k >= per + (xcd < rem ? 1 : 0)) return false;
+        tile = xcd * per + (xcd < rem ? xcd : rem) + k;
+    }
     int seen = 0;
     for (int e0 = 0; e0 < p.E; e0 += MTS_WAVE) {
         const int le = e0 + lane;
@@ -1520,10 +1545,21 @@ int64_t m_tiles(int64_t TK, int E) {
     return a < TK ? a : TK;
 }
 
+// MTS_XCD_RANGES=0 selects the round-robin deal of m-tiles to XCDs (tuning runs only)
+int xcd_ranges_choice() {
+    static int choice = -1;
+    if (choice < 0) {
+        const char* s = getenv("MTS_XCD_RANGES");
+        choice = (s && atoi(s) == 0) ? 0 : 1;
+    }
+    return choice;
+}
+
 template <class T, int EPI>
 dim3 rows_grid(RowsParams& p, int64_t TK) {
     const int per_block = (EPI == EPI_SWIGLU) ? T::BN / 2 : T::BN;
     p.n_tiles = (p.N + per_block - 1) / per_block;
+    p.xcd_ranges = xcd_ranges_choice();
     const int64_t m_groups = (m_tiles<T>(TK, p.E) + kXcds - 1) / kXcds;
     return dim3((unsigned)(m_groups * kXcds * p.n_tiles));
 }
@@ -1667,29 +1703,32 @@ extern "C" int mts_moe_ds_partials(int I) { return dy1_partials(I); }
 #endif
 
 extern "C" int MTS_GEMM_ENTRY(mts_moe_fwd_gateup_swiglu)(const void* x, const void* w1, const int32_t* x_gather,
-                                         const int32_t* expert_start, int64_t T, int K, int E,
+                                         const int32_t* expert_start, const void* weights,
+                                         const int32_t* s_scatter, int64_t T, int K, int E,
                                          int H, int I, int act_dtype, void* pre_act,
                                          void* post_act, void* stream) {
 #ifndef MTS_GEMM_F16
-    if (act_dtype == MTS_F16) return mts_moe_fwd_gateup_swiglu_f16(x, w1, x_gather, expert_start, T, K, E, H, I, act_dtype, pre_act, post_act, stream);
+    if (act_dtype == MTS_F16) return mts_moe_fwd_gateup_swiglu_f16(x, w1, x_gather, expert_start, weights, s_scatter, T, K, E, H, I, act_dtype, pre_act, post_act, stream);
 #endif
     if (!x || !w1 || !x_gather || !expert_start || !pre_act || !post_act) return MTS_ERR_NULL;
+    if ((weights != nullptr) != (s_scatter != nullptr)) return MTS_ERR_NULL;   // the routing weight needs the row -> entry map
     if (T <= 0 || K < 1) return MTS_ERR_SHAPE;
     if (act_dtype == MTS_F32) {
         if (E < 1 || E > MTS_MAX_EXPERTS || H < 1 || I < 1 || T * K > 0x7fffffffLL) return MTS_ERR_SHAPE;
         return mts_f32_rows(1, (const float*)x, H, x_gather, (const float*)w1, 2 * I, I, H, expert_start, E, T * K,
-                            (float*)pre_act, (float*)post_act, nullptr, nullptr, nullptr, nullptr, 0,
+                            (float*)pre_act, (float*)post_act, nullptr, (const float*)weights, s_scatter, nullptr, 0,
                             (hipStream_t)stream);
     }
     if (act_dtype != MTS_GEMM_DTYPE) return MTS_ERR_DTYPE;
     int rc = check_common(T * K, E, H, I);
     if (rc) return rc;
-    if (!mts_aligned16(x) || !mts_aligned16(w1)) return MTS_ERR_ALIGN;
+    if (!mts_aligned16(x) || !mts_aligned16(w1) || !mts_aligned16(pre_act) || !mts_aligned16(post_act)) return MTS_ERR_ALIGN;
     RowsParams p = {};
     p.A = (const bf16_t*)x; p.a_rows = T; p.lda = H; p.a_gather = x_gather;
     p.B = (const bf16_t*)w1; p.b_rows = 2 * I;
     p.N = I; p.Kdim = H; p.expert_start = expert_start; p.E = E;
     p.C = (bf16_t*)pre_act; p.C2 = (bf16_t*)post_act; p.TK = T * K;
+    p.route_w = (const bf16_t*)weights; p.s_scatter = s_scatter;
     return launch_rows_any<EPI_SWIGLU>(K_GATEUP, p, T * K, (hipStream_t)stream);
 }
 
@@ -1708,7 +1747,7 @@ extern "C" int MTS_GEMM_ENTRY(mts_moe_fwd_down)(const void* post_act, const void
     if (act_dtype != MTS_GEMM_DTYPE) return MTS_ERR_DTYPE;
     int rc = check_common(TK, E, H, I);
     if (rc) return rc;
-    if (!mts_aligned16(post_act) || !mts_aligned16(w2)) return MTS_ERR_ALIGN;
+    if (!mts_aligned16(post_act) || !mts_aligned16(w2) || !mts_aligned16(y)) return MTS_ERR_ALIGN;
     RowsParams p = {};
     p.A = (const bf16_t*)post_act; p.a_rows = TK; p.lda = I; p.a_gather = nullptr;
     p.B = (const bf16_t*)w2; p.b_rows = H;
@@ -1732,7 +1771,7 @@ extern "C" int MTS_GEMM_ENTRY(mts_moe_bwd_dy1)(const void* d_out, const void* w2
     if (act_dtype == MTS_F16) return mts_moe_bwd_dy1_f16(d_out, w2t, w2_as_stored, pre_act, weights, x_gather, s_scatter, expert_start, T, K, E, H, I, act_dtype, d_pre_act, weighted_act, ds_partial, stream);
 #endif
     if (!d_out || !w2t || !pre_act || !weights || !x_gather || !s_scatter || !expert_start ||
-        !d_pre_act || !weighted_act || !ds_partial)
+        !d_pre_act || !ds_partial)
         return MTS_ERR_NULL;
     if (T <= 0 || K < 1) return MTS_ERR_SHAPE;
     if (act_dtype == MTS_F32) {
@@ -1744,7 +1783,9 @@ extern "C" int MTS_GEMM_ENTRY(mts_moe_bwd_dy1)(const void* d_out, const void* w2
     if (act_dtype != MTS_GEMM_DTYPE) return MTS_ERR_DTYPE;
     int rc = check_common(T * K, E, H, I);
     if (rc) return rc;
-    if (!mts_aligned16(d_out) || !mts_aligned16(w2t)) return MTS_ERR_ALIGN;
+    if (!mts_aligned16(d_out) || !mts_aligned16(w2t) || !mts_aligned16(pre_act) || !mts_aligned16(d_pre_act) ||
+        !mts_aligned16(weighted_act))
+        return MTS_ERR_ALIGN;
     RowsParams p = {};
     p.A = (const bf16_t*)d_out; p.a_rows = T; p.lda = H; p.a_gather = x_gather;
     p.B = (const bf16_t*)w2t; p.b_rows = I;
@@ -1752,6 +1793,7 @@ extern "C" int MTS_GEMM_ENTRY(mts_moe_bwd_dy1)(const void* d_out, const void* w2
     p.C = (bf16_t*)d_pre_act; p.C2 = (bf16_t*)weighted_act;
     p.pre_act = (const bf16_t*)pre_act; p.route_w = (const bf16_t*)weights;
     p.s_scatter = s_scatter; p.ds_part = ds_partial; p.np = mts_moe_ds_partials(I); p.TK = T * K;
+    if (!weighted_act) return launch_rows_any<EPI_DY1N>(K_DY1, p, T * K, (hipStream_t)stream, w2_as_stored != 0);
     return launch_rows_any<EPI_DY1>(K_DY1, p, T * K, (hipStream_t)stream, w2_as_stored != 0);
 }
 
@@ -1771,7 +1813,7 @@ extern "C" int MTS_GEMM_ENTRY(mts_moe_bwd_dx)(const void* d_pre_act, const void*
     if (act_dtype != MTS_GEMM_DTYPE) return MTS_ERR_DTYPE;
     int rc = check_common(TK, E, H, I);
     if (rc) return rc;
-    if (!mts_aligned16(d_pre_act) || !mts_aligned16(w1t)) return MTS_ERR_ALIGN;
+    if (!mts_aligned16(d_pre_act) || !mts_aligned16(w1t) || !mts_aligned16(dx_expanded)) return MTS_ERR_ALIGN;
     RowsParams p = {};
     p.A = (const bf16_t*)d_pre_act; p.a_rows = TK; p.lda = 2 * I; p.a_gather = nullptr;
     p.B = (const bf16_t*)w1t; p.b_rows = H;
@@ -1804,7 +1846,7 @@ extern "C" int MTS_GEMM_ENTRY(mts_moe_bwd_dw2)(const void* d_out, const void* we
     if (act_dtype != MTS_GEMM_DTYPE) return MTS_ERR_DTYPE;
     int rc = check_common(T * K, E, H, I);
     if (rc) return rc;
-    if (!mts_aligned16(d_out) || !mts_aligned16(weighted_act)) return MTS_ERR_ALIGN;
+    if (!mts_aligned16(d_out) || !mts_aligned16(weighted_act) || !mts_aligned16(d_w2)) return MTS_ERR_ALIGN;
     DwParams p = {};
     p.P = (const bf16_t*)d_out; p.p_rows = T; p.p_gather = x_gather;
     p.Q = (const bf16_t*)weighted_act; p.q_rows = T * K; p.q_gather = nullptr;
@@ -1829,7 +1871,7 @@ extern "C" int MTS_GEMM_ENTRY(mts_moe_bwd_dw1)(const void* d_pre_act, const void
     if (act_dtype != MTS_GEMM_DTYPE) return MTS_ERR_DTYPE;
     int rc = check_common(T * K, E, H, I);
     if (rc) return rc;
-    if (!mts_aligned16(d_pre_act) || !mts_aligned16(x)) return MTS_ERR_ALIGN;
+    if (!mts_aligned16(d_pre_act) || !mts_aligned16(x) || !mts_aligned16(d_w1)) return MTS_ERR_ALIGN;
     DwParams p = {};
     p.P = (const bf16_t*)d_pre_act; p.p_rows = T * K; p.p_gather = nullptr;
     p.Q = (const bf16_t*)x; p.q_rows = T; p.q_gather = x_gather;
@@ -1866,7 +1908,7 @@ extern "C" int MTS_GEMM_ENTRY(mts_moe_bwd_joint)(const void* d_out, const void* 
     if (rc) return rc;
     if (!bwd_joint_ok(H, I)) return MTS_ERR_SHAPE;
     if (!mts_aligned16(d_out) || !mts_aligned16(weighted_act) || !mts_aligned16(d_pre_act) || !mts_aligned16(x) ||
-        !mts_aligned16(w1))
+        !mts_aligned16(w1) || !mts_aligned16(dx_expanded) || !mts_aligned16(d_w1) || !mts_aligned16(d_w2))
         return MTS_ERR_ALIGN;
     BwdJointParams q = {};
     q.dw1.P = (const bf16_t*)d_pre_act; q.dw1.p_rows = TK; q.dw1.p_gather = nullptr;

@@ -116,6 +116,7 @@ __global__ __launch_bounds__(kThreads) void rows_gemm_f32_kernel(Rows32 p) {
         const bool rok = row < rend;
         float s = 0.f, dsp = 0.f;
         if (EPI == E32_DY1 && rok) s = p.route_w[p.s_scatter[row]];
+        if (EPI == E32_SWIGLU) s = (rok && p.route_w) ? p.route_w[p.s_scatter[row]] : 1.f;   // post_act may carry the routing weight
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int n = n0 + tx * 4 + j;
@@ -126,7 +127,7 @@ __global__ __launch_bounds__(kThreads) void rows_gemm_f32_kernel(Rows32 p) {
                 const float g = acc[0][i][j], u = acc[NB - 1][i][j];
                 p.C[(int64_t)row * (2 * p.N) + n] = g;
                 p.C[(int64_t)row * (2 * p.N) + p.N + n] = u;
-                p.C2[(int64_t)row * p.N + n] = g * sigmoid32(g) * u;
+                p.C2[(int64_t)row * p.N + n] = g * sigmoid32(g) * u * s;
             } else {
                 const int64_t o = (int64_t)row * (2 * p.N) + n;
                 const float g = p.pre_act[o], u = p.pre_act[o + p.N];
@@ -135,7 +136,7 @@ __global__ __launch_bounds__(kThreads) void rows_gemm_f32_kernel(Rows32 p) {
                 const float silu = g * sig;
                 const float y1 = silu * u;
                 dsp += a * y1;
-                p.C2[(int64_t)row * p.N + n] = s * y1;
+                if (p.C2) p.C2[(int64_t)row * p.N + n] = s * y1;
                 const float da = a * s;
                 p.C[o] = da * (silu * (1.0f - sig) + sig) * u;
                 p.C[o + p.N] = da * silu;
@@ -239,6 +240,7 @@ int mts_f32_dw(const float* P, const int32_t* p_gather, const float* Q, const in
     if (grid.y > 65535 || grid.z > 65535) return MTS_ERR_SHAPE;
     if (grad_dtype == MTS_F32) dw_gemm_f32_kernel<float><<<grid, kThreads, 0, s>>>(p);
     else if (grad_dtype == MTS_BF16) dw_gemm_f32_kernel<bf16_t><<<grid, kThreads, 0, s>>>(p);
+    else if (grad_dtype == MTS_F16) dw_gemm_f32_kernel<mts_f16_t><<<grid, kThreads, 0, s>>>(p);
     else return MTS_ERR_DTYPE;
     MTS_CHECK_LAUNCH();
     return MTS_OK;

@@ -12,6 +12,7 @@ import re
 import shutil
 import subprocess
 import sys
+import tempfile
 
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(os.path.dirname(PKG_DIR), "csrc")
@@ -39,24 +40,45 @@ def find_hipcc() -> str:
     raise RuntimeError("hipcc not found; set HIPCC or install ROCm")
 
 
-def build_library(verbose: bool = False, resource_report: bool = False) -> str:
-    os.makedirs(LIB_DIR, exist_ok=True)
-    cmd = [find_hipcc(), *FLAGS, f"-I{INCLUDE}", f"-I{CSRC}"]
+def build_library(verbose: bool = False, resource_report: bool = False, out: str | None = None,
+                  defines: tuple = ()) -> str:
+    """Compile every source (one hipcc process each, side by side) and link the shared library."""
+    out = out or LIB_PATH
+    os.makedirs(os.path.dirname(out), exist_ok=True)
+    hipcc = find_hipcc()
+    objdir = tempfile.mkdtemp(prefix="mts_build_")
+    try:
+        base = [hipcc, *[f for f in FLAGS if f != "-shared"], f"-I{INCLUDE}", f"-I{CSRC}", *[f"-D{d}" for d in defines]]
+        if resource_report:
+            base.append("-Rpass-analysis=kernel-resource-usage")
+        procs = []
+        for src in SOURCES:
+            obj = os.path.join(objdir, src.replace(".hip", ".o"))
+            procs.append((obj, subprocess.Popen(base + ["-c", os.path.join(CSRC, src), "-o", obj],
+                                                stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)))
+        stderr = ""
+        for obj, proc in procs:
+            _, err = proc.communicate()
+            stderr += err
+            if proc.returncode != 0:
+                raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{_quiet(err)}")
+        tmp = out + ".tmp"
+        link = subprocess.run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *[o for o, _ in procs], "-o", tmp],
+                              capture_output=True, text=True)
+        if link.returncode != 0:
+            raise RuntimeError(f"link failed ({link.returncode}):\n{_quiet(link.stderr)}")
+        os.replace(tmp, out)
+    finally:
+        shutil.rmtree(objdir, ignore_errors=True)
     if resource_report:
-        cmd.append("-Rpass-analysis=kernel-resource-usage")
-    cmd += [os.path.join(CSRC, s) for s in SOURCES]
-    tmp = LIB_PATH + ".tmp"
-    cmd += ["-o", tmp]
-    proc = subprocess.run(cmd, capture_output=True, text=True)
-    err = "\n".join(l for l in proc.stderr.splitlines() if "packed-fp32-ops" not in l)
-    if proc.returncode != 0:
-        raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{err}")
-    os.replace(tmp, LIB_PATH)
-    if resource_report:
-        print(summarise_resources(proc.stderr))
-    elif verbose and err.strip():
-        print(err)
-    return LIB_PATH
+        print(summarise_resources(stderr))
+    elif verbose and _quiet(stderr).strip():
+        print(_quiet(stderr))
+    return out
+
+
+def _quiet(err: str) -> str:
+    return "\n".join(l for l in err.splitlines() if "packed-fp32-ops" not in l)
 
 
 def summarise_resources(text: str) -> str:

@@ -136,6 +136,8 @@ def expert_counts(topk_indices: torch.Tensor, E: int) -> torch.Tensor:
 _OVERLAP = os.environ.get("MTS_NO_OVERLAP", "0") != "1"
 # MTS_NO_JOINT_BWD=1 launches dW2, dW1 and dX separately (on the side streams) even where one launch could hold them
 _JOINT = os.environ.get("MTS_NO_JOINT_BWD", "0") != "1"
+# MTS_WEIGHTED_POST=0: the forward pass writes the unweighted activation and dY1 writes s * a again (tuning runs only)
+_WEIGHTED_POST = os.environ.get("MTS_WEIGHTED_POST", "1") != "0"
 _SIDE_STREAMS: dict = {}
 
 
@@ -197,10 +199,17 @@ class _FusedMoEFunction(torch.autograd.Function):
         w2 = _stage(lib, down_proj, False, x.dtype)
         pre_act = torch.empty(TK, 2 * I, dtype=x.dtype, device=dev)
         post_act = torch.empty(TK, I, dtype=x.dtype, device=dev)
+        weights_flat = top_k_weights.flatten().contiguous()
+        # The routing weight is applied where the activation is formed: post_act = s * silu(g) * u.  The
+        # down projection then yields s * y, the combine is a plain sum, and post_act is at the same time
+        # the `weighted_act` operand of the dW2 GEMM, so it is kept for the backward pass instead of being
+        # written again there (TK * I elements held from forward to backward, and as many fewer written).
+        weighted = _WEIGHTED_POST
         _lib.check(
             lib.mts_moe_fwd_gateup_swiglu(
-                x.data_ptr(), w1.data_ptr(), x_gather.data_ptr(), expert_start.data_ptr(), T, K, E, H, I, act,
-                pre_act.data_ptr(), post_act.data_ptr(), stream,
+                x.data_ptr(), w1.data_ptr(), x_gather.data_ptr(), expert_start.data_ptr(),
+                weights_flat.data_ptr() if weighted else None, s_scatter.data_ptr() if weighted else None,
+                T, K, E, H, I, act, pre_act.data_ptr(), post_act.data_ptr(), stream,
             ),
             "mts_moe_fwd_gateup_swiglu",
         )
@@ -211,18 +220,20 @@ class _FusedMoEFunction(torch.autograd.Function):
             ),
             "mts_moe_fwd_down",
         )
-        weights_flat = top_k_weights.flatten().contiguous()
         out = torch.empty(T, H, dtype=x.dtype, device=dev)
         _lib.check(
             lib.mts_moe_combine(
-                y.data_ptr(), weights_flat.data_ptr(), s_reverse.data_ptr(), T, K, H, act, out.data_ptr(), stream
+                y.data_ptr(), None if weighted else weights_flat.data_ptr(), s_reverse.data_ptr(), T, K, H, act,
+                out.data_ptr(), stream,
             ),
             "mts_moe_combine",
         )
 
         ctx.save_for_backward(
-            x, gate_up_proj, down_proj, pre_act, weights_flat, expert_start, x_gather, s_scatter, s_reverse
+            x, gate_up_proj, down_proj, pre_act, weights_flat, expert_start, x_gather, s_scatter, s_reverse,
+            *((post_act,) if weighted else ()),
         )
+        ctx.weighted = weighted
         ctx.dims = (T, K, E, H, I)
         # fp32 parameters under a bf16 activation dtype: the backward GEMMs that read the weights as
         # stored reuse the casts made here (38 MB a layer at the 768/1024 shape) instead of repeating them
@@ -239,7 +250,7 @@ class _FusedMoEFunction(torch.autograd.Function):
             return None, None, None, None, None
         lib = _lib.load()
         (x, gate_up_proj, down_proj, pre_act, weights_flat, expert_start, x_gather, s_scatter, s_reverse) = (
-            ctx.saved_tensors
+            ctx.saved_tensors[:9]
         )
         T, K, E, H, I = ctx.dims
         TK = T * K
@@ -293,7 +304,8 @@ class _FusedMoEFunction(torch.autograd.Function):
         else:
             w2_bwd = _stage(lib, down_proj, not as_stored, x.dtype)  # [E, H, I] as stored, else [E, I, H]
         d_pre_act = torch.empty(TK, 2 * I, dtype=x.dtype, device=dev)
-        weighted_act = torch.empty(TK, I, dtype=x.dtype, device=dev)
+        # s * silu(g) * u: the forward pass's post_act where it carries the routing weight, else written by dY1
+        weighted_act = ctx.saved_tensors[9] if ctx.weighted else torch.empty(TK, I, dtype=x.dtype, device=dev)
         n_part = lib.mts_moe_ds_partials(I)
         ds_part = torch.empty(TK, n_part, dtype=torch.float32, device=dev)
         _lib.check(
@@ -301,7 +313,7 @@ class _FusedMoEFunction(torch.autograd.Function):
                 dO.data_ptr(), w2_bwd.data_ptr(), int(as_stored), pre_act.data_ptr(), weights_flat.data_ptr(),
                 x_gather.data_ptr(),
                 s_scatter.data_ptr(), expert_start.data_ptr(), T, K, E, H, I, act, d_pre_act.data_ptr(),
-                weighted_act.data_ptr(), ds_part.data_ptr(), stream,
+                None if ctx.weighted else weighted_act.data_ptr(), ds_part.data_ptr(), stream,
             ),
             "mts_moe_bwd_dy1",
         )

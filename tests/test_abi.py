@@ -33,7 +33,7 @@ def test_library_exports_every_declared_symbol():
     for name in _declared():
         assert hasattr(lib, name), f"{name} is declared in mts_moe.h but not exported"
         assert name in _lib.SIGNATURES, f"{name} has no ctypes prototype"
-    assert lib.mts_version() == 1
+    assert lib.mts_version() == 2
     assert lib.mts_error_string(0) == b"ok"
     # argument checks run on the host before any launch: safe without a GPU
     assert lib.mts_router_fwd(None, 4, 8, 2, 1, None, None, None, None, None, None, None, None, None, 0, None, 0, None) == -1

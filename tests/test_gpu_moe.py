@@ -229,8 +229,89 @@ def test_full_size_configs(name, seed, T, imbalanced):
     ref = O.fused_moe(case["x"][pick], case["w1"], case["w2"], case["idx"][pick], case["w"][pick],
                       compute_dtype=torch.float32)
     assert_close_scaled(out[pick], ref, BF16_TOL, "sampled tokens vs CPU oracle")
+    # backward against the CPU oracle as well.  dX and dS of a token depend on that token alone: the sampled
+    # tokens go through the oracle's autograd.  dW1 / dW2 of one expert are sums over that expert's routes:
+    # float64 accumulation of the per-route outer products on the CPU, for a slice of each matrix.
+    _, grads = hip_moe_grads(case["x"], case["w1"], case["w2"], case["idx"], case["w"], case["g"])
+    _, ref_grads = oracle_moe_grads(case["x"][pick], case["w1"], case["w2"], case["idx"][pick], case["w"][pick],
+                                    case["g"][pick])
+    assert_close_scaled(grads[0].cpu()[pick], ref_grads[0], BF16_TOL, "sampled dX vs CPU oracle")
+    assert_close_scaled(grads[3].cpu()[pick], ref_grads[3], BF16_TOL, "sampled dS vs CPU oracle")
+    e = int(np.bincount(case["idx"].flatten().numpy(), minlength=E).argmin())   # the lightest expert: fewest rows
+    dw1_ref, dw2_ref = _expert_weight_gradients_f64(case, e, rows1=slice(0, 2 * I, 61), rows2=slice(0, H, 29))
+    assert_close_scaled(grads[1][e].cpu()[0:2 * I:61], dw1_ref, BF16_TOL, "dW1 slice of one expert vs float64 CPU sum")
+    assert_close_scaled(grads[2][e].cpu()[0:H:29], dw2_ref, BF16_TOL, "dW2 slice of one expert vs float64 CPU sum")
     if name == "config3":
         print("peak HBM allocated (MB):", torch.cuda.max_memory_allocated() / 2**20, flush=True)
+
+
+def _expert_weight_gradients_f64(case, e, rows1, rows2):
+    """Rows ``rows1`` of dW1[e] and ``rows2`` of dW2[e] from the definition (minitrain/kernels/torch_ops.py:
+    122-150 differentiated by hand), accumulated in float64 on the CPU over the routes of expert ``e``."""
+    x, w1, w2, idx, w, g = (case[k] for k in ("x", "w1", "w2", "idx", "w", "g"))
+    tok, k = (idx == e).nonzero(as_tuple=True)
+    xe, ge, se = x[tok].double(), g[tok].double(), w[tok, k].double()
+    W1, W2 = w1[e].double(), w2[e].double()
+    I = W2.shape[1]
+    pre = xe @ W1.T
+    gate, up = pre[:, :I], pre[:, I:]
+    sig = torch.sigmoid(gate)
+    silu = gate * sig
+    act = silu * up
+    d_act = (ge @ W2) * se[:, None]                                   # d loss / d act
+    d_pre = torch.cat([d_act * up * (sig + silu * (1 - sig)), d_act * silu], dim=1)
+    dw1 = d_pre.T[rows1] @ xe                                         # [rows1, H]
+    dw2 = (ge * se[:, None]).T[rows2] @ act                           # [rows2, I]
+    return dw1, dw2
+
+
+def test_unweighted_post_act_path(monkeypatch):
+    """The operator applies the routing weight in the gate/up epilogue and keeps post_act for dW2; the
+    other route through the same C ABI (plain post_act, weighted combine, dY1 writes s*a) stays
+    available to other bindings and must satisfy the same parity."""
+    print("moe unweighted post_act", flush=True)
+    import importlib
+
+    F = importlib.import_module("minitrain_amd.kernels.hip.fused_moe")
+    assert F._WEIGHTED_POST
+    for shape in ((1000, 128, 8, 256, 2), (700, 72, 3, 40, 2)):
+        case = routed_case(81, *shape)
+        args = (case["x"], case["w1"], case["w2"], case["idx"], case["w"], case["g"])
+        a = hip_moe_grads(*args)
+        with monkeypatch.context() as m:
+            m.setattr(F, "_WEIGHTED_POST", False)
+            _compare(case)
+            b = hip_moe_grads(*args)
+        assert_close_scaled(a[0], b[0], 1e-2, "out, weight in the epilogue vs in the combine")
+        for name, u, v in zip(NAMES, a[1], b[1]):
+            assert_close_scaled(u, v, 1e-2, name)
+        assert torch.equal(a[1][3], b[1][3])   # dS does not depend on where the weight is applied
+
+
+@pytest.mark.parametrize("T,H,E,I,skew", [(600, 64, 130, 64, 0.0), (900, 64, 130, 64, 0.6)])
+def test_more_experts_than_a_wave_holds(T, H, E, I, skew):
+    """E > 64: the tile and unit lookups of the GEMM kernels take more than one round of 64 experts
+    (with skew, row chunks of an over-full expert add workspace slots to the lookup)."""
+    print(f"moe many experts T={T} E={E} skew={skew}", flush=True)
+    case = routed_case(90 + T, T, H, E, I, 2)
+    if skew:
+        rng = np.random.Generator(np.random.Philox(T))
+        idx = case["idx"].clone()
+        heavy = torch.from_numpy(rng.random(T) < skew)
+        idx[heavy, 0] = 97                                  # an expert of the second round takes most first choices
+        idx[heavy & (idx[:, 1] == 97), 1] = 3
+        case.update(idx=idx)
+    _compare(case)
+
+
+@pytest.mark.parametrize("wdtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_fp32_activations_with_16bit_parameters(wdtype):
+    """fp32 activations take fp32, bf16 or fp16 expert parameters (widened once per call); the weight
+    gradients come back in the parameter's dtype."""
+    print(f"moe fp32 activations, {wdtype} parameters", flush=True)
+    case = routed_case(95, 300, 64, 4, 96, 2, dtype=torch.float32)
+    case.update(w1=case["w1"].to(wdtype), w2=case["w2"].to(wdtype))
+    _compare(case, tol=1e-5 if wdtype == torch.float32 else 4e-3)   # 16-bit gradients: one rounding of the result
 
 
 def test_moe_block_end_to_end():
