@@ -128,6 +128,22 @@ int mts_moe_route(const int32_t* top_k_index, int64_t T, int K, int E, int block
                   int32_t* tile_expert, int32_t* tile_count, void* workspace,
                   int64_t workspace_bytes, void* stream);
 
+/* mts_moe_route without a workspace argument, for callers that cannot allocate device memory
+ * (code under HIP graph capture, serving loops and harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference.  The chunk counters live in an array inside the library's device
+ * image, MTS_ROUTE_STATIC_BYTES per GPU the library is used on, held until the process ends; the
+ * call allocates and frees nothing.  Same arguments, results and errors as mts_moe_route
+ * otherwise; MTS_ERR_WORKSPACE when mts_moe_route_workspace_bytes(T, K, E) exceeds
+ * MTS_ROUTE_STATIC_BYTES (T*K*E <= 2^28, e.g. 4 M routes over 64 experts).  All calls on one GPU
+ * share that GPU's array: calls that overlap in time on one GPU (different streams) race; calls
+ * on one stream, or ordered by events, do not.  The first call on a device looks the array's
+ * address up (hipGetSymbolAddress), so make one call per device outside a graph capture.   */
+#define MTS_ROUTE_STATIC_BYTES (4 << 20)
+int mts_moe_route_static(const int32_t* top_k_index, int64_t T, int K, int E, int block_m,
+                         int32_t* counts, int32_t* expert_start, int32_t* s_scatter,
+                         int32_t* s_reverse, int32_t* x_gather, int32_t* tile_row_start,
+                         int32_t* tile_expert, int32_t* tile_count, void* stream);
+
 /* ---- capacity-limited dispatch --------------------------------------------
  * The selection rule of TopKRouter._capacity_mask (minitrain/model/moe_router.py:
  * 29-61): per expert, the `capacity` routes with the largest router weight are

@@ -15,6 +15,8 @@
 // of routes that were kept.
 #include "mts_common.h"
 
+#include <mutex>
+
 namespace {
 
 constexpr int kThreads = 256;
@@ -170,26 +172,19 @@ extern "C" int64_t mts_moe_route_workspace_bytes(int64_t T, int K, int E) {
     return n_chunks * E * (int64_t)sizeof(int32_t);
 }
 
-extern "C" int mts_moe_route(const int32_t* top_k_index, int64_t T, int K, int E, int block_m,
-                             int32_t* counts, int32_t* expert_start, int32_t* s_scatter,
-                             int32_t* s_reverse, int32_t* x_gather, int32_t* tile_row_start,
-                             int32_t* tile_expert, int32_t* tile_count, void* workspace,
-                             int64_t workspace_bytes, void* stream) {
-    // the three permutation arrays are optional as a group: without them only the counts,
-    // the expert offsets and (if asked for) the tile list are produced
-    const bool permute = s_scatter || s_reverse || x_gather;
-    if (!top_k_index || !counts || !expert_start || !workspace) return MTS_ERR_NULL;
-    if (permute && (!s_scatter || !s_reverse || !x_gather)) return MTS_ERR_NULL;
-    if (T <= 0 || K < 1 || E < 1 || E > MTS_MAX_EXPERTS || block_m < 1 ||
-        T * (int64_t)K > 0x7fffffffLL)
-        return MTS_ERR_SHAPE;
-    if (workspace_bytes < mts_moe_route_workspace_bytes(T, K, E)) return MTS_ERR_WORKSPACE;
-    hipStream_t s = (hipStream_t)stream;
+namespace {
+
+// the three launches; cnt holds n_chunks * E counters, every one of which is written by the
+// histogram kernel before the scan reads it (nothing has to start at zero)
+int route_launch(const int32_t* top_k_index, int64_t T, int K, int E, int block_m, int32_t* counts,
+                 int32_t* expert_start, int32_t* s_scatter, int32_t* s_reverse, int32_t* x_gather,
+                 int32_t* tile_row_start, int32_t* tile_expert, int32_t* tile_count, int32_t* cnt,
+                 hipStream_t s) {
+    const bool permute = s_scatter != nullptr;
     const int64_t TK = T * K;
     const int64_t n_chunks = (TK + kChunk - 1) / kChunk;
     const int grid = (int)((n_chunks + kWaves - 1) / kWaves);
     const size_t lds = (size_t)kWaves * E * sizeof(int32_t);
-    int32_t* cnt = (int32_t*)workspace;
     route_hist_kernel<<<grid, kThreads, lds, s>>>(top_k_index, TK, E, cnt);
     MTS_CHECK_LAUNCH();
     route_scan_kernel<<<1, 1024, 0, s>>>(cnt, n_chunks, E, TK, block_m, counts, expert_start,
@@ -200,4 +195,73 @@ extern "C" int mts_moe_route(const int32_t* top_k_index, int64_t T, int K, int E
                                                      s_scatter, s_reverse, x_gather);
     MTS_CHECK_LAUNCH();
     return MTS_OK;
+}
+
+// argument checks shared by the two entry points
+int route_check(const int32_t* top_k_index, int64_t T, int K, int E, int block_m, const int32_t* counts,
+                const int32_t* expert_start, const int32_t* s_scatter, const int32_t* s_reverse,
+                const int32_t* x_gather) {
+    // the three permutation arrays are optional as a group: without them only the counts,
+    // the expert offsets and (if asked for) the tile list are produced
+    const bool permute = s_scatter || s_reverse || x_gather;
+    if (!top_k_index || !counts || !expert_start) return MTS_ERR_NULL;
+    if (permute && (!s_scatter || !s_reverse || !x_gather)) return MTS_ERR_NULL;
+    if (T <= 0 || K < 1 || E < 1 || E > MTS_MAX_EXPERTS || block_m < 1 ||
+        T * (int64_t)K > 0x7fffffffLL)
+        return MTS_ERR_SHAPE;
+    return MTS_OK;
+}
+
+// Chunk counters of mts_moe_route_static: one array per GPU the library runs on, held until the
+// process ends.  In host code the symbol is only a handle; the device address is looked up once
+// per device (with that device current) and kept.
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) int32_t scratch[MTS_ROUTE_STATIC_BYTES / sizeof(int32_t)];
+std::mutex scratch_lock;
+int32_t* scratch_ptr[kMaxDevices] = {};
+
+int scratch_of_current_device(int32_t** out) {
+    int dev = -1;
+    hipError_t err = hipGetDevice(&dev);
+    if (err != hipSuccess) return (int)err;
+    if (dev < 0 || dev >= kMaxDevices) return (int)hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> guard(scratch_lock);
+    if (!scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (err != hipSuccess) return (int)err;
+        if (!ptr) return (int)hipErrorInvalidSymbol;
+        scratch_ptr[dev] = (int32_t*)ptr;
+    }
+    *out = scratch_ptr[dev];
+    return MTS_OK;
+}
+
+}  // namespace
+
+extern "C" int mts_moe_route(const int32_t* top_k_index, int64_t T, int K, int E, int block_m,
+                             int32_t* counts, int32_t* expert_start, int32_t* s_scatter,
+                             int32_t* s_reverse, int32_t* x_gather, int32_t* tile_row_start,
+                             int32_t* tile_expert, int32_t* tile_count, void* workspace,
+                             int64_t workspace_bytes, void* stream) {
+    if (!workspace) return MTS_ERR_NULL;
+    const int rc = route_check(top_k_index, T, K, E, block_m, counts, expert_start, s_scatter, s_reverse, x_gather);
+    if (rc) return rc;
+    if (workspace_bytes < mts_moe_route_workspace_bytes(T, K, E)) return MTS_ERR_WORKSPACE;
+    return route_launch(top_k_index, T, K, E, block_m, counts, expert_start, s_scatter, s_reverse, x_gather,
+                        tile_row_start, tile_expert, tile_count, (int32_t*)workspace, (hipStream_t)stream);
+}
+
+extern "C" int mts_moe_route_static(const int32_t* top_k_index, int64_t T, int K, int E, int block_m,
+                                    int32_t* counts, int32_t* expert_start, int32_t* s_scatter,
+                                    int32_t* s_reverse, int32_t* x_gather, int32_t* tile_row_start,
+                                    int32_t* tile_expert, int32_t* tile_count, void* stream) {
+    const int rc = route_check(top_k_index, T, K, E, block_m, counts, expert_start, s_scatter, s_reverse, x_gather);
+    if (rc) return rc;
+    if (mts_moe_route_workspace_bytes(T, K, E) > (int64_t)MTS_ROUTE_STATIC_BYTES) return MTS_ERR_WORKSPACE;
+    int32_t* cnt = nullptr;
+    const int err = scratch_of_current_device(&cnt);
+    if (err) return err;
+    return route_launch(top_k_index, T, K, E, block_m, counts, expert_start, s_scatter, s_reverse, x_gather,
+                        tile_row_start, tile_expert, tile_count, cnt, (hipStream_t)stream);
 }

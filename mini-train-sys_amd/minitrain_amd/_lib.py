@@ -37,6 +37,7 @@ SIGNATURES = {
     "mts_router_logits_bwd": (_i, [_p, _p, _p, _l, _i, _i, _i, _p, _p, _p, _l, _p]),
     "mts_moe_route_workspace_bytes": (_l, [_l, _i, _i]),
     "mts_moe_route": (_i, [_p, _l, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p, _p, _l, _p]),
+    "mts_moe_route_static": (_i, [_p, _l, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p, _p]),
     "mts_moe_capacity_workspace_bytes": (_l, [_l, _i, _i]),
     "mts_moe_capacity_mask": (_i, [_p, _p, _l, _i, _i, _l, _p, _p, _p, _p, _l, _p]),
     "mts_moe_stage_weights": (_i, [_p, _i, _p, _i, _i, _l, _l, _i, _p]),
