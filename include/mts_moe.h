@@ -105,6 +105,36 @@ int mts_router_logits_bwd(const float* dlogits, const void* x, const float* w_r,
                           int H, int E, int act_dtype, void* dx, float* d_w_r,
                           void* workspace, int64_t workspace_bytes, void* stream);
 
+/* ---- the layer's head in three launches -------------------------------------
+ * mts_router_logits_fwd + mts_router_fwd + mts_moe_route as one chain (router projection,
+ * post-process and routing metadata of minitrain/model/moe_router.py:64-90 and
+ * triton/fused_moe.py:74-154): the post-process runs on the logits while they are still in
+ * registers, the routes per expert it counts per block are the chunk histogram of the
+ * routing metadata, and one block reduces the statistics and scans the counts.  Outputs as in
+ * those three calls (logits [T,E] f32 are written for the backward pass; weights_act,
+ * load_balance and load_stats may be NULL).  E <= 16, H a multiple of 4 and at most 1024,
+ * K <= min(E, MTS_MAX_TOP_K).  The statistics are summed in a fixed order of their own: they agree
+ * with mts_router_fwd to rounding, indices and the permutation agree exactly.              */
+int64_t mts_moe_head_workspace_bytes(int64_t T, int K, int E);
+int mts_moe_head_fwd(const void* x, const float* w_r, int64_t T, int H, int E, int K, int normalize,
+                     int act_dtype, float* logits, float* weights, int32_t* indices, void* weights_act,
+                     float* prob_mean, float* z_loss, float* entropy, int32_t* counts,
+                     float* load_balance, float* load_stats, int32_t* expert_start, int32_t* s_scatter,
+                     int32_t* s_reverse, int32_t* x_gather, void* workspace, int64_t workspace_bytes,
+                     void* stream);
+
+/* mts_router_bwd chained into mts_router_logits_bwd: every block of the projection's backward
+ * kernel first forms the logit gradients of its rows from the post-process's saved tensors
+ * (same arithmetic as mts_router_bwd), so dlogits never goes through memory.  dx [T,H] in
+ * act_dtype, d_w_r [E,H] f32.  Gradient inputs may be NULL (zeros) as for mts_router_bwd.      */
+int64_t mts_moe_head_bwd_workspace_bytes(int64_t T, int H, int E);
+int mts_moe_head_bwd(const void* x, const float* w_r, const float* logits, const float* weights,
+                     const int32_t* indices, const int32_t* counts, const float* g_weights,
+                     const void* g_weights_act, const float* g_prob_mean, const float* g_z_loss,
+                     const float* g_load_balance, int64_t T, int H, int E, int K, int normalize,
+                     int act_dtype, void* dx, float* d_w_r, void* workspace, int64_t workspace_bytes,
+                     void* stream);
+
 /* ---- routing metadata ---------------------------------------------------
  * Replaces compute_routing_metadata (minitrain/kernels/triton/fused_moe.py:74-154)
  * and its three kernels (fused_moe_kernels.py:25-234): per-expert counts [E],
@@ -192,10 +222,12 @@ int mts_moe_fwd_down(const void* post_act, const void* w2, const int32_t* expert
                      int64_t TK, int E, int H, int I, int act_dtype, void* y, void* stream);
 
 /* Replaces _token_gather_weighted_sum_kernel (fused_moe_kernels.py:451-498):
- * out[t] = sum_k w[t,k] * y[s_reverse[t*K+k]]  (fp32 sum, one rounding);
- * weights == NULL gives the unweighted sum used for dx.                      */
-int mts_moe_combine(const void* y, const void* weights, const int32_t* s_reverse, int64_t T,
-                    int K, int H, int act_dtype, void* out, void* stream);
+ * out[t] = addend[t] + sum_k w[t,k] * y[s_reverse[t*K+k]]  (fp32 sum, one rounding);
+ * weights == NULL gives the unweighted sum used for dx; addend [T,H] (act_dtype) may be NULL
+ * (zeros): it is the other gradient that reaches x, the router projection's (the sum autograd
+ * forms for minitrain/model/blocks.py:89-96, where x feeds both the router and the experts). */
+int mts_moe_combine(const void* y, const void* weights, const void* addend, const int32_t* s_reverse,
+                    int64_t T, int K, int H, int act_dtype, void* out, void* stream);
 
 /* ---- backward -----------------------------------------------------------
  * Replaces _moe_bwd_down_proj_kernel (fused_moe_kernels.py:500-600):

@@ -27,8 +27,8 @@ struct Vec8<mts_f16_t> {
 
 template <typename ET, int KK, int UN>
 __global__ __launch_bounds__(kThreads) void combine_bf16_kernel(
-    const ET* __restrict__ y, const ET* __restrict__ w, const int32_t* __restrict__ s_rev,
-    int64_t T, int K, int H, ET* __restrict__ out) {
+    const ET* __restrict__ y, const ET* __restrict__ w, const ET* __restrict__ addend,
+    const int32_t* __restrict__ s_rev, int64_t T, int K, int H, ET* __restrict__ out) {
     typedef typename Vec8<ET>::type bf16x8;   // the build's 8-element vector
     const int vec_per_row = H / 8;
     const int64_t chunk = (T + UN - 1) / UN;           // tokens per unrolled slice
@@ -37,11 +37,12 @@ __global__ __launch_bounds__(kThreads) void combine_bf16_kernel(
          i += (int64_t)gridDim.x * kThreads) {
         const int64_t t0 = i / vec_per_row;
         const int c = (int)(i - t0 * vec_per_row);
-        bf16x8 v[UN][KK];
+        bf16x8 v[UN][KK], add[UN];
         float s[UN][KK];
 #pragma unroll
         for (int u = 0; u < UN; ++u) {
             const int64_t t = t0 + u * chunk;
+            add[u] = (addend && t < T) ? *reinterpret_cast<const bf16x8*>(addend + t * H + c * 8) : bf16x8{};
 #pragma unroll
             for (int k = 0; k < KK; ++k) {
                 const bool in = t < T && k < K;
@@ -60,7 +61,7 @@ __global__ __launch_bounds__(kThreads) void combine_bf16_kernel(
             if (t >= T) continue;
             float acc[8];
 #pragma unroll
-            for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+            for (int j = 0; j < 8; ++j) acc[j] = (float)add[u][j];
 #pragma unroll
             for (int k = 0; k < KK; ++k)
 #pragma unroll
@@ -76,8 +77,8 @@ __global__ __launch_bounds__(kThreads) void combine_bf16_kernel(
 // any K: the routes of a token are visited in a loop
 template <typename ET>
 __global__ __launch_bounds__(kThreads) void combine_bf16_anyk_kernel(
-    const ET* __restrict__ y, const ET* __restrict__ w, const int32_t* __restrict__ s_rev,
-    int64_t T, int K, int H, ET* __restrict__ out) {
+    const ET* __restrict__ y, const ET* __restrict__ w, const ET* __restrict__ addend,
+    const int32_t* __restrict__ s_rev, int64_t T, int K, int H, ET* __restrict__ out) {
     typedef typename Vec8<ET>::type bf16x8;
     const int vec_per_row = H / 8;
     const int64_t total = T * (int64_t)vec_per_row;
@@ -86,8 +87,9 @@ __global__ __launch_bounds__(kThreads) void combine_bf16_anyk_kernel(
         const int64_t t = i / vec_per_row;
         const int c = (int)(i - t * vec_per_row);
         float acc[8];
+        const bf16x8 add = addend ? *reinterpret_cast<const bf16x8*>(addend + t * H + c * 8) : bf16x8{};
 #pragma unroll
-        for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+        for (int j = 0; j < 8; ++j) acc[j] = (float)add[j];
         for (int k = 0; k < K; ++k) {
             const int64_t row = s_rev[t * K + k];
             if (row < 0) continue;
@@ -104,8 +106,8 @@ __global__ __launch_bounds__(kThreads) void combine_bf16_anyk_kernel(
 }
 
 __global__ __launch_bounds__(kThreads) void combine_f32_kernel(
-    const float* __restrict__ y, const float* __restrict__ w, const int32_t* __restrict__ s_rev,
-    int64_t T, int K, int H, float* __restrict__ out) {
+    const float* __restrict__ y, const float* __restrict__ w, const float* __restrict__ addend,
+    const int32_t* __restrict__ s_rev, int64_t T, int K, int H, float* __restrict__ out) {
     const int vec_per_row = H / 4;
     const int64_t total = T * (int64_t)vec_per_row;
     for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total;
@@ -113,6 +115,7 @@ __global__ __launch_bounds__(kThreads) void combine_f32_kernel(
         const int64_t t = i / vec_per_row;
         const int c = (int)(i - t * vec_per_row);
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        if (addend) acc = *reinterpret_cast<const f32x4*>(addend + t * H + c * 4);
         for (int k = 0; k < K; ++k) {
             const int64_t row = s_rev[t * K + k];
             if (row < 0) continue;
@@ -208,11 +211,11 @@ int grid_1d(int64_t total) {
 
 }  // namespace
 
-extern "C" int mts_moe_combine(const void* y, const void* weights, const int32_t* s_reverse,
+extern "C" int mts_moe_combine(const void* y, const void* weights, const void* addend, const int32_t* s_reverse,
                                int64_t T, int K, int H, int act_dtype, void* out, void* stream) {
     if (!y || !s_reverse || !out) return MTS_ERR_NULL;
     if (T <= 0 || K < 1 || H < 1) return MTS_ERR_SHAPE;
-    if (!mts_aligned16(y) || !mts_aligned16(out)) return MTS_ERR_ALIGN;
+    if (!mts_aligned16(y) || !mts_aligned16(out) || !mts_aligned16(addend)) return MTS_ERR_ALIGN;
     hipStream_t s = (hipStream_t)stream;
     if (act_dtype == MTS_BF16 || act_dtype == MTS_F16) {
         if (H % 8) return MTS_ERR_SHAPE;
@@ -222,13 +225,13 @@ extern "C" int mts_moe_combine(const void* y, const void* weights, const int32_t
     do {                                                                                                      \
         if (K <= 2)                                                                                           \
             combine_bf16_kernel<ET, 2, UN><<<grid_1d(sliced), kThreads, 0, s>>>(                              \
-                (const ET*)y, (const ET*)weights, s_reverse, T, K, H, (ET*)out);                              \
+                (const ET*)y, (const ET*)weights, (const ET*)addend, s_reverse, T, K, H, (ET*)out);                              \
         else if (K <= 4)                                                                                      \
             combine_bf16_kernel<ET, 4, UN><<<grid_1d(sliced), kThreads, 0, s>>>(                              \
-                (const ET*)y, (const ET*)weights, s_reverse, T, K, H, (ET*)out);                              \
+                (const ET*)y, (const ET*)weights, (const ET*)addend, s_reverse, T, K, H, (ET*)out);                              \
         else                                                                                                  \
             combine_bf16_anyk_kernel<ET><<<grid_1d(T * (int64_t)(H / 8)), kThreads, 0, s>>>(                  \
-                (const ET*)y, (const ET*)weights, s_reverse, T, K, H, (ET*)out);                              \
+                (const ET*)y, (const ET*)weights, (const ET*)addend, s_reverse, T, K, H, (ET*)out);                              \
     } while (0)
         if (act_dtype == MTS_BF16) MTS_COMBINE16(bf16_t);
         else MTS_COMBINE16(mts_f16_t);
@@ -236,7 +239,7 @@ extern "C" int mts_moe_combine(const void* y, const void* weights, const int32_t
     } else if (act_dtype == MTS_F32) {
         if (H % 4) return MTS_ERR_SHAPE;
         combine_f32_kernel<<<grid_1d(T * (int64_t)(H / 4)), kThreads, 0, s>>>(
-            (const float*)y, (const float*)weights, s_reverse, T, K, H, (float*)out);
+            (const float*)y, (const float*)weights, (const float*)addend, s_reverse, T, K, H, (float*)out);
     } else {
         return MTS_ERR_DTYPE;
     }

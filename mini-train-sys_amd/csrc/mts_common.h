@@ -75,3 +75,10 @@ int mts_f32_rows(int epi, const float* A, int lda, const int32_t* a_gather, cons
                  int np, hipStream_t s);
 int mts_f32_dw(const float* P, const int32_t* p_gather, const float* Q, const int32_t* q_gather, int M,
                int N, const int32_t* expert_start, int E, int grad_dtype, void* C, hipStream_t s);
+
+// chained router forward (mts_router_linear.hip), launched by mts_moe_head_fwd (mts_route.hip)
+#define MTS_HEAD_MAX_CHUNKS 512
+void mts_router_head_geometry(int64_t T, int* blocks, int* rows_per_wave);
+int mts_launch_router_head(const void* x, const float* w_r, int64_t T, int H, int E, int K, int normalize, int act_dtype,
+                           float* logits, float* weights, int32_t* indices, void* weights_act, float* partial,
+                           int32_t* cnt, hipStream_t s);

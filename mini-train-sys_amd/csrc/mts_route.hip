@@ -14,6 +14,7 @@
 // counted, gets no row, and its s_reverse entry is -1.  expert_start[E] is the number
 // of routes that were kept.
 #include "mts_common.h"
+#include "mts_router_row.h"
 
 #include <mutex>
 
@@ -51,8 +52,8 @@ __global__ __launch_bounds__(kThreads) void route_hist_kernel(const int32_t* __r
 
 // One block.  Wave w owns experts w, w+nw, ...: exclusive scan over chunks in
 // groups of 64, then an exclusive scan of the totals over experts.
-__global__ __launch_bounds__(1024) void route_scan_kernel(
-    int32_t* __restrict__ cnt, int64_t n_chunks, int E, int64_t TK, int block_m,
+__device__ __forceinline__ void route_scan_block(
+    int32_t* __restrict__ cnt, int64_t n_chunks, int E, int block_m,
     int32_t* __restrict__ counts, int32_t* __restrict__ expert_start,
     int32_t* __restrict__ tile_row_start, int32_t* __restrict__ tile_expert,
     int32_t* __restrict__ tile_count) {
@@ -122,27 +123,56 @@ __global__ __launch_bounds__(1024) void route_scan_kernel(
     }
 }
 
+__global__ __launch_bounds__(1024) void route_scan_kernel(
+    int32_t* __restrict__ cnt, int64_t n_chunks, int E, int64_t TK, int block_m,
+    int32_t* __restrict__ counts, int32_t* __restrict__ expert_start,
+    int32_t* __restrict__ tile_row_start, int32_t* __restrict__ tile_expert,
+    int32_t* __restrict__ tile_count) {
+    (void)TK;
+    route_scan_block(cnt, n_chunks, E, block_m, counts, expert_start, tile_row_start, tile_expert, tile_count);
+}
+
+// One block after the kernel that chains the router projection to the post-process: the scan over
+// that kernel's per-block route counts (the chunks of the scatter that follows) and the reduction
+// of its per-block statistics.
+__global__ __launch_bounds__(1024) void head_finish_kernel(
+    const float* __restrict__ partial, int32_t* __restrict__ cnt, int64_t n_chunks, int E, float inv_t,
+    float inv_routes, float* __restrict__ prob_mean, float* __restrict__ z_loss, float* __restrict__ entropy,
+    int32_t* __restrict__ counts, float* __restrict__ load_balance, float* __restrict__ load_stats,
+    int32_t* __restrict__ expert_start) {
+    // the statistics read the counts before the scan turns them into offsets
+    mts_router::stats_block<1024 / MTS_WAVE>(partial, cnt, (int)n_chunks, E, inv_t, inv_routes, prob_mean, z_loss, entropy,
+                                             nullptr, load_balance, load_stats, threadIdx.x / MTS_WAVE);
+    __syncthreads();
+    route_scan_block(cnt, n_chunks, E, 1, counts, expert_start, nullptr, nullptr, nullptr);
+}
+
+// chunk_len entries per wave (a multiple of 64 is not required); the chunks are the ones the
+// counters in cnt were taken over
 __global__ __launch_bounds__(kThreads) void route_scatter_kernel(
-    const int32_t* __restrict__ idx, int64_t TK, int K, int E, const int32_t* __restrict__ cnt,
+    const int32_t* __restrict__ idx, int64_t TK, int K, int E, int chunk_len, const int32_t* __restrict__ cnt,
     const int32_t* __restrict__ expert_start, int32_t* __restrict__ s_scatter,
     int32_t* __restrict__ s_reverse, int32_t* __restrict__ x_gather) {
     extern __shared__ int32_t lds[];  // [kWaves][E] next free row per expert
     const int wave = threadIdx.x / MTS_WAVE, lane = threadIdx.x % MTS_WAVE;
     const int64_t chunk = (int64_t)blockIdx.x * kWaves + wave;
-    const int64_t base = chunk * kChunk;
-    if (base >= TK) return;  // whole wave leaves; no block barrier below
+    const int64_t cbeg = chunk * chunk_len;
+    if (cbeg >= TK) return;  // whole wave leaves; no block barrier below
+    const int64_t cend = cbeg + chunk_len < TK ? cbeg + chunk_len : TK;
     volatile int32_t* next = lds + wave * E;
     for (int e = lane; e < E; e += MTS_WAVE) next[e] = expert_start[e] + cnt[chunk * E + e];
     const uint64_t lt = lanemask_lt();
+  for (int64_t base = cbeg; base < cend; base += kChunk) {   // kSteps x 64 entries at a time
     int ev[kSteps];
 #pragma unroll
-    for (int s = 0; s < kSteps; ++s) {  // all of the chunk's loads are in flight together
+    for (int s = 0; s < kSteps; ++s) {  // these loads are in flight together
         const int64_t n = base + s * MTS_WAVE + lane;
-        ev[s] = n < TK ? clamp_expert(idx[n], E) : -1;
+        ev[s] = n < cend ? clamp_expert(idx[n], E) : -1;
     }
 #pragma unroll
     for (int s = 0; s < kSteps; ++s) {
         const int64_t n = base + s * MTS_WAVE + lane;
+        if (base + s * MTS_WAVE >= cend) break;   // wave-uniform
         const int e = ev[s];
         const bool valid = e >= 0;
         int pos = -1;
@@ -156,12 +186,13 @@ __global__ __launch_bounds__(kThreads) void route_scatter_kernel(
             if (lane == leader) next[el] = first + __popcll(same);
             todo &= ~same;
         }
-        if (n < TK) s_reverse[n] = pos;
+        if (n < cend) s_reverse[n] = pos;
         if (valid) {
             s_scatter[pos] = (int32_t)n;
             x_gather[pos] = (int32_t)(n / K);
         }
     }
+  }
 }
 
 }  // namespace
@@ -191,7 +222,7 @@ int route_launch(const int32_t* top_k_index, int64_t T, int K, int E, int block_
                                          tile_row_start, tile_expert, tile_count);
     MTS_CHECK_LAUNCH();
     if (!permute) return MTS_OK;
-    route_scatter_kernel<<<grid, kThreads, lds, s>>>(top_k_index, TK, K, E, cnt, expert_start,
+    route_scatter_kernel<<<grid, kThreads, lds, s>>>(top_k_index, TK, K, E, kChunk, cnt, expert_start,
                                                      s_scatter, s_reverse, x_gather);
     MTS_CHECK_LAUNCH();
     return MTS_OK;
@@ -264,4 +295,42 @@ extern "C" int mts_moe_route_static(const int32_t* top_k_index, int64_t T, int K
     if (err) return err;
     return route_launch(top_k_index, T, K, E, block_m, counts, expert_start, s_scatter, s_reverse, x_gather,
                         tile_row_start, tile_expert, tile_count, cnt, (hipStream_t)stream);
+}
+
+extern "C" int64_t mts_moe_head_workspace_bytes(int64_t T, int K, int E) {
+    (void)T;
+    (void)K;
+    return (int64_t)MTS_HEAD_MAX_CHUNKS * (2 * E + 2) * (int64_t)sizeof(float);   // statistics partials, then route counts
+}
+
+extern "C" int mts_moe_head_fwd(const void* x, const float* w_r, int64_t T, int H, int E, int K, int normalize,
+                                int act_dtype, float* logits, float* weights, int32_t* indices, void* weights_act,
+                                float* prob_mean, float* z_loss, float* entropy, int32_t* counts, float* load_balance,
+                                float* load_stats, int32_t* expert_start, int32_t* s_scatter, int32_t* s_reverse,
+                                int32_t* x_gather, void* workspace, int64_t workspace_bytes, void* stream) {
+    if (!prob_mean || !z_loss || !entropy || !counts || !expert_start || !s_scatter || !s_reverse || !x_gather || !workspace)
+        return MTS_ERR_NULL;
+    if (weights_act && act_dtype == MTS_F32) return MTS_ERR_DTYPE;
+    if (T <= 0 || K < 1 || T * (int64_t)K > 0x7fffffffLL) return MTS_ERR_SHAPE;
+    if (workspace_bytes < mts_moe_head_workspace_bytes(T, K, E)) return MTS_ERR_WORKSPACE;
+    if (!mts_aligned16(workspace)) return MTS_ERR_ALIGN;
+    hipStream_t s = (hipStream_t)stream;
+    float* partial = (float*)workspace;
+    int32_t* cnt = (int32_t*)(partial + (int64_t)MTS_HEAD_MAX_CHUNKS * (E + 2));
+    const int rc = mts_launch_router_head(x, w_r, T, H, E, K, normalize, act_dtype, logits, weights, indices, weights_act,
+                                          partial, cnt, s);
+    if (rc) return rc;
+    int blocks, rows_per_wave;
+    mts_router_head_geometry(T, &blocks, &rows_per_wave);
+    const int64_t rows_per_chunk = (int64_t)rows_per_wave * 4;
+    const int64_t n_chunks = (T + rows_per_chunk - 1) / rows_per_chunk;
+    head_finish_kernel<<<1, 1024, 0, s>>>(partial, cnt, n_chunks, E, 1.0f / (float)T, 1.0f / ((float)T * (float)K),
+                                          prob_mean, z_loss, entropy, counts, load_balance, load_stats, expert_start);
+    MTS_CHECK_LAUNCH();
+    const int grid = (int)((n_chunks + kWaves - 1) / kWaves);
+    const size_t lds = (size_t)kWaves * E * sizeof(int32_t);
+    route_scatter_kernel<<<grid, kThreads, lds, s>>>(indices, T * (int64_t)K, K, E, (int)(rows_per_chunk * K), cnt,
+                                                     expert_start, s_scatter, s_reverse, x_gather);
+    MTS_CHECK_LAUNCH();
+    return MTS_OK;
 }

@@ -8,70 +8,14 @@
 // wave with a fixed shuffle tree, over the block through LDS and over blocks by a
 // second one-block kernel, so that results are bit-stable from run to run.
 #include "mts_common.h"
-
-#include <math.h>
+#include "mts_router_row.h"
 
 namespace {
 
+using namespace mts_router;
+
 constexpr int kThreads = 256;
 constexpr int kMaxBlocks = 256;
-constexpr float kLogFloor = -20.72326583694641f;  // log(1e-9): the entropy clamps p at 1e-9
-
-template <int G>
-__device__ __forceinline__ float group_sum(float v) {
-#pragma unroll
-    for (int o = G / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, MTS_WAVE);
-    return v;
-}
-template <int G>
-__device__ __forceinline__ float group_max(float v) {
-#pragma unroll
-    for (int o = G / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, MTS_WAVE));
-    return v;
-}
-
-template <int EP, int G>
-struct RowState {
-    float l[EP];
-    float p[EP];
-    float m, s, L;
-};
-
-template <int EP, int G>
-__device__ __forceinline__ void load_row(const float* __restrict__ logits, int64_t row, int E, int g,
-                                         RowState<EP, G>& r) {
-    const float* src = logits + row * (int64_t)E;
-    if (G == 1 && EP == 8 && E == 8) {
-        const f32x4* v = reinterpret_cast<const f32x4*>(src);
-        f32x4 a = v[0], b = v[1];
-        r.l[0] = a[0]; r.l[1] = a[1]; r.l[2] = a[2]; r.l[3] = a[3];
-        r.l[4 % EP] = b[0]; r.l[5 % EP] = b[1]; r.l[6 % EP] = b[2]; r.l[7 % EP] = b[3];
-    } else {
-#pragma unroll
-        for (int j = 0; j < EP; ++j) {
-            int e = j * G + g;
-            r.l[j] = (e < E) ? src[e] : -INFINITY;
-        }
-    }
-    float m = r.l[0];
-#pragma unroll
-    for (int j = 1; j < EP; ++j) m = fmaxf(m, r.l[j]);
-    m = group_max<G>(m);
-    float s = 0.f;
-#pragma unroll
-    for (int j = 0; j < EP; ++j) {
-        r.p[j] = expf(r.l[j] - m);
-        s += r.p[j];
-    }
-    s = group_sum<G>(s);
-    float inv = 1.0f / s;
-#pragma unroll
-    for (int j = 0; j < EP; ++j) r.p[j] *= inv;
-    r.m = m;
-    r.s = s;
-    r.L = m + logf(s);
-}
-
 template <int EP, int G>
 __global__ __launch_bounds__(kThreads) void router_fwd_kernel(
     const float* __restrict__ logits, int64_t T, int E, int K, int normalize,
@@ -95,48 +39,14 @@ __global__ __launch_bounds__(kThreads) void router_fwd_kernel(
         RowState<EP, G> r;
         load_row<EP, G>(logits, live ? row : 0, E, g, r);
 
-        uint32_t taken = 0;
-#pragma unroll
-        for (int j = 0; j < EP; ++j)
-            if (j * G + g >= E) taken |= 1u << j;
-
         float sel_p[MTS_MAX_TOP_K];
         int sel_e[MTS_MAX_TOP_K];
-        float mass = 0.f;
+        float mass;
+        select_top_k<EP, G>(r, E, K, g, sel_p, sel_e, mass);
 #pragma unroll
-        for (int k = 0; k < MTS_MAX_TOP_K; ++k) {
-            sel_p[k] = 0.f;
-            sel_e[k] = 0;
-            if (k < K) {
-                float bv = -INFINITY;
-                int be = 0x7fffffff;
+        for (int k = 0; k < MTS_MAX_TOP_K; ++k)
 #pragma unroll
-                for (int j = 0; j < EP; ++j) {
-                    int e = j * G + g;
-                    bool free_slot = !((taken >> j) & 1u);
-                    if (free_slot && (r.l[j] > bv || (r.l[j] == bv && e < be))) {
-                        bv = r.l[j];
-                        be = e;
-                    }
-                }
-#pragma unroll
-                for (int o = G / 2; o > 0; o >>= 1) {
-                    float ov = __shfl_xor(bv, o, MTS_WAVE);
-                    int oe = __shfl_xor(be, o, MTS_WAVE);
-                    if (ov > bv || (ov == bv && oe < be)) {
-                        bv = ov;
-                        be = oe;
-                    }
-                }
-                if (be % G == g) taken |= 1u << (be / G);
-#pragma unroll
-                for (int j = 0; j < EP; ++j) csum[j] += (live && j * G + g == be) ? 1 : 0;
-                float pk = expf(bv - r.m) / r.s;
-                sel_p[k] = pk;
-                sel_e[k] = be;
-                mass += pk;
-            }
-        }
+            for (int j = 0; j < EP; ++j) csum[j] += (live && k < K && j * G + g == sel_e[k]) ? 1 : 0;
         if (live && g == 0) {
             float inv = normalize ? 1.0f / fmaxf(mass, 1.1920928955078125e-07f) : 1.0f;
 #pragma unroll
@@ -211,95 +121,13 @@ __global__ __launch_bounds__(kThreads) void router_fwd_kernel(
     }
 }
 
-// One block: wave w reduces columns w, w+4, ...; lanes stride over the per-block
-// partials and the lane sums meet in a fixed shuffle tree (bit-stable).  Also the routes per
-// expert and, if asked for, the load-balancing term E * sum_e (routes_e / routes) * mean_prob_e.
 __global__ __launch_bounds__(kThreads) void router_stats_kernel(
     const float* __restrict__ partial, const int32_t* __restrict__ partial_counts, int nblocks, int E,
     float inv_t, float inv_routes, float* __restrict__ prob_mean, float* __restrict__ z_loss,
     float* __restrict__ entropy, int32_t* __restrict__ counts, float* __restrict__ load_balance,
     float* __restrict__ load_stats) {
-    __shared__ float prod[MTS_MAX_EXPERTS];   // fraction of routes x mean probability, per expert
-    __shared__ float share[MTS_MAX_EXPERTS];  // fraction of routes, per expert
-    __shared__ int routes_of[MTS_MAX_EXPERTS];
-    __shared__ float entropy_s;
-    const int wave = threadIdx.x / MTS_WAVE, lane = threadIdx.x % MTS_WAVE;
-    for (int i = wave; i < E + 2; i += kThreads / MTS_WAVE) {
-        float v = 0.f;
-        for (int b = lane; b < nblocks; b += MTS_WAVE) v += partial[(int64_t)b * (E + 2) + i];
-        v = wave_sum(v) * inv_t;
-        int c = 0;
-        if (i < E) {
-            for (int b = lane; b < nblocks; b += MTS_WAVE) c += partial_counts[(int64_t)b * E + i];
-#pragma unroll
-            for (int o = 32; o > 0; o >>= 1) c += __shfl_xor(c, o, MTS_WAVE);
-        }
-        if (lane == 0) {
-            if (i < E) {
-                prob_mean[i] = v;
-                prod[i] = (float)c * inv_routes * v;
-                share[i] = (float)c * inv_routes;
-                routes_of[i] = c;
-                if (counts) counts[i] = c;
-            } else if (i == E) {
-                z_loss[0] = v;
-            } else {
-                entropy[0] = v;
-                entropy_s = v;
-            }
-        }
-    }
-    if (!load_balance && !load_stats) return;
-    __syncthreads();
-    // E * sum_e f_e * pbar_e, summed in a fixed order by one wave
-    if (wave == 0 && load_balance) {
-        float v = 0.f;
-        for (int e = lane; e < E; e += MTS_WAVE) v += prod[e];
-        v = wave_sum(v);
-        if (lane == 0) load_balance[0] = (float)E * v;
-    }
-    // load statistics of the router module (minitrain/model/moe_router.py:113-135) from the route
-    // fractions: [0,E) the fractions, then the largest and smallest route count, the coefficient
-    // of variation (population standard deviation x E), largest fraction x E, the number of
-    // experts without a route, a zero (the dropped-route fraction of dropless routing) and the
-    // entropy over log E
-    if (wave == 1 % (kThreads / MTS_WAVE) && load_stats) {
-        float sum = 0.f, hi = 0.f, dead = 0.f;
-        int most = 0, fewest = 0x7fffffff;
-        for (int e = lane; e < E; e += MTS_WAVE) {
-            const float f = share[e];
-            load_stats[e] = f;
-            sum += f;
-            hi = fmaxf(hi, f);
-            most = max(most, routes_of[e]);
-            fewest = min(fewest, routes_of[e]);
-            dead += routes_of[e] == 0 ? 1.f : 0.f;
-        }
-        sum = wave_sum(sum);
-        dead = wave_sum(dead);
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) {
-            hi = fmaxf(hi, __shfl_xor(hi, o, MTS_WAVE));
-            most = max(most, __shfl_xor(most, o, MTS_WAVE));
-            fewest = min(fewest, __shfl_xor(fewest, o, MTS_WAVE));
-        }
-        const float mean = sum / (float)E;
-        float var = 0.f;
-        for (int e = lane; e < E; e += MTS_WAVE) {
-            const float d = share[e] - mean;
-            var += d * d;
-        }
-        var = wave_sum(var) / (float)E;
-        if (lane == 0) {
-            load_stats[E] = (float)most;
-            load_stats[E + 1] = (float)fewest;
-            load_stats[E + 2] = sqrtf(var) * (float)E;
-            load_stats[E + 3] = hi * (float)E;
-            load_stats[E + 4] = dead;
-            load_stats[E + 5] = 0.f;
-            load_stats[E + 6] = entropy_s / (E > 1 ? logf((float)E) : 1.0f);
-        }
-    }
+    stats_block<kThreads / MTS_WAVE>(partial, partial_counts, nblocks, E, inv_t, inv_routes, prob_mean, z_loss, entropy,
+                                     counts, load_balance, load_stats, threadIdx.x / MTS_WAVE);
 }
 
 template <int EP, int G>
@@ -336,37 +164,11 @@ __global__ __launch_bounds__(kThreads) void router_bwd_kernel(
         int64_t rr = live ? row : 0;
         RowState<EP, G> r;
         load_row<EP, G>(logits, rr, E, g, r);
-        float dp[EP], extra[EP];
-#pragma unroll
-        for (int j = 0; j < EP; ++j) {
-            dp[j] = gp[j];
-            extra[j] = 0.f;
-        }
-        float wdot = 0.f;
-        if (normalize) {
-            for (int k = 0; k < K; ++k) wdot += weights[rr * K + k] * grad_w(rr * K + k);
-        }
-        for (int k = 0; k < K; ++k) {
-            int e = indices[rr * K + k];
-            float gw = grad_w(rr * K + k);
-            float w = weights[rr * K + k];
-#pragma unroll
-            for (int j = 0; j < EP; ++j) {
-                if (j * G + g == e) {
-                    if (normalize) extra[j] += w * (gw - wdot);
-                    else dp[j] += gw;
-                }
-            }
-        }
-        float dot = 0.f;
-#pragma unroll
-        for (int j = 0; j < EP; ++j) dot += r.p[j] * dp[j];
-        dot = group_sum<G>(dot);
+        float o[EP];
+        row_logit_gradient<EP, G>(r, gp, gz, K, normalize, g, weights + rr * K, indices + rr * K,
+                                  [&](int k) { return grad_w(rr * K + k); }, o);
         if (live) {
             float* dst = dlogits + row * (int64_t)E;
-            float o[EP];
-#pragma unroll
-            for (int j = 0; j < EP; ++j) o[j] = r.p[j] * (dp[j] - dot) + gz * r.L * r.p[j] + extra[j];
             if (G == 1 && EP == 8 && E == 8) {
                 f32x4* v = reinterpret_cast<f32x4*>(dst);
                 v[0] = f32x4{o[0], o[1], o[2], o[3]};

@@ -3,6 +3,7 @@
 // copy of the activations is made; every sum runs in a fixed order (no float atomics).
 // All three kernels are VALU/HBM bound: 2*T*H*E FLOP forward, twice that backward.
 #include "mts_common.h"
+#include "mts_router_row.h"
 
 namespace {
 
@@ -163,6 +164,178 @@ __global__ __launch_bounds__(kFwdThreads) void router_logits_fwd_kernel(const XT
     }
 }
 
+// ---------------------------------------------------------------------------
+// The router projection chained to the post-process.  The block takes a contiguous range of
+// rows, a wave a contiguous part of it; the 4 rows x E logits a wave has just summed sit one per
+// lane (pair), so lanes 0..3 collect a row each with cross-lane reads and run the post-process
+// on it (softmax, top-k on the logits, weights) without the logits making a round trip through
+// memory; the logits are still written, for the backward pass.  Per block: the sums of the
+// statistics (fixed order) and the routes per expert, which are at the same time the chunk
+// histogram of the routing metadata (chunk = the entries of the block's rows).
+// ---------------------------------------------------------------------------
+template <typename XT, int EP, int PASSES>
+__global__ __launch_bounds__(kFwdThreads) void router_head_kernel(
+    const XT* __restrict__ x, const float* __restrict__ w, int64_t T, int H, int E, int K, int normalize,
+    int rows_per_wave, float* __restrict__ logits, float* __restrict__ weights, int32_t* __restrict__ indices,
+    void* __restrict__ weights_act, int act_dtype, float* __restrict__ partial, int32_t* __restrict__ cnt) {
+    using namespace mts_router;
+    extern __shared__ __attribute__((aligned(16))) float w_lds[];   // [E][H]
+#pragma unroll 8
+    for (int i = threadIdx.x * 4; i < E * H; i += kFwdThreads * 4)
+        *reinterpret_cast<f32x4*>(w_lds + i) = *reinterpret_cast<const f32x4*>(w + i);
+    constexpr int WAVES = kFwdThreads / MTS_WAVE;
+    const int lane = threadIdx.x % MTS_WAVE, wave = threadIdx.x / MTS_WAVE;
+    const int64_t beg = ((int64_t)blockIdx.x * WAVES + wave) * rows_per_wave;
+    const int64_t end = beg + rows_per_wave < T ? beg + rows_per_wave : T;
+    typedef typename RawVec<XT>::type raw_t;
+    raw_t cur[PASSES][kRows], nxt[PASSES][kRows];
+    auto load_group = [&](raw_t (&dst)[PASSES][kRows], int64_t r0) {
+#pragma unroll
+        for (int ps = 0; ps < PASSES; ++ps) {
+            const int c = lane * 4 + ps * MTS_WAVE * 4;
+#pragma unroll
+            for (int r = 0; r < kRows; ++r) {
+                const bool ok = c < H && r0 + r < end;
+                dst[ps][r] = load_raw(x + (ok ? (r0 + r) * H + c : 0));   // a masked lane reads element 0; its weights are skipped
+            }
+        }
+    };
+    if (beg < end) load_group(cur, beg);
+    __syncthreads();
+
+    // statistics of the rows this lane post-processes (lanes 0..3)
+    float psum[EP], zsum = 0.f, hsum = 0.f;
+    int csum[EP];
+#pragma unroll
+    for (int e = 0; e < EP; ++e) {
+        psum[e] = 0.f;
+        csum[e] = 0;
+    }
+    for (int64_t r0 = beg; r0 < end; r0 += kRows) {
+        if (r0 + kRows < end) load_group(nxt, r0 + kRows);
+        float acc[kRows][EP];
+#pragma unroll
+        for (int r = 0; r < kRows; ++r)
+#pragma unroll
+            for (int e = 0; e < EP; ++e) acc[r][e] = 0.f;
+#pragma unroll
+        for (int ps = 0; ps < PASSES; ++ps) {
+            const int c = lane * 4 + ps * MTS_WAVE * 4;
+            if (c < H) {
+                f32x4 xv[kRows];
+#pragma unroll
+                for (int r = 0; r < kRows; ++r) {
+                    const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+                    xv[r] = r0 + r < end ? widen(cur[ps][r]) : z;
+                }
+#pragma unroll
+                for (int e = 0; e < EP; ++e) {
+                    const f32x4 wv = *reinterpret_cast<const f32x4*>(w_lds + (e < E ? e : 0) * H + c);
+#pragma unroll
+                    for (int r = 0; r < kRows; ++r)
+                        acc[r][e] += xv[r][0] * wv[0] + xv[r][1] * wv[1] + xv[r][2] * wv[2] + xv[r][3] * wv[3];
+                }
+            }
+        }
+#pragma unroll
+        for (int ps = 0; ps < PASSES; ++ps)
+#pragma unroll
+            for (int r = 0; r < kRows; ++r) cur[ps][r] = nxt[ps][r];
+        static_assert(kRows * EP == 32 || kRows * EP == 64, "reduction layout");
+        constexpr int NV = kRows * EP;
+        float v[NV];
+#pragma unroll
+        for (int r = 0; r < kRows; ++r)
+#pragma unroll
+            for (int e = 0; e < EP; ++e) v[r * EP + e] = acc[r][e];
+        int idx = 0;
+        reduce_scatter<NV, NV, 32>(v, lane, idx);
+        const float mine = v[0];   // value `idx` of the group: row r0 + idx / EP, expert idx % EP
+        {
+            const int r = idx / EP, e = idx % EP;
+            const bool writer = NV == 64 ? true : (lane & 1) == 0;
+            if (writer && e < E && r0 + r < end) logits[(r0 + r) * E + e] = mine;
+        }
+        // value i of the group ends up in lane i (64 values) or in lanes 2i and 2i+1 (32 values):
+        // lane L < 4 collects the logits of row r0 + L
+        constexpr int SPREAD = NV == 64 ? 1 : 2;
+        const int my = lane & (kRows - 1);
+        RowState<EP, 1> rs;
+#pragma unroll
+        for (int e = 0; e < EP; ++e) {
+            const float got = __shfl(mine, (my * EP + e) * SPREAD, MTS_WAVE);
+            rs.l[e] = e < E ? got : -INFINITY;
+        }
+        const int64_t row = r0 + my;
+        const bool live = lane < kRows && row < end;
+        softmax_row<EP, 1>(rs);
+        float sel_p[MTS_MAX_TOP_K], mass;
+        int sel_e[MTS_MAX_TOP_K];
+        select_top_k<EP, 1>(rs, E, K, 0, sel_p, sel_e, mass);
+        if (live) {
+            const float inv = normalize ? 1.0f / fmaxf(mass, 1.1920928955078125e-07f) : 1.0f;
+#pragma unroll
+            for (int k = 0; k < MTS_MAX_TOP_K; ++k) {
+                if (k < K) {
+                    const float wk = sel_p[k] * inv;
+                    weights[row * K + k] = wk;
+                    indices[row * K + k] = sel_e[k];
+                    if (weights_act) {
+                        if (act_dtype == MTS_BF16) reinterpret_cast<bf16_t*>(weights_act)[row * K + k] = (bf16_t)wk;
+                        else reinterpret_cast<mts_f16_t*>(weights_act)[row * K + k] = (mts_f16_t)wk;
+                    }
+#pragma unroll
+                    for (int e = 0; e < EP; ++e) csum[e] += e == sel_e[k] ? 1 : 0;
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < EP; ++e) {
+                psum[e] += rs.p[e];
+                const float lp = fmaxf(rs.l[e] - rs.L, kLogFloor);
+                hsum -= (rs.p[e] > 0.f) ? rs.p[e] * lp : 0.f;
+            }
+            zsum += rs.L * rs.L;
+        }
+    }
+    // lanes 0..3 -> lane 0 (fixed order), waves -> block through LDS (fixed order)
+    __shared__ float red[WAVES][EP + 2];
+    __shared__ int32_t cred[WAVES][EP];
+#pragma unroll
+    for (int o = 1; o < kRows; o <<= 1) {
+#pragma unroll
+        for (int e = 0; e < EP; ++e) {
+            psum[e] += __shfl_xor(psum[e], o, MTS_WAVE);
+            csum[e] += __shfl_xor(csum[e], o, MTS_WAVE);
+        }
+        zsum += __shfl_xor(zsum, o, MTS_WAVE);
+        hsum += __shfl_xor(hsum, o, MTS_WAVE);
+    }
+    if (lane == 0) {
+#pragma unroll
+        for (int e = 0; e < EP; ++e) {
+            red[wave][e] = psum[e];
+            cred[wave][e] = csum[e];
+        }
+        red[wave][EP] = zsum;
+        red[wave][EP + 1] = hsum;
+    }
+    __syncthreads();
+    if ((int64_t)blockIdx.x * WAVES * rows_per_wave >= T) return;   // no rows: not a chunk
+    for (int i = threadIdx.x; i < E + 2; i += kFwdThreads) {
+        const int src = i < E ? i : EP + (i - E);
+        float sum = 0.f;
+#pragma unroll
+        for (int q = 0; q < WAVES; ++q) sum += red[q][src];
+        partial[(int64_t)blockIdx.x * (E + 2) + i] = sum;
+    }
+    for (int i = threadIdx.x; i < E; i += kFwdThreads) {
+        int32_t sum = 0;
+#pragma unroll
+        for (int q = 0; q < WAVES; ++q) sum += cred[q][i];
+        cnt[(int64_t)blockIdx.x * E + i] = sum;
+    }
+}
+
 // Backward: a thread owns 4 consecutive columns.  Per row it forms dx (in the activation
 // dtype) from the row's E logit gradients and its weight columns, and adds the row's
 // contribution to its E x 4 block of dW_r; every block writes its partial dW_r to the
@@ -176,13 +349,66 @@ __global__ __launch_bounds__(kFwdThreads) void router_logits_fwd_kernel(const XT
 // one partial: a quarter of the partials for the same number of waves in flight.
 constexpr int bwd_max_threads(int EP) { return EP <= 8 ? 768 : 384; }   // 16 experts need twice the registers
 
-template <typename XT, int EP, bool EXACT>
+// What the backward kernel needs to form the logit gradients itself (CHAIN): the saved outputs of
+// the post-process and the gradients that arrived at them (null = zeros).
+struct RouterGradIn {
+    const float* logits;
+    const float* weights;
+    const int32_t* indices;
+    const int32_t* counts;
+    const float* g_w;
+    const void* g_w_act;
+    const float* g_p;
+    const float* g_z;
+    const float* g_lb;
+    int act_dtype, K, normalize;
+};
+constexpr int kChainRows = 256;   // most rows a block of the chained kernel takes (their logit gradients sit in LDS)
+
+// CHAIN: `dl` is not read; the block first computes the logit gradients of its rows from the
+// post-process's saved tensors (one thread per row, the arithmetic of the stand-alone
+// post-process backward) into LDS, [row][EP] with zeros past E, and the row loop reads them there.
+template <typename XT, int EP, bool EXACT, bool CHAIN = false>
 __global__ __launch_bounds__(bwd_max_threads(EP)) void router_logits_bwd_kernel(const float* __restrict__ dl,
                                                                  const XT* __restrict__ x,
                                                                  const float* __restrict__ w, int64_t T, int H,
                                                                  int E, int rows_per_block, int groups,
-                                                                 XT* __restrict__ dx, float* __restrict__ part) {
+                                                                 XT* __restrict__ dx, float* __restrict__ part,
+                                                                 RouterGradIn rg = RouterGradIn()) {
     extern __shared__ __attribute__((aligned(16))) float set_sum[];   // [E][H]
+    __shared__ __attribute__((aligned(16))) float dl_lds[CHAIN ? kChainRows * EP : 4];
+    if constexpr (CHAIN) {
+        using namespace mts_router;
+        const int64_t b0 = (int64_t)blockIdx.x * rows_per_block;
+        const int64_t b1 = b0 + rows_per_block < T ? b0 + rows_per_block : T;
+        const float inv_t = 1.0f / (float)T;
+        const float gz = rg.g_z ? rg.g_z[0] * 2.0f * inv_t : 0.f;
+        float gp[EP];
+#pragma unroll
+        for (int e = 0; e < EP; ++e) {
+            gp[e] = (rg.g_p && e < E) ? rg.g_p[e] * inv_t : 0.f;
+            if (rg.g_lb && e < E)
+                gp[e] += rg.g_lb[0] * (float)E * ((float)rg.counts[e] / ((float)T * (float)rg.K)) * inv_t;
+        }
+        for (int64_t row = b0 + threadIdx.x; row < b1; row += blockDim.x) {
+            RowState<EP, 1> r;
+            load_row<EP, 1>(rg.logits, row, E, 0, r);
+            float o[EP];
+            auto grad_w = [&](int k) {
+                const int64_t i = row * rg.K + k;
+                float v = rg.g_w ? rg.g_w[i] : 0.f;
+                if (rg.g_w_act)
+                    v += rg.act_dtype == MTS_BF16 ? (float)reinterpret_cast<const bf16_t*>(rg.g_w_act)[i]
+                                                  : (float)reinterpret_cast<const mts_f16_t*>(rg.g_w_act)[i];
+                return v;
+            };
+            row_logit_gradient<EP, 1>(r, gp, gz, rg.K, rg.normalize, 0, rg.weights + row * rg.K, rg.indices + row * rg.K,
+                                      grad_w, o);
+#pragma unroll
+            for (int e = 0; e < EP; ++e) dl_lds[(row - b0) * EP + e] = e < E ? o[e] : 0.f;
+        }
+        __syncthreads();
+    }
     const int col_threads = blockDim.x / groups;
     const int grp = threadIdx.x / col_threads;
     const int c = (threadIdx.x % col_threads) * 4;
@@ -203,7 +429,14 @@ __global__ __launch_bounds__(bwd_max_threads(EP)) void router_logits_bwd_kernel(
     auto one_row = [&](int64_t row, raw_t raw) {
         const f32x4 xv = widen(raw);
         float g[EP];
-        if constexpr (EXACT) {
+        if constexpr (CHAIN) {
+            const float* src = dl_lds + (row - block_beg) * EP;   // the same address in every lane: a broadcast read
+#pragma unroll
+            for (int q = 0; q < EP / 4; ++q) {
+                const f32x4 v = *reinterpret_cast<const f32x4*>(src + q * 4);
+                g[q * 4] = v[0], g[q * 4 + 1] = v[1], g[q * 4 + 2] = v[2], g[q * 4 + 3] = v[3];
+            }
+        } else if constexpr (EXACT) {
 #pragma unroll
             for (int q = 0; q < EP / 4; ++q) {
                 const f32x4 v = *reinterpret_cast<const f32x4*>(dl + row * EP + q * 4);
@@ -295,6 +528,7 @@ __global__ __launch_bounds__(256) void router_dw_reduce_kernel(const float* __re
 constexpr int kMaxE = 16;
 constexpr int kMaxH = 1024;   // E*H floats of weights fit the 64 KiB of LDS a block may use by default
 constexpr int kBwdBlocks = 1024;
+constexpr int kHeadMaxBlocks = MTS_HEAD_MAX_CHUNKS;   // blocks of the chained forward kernel = chunks of the routing metadata
 
 int check(const void* x, const float* w, int64_t T, int H, int E, int act_dtype) {
     if (!x || !w) return MTS_ERR_NULL;
@@ -341,6 +575,57 @@ extern "C" int mts_router_logits_fwd(const void* x, const float* w_r, int64_t T,
     }
 #undef MTS_FWD_PASSES
 #undef MTS_FWD
+    MTS_CHECK_LAUNCH();
+    return MTS_OK;
+}
+
+// Geometry of the chained forward kernel: blocks, rows per wave (a multiple of kRows); a block's
+// rows are one chunk of the routing metadata.
+void mts_router_head_geometry(int64_t T, int* blocks, int* rows_per_wave) {
+    const int64_t groups = (T + kRows - 1) / kRows;
+    int64_t b = (groups + 3) / 4;
+    if (b > kHeadMaxBlocks) b = kHeadMaxBlocks;
+    const int64_t waves = b * (kFwdThreads / MTS_WAVE);
+    const int64_t per_wave = ((T + waves - 1) / waves + kRows - 1) / kRows * kRows;
+    *blocks = (int)b;
+    *rows_per_wave = (int)per_wave;
+}
+
+int mts_launch_router_head(const void* x, const float* w_r, int64_t T, int H, int E, int K, int normalize, int act_dtype,
+                           float* logits, float* weights, int32_t* indices, void* weights_act, float* partial,
+                           int32_t* cnt, hipStream_t s) {
+    const int rc = check(x, w_r, T, H, E, act_dtype);
+    if (rc != MTS_OK) return rc;
+    if (!logits || !weights || !indices || !partial || !cnt) return MTS_ERR_NULL;
+    if (K < 1 || K > E || K > MTS_MAX_TOP_K) return MTS_ERR_SHAPE;
+    int blocks, rows_per_wave;
+    mts_router_head_geometry(T, &blocks, &rows_per_wave);
+    const dim3 grid((unsigned)blocks);
+    const size_t lds = (size_t)E * H * sizeof(float);
+    const int passes = (H + MTS_WAVE * 4 - 1) / (MTS_WAVE * 4);
+    const int wa_dtype = act_dtype == MTS_F16 ? MTS_F16 : MTS_BF16;   // fp32 activations carry no weights_act (checked by the caller)
+#define MTS_HEAD(XT, EP, PS)                                                                                         \
+    router_head_kernel<XT, EP, PS><<<grid, kFwdThreads, lds, s>>>((const XT*)x, w_r, T, H, E, K, normalize, rows_per_wave, \
+                                                                  logits, weights, indices, weights_act, wa_dtype, partial, cnt)
+#define MTS_HEAD_PASSES(XT, EP)                    \
+    do {                                           \
+        if (passes == 1) MTS_HEAD(XT, EP, 1);      \
+        else if (passes == 2) MTS_HEAD(XT, EP, 2); \
+        else if (passes == 3) MTS_HEAD(XT, EP, 3); \
+        else MTS_HEAD(XT, EP, 4);                  \
+    } while (0)
+    if (act_dtype == MTS_BF16) {
+        if (E <= 8) MTS_HEAD_PASSES(bf16_t, 8);
+        else MTS_HEAD_PASSES(bf16_t, 16);
+    } else if (act_dtype == MTS_F16) {
+        if (E <= 8) MTS_HEAD_PASSES(mts_f16_t, 8);
+        else MTS_HEAD_PASSES(mts_f16_t, 16);
+    } else {
+        if (E <= 8) MTS_HEAD_PASSES(float, 8);
+        else MTS_HEAD_PASSES(float, 16);
+    }
+#undef MTS_HEAD_PASSES
+#undef MTS_HEAD
     MTS_CHECK_LAUNCH();
     return MTS_OK;
 }
@@ -396,6 +681,68 @@ extern "C" int mts_router_logits_bwd(const float* dlogits, const void* x, const 
     // every block has at least one row when nb <= T
     const int used = (int)((T + rows_per_block - 1) / rows_per_block);
     router_dw_reduce_kernel<<<(unsigned)((EH + per_block - 1) / per_block), 256, 0, s>>>(part, used, EH, d_w_r);
+    MTS_CHECK_LAUNCH();
+    return MTS_OK;
+}
+
+namespace {
+int64_t chain_blocks(int64_t T, int groups) {
+    int64_t nb = (bwd_blocks(T) + groups - 1) / groups;
+    const int64_t need = (T + kChainRows - 1) / kChainRows;   // a block's logit gradients sit in LDS
+    return nb > need ? nb : need;
+}
+}  // namespace
+
+extern "C" int64_t mts_moe_head_bwd_workspace_bytes(int64_t T, int H, int E) {
+    if (T <= 0 || H <= 0 || E <= 0) return 0;
+    return chain_blocks(T, 1) * E * H * (int64_t)sizeof(float);
+}
+
+extern "C" int mts_moe_head_bwd(const void* x, const float* w_r, const float* logits, const float* weights,
+                                const int32_t* indices, const int32_t* counts, const float* g_weights,
+                                const void* g_weights_act, const float* g_prob_mean, const float* g_z_loss,
+                                const float* g_load_balance, int64_t T, int H, int E, int K, int normalize,
+                                int act_dtype, void* dx, float* d_w_r, void* workspace, int64_t workspace_bytes,
+                                void* stream) {
+    const int rc = check(x, w_r, T, H, E, act_dtype);
+    if (rc != MTS_OK) return rc;
+    if (!logits || !weights || !indices || !dx || !d_w_r || !workspace) return MTS_ERR_NULL;
+    if (g_load_balance && !counts) return MTS_ERR_NULL;
+    if (g_weights_act && act_dtype == MTS_F32) return MTS_ERR_DTYPE;   // that gradient comes in a 16-bit activation dtype
+    if (K < 1 || K > E || K > MTS_MAX_TOP_K) return MTS_ERR_SHAPE;
+    if (workspace_bytes < mts_moe_head_bwd_workspace_bytes(T, H, E)) return MTS_ERR_WORKSPACE;
+    if (!mts_aligned16(workspace) || !mts_aligned16(d_w_r) || !mts_aligned16(dx) || (E == 8 && !mts_aligned16(logits)))
+        return MTS_ERR_ALIGN;
+    hipStream_t s = (hipStream_t)stream;
+    const int col_threads = ((H / 4 + MTS_WAVE - 1) / MTS_WAVE) * MTS_WAVE;
+    const int max_threads = bwd_max_threads(E <= 8 ? 8 : 16);
+    const int groups = max_threads / col_threads < 4 ? (max_threads / col_threads < 1 ? 1 : max_threads / col_threads) : 4;
+    const int threads = groups * col_threads;
+    int nb = (int)chain_blocks(T, groups);
+    const int rows_per_block = (int)((T + nb - 1) / nb);
+    nb = (int)((T + rows_per_block - 1) / rows_per_block);
+    const size_t lds = (size_t)E * H * sizeof(float);
+    float* part = (float*)workspace;
+    RouterGradIn rg = {logits, weights, indices, counts, g_weights, g_weights_act, g_prob_mean, g_z_loss, g_load_balance,
+                       act_dtype, K, normalize};
+#define MTS_CHAIN(XT, EP)                                                                                        \
+    router_logits_bwd_kernel<XT, EP, false, true><<<nb, threads, lds, s>>>(nullptr, (const XT*)x, w_r, T, H, E,    \
+                                                                            rows_per_block, groups, (XT*)dx, part, rg)
+    if (act_dtype == MTS_BF16) {
+        if (E <= 8) MTS_CHAIN(bf16_t, 8);
+        else MTS_CHAIN(bf16_t, 16);
+    } else if (act_dtype == MTS_F16) {
+        if (E <= 8) MTS_CHAIN(mts_f16_t, 8);
+        else MTS_CHAIN(mts_f16_t, 16);
+    } else {
+        if (E <= 8) MTS_CHAIN(float, 8);
+        else MTS_CHAIN(float, 16);
+    }
+#undef MTS_CHAIN
+    MTS_CHECK_LAUNCH();
+    const int64_t EH = (int64_t)E * H;
+    const int per_block = (256 / kSegs) * 4;
+    router_dw_reduce_kernel<<<(unsigned)((EH + per_block - 1) / per_block), 256, 0, s>>>(part, nb, EH, d_w_r);
     MTS_CHECK_LAUNCH();
     return MTS_OK;
 }

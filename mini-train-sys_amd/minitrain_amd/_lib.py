@@ -43,7 +43,11 @@ SIGNATURES = {
     "mts_moe_stage_weights": (_i, [_p, _i, _p, _i, _i, _l, _l, _i, _p]),
     "mts_moe_fwd_gateup_swiglu": (_i, [_p, _p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p, _p, _p]),
     "mts_moe_fwd_down": (_i, [_p, _p, _p, _l, _i, _i, _i, _i, _p, _p]),
-    "mts_moe_combine": (_i, [_p, _p, _p, _l, _i, _i, _i, _p, _p]),
+    "mts_moe_combine": (_i, [_p, _p, _p, _p, _l, _i, _i, _i, _p, _p]),
+    "mts_moe_head_workspace_bytes": (_l, [_l, _i, _i]),
+    "mts_moe_head_fwd": (_i, [_p, _p, _l, _i, _i, _i, _i, _i] + [_p] * 14 + [_p, _l, _p]),
+    "mts_moe_head_bwd_workspace_bytes": (_l, [_l, _i, _i]),
+    "mts_moe_head_bwd": (_i, [_p] * 11 + [_l, _i, _i, _i, _i, _i, _p, _p, _p, _l, _p]),
     "mts_moe_ds_partials": (_i, [_i]),
     "mts_moe_bwd_weights_as_stored": (_i, [_i, _i, _i]),
     "mts_moe_bwd_dy1": (_i, [_p, _p, _i, _p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p, _p, _p, _p]),

@@ -10,6 +10,7 @@ import os
 from minitrain_amd.kernels.dense_ops import DenseTorchOps
 from minitrain_amd.kernels.hip.capacity import capacity_mask, is_capacity_mask_supported
 from minitrain_amd.kernels.hip.fused_moe import expert_counts, fused_moe, is_fused_moe_supported
+from minitrain_amd.kernels.hip.moe_layer import moe_layer, moe_layer_violation
 from minitrain_amd.kernels.hip.router import (
     is_router_logits_supported,
     is_router_postprocess_supported,
@@ -44,6 +45,17 @@ class HipOpsBackend(DenseTorchOps):
             return None
         return capacity_mask(expert_indices, expert_weights, num_experts, capacity)
 
+    # MTS_NO_LAYER_NODE=1 keeps the layer on the three separate operators (for comparisons)
+    offers_moe_layer = os.environ.get("MTS_NO_LAYER_NODE", "0") != "1"
+
+    def moe_layer(self, x, router_weight, gate_up_proj, down_proj, top_k, *, normalize):
+        """Extension: router projection, post-process, routing metadata and the experts as one autograd
+        node (see ``kernels/hip/moe_layer.py``).  Returns None when the contract is not supported; the
+        caller then composes the layer from ``router_postprocess`` and ``fused_moe``."""
+        if not self.offers_moe_layer or moe_layer_violation(x, router_weight, gate_up_proj, down_proj, top_k) is not None:
+            return None
+        return moe_layer(x, router_weight, gate_up_proj, down_proj, top_k, normalize=normalize)
+
     def router_logits(self, hidden_states, weight):
         """Extension beyond the reference's operator interface: the router projection in fp32
         straight from the activation dtype.  Returns None when the contract is not supported,
@@ -62,6 +74,7 @@ __all__ = [
     "is_fused_moe_supported",
     "is_router_logits_supported",
     "is_router_postprocess_supported",
+    "moe_layer",
     "router_logits",
     "router_postprocess",
 ]

@@ -20,47 +20,78 @@ BLOCK_M_TOKEN = 64
 
 
 def ensure_contiguous(fn):
-    @functools.wraps(fn)
-    def wrapper(ctx, *args, **kwargs):
-        args = [a.contiguous() if isinstance(a, torch.Tensor) else a for a in args]
-        return fn(ctx, *args, **kwargs)
+    """Autograd-function decorator: every tensor argument reaches ``fn`` dense and row-major."""
 
-    return wrapper
+    @functools.wraps(fn)
+    def dense_call(ctx, *args):
+        return fn(ctx, *(a.contiguous() if torch.is_tensor(a) else a for a in args))
+
+    return dense_call
+
+
+def expert_contract(x, gate_up_proj, down_proj):
+    """``(holds, requirement)`` pairs for the activations and the expert parameters; the first one that
+    does not hold is what an error message names."""
+    tensors = (x, gate_up_proj, down_proj)
+    if not all(torch.is_tensor(t) for t in tensors):
+        return [(False, "x, gate_up_proj and down_proj are tensors")]
+    shapes_ok = x.ndim == 2 and gate_up_proj.ndim == 3 and down_proj.ndim == 3
+    if not shapes_ok:
+        return [(False, "x is [T,H], gate_up_proj [E,2I,H] and down_proj [E,H,I]")]
+    T, H = x.shape
+    E, two_i, h_w = gate_up_proj.shape
+    I = two_i // 2
+    wide = x.dtype == torch.float32
+    # expert parameters come in the activation dtype or as fp32 master weights; fp32 activations
+    # take 16-bit parameters as well (widened once per call)
+    param_dtypes = (torch.float32, torch.bfloat16, torch.float16) if wide else (x.dtype, torch.float32)
+    return [
+        (all(t.is_cuda for t in tensors) and len({t.device for t in tensors}) == 1, "all tensors on one GPU"),
+        (x.dtype in (torch.bfloat16, torch.float16, torch.float32), "activations are bf16, fp16 or fp32"),
+        (T > 0, "at least one token"),
+        (0 < E <= _MAX_EXPERTS, f"between 1 and {_MAX_EXPERTS} experts"),
+        (two_i % 2 == 0 and h_w == H and tuple(down_proj.shape) == (E, H, I),
+         "gate_up_proj is [E,2I,H] and down_proj [E,H,I] for x [T,H]"),
+        (gate_up_proj.dtype in param_dtypes and down_proj.dtype in param_dtypes,
+         "expert parameters in the activation dtype or fp32 (any of fp32/bf16/fp16 under fp32 activations)"),
+        (H % (4 if wide else 8) == 0, "hidden size a multiple of 8 (4 for fp32 activations)"),
+        (wide or I % 8 == 0, "expert width a multiple of 8 for 16-bit activations"),
+    ]
+
+
+def routing_contract(x, gate_up_proj, top_k_index, top_k_weights):
+    if not (torch.is_tensor(top_k_index) and torch.is_tensor(top_k_weights)):
+        return [(False, "top_k_index and top_k_weights are tensors")]
+    if top_k_index.ndim != 2:
+        return [(False, "top_k_index is [T,K]")]
+    K = top_k_index.shape[1]
+    return [
+        (top_k_index.is_cuda and top_k_weights.is_cuda and top_k_index.device == x.device == top_k_weights.device,
+         "routing tensors on the activations' GPU"),
+        (top_k_weights.shape == top_k_index.shape and top_k_index.shape[0] == x.shape[0], "top_k_index and top_k_weights are [T,K]"),
+        (0 < K <= min(gate_up_proj.shape[0], 32768), "1 <= K <= number of experts"),
+        (x.shape[0] * K < 2**31, "fewer than 2^31 routes"),
+        (top_k_index.dtype == torch.int32, "int32 expert indices"),
+        (top_k_weights.dtype == x.dtype, "routing weights in the activation dtype"),
+    ]
+
+
+def first_violation(pairs):
+    for holds, requirement in pairs:
+        if not holds:
+            return requirement
+    return None
+
+
+def fused_moe_violation(x, gate_up_proj, down_proj, top_k_index, top_k_weights):
+    """The first requirement of the operator's tensor contract that the arguments miss, or None."""
+    missed = first_violation(expert_contract(x, gate_up_proj, down_proj))
+    return missed if missed is not None else first_violation(routing_contract(x, gate_up_proj, top_k_index, top_k_weights))
 
 
 def is_fused_moe_supported(x, gate_up_proj, down_proj, top_k_index, top_k_weights) -> bool:
-    tensors = (x, gate_up_proj, down_proj, top_k_index, top_k_weights)
-    if not all(t.is_cuda for t in tensors):
-        return False
-    if len({t.device for t in tensors}) != 1:
-        return False
-    if x.ndim != 2 or gate_up_proj.ndim != 3 or down_proj.ndim != 3:
-        return False
-    if top_k_index.ndim != 2 or top_k_weights.shape != top_k_index.shape:
-        return False
-    tokens, hidden = x.shape
-    experts, twice_intermediate, weight_hidden = gate_up_proj.shape
-    intermediate = twice_intermediate // 2
-    # expert parameters come in the activation dtype or as fp32 master weights; fp32 activations
-    # take 16-bit parameters as well (widened once per call)
-    weight_dtypes = (x.dtype, torch.float32) if x.dtype != torch.float32 else (torch.float32, torch.bfloat16, torch.float16)
-    return (
-        tokens > 0
-        and 0 < experts <= _MAX_EXPERTS
-        and twice_intermediate % 2 == 0
-        and weight_hidden == hidden
-        and down_proj.shape == (experts, hidden, intermediate)
-        and top_k_index.shape[0] == tokens
-        and 0 < top_k_index.shape[1] <= min(experts, 32768)
-        and tokens * top_k_index.shape[1] < 2**31
-        and top_k_index.dtype == torch.int32
-        and top_k_weights.dtype == x.dtype
-        and x.dtype in (torch.bfloat16, torch.float16, torch.float32)
-        and gate_up_proj.dtype in weight_dtypes
-        and down_proj.dtype in weight_dtypes
-        and hidden % (4 if x.dtype == torch.float32 else 8) == 0
-        and (intermediate % 8 == 0 or x.dtype == torch.float32)
-    )
+    """Counterpart of the reference's predicate (minitrain/kernels/triton/fused_moe.py:37-71)."""
+    return fused_moe_violation(x, gate_up_proj, down_proj, top_k_index, top_k_weights) is None
 
 
 def compute_routing_metadata(topk_indices: torch.Tensor, E: int, block_m_token: int = BLOCK_M_TOKEN):
@@ -178,67 +209,262 @@ def _stage(lib, w: torch.Tensor, transpose: bool, dtype: torch.dtype, stream: in
     return out
 
 
+class _Saved:
+    """What the forward pass leaves for the backward pass (the tensors travel through
+    ``ctx.save_for_backward``; the rest are plain attributes)."""
+
+    __slots__ = ("dims", "staged", "weighted")
+
+
+def moe_forward(x, gate_up_proj, down_proj, weights_flat, routing):
+    """Gate/up + SwiGLU, down projection and combine for routes that are already sorted.
+
+    ``routing`` = ``(expert_start, x_gather, s_scatter, s_reverse)``.  Returns the output, the tensors
+    to save for :func:`moe_backward` and the non-tensor state."""
+    lib = _lib.load()
+    expert_start, x_gather, s_scatter, s_reverse = routing
+    T, H = x.shape
+    E = gate_up_proj.shape[0]
+    I = gate_up_proj.shape[1] // 2
+    TK = weights_flat.numel()
+    K = TK // T
+    dev = x.device
+    act = _lib.dtype_code(x.dtype)
+    stream = _lib.stream_of(x)
+
+    w1 = _stage(lib, gate_up_proj, False, x.dtype)
+    w2 = _stage(lib, down_proj, False, x.dtype)
+    pre_act = torch.empty(TK, 2 * I, dtype=x.dtype, device=dev)
+    post_act = torch.empty(TK, I, dtype=x.dtype, device=dev)
+    # The routing weight is applied where the activation is formed: post_act = s * silu(g) * u.  The
+    # down projection then yields s * y, the combine is a plain sum, and post_act is at the same time
+    # the `weighted_act` operand of the dW2 GEMM, so it is kept for the backward pass instead of being
+    # written again there (TK * I elements held from forward to backward, and as many fewer written).
+    weighted = _WEIGHTED_POST
+    _lib.check(
+        lib.mts_moe_fwd_gateup_swiglu(
+            x.data_ptr(), w1.data_ptr(), x_gather.data_ptr(), expert_start.data_ptr(),
+            weights_flat.data_ptr() if weighted else None, s_scatter.data_ptr() if weighted else None,
+            T, K, E, H, I, act, pre_act.data_ptr(), post_act.data_ptr(), stream,
+        ),
+        "mts_moe_fwd_gateup_swiglu",
+    )
+    y = torch.empty(TK, H, dtype=x.dtype, device=dev)
+    _lib.check(
+        lib.mts_moe_fwd_down(
+            post_act.data_ptr(), w2.data_ptr(), expert_start.data_ptr(), TK, E, H, I, act, y.data_ptr(), stream
+        ),
+        "mts_moe_fwd_down",
+    )
+    out = torch.empty(T, H, dtype=x.dtype, device=dev)
+    _lib.check(
+        lib.mts_moe_combine(
+            y.data_ptr(), None if weighted else weights_flat.data_ptr(), None, s_reverse.data_ptr(), T, K, H, act,
+            out.data_ptr(), stream,
+        ),
+        "mts_moe_combine",
+    )
+    tensors = (x, gate_up_proj, down_proj, pre_act, weights_flat, expert_start, x_gather, s_scatter, s_reverse,
+               *((post_act,) if weighted else ()))
+    state = _Saved()
+    state.dims = (T, K, E, H, I)
+    state.weighted = weighted
+    # fp32 parameters under a bf16 activation dtype: the backward GEMMs that read the weights as
+    # stored reuse the casts made here (38 MB a layer at the 768/1024 shape) instead of repeating them
+    keep = bool(lib.mts_moe_bwd_weights_as_stored(act, H, I))
+    state.staged = (w1 if keep and w1 is not gate_up_proj else None, w2 if keep and w2 is not down_proj else None)
+    return out, tensors, state
+
+
+def moe_backward(tensors, state, dO, needs, x_addend=None):
+    """``(dx, dW1, dW2, dS)`` for ``needs = (x, W1, W2, S)``.
+
+    ``x_addend``: called with ``dS`` (on the caller's stream) once it exists and before the dX combine;
+    what it returns ([T,H], activation dtype, or None) is added to ``dx`` inside the combine kernel.
+    It is how a caller that owns another path from ``x`` to the loss (the router) avoids a separate
+    sum of the two gradients."""
+    lib = _lib.load()
+    (x, gate_up_proj, down_proj, pre_act, weights_flat, expert_start, x_gather, s_scatter, s_reverse) = tensors[:9]
+    T, K, E, H, I = state.dims
+    TK = T * K
+    dev = dO.device
+    if dO.dtype != x.dtype:
+        dO = dO.to(x.dtype)
+    act = _lib.dtype_code(x.dtype)
+    stream = _lib.stream_of(dO)
+    need_x, need_w1, need_w2, need_s = needs
+
+    # Kernels that do not depend on one another run side by side: the transposed copy of W1 (needed
+    # by dX only) next to the dO*W2 GEMM, and then dW2, dW1 and dX, which depend only on what that
+    # GEMM wrote; the two weight-gradient GEMMs have fewer tiles than the chip has CUs.  Two side
+    # streams (default priority) are forked from and joined to the caller's stream with events;
+    # everything they read stays referenced until the join has been enqueued.
+    main = torch.cuda.current_stream(dev)
+    overlap = _OVERLAP
+    side = [_side_stream(dev, 0), _side_stream(dev, 1)] if overlap else [main, main]
+
+    def fork(*to):
+        # one marker on the caller's stream, however many side streams wait for it
+        if overlap:
+            ev = torch.cuda.Event()
+            ev.record(main)
+            for s in to:
+                s.wait_event(ev)
+
+    def join(frm):
+        if overlap:
+            ev = torch.cuda.Event()
+            ev.record(frm)
+            main.wait_event(ev)
+
+    # The ring kernels read the weights in their stored layout (bf16, whole 64-wide k-tiles);
+    # other contracts get transposed copies, W1's made on a side stream next to the dO*W2 GEMM.
+    as_stored = bool(lib.mts_moe_bwd_weights_as_stored(act, H, I))
+    w1_bwd = None
+    if need_x:
+        if as_stored:
+            # [E, 2I, H]: the parameter itself, or the forward pass's cast of an fp32 parameter
+            w1_bwd = state.staged[0] if state.staged[0] is not None else _stage(lib, gate_up_proj, False, x.dtype)
+        else:
+            fork(side[0])
+            w1_bwd = _stage(lib, gate_up_proj, True, x.dtype, side[0].cuda_stream)  # [E, H, 2I]
+            w1t_ready = torch.cuda.Event() if overlap else None
+            if overlap:
+                w1t_ready.record(side[0])
+
+    if as_stored and state.staged[1] is not None:
+        w2_bwd = state.staged[1]
+    else:
+        w2_bwd = _stage(lib, down_proj, not as_stored, x.dtype)  # [E, H, I] as stored, else [E, I, H]
+    d_pre_act = torch.empty(TK, 2 * I, dtype=x.dtype, device=dev)
+    # s * silu(g) * u: the forward pass's post_act where it carries the routing weight, else written by dY1
+    weighted_act = tensors[9] if state.weighted else torch.empty(TK, I, dtype=x.dtype, device=dev)
+    n_part = lib.mts_moe_ds_partials(I)
+    ds_part = torch.empty(TK, n_part, dtype=torch.float32, device=dev)
+    _lib.check(
+        lib.mts_moe_bwd_dy1(
+            dO.data_ptr(), w2_bwd.data_ptr(), int(as_stored), pre_act.data_ptr(), weights_flat.data_ptr(),
+            x_gather.data_ptr(),
+            s_scatter.data_ptr(), expert_start.data_ptr(), T, K, E, H, I, act, d_pre_act.data_ptr(),
+            None if state.weighted else weighted_act.data_ptr(), ds_part.data_ptr(), stream,
+        ),
+        "mts_moe_bwd_dy1",
+    )
+
+    ddown_proj = None
+    ws1, ws1_ptr, ws1_bytes = _dw_workspace(lib, 1, E, H, I, x.dtype, dev) if need_w1 else (None, 0, 0)
+    ws2, ws2_ptr, ws2_bytes = _dw_workspace(lib, 2, E, H, I, x.dtype, dev) if need_w2 else (None, 0, 0)
+
+    def combine_dx(dx_expanded, d_weights):
+        addend = x_addend(d_weights) if x_addend is not None else None
+        dx = torch.empty(T, H, dtype=x.dtype, device=dev)
+        _lib.check(
+            lib.mts_moe_combine(
+                dx_expanded.data_ptr(), None, _lib.ptr(addend), s_reverse.data_ptr(), T, K, H, act, dx.data_ptr(), stream
+            ),
+            "mts_moe_combine",
+        )
+        return dx
+
+    # When every gradient is wanted, dW1, dW2, dX and the dS reduction go out as ONE launch whose block
+    # order starts the long weight-gradient tiles first; no side stream is involved.
+    if (
+        _JOINT and need_x and need_w1 and need_w2 and need_s and as_stored
+        and gate_up_proj.dtype == down_proj.dtype and lib.mts_moe_bwd_joint_supported(act, H, I)
+    ):
+        dgate_up_proj, ddown_proj = torch.empty_like(gate_up_proj), torch.empty_like(down_proj)
+        d_weights = torch.empty(T, K, dtype=weights_flat.dtype, device=dev)
+        dx_expanded = torch.empty(TK, H, dtype=x.dtype, device=dev)
+        _lib.check(
+            lib.mts_moe_bwd_joint(
+                dO.data_ptr(), weighted_act.data_ptr(), d_pre_act.data_ptr(), x.data_ptr(), w1_bwd.data_ptr(),
+                x_gather.data_ptr(), expert_start.data_ptr(), s_reverse.data_ptr(), ds_part.data_ptr(), T, K, E, H, I,
+                act, _lib.dtype_code(gate_up_proj.dtype), dx_expanded.data_ptr(), dgate_up_proj.data_ptr(),
+                ddown_proj.data_ptr(), d_weights.data_ptr(), ws1_ptr, ws1_bytes, ws2_ptr, ws2_bytes, stream,
+            ),
+            "mts_moe_bwd_joint",
+        )
+        return combine_dx(dx_expanded, d_weights), dgate_up_proj, ddown_proj, d_weights
+
+    if need_w1 and need_w2:
+        fork(side[0], side[1])
+    elif need_w2:
+        fork(side[0])
+    elif need_w1:
+        fork(side[1])
+    # the routing-weight gradient is needed after the join only: it leads one of the side streams
+    # (when there is one) so that dX follows the dO*W2 GEMM directly on the caller's stream; a caller
+    # that takes it before the dX combine gets it on its own stream
+    d_weights = None
+    if need_s:
+        ds_stream = stream if x_addend is not None else (
+            side[0].cuda_stream if need_w2 else (side[1].cuda_stream if need_w1 else stream))
+        d_weights = torch.empty(T, K, dtype=weights_flat.dtype, device=dev)
+        _lib.check(
+            lib.mts_moe_bwd_ds(
+                ds_part.data_ptr(), s_reverse.data_ptr(), TK, I, act, d_weights.data_ptr(), ds_stream
+            ),
+            "mts_moe_bwd_ds",
+        )
+
+    if need_w2:
+        ddown_proj = torch.empty_like(down_proj)
+        _lib.check(
+            lib.mts_moe_bwd_dw2(
+                dO.data_ptr(), weighted_act.data_ptr(), x_gather.data_ptr(), expert_start.data_ptr(), T, K, E, H,
+                I, act, _lib.dtype_code(down_proj.dtype), ddown_proj.data_ptr(), ws2_ptr, ws2_bytes,
+                side[0].cuda_stream,
+            ),
+            "mts_moe_bwd_dw2",
+        )
+
+    dgate_up_proj = None
+    if need_w1:
+        dgate_up_proj = torch.empty_like(gate_up_proj)
+        _lib.check(
+            lib.mts_moe_bwd_dw1(
+                d_pre_act.data_ptr(), x.data_ptr(), x_gather.data_ptr(), expert_start.data_ptr(), T, K, E, H, I,
+                act, _lib.dtype_code(gate_up_proj.dtype), dgate_up_proj.data_ptr(), ws1_ptr, ws1_bytes,
+                side[1].cuda_stream,
+            ),
+            "mts_moe_bwd_dw1",
+        )
+
+    dx = None
+    if need_x:
+        if overlap and not as_stored:
+            main.wait_event(w1t_ready)
+        dx_expanded = torch.empty(TK, H, dtype=x.dtype, device=dev)
+        _lib.check(
+            lib.mts_moe_bwd_dx(
+                d_pre_act.data_ptr(), w1_bwd.data_ptr(), int(as_stored), expert_start.data_ptr(), TK, E, H, I,
+                act, dx_expanded.data_ptr(), stream,
+            ),
+            "mts_moe_bwd_dx",
+        )
+        dx = combine_dx(dx_expanded, d_weights)
+
+    if need_w2 or need_x:
+        join(side[0])
+    if need_w1:
+        join(side[1])
+
+    return dx, dgate_up_proj, ddown_proj, d_weights
+
+
 class _FusedMoEFunction(torch.autograd.Function):
     @staticmethod
     @ensure_contiguous
     def forward(ctx, x, gate_up_proj, down_proj, top_k_index, top_k_weights):
-        lib = _lib.load()
         T, K = top_k_index.shape
         E = gate_up_proj.shape[0]
-        H = x.shape[1]
-        I = gate_up_proj.shape[1] // 2
-        TK = T * K
-        dev = x.device
-        act = _lib.dtype_code(x.dtype)
-        stream = _lib.stream_of(x)
-
         with torch.no_grad():
             (_, expert_start, x_gather, s_scatter, s_reverse, _, _, _) = compute_routing_metadata(top_k_index, E)
-
-        w1 = _stage(lib, gate_up_proj, False, x.dtype)
-        w2 = _stage(lib, down_proj, False, x.dtype)
-        pre_act = torch.empty(TK, 2 * I, dtype=x.dtype, device=dev)
-        post_act = torch.empty(TK, I, dtype=x.dtype, device=dev)
         weights_flat = top_k_weights.flatten().contiguous()
-        # The routing weight is applied where the activation is formed: post_act = s * silu(g) * u.  The
-        # down projection then yields s * y, the combine is a plain sum, and post_act is at the same time
-        # the `weighted_act` operand of the dW2 GEMM, so it is kept for the backward pass instead of being
-        # written again there (TK * I elements held from forward to backward, and as many fewer written).
-        weighted = _WEIGHTED_POST
-        _lib.check(
-            lib.mts_moe_fwd_gateup_swiglu(
-                x.data_ptr(), w1.data_ptr(), x_gather.data_ptr(), expert_start.data_ptr(),
-                weights_flat.data_ptr() if weighted else None, s_scatter.data_ptr() if weighted else None,
-                T, K, E, H, I, act, pre_act.data_ptr(), post_act.data_ptr(), stream,
-            ),
-            "mts_moe_fwd_gateup_swiglu",
-        )
-        y = torch.empty(TK, H, dtype=x.dtype, device=dev)
-        _lib.check(
-            lib.mts_moe_fwd_down(
-                post_act.data_ptr(), w2.data_ptr(), expert_start.data_ptr(), TK, E, H, I, act, y.data_ptr(), stream
-            ),
-            "mts_moe_fwd_down",
-        )
-        out = torch.empty(T, H, dtype=x.dtype, device=dev)
-        _lib.check(
-            lib.mts_moe_combine(
-                y.data_ptr(), None if weighted else weights_flat.data_ptr(), s_reverse.data_ptr(), T, K, H, act,
-                out.data_ptr(), stream,
-            ),
-            "mts_moe_combine",
-        )
-
-        ctx.save_for_backward(
-            x, gate_up_proj, down_proj, pre_act, weights_flat, expert_start, x_gather, s_scatter, s_reverse,
-            *((post_act,) if weighted else ()),
-        )
-        ctx.weighted = weighted
-        ctx.dims = (T, K, E, H, I)
-        # fp32 parameters under a bf16 activation dtype: the backward GEMMs that read the weights as
-        # stored reuse the casts made here (38 MB a layer at the 768/1024 shape) instead of repeating them
-        keep = bool(lib.mts_moe_bwd_weights_as_stored(act, H, I))
-        ctx.staged = (w1 if keep and w1 is not gate_up_proj else None, w2 if keep and w2 is not down_proj else None)
+        out, tensors, state = moe_forward(x, gate_up_proj, down_proj, weights_flat,
+                                          (expert_start, x_gather, s_scatter, s_reverse))
+        ctx.save_for_backward(*tensors)
+        ctx.state = state
         ctx.mark_non_differentiable(top_k_index)
         ctx.set_materialize_grads(False)
         return out
@@ -248,176 +474,13 @@ class _FusedMoEFunction(torch.autograd.Function):
     def backward(ctx, dO):
         if dO is None:
             return None, None, None, None, None
-        lib = _lib.load()
-        (x, gate_up_proj, down_proj, pre_act, weights_flat, expert_start, x_gather, s_scatter, s_reverse) = (
-            ctx.saved_tensors[:9]
-        )
-        T, K, E, H, I = ctx.dims
-        TK = T * K
-        dev = dO.device
-        if dO.dtype != x.dtype:
-            dO = dO.to(x.dtype)
-        act = _lib.dtype_code(x.dtype)
-        stream = _lib.stream_of(dO)
         need_x, need_w1, need_w2, _, need_s = ctx.needs_input_grad
-
-        # Kernels that do not depend on one another run side by side: the transposed copy of W1 (needed
-        # by dX only) next to the dO*W2 GEMM, and then dW2, dW1 and dX, which depend only on what that
-        # GEMM wrote; the two weight-gradient GEMMs have fewer tiles than the chip has CUs.  Two side
-        # streams (default priority) are forked from and joined to the caller's stream with events;
-        # everything they read stays referenced until the join has been enqueued.
-        main = torch.cuda.current_stream(dev)
-        overlap = _OVERLAP
-        side = [_side_stream(dev, 0), _side_stream(dev, 1)] if overlap else [main, main]
-
-        def fork(*to):
-            # one marker on the caller's stream, however many side streams wait for it
-            if overlap:
-                ev = torch.cuda.Event()
-                ev.record(main)
-                for s in to:
-                    s.wait_event(ev)
-
-        def join(frm):
-            if overlap:
-                ev = torch.cuda.Event()
-                ev.record(frm)
-                main.wait_event(ev)
-
-        # The ring kernels read the weights in their stored layout (bf16, whole 64-wide k-tiles);
-        # other contracts get transposed copies, W1's made on a side stream next to the dO*W2 GEMM.
-        as_stored = bool(lib.mts_moe_bwd_weights_as_stored(act, H, I))
-        w1_bwd = None
-        if need_x:
-            if as_stored:
-                # [E, 2I, H]: the parameter itself, or the forward pass's cast of an fp32 parameter
-                w1_bwd = ctx.staged[0] if ctx.staged[0] is not None else _stage(lib, gate_up_proj, False, x.dtype)
-            else:
-                fork(side[0])
-                w1_bwd = _stage(lib, gate_up_proj, True, x.dtype, side[0].cuda_stream)  # [E, H, 2I]
-                w1t_ready = torch.cuda.Event() if overlap else None
-                if overlap:
-                    w1t_ready.record(side[0])
-
-        if as_stored and ctx.staged[1] is not None:
-            w2_bwd = ctx.staged[1]
-        else:
-            w2_bwd = _stage(lib, down_proj, not as_stored, x.dtype)  # [E, H, I] as stored, else [E, I, H]
-        d_pre_act = torch.empty(TK, 2 * I, dtype=x.dtype, device=dev)
-        # s * silu(g) * u: the forward pass's post_act where it carries the routing weight, else written by dY1
-        weighted_act = ctx.saved_tensors[9] if ctx.weighted else torch.empty(TK, I, dtype=x.dtype, device=dev)
-        n_part = lib.mts_moe_ds_partials(I)
-        ds_part = torch.empty(TK, n_part, dtype=torch.float32, device=dev)
-        _lib.check(
-            lib.mts_moe_bwd_dy1(
-                dO.data_ptr(), w2_bwd.data_ptr(), int(as_stored), pre_act.data_ptr(), weights_flat.data_ptr(),
-                x_gather.data_ptr(),
-                s_scatter.data_ptr(), expert_start.data_ptr(), T, K, E, H, I, act, d_pre_act.data_ptr(),
-                None if ctx.weighted else weighted_act.data_ptr(), ds_part.data_ptr(), stream,
-            ),
-            "mts_moe_bwd_dy1",
-        )
-
-        ddown_proj = None
-        ws1, ws1_ptr, ws1_bytes = _dw_workspace(lib, 1, E, H, I, x.dtype, dev) if need_w1 else (None, 0, 0)
-        ws2, ws2_ptr, ws2_bytes = _dw_workspace(lib, 2, E, H, I, x.dtype, dev) if need_w2 else (None, 0, 0)
-
-        # When every gradient is wanted, dW1, dW2, dX and the dS reduction go out as ONE launch whose block
-        # order starts the long weight-gradient tiles first; no side stream is involved.
-        if (
-            _JOINT and need_x and need_w1 and need_w2 and need_s and as_stored
-            and gate_up_proj.dtype == down_proj.dtype and lib.mts_moe_bwd_joint_supported(act, H, I)
-        ):
-            dgate_up_proj, ddown_proj = torch.empty_like(gate_up_proj), torch.empty_like(down_proj)
-            d_weights = torch.empty(T, K, dtype=weights_flat.dtype, device=dev)
-            dx_expanded = torch.empty(TK, H, dtype=x.dtype, device=dev)
-            _lib.check(
-                lib.mts_moe_bwd_joint(
-                    dO.data_ptr(), weighted_act.data_ptr(), d_pre_act.data_ptr(), x.data_ptr(), w1_bwd.data_ptr(),
-                    x_gather.data_ptr(), expert_start.data_ptr(), s_reverse.data_ptr(), ds_part.data_ptr(), T, K, E, H, I,
-                    act, _lib.dtype_code(gate_up_proj.dtype), dx_expanded.data_ptr(), dgate_up_proj.data_ptr(),
-                    ddown_proj.data_ptr(), d_weights.data_ptr(), ws1_ptr, ws1_bytes, ws2_ptr, ws2_bytes, stream,
-                ),
-                "mts_moe_bwd_joint",
-            )
-            dx = torch.empty(T, H, dtype=x.dtype, device=dev)
-            _lib.check(
-                lib.mts_moe_combine(dx_expanded.data_ptr(), None, s_reverse.data_ptr(), T, K, H, act, dx.data_ptr(), stream),
-                "mts_moe_combine",
-            )
-            return dx, dgate_up_proj, ddown_proj, None, d_weights
-
-        if need_w1 and need_w2:
-            fork(side[0], side[1])
-        elif need_w2:
-            fork(side[0])
-        elif need_w1:
-            fork(side[1])
-        # the routing-weight gradient is needed after the join only: it leads one of the side streams
-        # (when there is one) so that dX follows the dO*W2 GEMM directly on the caller's stream
-        d_weights = None
-        if need_s:
-            ds_stream = side[0].cuda_stream if need_w2 else (side[1].cuda_stream if need_w1 else stream)
-            d_weights = torch.empty(T, K, dtype=weights_flat.dtype, device=dev)
-            _lib.check(
-                lib.mts_moe_bwd_ds(
-                    ds_part.data_ptr(), s_reverse.data_ptr(), TK, I, act, d_weights.data_ptr(), ds_stream
-                ),
-                "mts_moe_bwd_ds",
-            )
-
-        if need_w2:
-            ddown_proj = torch.empty_like(down_proj)
-            _lib.check(
-                lib.mts_moe_bwd_dw2(
-                    dO.data_ptr(), weighted_act.data_ptr(), x_gather.data_ptr(), expert_start.data_ptr(), T, K, E, H,
-                    I, act, _lib.dtype_code(down_proj.dtype), ddown_proj.data_ptr(), ws2_ptr, ws2_bytes,
-                    side[0].cuda_stream,
-                ),
-                "mts_moe_bwd_dw2",
-            )
-
-        dgate_up_proj = None
-        if need_w1:
-            dgate_up_proj = torch.empty_like(gate_up_proj)
-            _lib.check(
-                lib.mts_moe_bwd_dw1(
-                    d_pre_act.data_ptr(), x.data_ptr(), x_gather.data_ptr(), expert_start.data_ptr(), T, K, E, H, I,
-                    act, _lib.dtype_code(gate_up_proj.dtype), dgate_up_proj.data_ptr(), ws1_ptr, ws1_bytes,
-                    side[1].cuda_stream,
-                ),
-                "mts_moe_bwd_dw1",
-            )
-
-        dx = None
-        if need_x:
-            if overlap and not as_stored:
-                main.wait_event(w1t_ready)
-            dx_expanded = torch.empty(TK, H, dtype=x.dtype, device=dev)
-            _lib.check(
-                lib.mts_moe_bwd_dx(
-                    d_pre_act.data_ptr(), w1_bwd.data_ptr(), int(as_stored), expert_start.data_ptr(), TK, E, H, I,
-                    act, dx_expanded.data_ptr(), stream,
-                ),
-                "mts_moe_bwd_dx",
-            )
-            dx = torch.empty(T, H, dtype=x.dtype, device=dev)
-            _lib.check(
-                lib.mts_moe_combine(
-                    dx_expanded.data_ptr(), None, s_reverse.data_ptr(), T, K, H, act, dx.data_ptr(), stream
-                ),
-                "mts_moe_combine",
-            )
-
-        if need_w2 or need_x:
-            join(side[0])
-        if need_w1:
-            join(side[1])
-
-        return dx, dgate_up_proj, ddown_proj, None, d_weights
+        dx, dw1, dw2, ds = moe_backward(ctx.saved_tensors, ctx.state, dO, (need_x, need_w1, need_w2, need_s))
+        return dx, dw1, dw2, None, ds
 
 
 def fused_moe(x, gate_up_proj, down_proj, top_k_index, top_k_weights):
-    if not is_fused_moe_supported(x, gate_up_proj, down_proj, top_k_index, top_k_weights):
-        raise RuntimeError("Unsupported tensor contract for hip fused MoE")
+    missed = fused_moe_violation(x, gate_up_proj, down_proj, top_k_index, top_k_weights)
+    if missed is not None:
+        raise RuntimeError(f"Unsupported tensor contract for hip fused MoE: it requires {missed}")
     return _FusedMoEFunction.apply(x, gate_up_proj, down_proj, top_k_index, top_k_weights)

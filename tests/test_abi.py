@@ -78,7 +78,7 @@ def test_contract_violations_are_reported_before_any_launch():
     assert joint(*(ok_args[:12] + [72, 40] + ok_args[14:])) == SHAPE                          # 2I = 80 has no whole k-tile
     assert joint(*(ok_args[:20] + [fake, 16] + ok_args[22:])) == WORKSPACE
     # unknown element type
-    assert lib.mts_moe_combine(fake, None, fake, 8, 2, 64, 7, fake, None) == -3
+    assert lib.mts_moe_combine(fake, None, None, fake, 8, 2, 64, 7, fake, None) == -3
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
