@@ -134,17 +134,75 @@ __global__ __launch_bounds__(1024) void route_scan_kernel(
 
 // One block after the kernel that chains the router projection to the post-process: the scan over
 // that kernel's per-block route counts (the chunks of the scatter that follows) and the reduction
-// of its per-block statistics.
+// of its per-block statistics.  The E per-expert scans over the chunks and the E + 2 column sums of
+// the statistics are independent jobs spread over the 16 waves, every job with all its loads issued
+// up front (at most kFinishChunks chunks: 8 per lane); one barrier later a few waves finish up.
+constexpr int kFinishChunks = MTS_HEAD_MAX_CHUNKS;
+constexpr int kFinishMaxE = 64;
 __global__ __launch_bounds__(1024) void head_finish_kernel(
-    const float* __restrict__ partial, int32_t* __restrict__ cnt, int64_t n_chunks, int E, float inv_t,
+    const float* __restrict__ partial, int32_t* __restrict__ cnt, int n_chunks, int E, float inv_t,
     float inv_routes, float* __restrict__ prob_mean, float* __restrict__ z_loss, float* __restrict__ entropy,
     int32_t* __restrict__ counts, float* __restrict__ load_balance, float* __restrict__ load_stats,
     int32_t* __restrict__ expert_start) {
-    // the statistics read the counts before the scan turns them into offsets
-    mts_router::stats_block<1024 / MTS_WAVE>(partial, cnt, (int)n_chunks, E, inv_t, inv_routes, prob_mean, z_loss, entropy,
-                                             nullptr, load_balance, load_stats, threadIdx.x / MTS_WAVE);
+    __shared__ mts_router::StatsShared sh;
+    __shared__ float col_mean[kFinishMaxE + 2];
+    __shared__ int32_t total[kFinishMaxE];
+    constexpr int NW = 1024 / MTS_WAVE, PER_LANE = kFinishChunks / MTS_WAVE;
+    const int wave = threadIdx.x / MTS_WAVE, lane = threadIdx.x % MTS_WAVE;
+    for (int job = wave; job < 2 * E + 2; job += NW) {
+        if (job < E + 2) {   // a column of the statistics
+            float v[PER_LANE];
+#pragma unroll
+            for (int q = 0; q < PER_LANE; ++q) {
+                const int b = q * MTS_WAVE + lane;
+                v[q] = b < n_chunks ? partial[(int64_t)b * (E + 2) + job] : 0.f;
+            }
+            float sum = 0.f;
+#pragma unroll
+            for (int q = 0; q < PER_LANE; ++q) sum += v[q];
+            sum = wave_sum(sum) * inv_t;
+            if (lane == 0) col_mean[job] = sum;
+        } else {             // an expert's routes per chunk -> routes in earlier chunks
+            const int e = job - (E + 2);
+            int32_t v[PER_LANE];
+#pragma unroll
+            for (int q = 0; q < PER_LANE; ++q) {
+                const int c = q * MTS_WAVE + lane;
+                v[q] = c < n_chunks ? cnt[(int64_t)c * E + e] : 0;
+            }
+            int32_t carry = 0;
+#pragma unroll
+            for (int q = 0; q < PER_LANE; ++q) {
+                int32_t incl = v[q];
+#pragma unroll
+                for (int o = 1; o < MTS_WAVE; o <<= 1) {
+                    const int32_t up = __shfl_up(incl, o, MTS_WAVE);
+                    if (lane >= o) incl += up;
+                }
+                const int c = q * MTS_WAVE + lane;
+                if (c < n_chunks) cnt[(int64_t)c * E + e] = carry + incl - v[q];
+                carry += __shfl(incl, MTS_WAVE - 1, MTS_WAVE);
+            }
+            if (lane == 0) total[e] = carry;
+        }
+    }
     __syncthreads();
-    route_scan_block(cnt, n_chunks, E, 1, counts, expert_start, nullptr, nullptr, nullptr);
+    if (threadIdx.x < E + 2)
+        mts_router::stats_column(sh, threadIdx.x, col_mean[threadIdx.x], threadIdx.x < E ? total[threadIdx.x] : 0, E,
+                                 inv_routes, prob_mean, z_loss, entropy, counts);
+    if (wave == NW - 1) {   // exclusive scan of the routes per expert (E <= 64: one lane per expert)
+        const int32_t v = lane < E ? total[lane] : 0;
+        int32_t incl = v;
+#pragma unroll
+        for (int o = 1; o < MTS_WAVE; o <<= 1) {
+            const int32_t up = __shfl_up(incl, o, MTS_WAVE);
+            if (lane >= o) incl += up;
+        }
+        if (lane < E) expert_start[lane] = incl - v;
+        if (lane == E - 1) expert_start[E] = incl;
+    }
+    __syncthreads();
+    mts_router::stats_finalize(sh, wave, 1, 2, E, load_balance, load_stats);
 }
 
 // chunk_len entries per wave (a multiple of 64 is not required); the chunks are the ones the
@@ -324,7 +382,8 @@ extern "C" int mts_moe_head_fwd(const void* x, const float* w_r, int64_t T, int 
     mts_router_head_geometry(T, &blocks, &rows_per_wave);
     const int64_t rows_per_chunk = (int64_t)rows_per_wave * 4;
     const int64_t n_chunks = (T + rows_per_chunk - 1) / rows_per_chunk;
-    head_finish_kernel<<<1, 1024, 0, s>>>(partial, cnt, n_chunks, E, 1.0f / (float)T, 1.0f / ((float)T * (float)K),
+    if (n_chunks > kFinishChunks || E > kFinishMaxE) return MTS_ERR_SHAPE;   // cannot happen: the geometry caps the chunks, the projection E
+    head_finish_kernel<<<1, 1024, 0, s>>>(partial, cnt, (int)n_chunks, E, 1.0f / (float)T, 1.0f / ((float)T * (float)K),
                                           prob_mean, z_loss, entropy, counts, load_balance, load_stats, expert_start);
     MTS_CHECK_LAUNCH();
     const int grid = (int)((n_chunks + kWaves - 1) / kWaves);

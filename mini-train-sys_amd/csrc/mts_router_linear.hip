@@ -203,14 +203,20 @@ __global__ __launch_bounds__(kFwdThreads) void router_head_kernel(
     if (beg < end) load_group(cur, beg);
     __syncthreads();
 
-    // statistics of the rows this lane post-processes (lanes 0..3)
-    float psum[EP], zsum = 0.f, hsum = 0.f;
+    // The logits of up to 64 rows are parked in LDS (row stride EP + 1: a lane per row reads without
+    // bank conflicts); then lane L runs the post-process of row L, so a wave pays for the post-process
+    // once per 64 rows, not once per group of kRows.
+    constexpr int LROW = EP + 1;
+    __shared__ float parked[WAVES][MTS_WAVE * LROW];
+    float* mine_rows = parked[wave];
+    float psum[EP], zsum = 0.f, hsum = 0.f;   // statistics of the rows this lane post-processes
     int csum[EP];
 #pragma unroll
     for (int e = 0; e < EP; ++e) {
         psum[e] = 0.f;
         csum[e] = 0;
     }
+    int64_t pass_base = beg;
     for (int64_t r0 = beg; r0 < end; r0 += kRows) {
         if (r0 + kRows < end) load_group(nxt, r0 + kRows);
         float acc[kRows][EP];
@@ -255,19 +261,16 @@ __global__ __launch_bounds__(kFwdThreads) void router_head_kernel(
             const int r = idx / EP, e = idx % EP;
             const bool writer = NV == 64 ? true : (lane & 1) == 0;
             if (writer && e < E && r0 + r < end) logits[(r0 + r) * E + e] = mine;
+            if (writer) mine_rows[(int)(r0 - pass_base + r) * LROW + e] = e < E ? mine : -INFINITY;
         }
-        // value i of the group ends up in lane i (64 values) or in lanes 2i and 2i+1 (32 values):
-        // lane L < 4 collects the logits of row r0 + L
-        constexpr int SPREAD = NV == 64 ? 1 : 2;
-        const int my = lane & (kRows - 1);
+        const int64_t parked_to = r0 + kRows < end ? r0 + kRows : end;
+        if (parked_to - pass_base < MTS_WAVE && parked_to < end) continue;   // wave-uniform: park more rows first
+        __builtin_amdgcn_wave_barrier();
+        const int64_t row = pass_base + lane;
+        const bool live = row < parked_to;
         RowState<EP, 1> rs;
 #pragma unroll
-        for (int e = 0; e < EP; ++e) {
-            const float got = __shfl(mine, (my * EP + e) * SPREAD, MTS_WAVE);
-            rs.l[e] = e < E ? got : -INFINITY;
-        }
-        const int64_t row = r0 + my;
-        const bool live = lane < kRows && row < end;
+        for (int e = 0; e < EP; ++e) rs.l[e] = live ? mine_rows[lane * LROW + e] : (e == 0 ? 0.f : -INFINITY);
         softmax_row<EP, 1>(rs);
         float sel_p[MTS_MAX_TOP_K], mass;
         int sel_e[MTS_MAX_TOP_K];
@@ -296,20 +299,20 @@ __global__ __launch_bounds__(kFwdThreads) void router_head_kernel(
             }
             zsum += rs.L * rs.L;
         }
+        pass_base = parked_to;
+        __builtin_amdgcn_wave_barrier();
     }
-    // lanes 0..3 -> lane 0 (fixed order), waves -> block through LDS (fixed order)
+    // lanes -> lane 0 (fixed shuffle tree), waves -> block through LDS (fixed order)
     __shared__ float red[WAVES][EP + 2];
     __shared__ int32_t cred[WAVES][EP];
 #pragma unroll
-    for (int o = 1; o < kRows; o <<= 1) {
+    for (int e = 0; e < EP; ++e) {
+        psum[e] = wave_sum(psum[e]);
 #pragma unroll
-        for (int e = 0; e < EP; ++e) {
-            psum[e] += __shfl_xor(psum[e], o, MTS_WAVE);
-            csum[e] += __shfl_xor(csum[e], o, MTS_WAVE);
-        }
-        zsum += __shfl_xor(zsum, o, MTS_WAVE);
-        hsum += __shfl_xor(hsum, o, MTS_WAVE);
+        for (int o = 32; o > 0; o >>= 1) csum[e] += __shfl_xor(csum[e], o, MTS_WAVE);
     }
+    zsum = wave_sum(zsum);
+    hsum = wave_sum(hsum);
     if (lane == 0) {
 #pragma unroll
         for (int e = 0; e < EP; ++e) {

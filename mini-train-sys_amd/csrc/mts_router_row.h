@@ -157,72 +157,60 @@ __device__ __forceinline__ void row_logit_gradient(const RowState<EP, G>& r, con
     for (int j = 0; j < EP; ++j) o[j] = r.p[j] * (dp[j] - dot) + gz * r.L * r.p[j] + extra[j];
 }
 
-// One block: wave w reduces columns w, w+4, ...; lanes stride over the per-block
-// partials and the lane sums meet in a fixed shuffle tree (bit-stable).  Also the routes per
-// expert and, if asked for, the load-balancing term E * sum_e (routes_e / routes) * mean_prob_e.
-// NWAVES waves of the block call this with their own `wave` index (any one-to-one numbering); it
-// ends with the block in step (a barrier inside when the load statistics are asked for).
-template <int NWAVES>
-__device__ __forceinline__ void stats_block(
-    const float* __restrict__ partial, const int32_t* __restrict__ partial_counts, int nblocks, int E,
-    float inv_t, float inv_routes, float* __restrict__ prob_mean, float* __restrict__ z_loss,
-    float* __restrict__ entropy, int32_t* __restrict__ counts, float* __restrict__ load_balance,
-    float* __restrict__ load_stats, int wave) {
-    __shared__ float prod[MTS_MAX_EXPERTS];   // fraction of routes x mean probability, per expert
-    __shared__ float share[MTS_MAX_EXPERTS];  // fraction of routes, per expert
-    __shared__ int routes_of[MTS_MAX_EXPERTS];
-    __shared__ float entropy_s;
-    const int lane = threadIdx.x % MTS_WAVE;
-    for (int i = wave; i < E + 2; i += NWAVES) {
-        float v = 0.f;
-        for (int b = lane; b < nblocks; b += MTS_WAVE) v += partial[(int64_t)b * (E + 2) + i];
-        v = wave_sum(v) * inv_t;
-        int c = 0;
-        if (i < E) {
-            for (int b = lane; b < nblocks; b += MTS_WAVE) c += partial_counts[(int64_t)b * E + i];
-#pragma unroll
-            for (int o = 32; o > 0; o >>= 1) c += __shfl_xor(c, o, MTS_WAVE);
-        }
-        if (lane == 0) {
-            if (i < E) {
-                prob_mean[i] = v;
-                prod[i] = (float)c * inv_routes * v;
-                share[i] = (float)c * inv_routes;
-                routes_of[i] = c;
-                if (counts) counts[i] = c;
-            } else if (i == E) {
-                z_loss[0] = v;
-            } else {
-                entropy[0] = v;
-                entropy_s = v;
-            }
-        }
+// ---- reduction of the routing statistics (one block) ----------------------------------------
+// Column i < E of the per-block partials is the probability mass of expert i, column E the sum
+// of squared log-partitions, column E+1 the entropy sum.  Sums run in a fixed order (bit-stable).
+struct StatsShared {
+    float prod[MTS_MAX_EXPERTS];    // fraction of routes x mean probability, per expert
+    float share[MTS_MAX_EXPERTS];   // fraction of routes, per expert
+    int routes_of[MTS_MAX_EXPERTS];
+    float entropy_s;
+};
+
+// what one thread does with the mean `v` of column i and, for i < E, the routes `c` of expert i
+__device__ __forceinline__ void stats_column(StatsShared& sh, int i, float v, int c, int E, float inv_routes,
+                                             float* __restrict__ prob_mean, float* __restrict__ z_loss,
+                                             float* __restrict__ entropy, int32_t* __restrict__ counts) {
+    if (i < E) {
+        prob_mean[i] = v;
+        sh.prod[i] = (float)c * inv_routes * v;
+        sh.share[i] = (float)c * inv_routes;
+        sh.routes_of[i] = c;
+        if (counts) counts[i] = c;
+    } else if (i == E) {
+        z_loss[0] = v;
+    } else {
+        entropy[0] = v;
+        sh.entropy_s = v;
     }
-    if (!load_balance && !load_stats) return;   // block-uniform
-    __syncthreads();
-    // E * sum_e f_e * pbar_e, summed in a fixed order by one wave
-    if (wave == 0 && load_balance) {
+}
+
+// After a block barrier behind the stats_column calls: wave `lb_wave` writes the load-balancing term
+// E * sum_e (routes_e / routes) * mean_prob_e, wave `ls_wave` the load statistics of the router module
+// (minitrain/model/moe_router.py:113-135) from the route fractions: [0,E) the fractions, then the
+// largest and smallest route count, the coefficient of variation (population standard deviation x E),
+// largest fraction x E, the number of experts without a route, a zero (the dropped-route fraction of
+// dropless routing) and the entropy over log E.  Either output may be NULL.
+__device__ __forceinline__ void stats_finalize(const StatsShared& sh, int wave, int lb_wave, int ls_wave, int E,
+                                               float* __restrict__ load_balance, float* __restrict__ load_stats) {
+    const int lane = threadIdx.x % MTS_WAVE;
+    if (wave == lb_wave && load_balance) {
         float v = 0.f;
-        for (int e = lane; e < E; e += MTS_WAVE) v += prod[e];
+        for (int e = lane; e < E; e += MTS_WAVE) v += sh.prod[e];
         v = wave_sum(v);
         if (lane == 0) load_balance[0] = (float)E * v;
     }
-    // load statistics of the router module (minitrain/model/moe_router.py:113-135) from the route
-    // fractions: [0,E) the fractions, then the largest and smallest route count, the coefficient
-    // of variation (population standard deviation x E), largest fraction x E, the number of
-    // experts without a route, a zero (the dropped-route fraction of dropless routing) and the
-    // entropy over log E
-    if (wave == 1 % NWAVES && load_stats) {
+    if (wave == ls_wave && load_stats) {
         float sum = 0.f, hi = 0.f, dead = 0.f;
         int most = 0, fewest = 0x7fffffff;
         for (int e = lane; e < E; e += MTS_WAVE) {
-            const float f = share[e];
+            const float f = sh.share[e];
             load_stats[e] = f;
             sum += f;
             hi = fmaxf(hi, f);
-            most = max(most, routes_of[e]);
-            fewest = min(fewest, routes_of[e]);
-            dead += routes_of[e] == 0 ? 1.f : 0.f;
+            most = max(most, sh.routes_of[e]);
+            fewest = min(fewest, sh.routes_of[e]);
+            dead += sh.routes_of[e] == 0 ? 1.f : 0.f;
         }
         sum = wave_sum(sum);
         dead = wave_sum(dead);
@@ -235,7 +223,7 @@ __device__ __forceinline__ void stats_block(
         const float mean = sum / (float)E;
         float var = 0.f;
         for (int e = lane; e < E; e += MTS_WAVE) {
-            const float d = share[e] - mean;
+            const float d = sh.share[e] - mean;
             var += d * d;
         }
         var = wave_sum(var) / (float)E;
@@ -246,10 +234,43 @@ __device__ __forceinline__ void stats_block(
             load_stats[E + 3] = hi * (float)E;
             load_stats[E + 4] = dead;
             load_stats[E + 5] = 0.f;
-            load_stats[E + 6] = entropy_s / (E > 1 ? logf((float)E) : 1.0f);
+            load_stats[E + 6] = sh.entropy_s / (E > 1 ? logf((float)E) : 1.0f);
         }
     }
 }
 
+// mean of column i of the partials over nblocks blocks: lanes stride over the blocks, the lane sums
+// meet in a fixed shuffle tree
+__device__ __forceinline__ float stats_column_mean(const float* __restrict__ partial, int nblocks, int E, int i,
+                                                   float inv_t) {
+    const int lane = threadIdx.x % MTS_WAVE;
+    float v = 0.f;
+    for (int b = lane; b < nblocks; b += MTS_WAVE) v += partial[(int64_t)b * (E + 2) + i];
+    return wave_sum(v) * inv_t;
+}
+
+// The whole reduction by one block of NWAVES waves: wave w takes columns w, w + NWAVES, ...
+template <int NWAVES>
+__device__ __forceinline__ void stats_block(
+    const float* __restrict__ partial, const int32_t* __restrict__ partial_counts, int nblocks, int E,
+    float inv_t, float inv_routes, float* __restrict__ prob_mean, float* __restrict__ z_loss,
+    float* __restrict__ entropy, int32_t* __restrict__ counts, float* __restrict__ load_balance,
+    float* __restrict__ load_stats, int wave) {
+    __shared__ StatsShared sh;
+    const int lane = threadIdx.x % MTS_WAVE;
+    for (int i = wave; i < E + 2; i += NWAVES) {
+        const float v = stats_column_mean(partial, nblocks, E, i, inv_t);
+        int c = 0;
+        if (i < E) {
+            for (int b = lane; b < nblocks; b += MTS_WAVE) c += partial_counts[(int64_t)b * E + i];
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) c += __shfl_xor(c, o, MTS_WAVE);
+        }
+        if (lane == 0) stats_column(sh, i, v, c, E, inv_routes, prob_mean, z_loss, entropy, counts);
+    }
+    if (!load_balance && !load_stats) return;   // block-uniform
+    __syncthreads();
+    stats_finalize(sh, wave, 0, 1 % NWAVES, E, load_balance, load_stats);
+}
 
 }  // namespace mts_router
