@@ -37,9 +37,13 @@ import torch.nn.functional as F
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
-# HBM-side bytes per launch (fetch + write) of the GEMM and combine stages at this workload, from the
-# two rocprofv3 counter runs summarised in profiles/moe_layer_24x1024_hbm_traffic.txt (FETCH_SIZE
-# scaled by 2.0, WRITE_SIZE by 1.0 against a plain copy kernel of known size).  Not measured live.
+RIDGE_FLOP_PER_BYTE = PEAK_BF16_TFLOPS * 1e12 / (PEAK_HBM_GBS * 1e9)   # 312.5: below it a kernel is HBM-bound
+
+# HBM-side bytes per launch (fetch + write) of the GEMM and combine stages at this workload.  They come
+# from two rocprofv3 counter runs (FETCH_SIZE, then WRITE_SIZE; FETCH_SIZE scaled by 2.0 and WRITE_SIZE by
+# 1.0 against a plain copy kernel of known size) and are NOT measured live: `traffic_source` in the bench
+# line names the file that holds the runs' commands and tables.
+TRAFFIC_SOURCE = "profiles/moe_layer_24x1024_hbm_traffic.txt"
 MEASURED_TRAFFIC_BYTES = {
     "fwd_gateup_swiglu": 694.8e6, "fwd_down": 303.4e6, "bwd_dy1": 710.5e6, "bwd_joint": 1115.7e6,
     "combine": 115.2e6, "dx_combine": 114.4e6,
@@ -104,6 +108,19 @@ class Layer:
         return out
 
 
+def settle(layer, seconds=0.4, at_least=30):
+    """Untimed steps until the clocks have settled: the first steps after an idle period run 5-15 % slower
+    on this chip, however few warm-up steps the caller asks for.  Returns the number of steps run."""
+    n, t_end = 0, time.perf_counter() + seconds
+    while n < at_least or time.perf_counter() < t_end:
+        layer.step()
+        n += 1
+        if n % 10 == 0:
+            torch.cuda.synchronize()
+    torch.cuda.synchronize()
+    return n
+
+
 def time_layer(layer, steps, warmup):
     for _ in range(warmup):
         layer.step()
@@ -116,9 +133,12 @@ def time_layer(layer, steps, warmup):
 
 
 def stage_breakdown(layer, steps):
-    """Launch every kernel stage through the C ABI with HIP events around each launch."""
+    """Launch every stage of the layer step through the C ABI, in the order the layer node issues them,
+    with HIP events (recorded on the launching stream) around each call.
+
+    Every stage carries its algorithmic FLOPs and its algorithmic bytes (what one launch must read and
+    write once); the binding roofline follows from their ratio against the ridge of the chip."""
     from minitrain_amd import _lib
-    from minitrain_amd.kernels.hip.fused_moe import compute_routing_metadata
 
     lib = _lib.load()
     w = WORKLOAD
@@ -126,61 +146,57 @@ def stage_breakdown(layer, steps):
     TK = T * K
     dev = layer.x.device
     bf = dict(dtype=torch.bfloat16, device=dev)
-    x, w1, w2, g = layer.x.detach(), layer.w1.detach(), layer.w2.detach(), layer.g
-    logits = F.linear(x.float(), layer.w_r.detach())
-    route = layer.ops.router_postprocess(logits, K, normalize=True)
-    idx, wts = route.expert_indices, route.expert_weights.bfloat16().flatten().contiguous()
-    (_, es, xg, ss, sr, _, _, _) = compute_routing_metadata(idx, E)
-    pre, post, y, out = torch.empty(TK, 2 * I, **bf), torch.empty(TK, I, **bf), torch.empty(TK, H, **bf), torch.empty(T, H, **bf)
-    dpre, dxe, dx = torch.empty(TK, 2 * I, **bf), torch.empty(TK, H, **bf), torch.empty(T, H, **bf)
-    npart = lib.mts_moe_ds_partials(I)
-    dsp = torch.empty(TK, npart, dtype=torch.float32, device=dev)
-    dwts = torch.empty(T, K, **bf)
-    dw1, dw2 = torch.empty_like(w1), torch.empty_like(w2)
-    # chunk partials of the weight-gradient GEMMs, as the operator passes them
-    dws1 = torch.empty(lib.mts_moe_bwd_dw_workspace_bytes(1, E, H, I), dtype=torch.uint8, device=dev)
-    dws2 = torch.empty(lib.mts_moe_bwd_dw_workspace_bytes(2, E, H, I), dtype=torch.uint8, device=dev)
-    rw = torch.empty(lib.mts_router_workspace_bytes(T, E), dtype=torch.uint8, device=dev)
-    rws = torch.empty(max(4, lib.mts_moe_route_workspace_bytes(T, K, E)), dtype=torch.uint8, device=dev)
-    r_w, r_i = torch.empty(T, K, dtype=torch.float32, device=dev), torch.empty(T, K, dtype=torch.int32, device=dev)
-    r_wa = torch.empty(T, K, **bf)
-    r_stats = torch.empty(2 * E + 10, dtype=torch.float32, device=dev)
-    i32 = dict(dtype=torch.int32, device=dev)
-    cnt, es2, a1, a2, a3 = torch.empty(E, **i32), torch.empty(E + 1, **i32), torch.empty(TK, **i32), torch.empty(TK, **i32), torch.empty(TK, **i32)
-    dlog = torch.empty_like(logits)
-    gw, gp, gz = torch.randn(T, K, device=dev), torch.randn(E, device=dev), torch.ones((), device=dev)
+    f32, i32 = dict(dtype=torch.float32, device=dev), dict(dtype=torch.int32, device=dev)
+    x, w_r, w1, w2, g = layer.x.detach(), layer.w_r.detach(), layer.w1.detach(), layer.w2.detach(), layer.g
     st = torch.cuda.current_stream().cuda_stream
     p = lambda t: t.data_ptr()
     B = _lib.MTS_BF16
-    gemm = lambda mult: 2.0 * TK * H * I * mult
     esz = 2
-    w_r = layer.w_r.detach()
-    lws = torch.empty(max(4, lib.mts_router_logits_bwd_workspace_bytes(T, H, E)), dtype=torch.uint8, device=dev)
-    dx_r, dw_r, logits2 = torch.empty(T, H, **bf), torch.empty_like(w_r), torch.empty_like(logits)
+    # head outputs
+    logits, r_w, r_i, r_wa = torch.empty(T, E, **f32), torch.empty(T, K, **f32), torch.empty(T, K, **i32), torch.empty(T, K, **bf)
+    r_stats = torch.empty(2 * E + 10, **f32)
+    cnt, es = torch.empty(E, **i32), torch.empty(E + 1, **i32)
+    ss, sr, xg = torch.empty(TK, **i32), torch.empty(TK, **i32), torch.empty(TK, **i32)
+    hws = torch.empty(lib.mts_moe_head_workspace_bytes(T, K, E), dtype=torch.uint8, device=dev)
+    # expert path
+    pre, post, y, out = torch.empty(TK, 2 * I, **bf), torch.empty(TK, I, **bf), torch.empty(TK, H, **bf), torch.empty(T, H, **bf)
+    dpre, dxe, dx = torch.empty(TK, 2 * I, **bf), torch.empty(TK, H, **bf), torch.empty(T, H, **bf)
+    npart = lib.mts_moe_ds_partials(I)
+    dsp = torch.empty(TK, npart, **f32)
+    dwts = torch.empty(T, K, **bf)
+    dw1, dw2 = torch.empty_like(w1), torch.empty_like(w2)
+    dws1 = torch.empty(lib.mts_moe_bwd_dw_workspace_bytes(1, E, H, I), dtype=torch.uint8, device=dev)
+    dws2 = torch.empty(lib.mts_moe_bwd_dw_workspace_bytes(2, E, H, I), dtype=torch.uint8, device=dev)
+    # router backward
+    gp, gz = torch.randn(E, device=dev), torch.ones((), device=dev)
+    bws = torch.empty(lib.mts_moe_head_bwd_workspace_bytes(T, H, E), dtype=torch.uint8, device=dev)
+    dx_r, dw_r = torch.empty(T, H, **bf), torch.empty_like(w_r)
+
+    unit = 2.0 * TK * H * I                  # FLOPs of one [TK,H] x [H,I] product
+    w1_b, w2_b = E * 2 * I * H * esz, E * H * I * esz
+    rows_h, rows_i = TK * H * esz, TK * I * esz
     stages = [
-        ("router_logits_fwd", "hbm", T * H * esz + T * E * 4 + E * H * 4,
-         lambda: lib.mts_router_logits_fwd(p(x), p(w_r), T, H, E, B, p(logits2), st)),
-        ("router_fwd", "hbm", T * E * 4 + T * K * 8 + T * K * esz,
-         lambda: lib.mts_router_fwd(p(logits), T, E, K, 1, p(r_w), p(r_i), p(r_stats), p(r_stats) + 4 * E, p(r_stats) + 4 * E + 4, p(cnt), p(r_stats) + 4 * E + 8, p(r_stats) + 4 * E + 12, p(r_wa), B, p(rw), rw.numel(), st)),
-        ("route_metadata", "hbm", TK * 4 * 2 + 3 * TK * 4,
-         lambda: lib.mts_moe_route(p(idx), T, K, E, 64, p(cnt), p(es2), p(a1), p(a2), p(a3), None, None, None, p(rws), rws.numel(), st)),
-        ("fwd_gateup_swiglu", "mfma", gemm(2),
-         lambda: lib.mts_moe_fwd_gateup_swiglu(p(x), p(w1), p(xg), p(es), p(wts), p(ss), T, K, E, H, I, B, p(pre), p(post), st)),
-        ("fwd_down", "mfma", gemm(1), lambda: lib.mts_moe_fwd_down(p(post), p(w2), p(es), TK, E, H, I, B, p(y), st)),
-        ("combine", "hbm", TK * H * esz + T * H * esz + TK * 4,
+        # name, FLOPs, algorithmic bytes, call
+        ("head_fwd", 2.0 * T * H * E, T * H * esz + E * H * 4 + T * E * 4 + T * K * (4 + 4 + esz) + TK * 4 * 4,
+         lambda: lib.mts_moe_head_fwd(p(x), p(w_r), T, H, E, K, 1, B, p(logits), p(r_w), p(r_i), p(r_wa), p(r_stats),
+                                      p(r_stats) + 4 * E, p(r_stats) + 4 * E + 4, p(cnt), p(r_stats) + 4 * E + 8,
+                                      p(r_stats) + 4 * E + 12, p(es), p(ss), p(sr), p(xg), p(hws), hws.numel(), st)),
+        ("fwd_gateup_swiglu", 2 * unit, rows_h + w1_b + 3 * rows_i + TK * (4 + 4 + esz),
+         lambda: lib.mts_moe_fwd_gateup_swiglu(p(x), p(w1), p(xg), p(es), p(r_wa), p(ss), T, K, E, H, I, B, p(pre), p(post), st)),
+        ("fwd_down", unit, rows_i + w2_b + rows_h, lambda: lib.mts_moe_fwd_down(p(post), p(w2), p(es), TK, E, H, I, B, p(y), st)),
+        ("combine", 1.0 * TK * H, rows_h + T * H * esz + TK * 4,
          lambda: lib.mts_moe_combine(p(y), None, None, p(sr), T, K, H, B, p(out), st)),
-        ("bwd_dy1", "mfma", gemm(1),
-         lambda: lib.mts_moe_bwd_dy1(p(g), p(w2), 1, p(pre), p(wts), p(xg), p(ss), p(es), T, K, E, H, I, B, p(dpre), None, p(dsp), st)),
+        ("bwd_dy1", unit, rows_h + w2_b + 2 * rows_i + 2 * rows_i + TK * npart * 4 + TK * (4 + 4 + esz),
+         lambda: lib.mts_moe_bwd_dy1(p(g), p(w2), 1, p(pre), p(r_wa), p(xg), p(ss), p(es), T, K, E, H, I, B, p(dpre), None, p(dsp), st)),
         # dW1, dW2, dX and the dS reduction: one launch (plus the chunk sum), as the operator issues them
-        ("bwd_joint", "mfma", gemm(5),
+        ("bwd_joint", 5 * unit, 2 * (2 * rows_i) + 2 * rows_h + rows_i + w1_b + rows_h + w1_b + w2_b + TK * npart * 4,
          lambda: lib.mts_moe_bwd_joint(p(g), p(post), p(dpre), p(x), p(w1), p(xg), p(es), p(sr), p(dsp), T, K, E, H, I, B, B,
                                        p(dxe), p(dw1), p(dw2), p(dwts), p(dws1), dws1.numel(), p(dws2), dws2.numel(), st)),
-        ("dx_combine", "hbm", TK * H * esz + 2 * T * H * esz + TK * 4,
+        ("head_bwd", 4.0 * T * H * E, 2 * T * H * esz + T * E * 4 + T * K * (4 + 4 + esz) + 2 * E * H * 4,
+         lambda: lib.mts_moe_head_bwd(p(x), p(w_r), p(logits), p(r_w), p(r_i), p(cnt), None, p(dwts), p(gp), p(gz), p(gz), T, H, E, K,
+                                      1, B, p(dx_r), p(dw_r), p(bws), bws.numel(), st)),
+        ("dx_combine", 1.0 * TK * H, rows_h + 2 * T * H * esz + TK * 4,
          lambda: lib.mts_moe_combine(p(dxe), None, p(dx_r), p(sr), T, K, H, B, p(dx), st)),
-        ("router_bwd", "hbm", T * E * 4 * 2 + T * K * 8 + T * K * esz,
-         lambda: lib.mts_router_bwd(p(logits), p(r_w), p(r_i), None, p(dwts), B, p(gp), p(gz), p(gz), p(cnt), T, E, K, 1, p(dlog), st)),
-        ("router_logits_bwd", "hbm", 2 * T * H * esz + T * E * 4 + 2 * E * H * 4,
-         lambda: lib.mts_router_logits_bwd(p(dlog), p(x), p(w_r), T, H, E, B, p(dx_r), p(dw_r), p(lws), lws.numel(), st)),
     ]
     ev = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in stages] for _ in range(steps)]
     for it in range(2 + steps):
@@ -194,16 +210,19 @@ def stage_breakdown(layer, steps):
                 raise RuntimeError(f"{name} returned {rc}")
     torch.cuda.synchronize()
     rows = []
-    for j, (name, bound, work, _) in enumerate(stages):
+    for j, (name, flops, nbytes, _) in enumerate(stages):
         ms = float(np.mean([ev[i][j][0].elapsed_time(ev[i][j][1]) for i in range(steps)]))
+        intensity = flops / nbytes
+        bound = "mfma" if intensity >= RIDGE_FLOP_PER_BYTE else "hbm"
+        tflops, gbs = flops / (ms * 1e-3) / 1e12, nbytes / (ms * 1e-3) / 1e9
+        row = dict(stage=name, bound=bound, avg_ms=round(ms, 4), flops=flops, algorithmic_bytes=int(nbytes),
+                   intensity_flop_per_byte=round(intensity, 1), tflops=round(tflops, 2), frac_mfma=round(tflops / PEAK_BF16_TFLOPS, 4),
+                   gbs=round(gbs, 1), frac_hbm=round(gbs / PEAK_HBM_GBS, 4))
         if bound == "mfma":
-            ach = work / (ms * 1e-3) / 1e12
-            rows.append(dict(stage=name, bound=bound, avg_ms=round(ms, 4), achieved=round(ach, 2), peak=PEAK_BF16_TFLOPS,
-                             unit="TFLOP/s", frac=round(ach / PEAK_BF16_TFLOPS, 4), work=work))
+            row.update(achieved=row["tflops"], peak=PEAK_BF16_TFLOPS, unit="TFLOP/s", frac=row["frac_mfma"])
         else:
-            ach = work / (ms * 1e-3) / 1e9
-            rows.append(dict(stage=name, bound=bound, avg_ms=round(ms, 4), achieved=round(ach, 1), peak=PEAK_HBM_GBS,
-                             unit="GB/s", frac=round(ach / PEAK_HBM_GBS, 4), work=work))
+            row.update(achieved=row["gbs"], peak=PEAK_HBM_GBS, unit="GB/s", frac=row["frac_hbm"])
+        rows.append(row)
     return rows
 
 
@@ -244,6 +263,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-breakdown", action="store_true")
+    ap.add_argument("--no-settle", action="store_true", help="skip the untimed clock-settling steps before the warm-up")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 256 MiB -> 256 MiB elementwise copy (the known-size kernel that "
                          "FETCH_SIZE / WRITE_SIZE counter runs are scaled by)")
@@ -260,6 +280,7 @@ def main():
     w = WORKLOAD
     ops = get_ops_backend("hip")
     layer = Layer(ops, *make_inputs(w["seed"], w["T"], w["H"], w["E"], w["I"]), w["K"])
+    settled = 0 if args.no_settle else settle(layer)
     sec = time_layer(layer, args.steps, args.warmup)
     tokens_per_s = w["T"] / sec
     gemm_flops = 18.0 * w["T"] * w["K"] * w["H"] * w["I"]
@@ -271,6 +292,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "settle_steps": settled,
         "ms_per_step": round(sec * 1e3, 4),
         "higher_is_better": True,
         "scaling": "weak",
@@ -278,24 +300,31 @@ def main():
         "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": w["name"], "tokens": w["T"], "d_model": w["H"], "experts": w["E"], "top_k": w["K"],
-                   "d_ff": w["I"], "seed": w["seed"], "step": "router GEMM + router post-process + fused MoE, fwd + full bwd"},
+                   "d_ff": w["I"], "seed": w["seed"],
+                   "step": "router projection + router post-process + routing metadata + fused MoE, fwd + full bwd",
+                   "timing": "untimed clock-settling steps (settle_steps), then `warmup` untimed steps, then `steps` timed steps"},
         "layer_gemm_tflops": round(gemm_flops / sec / 1e12, 2),
     }
     if not args.no_breakdown:
         rows = stage_breakdown(layer, max(5, min(args.steps, 20)))
         result["kernels"] = rows
         dom = max(rows, key=lambda r: r["avg_ms"])
+        traffic = MEASURED_TRAFFIC_BYTES.get(dom["stage"])
         result["roofline"] = {"kernel": dom["stage"], "bound": dom["bound"], "achieved": dom["achieved"], "peak": dom["peak"],
-                              "unit": dom["unit"], "frac": dom["frac"], "traffic": MEASURED_TRAFFIC_BYTES.get(dom["stage"]),
-                              "algorithmic": dom["work"], "avg_ms": dom["avg_ms"]}
-        gemm_rows = [r for r in rows if r["bound"] == "mfma"]
+                              "unit": dom["unit"], "frac": dom["frac"], "avg_ms": dom["avg_ms"],
+                              "algorithmic_flops": dom["flops"], "algorithmic_bytes": dom["algorithmic_bytes"],
+                              "intensity_flop_per_byte": dom["intensity_flop_per_byte"], "ridge_flop_per_byte": RIDGE_FLOP_PER_BYTE,
+                              "frac_mfma": dom["frac_mfma"], "frac_hbm": dom["frac_hbm"],
+                              "traffic": traffic, "traffic_source": TRAFFIC_SOURCE if traffic is not None else None,
+                              "traffic_over_algorithmic": round(traffic / dom["algorithmic_bytes"], 3) if traffic else None}
+        gemm_rows = [r for r in rows if r["stage"] in ("fwd_gateup_swiglu", "fwd_down", "bwd_dy1", "bwd_joint")]
         g_ms = sum(r["avg_ms"] for r in gemm_rows)
-        g_ach = sum(r["work"] for r in gemm_rows) / (g_ms * 1e-3) / 1e12
+        g_ach = sum(r["flops"] for r in gemm_rows) / (g_ms * 1e-3) / 1e12
         result["gemm_roofline"] = {"bound": "mfma", "achieved": round(g_ach, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                                    "frac": round(g_ach / PEAK_BF16_TFLOPS, 4), "sum_ms": round(g_ms, 4)}
         c_rows = [r for r in rows if r["stage"] in ("combine", "dx_combine")]
         c_ms = sum(r["avg_ms"] for r in c_rows)
-        c_ach = sum(r["work"] for r in c_rows) / (c_ms * 1e-3) / 1e9
+        c_ach = sum(r["algorithmic_bytes"] for r in c_rows) / (c_ms * 1e-3) / 1e9
         result["combine_roofline"] = {"bound": "hbm", "achieved": round(c_ach, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                                       "frac": round(c_ach / PEAK_HBM_GBS, 4), "sum_ms": round(c_ms, 4)}
         result["kernel_sum_ms"] = round(sum(r["avg_ms"] for r in rows), 4)

@@ -5,7 +5,6 @@ global-norm clipping, AdamW with weight decay on matrices only
 """
 
 import contextlib
-import math
 
 import torch
 
@@ -21,8 +20,14 @@ def build_optimizer(model: torch.nn.Module, *, lr: float = 3e-4, weight_decay: f
 
 def train_step(model: torch.nn.Module, optimizer: torch.optim.Optimizer, batch: dict, *,
                autocast_dtype: torch.dtype | None = torch.bfloat16, grad_clip_norm: float | None = 1.0,
-               use_fused_loss: bool = False) -> torch.Tensor:
-    """Forward, backward, clipping and the optimizer update, exactly once; returns the loss."""
+               use_fused_loss: bool = False, check_finite: bool = True) -> torch.Tensor:
+    """Forward, backward, clipping and the optimizer update, exactly once; returns the loss.
+
+    A non-finite loss or gradient norm raises ``FloatingPointError`` from the host before the optimizer
+    runs (the conditions the reference tests, minitrain/train/trainer.py:77-78,101-106).  The test is one flag
+    computed on the device and read once per step; nothing on the device asserts or traps.
+    ``check_finite=False`` skips the read (and its synchronisation) for callers that check at their own
+    interval."""
     model.train()
     device = next(model.parameters()).device
     input_ids = batch["input_ids"].to(device, non_blocking=True)
@@ -34,15 +39,14 @@ def train_step(model: torch.nn.Module, optimizer: torch.optim.Optimizer, batch: 
     )
     with ctx:
         loss, _ = model(input_ids, targets=targets, use_fused_loss=use_fused_loss)
-    if loss.is_cuda and hasattr(torch, "_assert_async"):
-        torch._assert_async(torch.isfinite(loss.detach()), "non-finite training loss")
-    elif not bool(torch.isfinite(loss.detach())):
-        raise FloatingPointError("non-finite training loss")
+    finite = torch.isfinite(loss.detach())
     loss.backward()
     if grad_clip_norm is not None:
         norm = torch.nn.utils.clip_grad_norm_(model.parameters(), grad_clip_norm)
-        if not loss.is_cuda and not math.isfinite(float(norm)):
-            raise FloatingPointError("non-finite global gradient norm")
+        finite = finite & torch.isfinite(norm)
+    if check_finite and not bool(finite):   # one host read per step
+        optimizer.zero_grad(set_to_none=True)
+        raise FloatingPointError("non-finite training loss or global gradient norm")
     optimizer.step()
     optimizer.zero_grad(set_to_none=True)
     return loss.detach()
