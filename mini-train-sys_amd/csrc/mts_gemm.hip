@@ -61,8 +61,12 @@ constexpr int BK = 64;                       // k extent of an LDS tile (8 chunk
 constexpr uint32_t kInvalid = 0x80000000u;   // buffer offset that is out of range for every operand
 constexpr int64_t kMaxOperandBytes = 0x7fffffffLL;
 
+// Raw buffer descriptor over `bytes` bytes at p.  Lane offsets are 32-bit and kInvalid (2^31) must stay
+// out of range, so a descriptor spans at most 2^31 - 1 bytes: operands that can be larger are addressed
+// through a descriptor that starts at the block's own tile (a 64-bit base, small offsets).
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, int64_t bytes) {
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)bytes, 0x00020000);
+    const int64_t span = bytes < 0 ? 0 : (bytes > kMaxOperandBytes ? kMaxOperandBytes : bytes);
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)span, 0x00020000);
 }
 __device__ __forceinline__ u32x4 buf_load16(__amdgpu_buffer_rsrc_t r, uint32_t byte_off) {
     return __builtin_amdgcn_raw_buffer_load_b128(r, (int)byte_off, 0, 0);
@@ -341,7 +345,8 @@ __device__ __forceinline__ void stage4(bf16_t* dst, float a, float b, float c, f
     *reinterpret_cast<bf16x4*>(dst) = v;
 }
 
-// staged [32][COLS] tile -> global rows rowg0.., columns col.. of a matrix with leading dimension ldc
+// staged [32][COLS] tile -> rows rowg0.. (counted from the start of the descriptor, rend of them exist),
+// columns col.. of a matrix with leading dimension ldc
 template <int COLS>
 __device__ __forceinline__ void flush_tile(const bf16_t* buf, __amdgpu_buffer_rsrc_t rs, uint32_t ldc, uint32_t col,
                                            int rowg0, int rend, int ncol0, int N) {
@@ -377,9 +382,16 @@ __device__ __forceinline__ void rows_epilogue(const RowsParams& p, f32x16 (&acc)
     bf16_t* bufu = WACT ? buf2 : buf1;
     const int ncol0 = n0 + wn * COLS;  // first output column of this wave
     const uint32_t N = (uint32_t)p.N;
-    const __amdgpu_buffer_rsrc_t rs_c = make_rsrc(p.C, p.TK * (int64_t)(EPI == EPI_PLAIN ? N : 2 * N) * 2);
-    const __amdgpu_buffer_rsrc_t rs_c2 = make_rsrc(p.C2, (EPI == EPI_PLAIN || EPI == EPI_DY1N) ? 0 : p.TK * (int64_t)N * 2);
-    const __amdgpu_buffer_rsrc_t rs_pre = make_rsrc(p.pre_act, DY1 ? p.TK * (int64_t)N * 4 : 0);
+    // The [TK, ...] outputs (and the saved pre-activations) may exceed what one descriptor spans: the
+    // descriptors start at the tile's first row and end at the expert's last row, and rows are
+    // counted from row0 below.
+    const int64_t left = rend - row0;
+    const int64_t ldc = EPI == EPI_PLAIN ? N : 2 * N;
+    const bool has_c2 = EPI == EPI_SWIGLU || EPI == EPI_DY1;
+    const __amdgpu_buffer_rsrc_t rs_c = make_rsrc(p.C + (int64_t)row0 * ldc, left * ldc * 2);
+    const __amdgpu_buffer_rsrc_t rs_c2 = make_rsrc(has_c2 ? p.C2 + (int64_t)row0 * N : nullptr, has_c2 ? left * (int64_t)N * 2 : 0);
+    const __amdgpu_buffer_rsrc_t rs_pre = make_rsrc(DY1 ? p.pre_act + (int64_t)row0 * 2 * N : nullptr, DY1 ? left * (int64_t)N * 4 : 0);
+    const int rrel = rend - row0;   // rows of the tile that exist
 
     // routing weight of each of the lane's rows (dY1; SwiGLU when post_act carries the weight): two
     // dependent loads, issued for all rows up front
@@ -393,8 +405,8 @@ __device__ __forceinline__ void rows_epilogue(const RowsParams& p, f32x16 (&acc)
         const int c = (lane % PRE_LPR) * 8;
 #pragma unroll
         for (int it = 0; it < PRE_IT; ++it) {
-            const int grow = row0 + wm * T::WM + mf * 32 + it * PRE_RPI + lane / PRE_LPR;
-            const bool ok = grow < rend && ncol0 + c < p.N;
+            const int grow = wm * T::WM + mf * 32 + it * PRE_RPI + lane / PRE_LPR;   // row inside the tile
+            const bool ok = grow < rrel && ncol0 + c < p.N;
             const uint32_t po = ok ? ((uint32_t)grow * 2u * N + (uint32_t)(ncol0 + c)) * 2u : kInvalid;
             gv[it] = buf_load16(rs_pre, po);
             uv[it] = buf_load16(rs_pre, po == kInvalid ? kInvalid : po + N * 2u);
@@ -411,7 +423,7 @@ __device__ __forceinline__ void rows_epilogue(const RowsParams& p, f32x16 (&acc)
     }
 #pragma unroll
     for (int mf = 0; mf < T::MF; ++mf) {
-        const int rowg0 = row0 + wm * T::WM + mf * 32;
+        const int rowg0 = wm * T::WM + mf * 32;   // first row of the slab, counted from row0
         if (EPI == EPI_PLAIN) {
 #pragma unroll
             for (int nf = 0; nf < T::NF; ++nf)
@@ -419,7 +431,7 @@ __device__ __forceinline__ void rows_epilogue(const RowsParams& p, f32x16 (&acc)
                 for (int j = 0; j < 4; ++j)
                     stage4(buf0 + ml * LDW + nf * 32 + 8 * j + nq, acc[mf][nf][4 * j], acc[mf][nf][4 * j + 1],
                            acc[mf][nf][4 * j + 2], acc[mf][nf][4 * j + 3]);
-            flush_tile<COLS>(buf0, rs_c, N, ncol0, rowg0, rend, ncol0, p.N);
+            flush_tile<COLS>(buf0, rs_c, N, ncol0, rowg0, rrel, ncol0, p.N);
         } else if (EPI == EPI_SWIGLU) {
             constexpr int HALF = T::NF / 2;
             const float s = srow[mf];
@@ -439,11 +451,11 @@ __device__ __forceinline__ void rows_epilogue(const RowsParams& p, f32x16 (&acc)
                     stage4(buf1 + o, u[0], u[1], u[2], u[3]);
                     stage4(buf2 + o, a[0], a[1], a[2], a[3]);
                 }
-            flush_tile<COLS>(buf0, rs_c, 2 * N, ncol0, rowg0, rend, ncol0, p.N);
-            flush_tile<COLS>(buf1, rs_c, 2 * N, N + ncol0, rowg0, rend, ncol0, p.N);
-            flush_tile<COLS>(buf2, rs_c2, N, ncol0, rowg0, rend, ncol0, p.N);
+            flush_tile<COLS>(buf0, rs_c, 2 * N, ncol0, rowg0, rrel, ncol0, p.N);
+            flush_tile<COLS>(buf1, rs_c, 2 * N, N + ncol0, rowg0, rrel, ncol0, p.N);
+            flush_tile<COLS>(buf2, rs_c2, N, ncol0, rowg0, rrel, ncol0, p.N);
         } else {  // dY1
-            const int row = rowg0 + ml;
+            const int row = row0 + rowg0 + ml;
             const bool rok = row < rend;
             const float s = srow[mf];
             // the slab's pre-activations go to the buffers that take d_gate and d_up afterwards (a
@@ -458,7 +470,7 @@ __device__ __forceinline__ void rows_epilogue(const RowsParams& p, f32x16 (&acc)
                         *reinterpret_cast<u32x4*>(bufu + r * LDW + c) = uv[it];
                     } else {   // load and hand over one row group at a time: few registers live
                         const int grow = rowg0 + r;
-                        const bool ok = grow < rend && ncol0 + c < p.N;
+                        const bool ok = grow < rrel && ncol0 + c < p.N;
                         const uint32_t po = ok ? ((uint32_t)grow * 2u * N + (uint32_t)(ncol0 + c)) * 2u : kInvalid;
                         const u32x4 g16 = buf_load16(rs_pre, po);
                         const u32x4 u16 = buf_load16(rs_pre, po == kInvalid ? kInvalid : po + N * 2u);
@@ -507,9 +519,9 @@ __device__ __forceinline__ void rows_epilogue(const RowsParams& p, f32x16 (&acc)
                 for (int q = 0; q < T::WN / 64; ++q)
                     if (slot + q < p.np) p.ds_part[(int64_t)row * p.np + slot + q] = q == 0 ? dsp : 0.f;
             }
-            if (WACT) flush_tile<COLS>(buf0, rs_c2, N, ncol0, rowg0, rend, ncol0, p.N);
-            flush_tile<COLS>(bufg, rs_c, 2 * N, ncol0, rowg0, rend, ncol0, p.N);
-            flush_tile<COLS>(bufu, rs_c, 2 * N, N + ncol0, rowg0, rend, ncol0, p.N);
+            if (WACT) flush_tile<COLS>(buf0, rs_c2, N, ncol0, rowg0, rrel, ncol0, p.N);
+            flush_tile<COLS>(bufg, rs_c, 2 * N, ncol0, rowg0, rrel, ncol0, p.N);
+            flush_tile<COLS>(bufu, rs_c, 2 * N, N + ncol0, rowg0, rrel, ncol0, p.N);
         }
     }
 }
@@ -592,7 +604,9 @@ __global__ __launch_bounds__(T::NT) void rows_gemm_kernel(RowsParams p) {
     KMajorLoader<T::BM, T::NT> la;
     KMajorLoader<T::BN, T::NT> lb;
     la.chunk = lb.chunk = threadIdx.x % 8;
-    la.rsrc = make_rsrc(p.A, p.a_rows * p.lda * 2);
+    // an operand read in place is addressed from the tile's first row (it may be larger than a descriptor spans)
+    la.rsrc = p.a_gather ? make_rsrc(p.A, p.a_rows * p.lda * 2)
+                         : make_rsrc(p.A + (int64_t)row0 * p.lda, (int64_t)(rend - row0) * p.lda * 2);
     lb.rsrc = make_rsrc(p.B + (int64_t)e * p.b_rows * p.Kdim, (int64_t)p.b_rows * p.Kdim * 2);
     {
         const int r = threadIdx.x / 8;
@@ -600,7 +614,7 @@ __global__ __launch_bounds__(T::NT) void rows_gemm_kernel(RowsParams p) {
         for (int q = 0; q < la.LOADS; ++q) {
             int row = row0 + q * (T::NT / 8) + r;
             int lrow = row < rend ? row : rend - 1;          // keep the index load in range
-            int src = p.a_gather ? p.a_gather[lrow] : lrow;
+            int src = p.a_gather ? p.a_gather[lrow] : lrow - row0;
             la.voff[q] = row < rend ? ((uint32_t)src * (uint32_t)p.lda + la.chunk * 8) * 2u : kInvalid;
         }
 #pragma unroll
@@ -706,7 +720,9 @@ __global__ __launch_bounds__(T::NT, T::WAVES_PER_EU) void rows_gemm_ring_kernel(
 
     constexpr int CPR_B = T::BN / 8, RPI_B = MTS_WAVE / CPR_B;   // k-major B: chunks per tile row, rows per instruction
     static_assert(!BKM || (EPI != EPI_SWIGLU && T::BKS / RPI_B / T::NWAVES == T::B_INSTR), "k-major B loader split");
-    const __amdgpu_buffer_rsrc_t rs_a = make_rsrc(p.A, p.a_rows * p.lda * 2);
+    // an operand read in place is addressed from the tile's first row (it may be larger than a descriptor spans)
+    const __amdgpu_buffer_rsrc_t rs_a = p.a_gather ? make_rsrc(p.A, p.a_rows * p.lda * 2)
+                                                   : make_rsrc(p.A + (int64_t)row0 * p.lda, (int64_t)(rend - row0) * p.lda * 2);
     const __amdgpu_buffer_rsrc_t rs_b =
         make_rsrc(p.B + (int64_t)e * p.b_rows * p.Kdim, (int64_t)p.b_rows * p.Kdim * 2);
     uint32_t voff_a[T::A_INSTR], voff_b[T::B_INSTR];
@@ -718,7 +734,7 @@ __global__ __launch_bounds__(T::NT, T::WAVES_PER_EU) void rows_gemm_ring_kernel(
             const int chunk = slot ^ (T::CHUNKS == 8 ? (tr >> 1) & 7 : (tr >> 2) & 3);
             const int row = row0 + tr;
             const int lrow = row < rend ? row : rend - 1;
-            const int src = p.a_gather ? p.a_gather[lrow] : lrow;
+            const int src = p.a_gather ? p.a_gather[lrow] : lrow - row0;
             voff_a[j] = row < rend ? ((uint32_t)src * (uint32_t)p.lda + chunk * 8) * 2u : kInvalid;
         }
 #pragma unroll
@@ -839,7 +855,9 @@ __device__ __forceinline__ void rows_gemm_ws_block(const RowsParams& p, bf16_t* 
     if (wave >= T::NWAVES) {
         // ------------------------------ producer ------------------------------
         const int pw = wave - T::NWAVES;
-        const __amdgpu_buffer_rsrc_t rs_a = make_rsrc(p.A, p.a_rows * p.lda * 2);
+        // an operand read in place is addressed from the tile's first row (it may be larger than a descriptor spans)
+        const __amdgpu_buffer_rsrc_t rs_a = p.a_gather ? make_rsrc(p.A, p.a_rows * p.lda * 2)
+                                                       : make_rsrc(p.A + (int64_t)row0 * p.lda, (int64_t)(rend - row0) * p.lda * 2);
         const __amdgpu_buffer_rsrc_t rs_b =
             make_rsrc(p.B + (int64_t)e * p.b_rows * p.Kdim, (int64_t)p.b_rows * p.Kdim * 2);
         uint32_t voff_a[T::A_INSTR], voff_b[T::B_INSTR];
@@ -852,7 +870,7 @@ __device__ __forceinline__ void rows_gemm_ws_block(const RowsParams& p, bf16_t* 
             const int chunk = slot ^ (T::CHUNKS == 8 ? (tr >> 1) & 7 : (tr >> 2) & 3);
             const int row = row0 + tr;
             const int lrow = row < rend ? row : rend - 1;
-            const int src = p.a_gather ? p.a_gather[lrow] : lrow;
+            const int src = p.a_gather ? p.a_gather[lrow] : lrow - row0;
             voff_a[j] = row < rend ? ((uint32_t)src * (uint32_t)p.lda + chunk * 8) * 2u : kInvalid;
         }
 #pragma unroll
@@ -1090,22 +1108,26 @@ struct MMajorLoader {
     u32x4 reg[PER_WAVE][8];
 
     __device__ __forceinline__ void init(const DwParams& p) {
-        rs_p = make_rsrc(p.P, p.p_rows * p.M * 2);
-        rs_q = make_rsrc(p.Q, p.q_rows * p.N * 2);
         gp = p.p_gather != nullptr;
         gq = p.q_gather != nullptr;
+        rs_p = make_rsrc(p.P, gp ? p.p_rows * p.M * 2 : 0);   // an operand read in place gets its descriptor per k-tile
+        rs_q = make_rsrc(p.Q, gq ? p.q_rows * p.N * 2 : 0);
         rs_gp = make_rsrc(p.p_gather, gp ? p.TK * 4 : 0);
         rs_gq = make_rsrc(p.q_gather, gq ? p.TK * 4 : 0);
     }
-    // source rows for the tile starting at row r0 (rows past the end read index 0; they are masked later)
+    // source rows for the tile starting at row r0 (rows past the end read index 0; they are masked later);
+    // an operand read in place is addressed from the tile's first row, so its row index is the k-row itself
     __device__ __forceinline__ void fetch_index(int r0) {
         const int lane = threadIdx.x % MTS_WAVE;
-        tok_p = gp ? buf_load4(rs_gp, (uint32_t)(r0 + lane) * 4u) : r0 + lane;
-        tok_q = gq ? buf_load4(rs_gq, (uint32_t)(r0 + lane) * 4u) : r0 + lane;
+        tok_p = gp ? buf_load4(rs_gp, (uint32_t)(r0 + lane) * 4u) : lane;
+        tok_q = gq ? buf_load4(rs_gq, (uint32_t)(r0 + lane) * 4u) : lane;
     }
     __device__ __forceinline__ void fetch(const DwParams& p, int m0, int n0, int r0, int rend) {
         const int wave = threadIdx.x / MTS_WAVE, lane = threadIdx.x % MTS_WAVE;
         const int kgrp = lane % 8, mc = lane / 8;
+        const int left = rend > r0 ? rend - r0 : 0;
+        const __amdgpu_buffer_rsrc_t tp = gp ? rs_p : make_rsrc(p.P + (int64_t)r0 * p.M, (int64_t)left * p.M * 2);
+        const __amdgpu_buffer_rsrc_t tq = gq ? rs_q : make_rsrc(p.Q + (int64_t)r0 * p.N, (int64_t)left * p.N * 2);
 #pragma unroll
         for (int q = 0; q < PER_WAVE; ++q) {
             const int item = q * T::NWAVES + wave;
@@ -1120,7 +1142,7 @@ struct MMajorLoader {
                 const int src = __shfl(tok, kr, MTS_WAVE);
                 const bool ok = (r0 + kr < rend) && (c < dim);
                 const uint32_t off = ok ? ((uint32_t)src * (uint32_t)dim + (uint32_t)c) * 2u : kInvalid;
-                reg[q][i] = buf_load16(isA ? rs_p : rs_q, off);
+                reg[q][i] = buf_load16(isA ? tp : tq, off);
             }
         }
     }
@@ -1528,13 +1550,15 @@ int tile_choice(int kind) {
     return choice[kind];
 }
 
-int check_common(int64_t TK, int E, int H, int I) {
+// `gathered_rows`: rows of the [T,H] operand that is read through the token gather (0: none).  Lane
+// offsets are 32-bit: one expert's weights and an operand whose rows are gathered from anywhere must
+// fit a single descriptor; the [TK, ...] operands are addressed tile by tile and may be larger.
+int check_common(int64_t TK, int E, int H, int I, int64_t gathered_rows) {
     if (TK <= 0 || TK > 0x7fffffffLL || E < 1 || E > MTS_MAX_EXPERTS || H < 8 || I < 8 || H % 8 ||
         I % 8)
         return MTS_ERR_SHAPE;
-    // every operand is addressed through a 32-bit buffer offset
-    if (TK * (int64_t)(2 * I) * 2 > kMaxOperandBytes || TK * (int64_t)H * 2 > kMaxOperandBytes ||
-        (int64_t)2 * I * H * 2 > kMaxOperandBytes)
+    if ((int64_t)2 * I * H * 2 > kMaxOperandBytes || gathered_rows * (int64_t)H * 2 > kMaxOperandBytes ||
+        TK * 4 > kMaxOperandBytes)   // the index arrays are read through descriptors as well
         return MTS_ERR_SHAPE;
     return MTS_OK;
 }
@@ -1720,7 +1744,7 @@ extern "C" int MTS_GEMM_ENTRY(mts_moe_fwd_gateup_swiglu)(const void* x, const vo
                             (hipStream_t)stream);
     }
     if (act_dtype != MTS_GEMM_DTYPE) return MTS_ERR_DTYPE;
-    int rc = check_common(T * K, E, H, I);
+    int rc = check_common(T * K, E, H, I, T);
     if (rc) return rc;
     if (!mts_aligned16(x) || !mts_aligned16(w1) || !mts_aligned16(pre_act) || !mts_aligned16(post_act)) return MTS_ERR_ALIGN;
     RowsParams p = {};
@@ -1745,7 +1769,7 @@ extern "C" int MTS_GEMM_ENTRY(mts_moe_fwd_down)(const void* post_act, const void
                             (float*)y, nullptr, nullptr, nullptr, nullptr, nullptr, 0, (hipStream_t)stream);
     }
     if (act_dtype != MTS_GEMM_DTYPE) return MTS_ERR_DTYPE;
-    int rc = check_common(TK, E, H, I);
+    int rc = check_common(TK, E, H, I, 0);
     if (rc) return rc;
     if (!mts_aligned16(post_act) || !mts_aligned16(w2) || !mts_aligned16(y)) return MTS_ERR_ALIGN;
     RowsParams p = {};
@@ -1781,7 +1805,7 @@ extern "C" int MTS_GEMM_ENTRY(mts_moe_bwd_dy1)(const void* d_out, const void* w2
                             s_scatter, ds_partial, mts_moe_ds_partials(I), (hipStream_t)stream);
     }
     if (act_dtype != MTS_GEMM_DTYPE) return MTS_ERR_DTYPE;
-    int rc = check_common(T * K, E, H, I);
+    int rc = check_common(T * K, E, H, I, T);
     if (rc) return rc;
     if (!mts_aligned16(d_out) || !mts_aligned16(w2t) || !mts_aligned16(pre_act) || !mts_aligned16(d_pre_act) ||
         !mts_aligned16(weighted_act))
@@ -1811,7 +1835,7 @@ extern "C" int MTS_GEMM_ENTRY(mts_moe_bwd_dx)(const void* d_pre_act, const void*
                             (hipStream_t)stream);
     }
     if (act_dtype != MTS_GEMM_DTYPE) return MTS_ERR_DTYPE;
-    int rc = check_common(TK, E, H, I);
+    int rc = check_common(TK, E, H, I, 0);
     if (rc) return rc;
     if (!mts_aligned16(d_pre_act) || !mts_aligned16(w1t) || !mts_aligned16(dx_expanded)) return MTS_ERR_ALIGN;
     RowsParams p = {};
@@ -1844,7 +1868,7 @@ extern "C" int MTS_GEMM_ENTRY(mts_moe_bwd_dw2)(const void* d_out, const void* we
                           grad_dtype, d_w2, (hipStream_t)stream);
     }
     if (act_dtype != MTS_GEMM_DTYPE) return MTS_ERR_DTYPE;
-    int rc = check_common(T * K, E, H, I);
+    int rc = check_common(T * K, E, H, I, T);
     if (rc) return rc;
     if (!mts_aligned16(d_out) || !mts_aligned16(weighted_act) || !mts_aligned16(d_w2)) return MTS_ERR_ALIGN;
     DwParams p = {};
@@ -1869,7 +1893,7 @@ extern "C" int MTS_GEMM_ENTRY(mts_moe_bwd_dw1)(const void* d_pre_act, const void
                           grad_dtype, d_w1, (hipStream_t)stream);
     }
     if (act_dtype != MTS_GEMM_DTYPE) return MTS_ERR_DTYPE;
-    int rc = check_common(T * K, E, H, I);
+    int rc = check_common(T * K, E, H, I, T);
     if (rc) return rc;
     if (!mts_aligned16(d_pre_act) || !mts_aligned16(x) || !mts_aligned16(d_w1)) return MTS_ERR_ALIGN;
     DwParams p = {};
@@ -1904,7 +1928,7 @@ extern "C" int MTS_GEMM_ENTRY(mts_moe_bwd_joint)(const void* d_out, const void* 
     if (act_dtype != MTS_GEMM_DTYPE) return MTS_ERR_DTYPE;
     if (T <= 0 || K < 1) return MTS_ERR_SHAPE;
     const int64_t TK = T * K;
-    int rc = check_common(TK, E, H, I);
+    int rc = check_common(TK, E, H, I, T);
     if (rc) return rc;
     if (!bwd_joint_ok(H, I)) return MTS_ERR_SHAPE;
     if (!mts_aligned16(d_out) || !mts_aligned16(weighted_act) || !mts_aligned16(d_pre_act) || !mts_aligned16(x) ||

@@ -55,6 +55,9 @@ def expert_contract(x, gate_up_proj, down_proj):
         (gate_up_proj.dtype in param_dtypes and down_proj.dtype in param_dtypes,
          "expert parameters in the activation dtype or fp32 (any of fp32/bf16/fp16 under fp32 activations)"),
         (H % (4 if wide else 8) == 0, "hidden size a multiple of 8 (4 for fp32 activations)"),
+        # rows of x and of dO are gathered from anywhere through 32-bit offsets; the [T*K, ...] intermediates are
+        # addressed tile by tile and may be larger
+        (wide or (T * H * 2 < 2**31 and 2 * I * H * 2 < 2**31), "16-bit activations and one expert's weights smaller than 2 GiB each"),
         (wide or I % 8 == 0, "expert width a multiple of 8 for 16-bit activations"),
     ]
 

@@ -253,12 +253,15 @@ def _expert_weight_gradients_f64(case, e, rows1, rows2):
     xe, ge, se = x[tok].double(), g[tok].double(), w[tok, k].double()
     W1, W2 = w1[e].double(), w2[e].double()
     I = W2.shape[1]
-    pre = xe @ W1.T
+    # per-row quantities: float64, or float32 products widened afterwards where the expert holds very many rows
+    # (a 768-term dot product in fp32 is good to 1e-6); the sums over the rows below are always float64
+    wide = torch.float64 if len(tok) <= 40000 else torch.float32
+    pre = (xe.to(wide) @ W1.to(wide).T).double()
     gate, up = pre[:, :I], pre[:, I:]
     sig = torch.sigmoid(gate)
     silu = gate * sig
     act = silu * up
-    d_act = (ge @ W2) * se[:, None]                                   # d loss / d act
+    d_act = (ge.to(wide) @ W2.to(wide)).double() * se[:, None]          # d loss / d act
     d_pre = torch.cat([d_act * up * (sig + silu * (1 - sig)), d_act * silu], dim=1)
     dw1 = d_pre.T[rows1] @ xe                                         # [rows1, H]
     dw2 = (ge * se[:, None]).T[rows2] @ act                           # [rows2, I]
@@ -312,6 +315,31 @@ def test_fp32_activations_with_16bit_parameters(wdtype):
     case = routed_case(95, 300, 64, 4, 96, 2, dtype=torch.float32)
     case.update(w1=case["w1"].to(wdtype), w2=case["w2"].to(wdtype))
     _compare(case, tol=1e-5 if wdtype == torch.float32 else 4e-3)   # 16-bit gradients: one rounding of the result
+
+
+def test_intermediates_beyond_2_gib():
+    """270 336 tokens at the layer shape: pre_act and d_pre_act ([T*K, 2I] bf16) are 2.2 GB each, more than
+    one buffer descriptor spans, so the kernels address them tile by tile (the reference carries int64 row
+    offsets for the same reason, minitrain/kernels/triton/fused_moe_kernels.py:314,413,474).  Checked on
+    the CPU: forward, dX and dS of sampled tokens, and slices of dW1 / dW2 of the LAST expert, whose rows
+    sit behind the 2 GiB mark."""
+    print("moe intermediates beyond 2 GiB", flush=True)
+    T, H, E, I, K = 270336, 768, 8, 1024, 2
+    assert T * K * 2 * I * 2 > 2**31
+    case = routed_case(9, T, H, E, I, K)
+    out, grads = hip_moe_grads(case["x"], case["w1"], case["w2"], case["idx"], case["w"], case["g"])
+    rng = np.random.Generator(np.random.Philox(9))
+    last = (case["idx"] == E - 1).any(dim=1).nonzero().flatten()             # tokens with a route to the last expert
+    pick = torch.cat([torch.from_numpy(rng.choice(T, size=128, replace=False)), last[torch.from_numpy(rng.choice(len(last), size=64, replace=False))]])
+    ref_out, ref_grads = oracle_moe_grads(case["x"][pick], case["w1"], case["w2"], case["idx"][pick], case["w"][pick],
+                                          case["g"][pick])
+    assert_close_scaled(out.cpu()[pick], ref_out, BF16_TOL, "sampled tokens vs CPU oracle")
+    assert_close_scaled(grads[0].cpu()[pick], ref_grads[0], BF16_TOL, "sampled dX vs CPU oracle")
+    assert_close_scaled(grads[3].cpu()[pick], ref_grads[3], BF16_TOL, "sampled dS vs CPU oracle")
+    dw1_ref, dw2_ref = _expert_weight_gradients_f64(case, E - 1, rows1=slice(0, 2 * I, 127), rows2=slice(0, H, 61))
+    assert_close_scaled(grads[1][E - 1].cpu()[0:2 * I:127], dw1_ref, BF16_TOL, "dW1 slice of the last expert")
+    assert_close_scaled(grads[2][E - 1].cpu()[0:H:61], dw2_ref, BF16_TOL, "dW2 slice of the last expert")
+    assert all(torch.isfinite(t.float()).all() for t in grads)
 
 
 def test_moe_block_end_to_end():
