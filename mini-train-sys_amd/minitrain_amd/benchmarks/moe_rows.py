@@ -187,6 +187,36 @@ def correctness(op, case):
     return row
 
 
+def operator_rows(profile="layer", tokens=24576, iters=20, warmup=5, seed=1, with_torch=True, zipf=False,
+                  capacity_factor=None):
+    """The benchmark rows as dictionaries: ``hip`` first, then ``hip_zero_weight`` (capacity runs) and ``torch``."""
+    from minitrain_amd.model.ops import get_ops_backend
+
+    H, I, E, K = PROFILES[profile]
+    ops = get_ops_backend("hip")
+    case = make_case(tokens, H, I, E, K, torch.bfloat16, seed, zipf=zipf)
+    common = dict(op="fused_moe", profile=profile, size=tokens, hidden=H, expert_width=I, experts=E,
+                  top_k=K, dtype="bf16", device=torch.cuda.get_device_name(0), timer="cuda_events",
+                  routing="zipf" if zipf else "uniform")
+    extra_rows = []
+    if capacity_factor is not None:
+        capacity, dropped, accepted = limit_capacity(case, ops, E, capacity_factor)
+        p50, p95 = _time(lambda: ops.capacity_mask(case["idx_all"], case["w32"], E, capacity), iters, warmup)
+        common.update(capacity_factor=capacity_factor, capacity=capacity, dropped_route_fraction=dropped,
+                      accepted_per_expert=accepted, capacity_mask_p50_ms=p50, capacity_mask_p95_ms=p95)
+        extra_rows.append(measure("hip_zero_weight", ops.fused_moe, case, iters, warmup, idx_key="idx_all"))
+    hip = measure("hip", ops.fused_moe, case, iters, warmup)
+    hip.update(correctness(ops.fused_moe, case))
+    rows = [hip] + extra_rows
+    if with_torch:
+        ref = measure("torch", torch_expert_loop, case, max(3, iters // 4), 2, idx_key="idx_all")
+        for m in ("fwd", "bwd", "full"):
+            hip[f"{m}_speedup"] = ref[f"{m}_p50_ms"] / hip[f"{m}_p50_ms"]
+            ref[f"{m}_speedup"] = 1.0
+        rows.append(ref)
+    return [{**common, **r} for r in rows]
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--profile", choices=sorted(PROFILES), default="layer")
@@ -198,32 +228,9 @@ def main():
     ap.add_argument("--zipf", action="store_true", help="routing skewed towards the low expert ids")
     ap.add_argument("--capacity-factor", type=float, default=None)
     args = ap.parse_args()
-    from minitrain_amd.model.ops import get_ops_backend
-
-    H, I, E, K = PROFILES[args.profile]
-    ops = get_ops_backend("hip")
-    case = make_case(args.tokens, H, I, E, K, torch.bfloat16, args.seed, zipf=args.zipf)
-    common = dict(op="fused_moe", profile=args.profile, size=args.tokens, hidden=H, expert_width=I, experts=E,
-                  top_k=K, dtype="bf16", device=torch.cuda.get_device_name(0), timer="cuda_events",
-                  routing="zipf" if args.zipf else "uniform")
-    extra_rows = []
-    if args.capacity_factor is not None:
-        capacity, dropped, accepted = limit_capacity(case, ops, E, args.capacity_factor)
-        p50, p95 = _time(lambda: ops.capacity_mask(case["idx_all"], case["w32"], E, capacity), args.iters, args.warmup)
-        common.update(capacity_factor=args.capacity_factor, capacity=capacity, dropped_route_fraction=dropped,
-                      accepted_per_expert=accepted, capacity_mask_p50_ms=p50, capacity_mask_p95_ms=p95)
-        extra_rows.append(measure("hip_zero_weight", ops.fused_moe, case, args.iters, args.warmup, idx_key="idx_all"))
-    hip = measure("hip", ops.fused_moe, case, args.iters, args.warmup)
-    hip.update(correctness(ops.fused_moe, case))
-    rows = [hip] + extra_rows
-    if not args.no_torch:
-        ref = measure("torch", torch_expert_loop, case, max(3, args.iters // 4), 2, idx_key="idx_all")
-        for m in ("fwd", "bwd", "full"):
-            hip[f"{m}_speedup"] = ref[f"{m}_p50_ms"] / hip[f"{m}_p50_ms"]
-            ref[f"{m}_speedup"] = 1.0
-        rows.append(ref)
-    for r in rows:
-        print(json.dumps({**common, **r}))
+    for row in operator_rows(args.profile, args.tokens, args.iters, args.warmup, args.seed, not args.no_torch, args.zipf,
+                             args.capacity_factor):
+        print(json.dumps(row))
 
 
 if __name__ == "__main__":

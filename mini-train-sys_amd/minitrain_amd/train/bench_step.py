@@ -65,6 +65,44 @@ class MoeRanges:
         return t
 
 
+def run(layers=12, batch=24, seq=1024, vocab=50257, steps=5, warmup=2, seed=4, fused_loss=False) -> dict:
+    """Builds the decoder, trains ``warmup + steps`` steps on one synthetic batch and returns the record."""
+    torch.manual_seed(seed)
+    cfg = ModelConfig(vocab_size=vocab, seq_len=seq, n_layers=layers, n_heads=12, hidden_size=768,
+                      intermediate_size=1024, dropout=0.0, tie_word_embeddings=True, ffn_type="moe",
+                      num_experts=8, experts_per_token=2)
+    model = MiniTransformer(cfg, get_ops_backend("hip"), activation_dtype=torch.bfloat16).cuda()
+    opt = build_optimizer(model)
+    ranges = MoeRanges(model)
+    g = torch.Generator().manual_seed(seed)
+    ids = torch.randint(0, vocab, (batch, seq + 1), generator=g)
+    data = {"input_ids": ids[:, :-1].contiguous(), "targets": ids[:, 1:].contiguous()}
+    losses = []
+    for _ in range(warmup):
+        losses.append(float(train_step(model, opt, data, use_fused_loss=fused_loss)))
+    ranges.total_ms()
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        losses.append(float(train_step(model, opt, data, use_fused_loss=fused_loss)))
+    torch.cuda.synchronize()
+    step_ms = (time.perf_counter() - t0) / max(steps, 1) * 1e3
+    moe_ms = ranges.total_ms() / max(steps, 1)
+    tokens = batch * seq
+    return {
+        "metric": "decoder training step tokens/s (hip MoE layer via OpsBackend)",
+        "value": tokens / (step_ms * 1e-3), "unit": "tokens/s", "ms_per_step": step_ms,
+        "moe_ms_per_step": moe_ms, "moe_share_of_step": moe_ms / step_ms,
+        "parameters": sum(p.numel() for p in model.parameters()),
+        "peak_allocated_gib": torch.cuda.max_memory_allocated() / 2**30,
+        "losses": losses,
+        "config": {"layers": layers, "batch": batch, "seq_len": seq, "vocab": vocab,
+                   "d_model": 768, "heads": 12, "experts": 8, "top_k": 2, "d_ff": 1024, "dtype": "bf16 autocast, fp32 params",
+                   "optimizer": "AdamW", "data": "synthetic token ids, uniform", "seed": seed},
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--layers", type=int, default=12)
@@ -76,41 +114,7 @@ def main():
     ap.add_argument("--seed", type=int, default=4)
     ap.add_argument("--fused-loss", action="store_true")
     args = ap.parse_args()
-
-    torch.manual_seed(args.seed)
-    cfg = ModelConfig(vocab_size=args.vocab, seq_len=args.seq, n_layers=args.layers, n_heads=12, hidden_size=768,
-                      intermediate_size=1024, dropout=0.0, tie_word_embeddings=True, ffn_type="moe",
-                      num_experts=8, experts_per_token=2)
-    model = MiniTransformer(cfg, get_ops_backend("hip"), activation_dtype=torch.bfloat16).cuda()
-    opt = build_optimizer(model)
-    ranges = MoeRanges(model)
-    g = torch.Generator().manual_seed(args.seed)
-    ids = torch.randint(0, args.vocab, (args.batch, args.seq + 1), generator=g)
-    batch = {"input_ids": ids[:, :-1].contiguous(), "targets": ids[:, 1:].contiguous()}
-    losses = []
-    for _ in range(args.warmup):
-        losses.append(float(train_step(model, opt, batch, use_fused_loss=args.fused_loss)))
-    ranges.total_ms()
-    torch.cuda.synchronize()
-    torch.cuda.reset_peak_memory_stats()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        losses.append(float(train_step(model, opt, batch, use_fused_loss=args.fused_loss)))
-    torch.cuda.synchronize()
-    step_ms = (time.perf_counter() - t0) / args.steps * 1e3
-    moe_ms = ranges.total_ms() / args.steps
-    tokens = args.batch * args.seq
-    print(json.dumps({
-        "metric": "decoder training step tokens/s (hip MoE layer via OpsBackend)",
-        "value": tokens / (step_ms * 1e-3), "unit": "tokens/s", "ms_per_step": step_ms,
-        "moe_ms_per_step": moe_ms, "moe_share_of_step": moe_ms / step_ms,
-        "parameters": sum(p.numel() for p in model.parameters()),
-        "peak_allocated_gib": torch.cuda.max_memory_allocated() / 2**30,
-        "losses": losses,
-        "config": {"layers": args.layers, "batch": args.batch, "seq_len": args.seq, "vocab": args.vocab,
-                   "d_model": 768, "heads": 12, "experts": 8, "top_k": 2, "d_ff": 1024, "dtype": "bf16 autocast, fp32 params",
-                   "optimizer": "AdamW", "data": "synthetic token ids, uniform", "seed": args.seed},
-    }))
+    print(json.dumps(run(args.layers, args.batch, args.seq, args.vocab, args.steps, args.warmup, args.seed, args.fused_loss)))
 
 
 if __name__ == "__main__":

@@ -1,0 +1,60 @@
+"""The operator benchmark rows in the reference's schema (benchmarks/operators/measurement.py:25-38,
+485-496; moe_runner.py:53,176-193) and the decoder training step at its real size (config 5)."""
+
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+TIMING = ("fwd_p50_ms", "fwd_p95_ms", "bwd_p50_ms", "bwd_p95_ms", "full_p50_ms", "full_p95_ms")
+MEMORY = ("fwd_peak_mem_mb", "bwd_peak_mem_mb", "full_peak_mem_mb")
+PARITY = ("max_abs", "max_rel", "relative_l2", "cosine_similarity")
+
+
+@pytest.mark.parametrize("tokens,zipf,capacity_factor", [(2048, False, None), (4096, True, 1.0)])
+def test_operator_rows_schema_and_acceptance(tokens, zipf, capacity_factor):
+    print(f"moe rows tokens={tokens} zipf={zipf} capacity_factor={capacity_factor}", flush=True)
+    from minitrain_amd.benchmarks.moe_rows import operator_rows
+
+    rows = operator_rows("layer", tokens, iters=3, warmup=1, seed=1, with_torch=True, zipf=zipf,
+                         capacity_factor=capacity_factor)
+    by = {r["provider"]: r for r in rows}
+    assert set(by) >= {"hip", "torch"}
+    for r in rows:
+        assert r["op"] == "fused_moe" and r["size"] == tokens and r["dtype"] == "bf16" and r["timer"] == "cuda_events"
+        for key in TIMING + MEMORY:
+            assert key in r and math.isfinite(r[key]) and r[key] >= 0, (r["provider"], key)
+        assert r["fwd_p50_ms"] > 0 and r["full_p50_ms"] >= r["fwd_p50_ms"] * 0.5
+    hip = by["hip"]
+    for side in ("fwd", "bwd"):
+        for key in PARITY:
+            assert f"{side}_{key}" in hip
+        # the reference's gate for this operator (moe_runner.py:176-193)
+        assert hip[f"{side}_relative_l2"] <= 1e-2 and hip[f"{side}_cosine_similarity"] >= 0.9999, hip
+        assert hip[f"{side}_correct"] is True
+    for m in ("fwd", "bwd", "full"):
+        assert hip[f"{m}_speedup"] > 0 and by["torch"][f"{m}_speedup"] == 1.0
+    if capacity_factor is not None:
+        assert "hip_zero_weight" in by and 0.0 < hip["dropped_route_fraction"] < 1.0
+        assert hip["capacity"] == max(4, math.ceil(capacity_factor * tokens * 2 / 8))
+        assert all(a <= hip["capacity"] for a in hip["accepted_per_expert"])
+
+
+def test_decoder_step_at_the_real_size():
+    """Config 5: 12 layers, 24 x 1024 tokens, 293 494 272 parameters, bf16 autocast over fp32 parameters,
+    AdamW: one warm-up step and two timed ones on one batch; the loss is finite and falls, and the MoE
+    blocks report their share of the step."""
+    print("decoder step, 12 layers, 24x1024", flush=True)
+    from minitrain_amd.train.bench_step import run
+
+    rec = run(layers=12, batch=24, seq=1024, vocab=50257, steps=2, warmup=1, seed=4)
+    assert rec["parameters"] == 293_494_272
+    losses = rec["losses"]
+    assert len(losses) == 3 and all(math.isfinite(v) for v in losses)
+    assert losses[0] > math.log(50257) * 0.9            # an untrained model starts near the uniform entropy
+    assert losses[-1] < losses[0]
+    assert 0.0 < rec["moe_share_of_step"] < 1.0 and rec["moe_ms_per_step"] > 0
+    assert rec["value"] > 0 and rec["config"]["layers"] == 12
+    torch.cuda.empty_cache()
