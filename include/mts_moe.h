@@ -42,7 +42,9 @@ extern "C" {
 #define MTS_ERR_WORKSPACE (-4)   /* workspace too small                             */
 #define MTS_ERR_ALIGN (-5)       /* a pointer or leading dimension is not 16-byte aligned */
 
-#define MTS_MAX_EXPERTS 1024
+#define MTS_MAX_EXPERTS 1024          /* router post-process, capacity mask                      */
+#define MTS_MAX_MOE_EXPERTS 65534     /* routing metadata and the grouped GEMMs (the reference's
+                                         limit, minitrain/kernels/triton/fused_moe.py:55-70)      */
 #define MTS_MAX_TOP_K 8
 
 int mts_version(void);
@@ -149,7 +151,8 @@ int mts_moe_head_bwd(const void* x, const float* w_r, const float* logits, const
  * counted and gets no row, its s_reverse entry is -1, and expert_start[E] is the
  * number of kept routes; every kernel below works on the kept rows only, combine
  * and the routing-weight gradient skip the -1 entries.
- * Returns MTS_ERR_SHAPE if E > MTS_MAX_EXPERTS; indices >= E are a caller error:
+ * Returns MTS_ERR_SHAPE if E > MTS_MAX_MOE_EXPERTS (beyond MTS_MAX_EXPERTS the three kernels run
+ * once per window of MTS_MAX_EXPERTS experts); indices >= E are a caller error:
  * they are clamped into range (memory-safe, result undefined).                  */
 int64_t mts_moe_route_workspace_bytes(int64_t T, int K, int E);
 int mts_moe_route(const int32_t* top_k_index, int64_t T, int K, int E, int block_m,

@@ -1554,7 +1554,7 @@ int tile_choice(int kind) {
 // offsets are 32-bit: one expert's weights and an operand whose rows are gathered from anywhere must
 // fit a single descriptor; the [TK, ...] operands are addressed tile by tile and may be larger.
 int check_common(int64_t TK, int E, int H, int I, int64_t gathered_rows) {
-    if (TK <= 0 || TK > 0x7fffffffLL || E < 1 || E > MTS_MAX_EXPERTS || H < 8 || I < 8 || H % 8 ||
+    if (TK <= 0 || TK > 0x7fffffffLL || E < 1 || E > MTS_MAX_MOE_EXPERTS || H < 8 || I < 8 || H % 8 ||
         I % 8)
         return MTS_ERR_SHAPE;
     if ((int64_t)2 * I * H * 2 > kMaxOperandBytes || gathered_rows * (int64_t)H * 2 > kMaxOperandBytes ||
@@ -1705,16 +1705,15 @@ int launch_bwd_joint(BwdJointParams q, int E, int grad_dtype, void* ws1, int64_t
     if (grad_dtype == MTS_GEMM_DTYPE) bwd_joint_kernel<bf16_t><<<grid, WsLarge::NT, 0, s>>>(q);
     else bwd_joint_kernel<float><<<grid, WsLarge::NT, 0, s>>>(q);
     MTS_CHECK_LAUNCH();
-    if (q.dw1.part && q.dw2.part) {
+    if (q.dw1.part && q.dw2.part && 2 * E <= 65535) {
         const int t = q.dw1.tiles_per_expert > q.dw2.tiles_per_expert ? q.dw1.tiles_per_expert : q.dw2.tiles_per_expert;
         const int64_t want = ((int64_t)t * (T::BM * T::BN / 4) + 255) / 256;
         const dim3 sum_grid((unsigned)(want < 256 ? want : 256), (unsigned)(2 * E));
         if (grad_dtype == MTS_GEMM_DTYPE) dw_chunk_sum_pair_kernel<T::BM, T::BN, bf16_t><<<sum_grid, 256, 0, s>>>(q.dw1, q.dw2);
         else dw_chunk_sum_pair_kernel<T::BM, T::BN, float><<<sum_grid, 256, 0, s>>>(q.dw1, q.dw2);
-    } else if (q.dw1.part) {
-        launch_dw_chunk_sum(q.dw1, E, grad_dtype, s);
-    } else if (q.dw2.part) {
-        launch_dw_chunk_sum(q.dw2, E, grad_dtype, s);
+    } else {   // one of the two, or more experts than a grid holds in y twice over
+        if (q.dw1.part) launch_dw_chunk_sum(q.dw1, E, grad_dtype, s);
+        if (q.dw2.part) launch_dw_chunk_sum(q.dw2, E, grad_dtype, s);
     }
     MTS_CHECK_LAUNCH();
     return MTS_OK;
@@ -1738,7 +1737,7 @@ extern "C" int MTS_GEMM_ENTRY(mts_moe_fwd_gateup_swiglu)(const void* x, const vo
     if ((weights != nullptr) != (s_scatter != nullptr)) return MTS_ERR_NULL;   // the routing weight needs the row -> entry map
     if (T <= 0 || K < 1) return MTS_ERR_SHAPE;
     if (act_dtype == MTS_F32) {
-        if (E < 1 || E > MTS_MAX_EXPERTS || H < 1 || I < 1 || T * K > 0x7fffffffLL) return MTS_ERR_SHAPE;
+        if (E < 1 || E > MTS_MAX_MOE_EXPERTS || H < 1 || I < 1 || T * K > 0x7fffffffLL) return MTS_ERR_SHAPE;
         return mts_f32_rows(1, (const float*)x, H, x_gather, (const float*)w1, 2 * I, I, H, expert_start, E, T * K,
                             (float*)pre_act, (float*)post_act, nullptr, (const float*)weights, s_scatter, nullptr, 0,
                             (hipStream_t)stream);
@@ -1764,7 +1763,7 @@ extern "C" int MTS_GEMM_ENTRY(mts_moe_fwd_down)(const void* post_act, const void
 #endif
     if (!post_act || !w2 || !expert_start || !y) return MTS_ERR_NULL;
     if (act_dtype == MTS_F32) {
-        if (TK <= 0 || TK > 0x7fffffffLL || E < 1 || E > MTS_MAX_EXPERTS || H < 1 || I < 1) return MTS_ERR_SHAPE;
+        if (TK <= 0 || TK > 0x7fffffffLL || E < 1 || E > MTS_MAX_MOE_EXPERTS || H < 1 || I < 1) return MTS_ERR_SHAPE;
         return mts_f32_rows(0, (const float*)post_act, I, nullptr, (const float*)w2, H, H, I, expert_start, E, TK,
                             (float*)y, nullptr, nullptr, nullptr, nullptr, nullptr, 0, (hipStream_t)stream);
     }
@@ -1799,7 +1798,7 @@ extern "C" int MTS_GEMM_ENTRY(mts_moe_bwd_dy1)(const void* d_out, const void* w2
         return MTS_ERR_NULL;
     if (T <= 0 || K < 1) return MTS_ERR_SHAPE;
     if (act_dtype == MTS_F32) {
-        if (E < 1 || E > MTS_MAX_EXPERTS || H < 1 || I < 1 || T * K > 0x7fffffffLL || w2_as_stored) return MTS_ERR_SHAPE;
+        if (E < 1 || E > MTS_MAX_MOE_EXPERTS || H < 1 || I < 1 || T * K > 0x7fffffffLL || w2_as_stored) return MTS_ERR_SHAPE;
         return mts_f32_rows(2, (const float*)d_out, H, x_gather, (const float*)w2t, I, I, H, expert_start, E, T * K,
                             (float*)d_pre_act, (float*)weighted_act, (const float*)pre_act, (const float*)weights,
                             s_scatter, ds_partial, mts_moe_ds_partials(I), (hipStream_t)stream);
@@ -1829,7 +1828,7 @@ extern "C" int MTS_GEMM_ENTRY(mts_moe_bwd_dx)(const void* d_pre_act, const void*
 #endif
     if (!d_pre_act || !w1t || !expert_start || !dx_expanded) return MTS_ERR_NULL;
     if (act_dtype == MTS_F32) {
-        if (TK <= 0 || TK > 0x7fffffffLL || E < 1 || E > MTS_MAX_EXPERTS || H < 1 || I < 1 || w1_as_stored) return MTS_ERR_SHAPE;
+        if (TK <= 0 || TK > 0x7fffffffLL || E < 1 || E > MTS_MAX_MOE_EXPERTS || H < 1 || I < 1 || w1_as_stored) return MTS_ERR_SHAPE;
         return mts_f32_rows(0, (const float*)d_pre_act, 2 * I, nullptr, (const float*)w1t, H, H, 2 * I, expert_start, E,
                             TK, (float*)dx_expanded, nullptr, nullptr, nullptr, nullptr, nullptr, 0,
                             (hipStream_t)stream);
@@ -1863,7 +1862,7 @@ extern "C" int MTS_GEMM_ENTRY(mts_moe_bwd_dw2)(const void* d_out, const void* we
     if (!d_out || !weighted_act || !x_gather || !expert_start || !d_w2) return MTS_ERR_NULL;
     if (T <= 0 || K < 1) return MTS_ERR_SHAPE;
     if (act_dtype == MTS_F32) {
-        if (E < 1 || E > MTS_MAX_EXPERTS || H < 1 || I < 1) return MTS_ERR_SHAPE;
+        if (E < 1 || E > MTS_MAX_MOE_EXPERTS || H < 1 || I < 1) return MTS_ERR_SHAPE;
         return mts_f32_dw((const float*)d_out, x_gather, (const float*)weighted_act, nullptr, H, I, expert_start, E,
                           grad_dtype, d_w2, (hipStream_t)stream);
     }
@@ -1888,7 +1887,7 @@ extern "C" int MTS_GEMM_ENTRY(mts_moe_bwd_dw1)(const void* d_pre_act, const void
     if (!d_pre_act || !x || !x_gather || !expert_start || !d_w1) return MTS_ERR_NULL;
     if (T <= 0 || K < 1) return MTS_ERR_SHAPE;
     if (act_dtype == MTS_F32) {
-        if (E < 1 || E > MTS_MAX_EXPERTS || H < 1 || I < 1) return MTS_ERR_SHAPE;
+        if (E < 1 || E > MTS_MAX_MOE_EXPERTS || H < 1 || I < 1) return MTS_ERR_SHAPE;
         return mts_f32_dw((const float*)d_pre_act, nullptr, (const float*)x, x_gather, 2 * I, H, expert_start, E,
                           grad_dtype, d_w1, (hipStream_t)stream);
     }

@@ -29,34 +29,42 @@ constexpr int kSteps = kChunk / MTS_WAVE;
 // them can leave the output arrays.  Negative ids (dropped routes) stay negative.
 __device__ __forceinline__ int clamp_expert(int e, int E) { return e >= E ? E - 1 : e; }
 
+// Experts are handled in windows of at most MTS_MAX_EXPERTS ids, [e0, e0 + EW): one pass of the
+// three kernels per window, so that the per-wave counters fit LDS whatever E is.  A pass counts and
+// places the routes of its window only; row offsets and the tile list carry on from the pass before
+// (expert_start[e0] and tile_count[0] hold what the earlier windows used).  Up to MTS_MAX_EXPERTS
+// experts are one window: e0 = 0, EW = E.
 __global__ __launch_bounds__(kThreads) void route_hist_kernel(const int32_t* __restrict__ idx,
-                                                              int64_t TK, int E,
+                                                              int64_t TK, int E, int e0, int EW,
                                                               int32_t* __restrict__ cnt) {
-    extern __shared__ int32_t lds[];  // [kWaves][E]
-    for (int i = threadIdx.x; i < kWaves * E; i += kThreads) lds[i] = 0;
+    extern __shared__ int32_t lds[];  // [kWaves][EW]
+    for (int i = threadIdx.x; i < kWaves * EW; i += kThreads) lds[i] = 0;
     __syncthreads();
     const int wave = threadIdx.x / MTS_WAVE, lane = threadIdx.x % MTS_WAVE;
     const int64_t chunk = (int64_t)blockIdx.x * kWaves + wave;
     const int64_t base = chunk * kChunk;
-    int32_t* mine = lds + wave * E;
+    int32_t* mine = lds + wave * EW;
     for (int i = lane; i < kChunk; i += MTS_WAVE) {
         int64_t n = base + i;
-        const int e = n < TK ? clamp_expert(idx[n], E) : -1;
-        if (e >= 0) atomicAdd(&mine[e], 1);
+        const int e = (n < TK ? clamp_expert(idx[n], E) : -1) - e0;   // a dropped route stays negative
+        if (e >= 0 && e < EW) atomicAdd(&mine[e], 1);
     }
     __syncthreads();
     if (base < TK) {
-        for (int e = lane; e < E; e += MTS_WAVE) cnt[chunk * E + e] = mine[e];
+        for (int e = lane; e < EW; e += MTS_WAVE) cnt[chunk * EW + e] = mine[e];
     }
 }
 
 // One block.  Wave w owns experts w, w+nw, ...: exclusive scan over chunks in
 // groups of 64, then an exclusive scan of the totals over experts.
+// E: experts of this window; counts / expert_start point at the window's first expert, whose id is e0.
+// For e0 > 0 the rows and tiles used by the earlier windows are read from expert_start[0] (the
+// sentinel the pass before wrote) and tile_count[0].
 __device__ __forceinline__ void route_scan_block(
     int32_t* __restrict__ cnt, int64_t n_chunks, int E, int block_m,
     int32_t* __restrict__ counts, int32_t* __restrict__ expert_start,
     int32_t* __restrict__ tile_row_start, int32_t* __restrict__ tile_expert,
-    int32_t* __restrict__ tile_count) {
+    int32_t* __restrict__ tile_count, int e0 = 0) {
     __shared__ int32_t total[MTS_MAX_EXPERTS];
     __shared__ int32_t start[MTS_MAX_EXPERTS + 1];
     __shared__ int32_t tile_off[MTS_MAX_EXPERTS + 1];
@@ -80,9 +88,9 @@ __device__ __forceinline__ void route_scan_block(
     }
     __syncthreads();
     if (wave == 0) {
-        int32_t carry = 0, tcarry = 0;
-        for (int e0 = 0; e0 < E; e0 += MTS_WAVE) {
-            int e = e0 + lane;
+        int32_t carry = e0 > 0 ? expert_start[0] : 0, tcarry = (e0 > 0 && tile_count) ? tile_count[0] : 0;
+        for (int eb = 0; eb < E; eb += MTS_WAVE) {
+            int e = eb + lane;
             int32_t v = (e < E) ? total[e] : 0;
             int32_t tv = (v + block_m - 1) / block_m;
             int32_t incl = v, tincl = tv;
@@ -117,7 +125,7 @@ __device__ __forceinline__ void route_scan_block(
             int32_t nt = tile_off[e + 1] - tile_off[e];
             for (int j = lane; j < nt; j += MTS_WAVE) {
                 tile_row_start[tile_off[e] + j] = start[e] + j * block_m;
-                tile_expert[tile_off[e] + j] = e;
+                tile_expert[tile_off[e] + j] = e0 + e;
             }
         }
     }
@@ -127,9 +135,9 @@ __global__ __launch_bounds__(1024) void route_scan_kernel(
     int32_t* __restrict__ cnt, int64_t n_chunks, int E, int64_t TK, int block_m,
     int32_t* __restrict__ counts, int32_t* __restrict__ expert_start,
     int32_t* __restrict__ tile_row_start, int32_t* __restrict__ tile_expert,
-    int32_t* __restrict__ tile_count) {
+    int32_t* __restrict__ tile_count, int e0) {
     (void)TK;
-    route_scan_block(cnt, n_chunks, E, block_m, counts, expert_start, tile_row_start, tile_expert, tile_count);
+    route_scan_block(cnt, n_chunks, E, block_m, counts, expert_start, tile_row_start, tile_expert, tile_count, e0);
 }
 
 // One block after the kernel that chains the router projection to the post-process: the scan over
@@ -207,9 +215,10 @@ __global__ __launch_bounds__(1024) void head_finish_kernel(
 
 // chunk_len entries per wave (a multiple of 64 is not required); the chunks are the ones the
 // counters in cnt were taken over
+// E: all experts; [e0, e0 + EW): the window of this pass (cnt is [chunk][EW], expert_start points at expert e0)
 __global__ __launch_bounds__(kThreads) void route_scatter_kernel(
-    const int32_t* __restrict__ idx, int64_t TK, int K, int E, int chunk_len, const int32_t* __restrict__ cnt,
-    const int32_t* __restrict__ expert_start, int32_t* __restrict__ s_scatter,
+    const int32_t* __restrict__ idx, int64_t TK, int K, int E, int e0, int EW, int chunk_len,
+    const int32_t* __restrict__ cnt, const int32_t* __restrict__ expert_start, int32_t* __restrict__ s_scatter,
     int32_t* __restrict__ s_reverse, int32_t* __restrict__ x_gather) {
     extern __shared__ int32_t lds[];  // [kWaves][E] next free row per expert
     const int wave = threadIdx.x / MTS_WAVE, lane = threadIdx.x % MTS_WAVE;
@@ -217,15 +226,17 @@ __global__ __launch_bounds__(kThreads) void route_scatter_kernel(
     const int64_t cbeg = chunk * chunk_len;
     if (cbeg >= TK) return;  // whole wave leaves; no block barrier below
     const int64_t cend = cbeg + chunk_len < TK ? cbeg + chunk_len : TK;
-    volatile int32_t* next = lds + wave * E;
-    for (int e = lane; e < E; e += MTS_WAVE) next[e] = expert_start[e] + cnt[chunk * E + e];
+    volatile int32_t* next = lds + wave * EW;
+    for (int e = lane; e < EW; e += MTS_WAVE) next[e] = expert_start[e] + cnt[chunk * EW + e];
     const uint64_t lt = lanemask_lt();
   for (int64_t base = cbeg; base < cend; base += kChunk) {   // kSteps x 64 entries at a time
     int ev[kSteps];
 #pragma unroll
     for (int s = 0; s < kSteps; ++s) {  // these loads are in flight together
         const int64_t n = base + s * MTS_WAVE + lane;
-        ev[s] = n < cend ? clamp_expert(idx[n], E) : -1;
+        const int e = n < cend ? clamp_expert(idx[n], E) : -1;
+        // window-relative id; -1: dropped route (its -1 goes to s_reverse in the first pass), -2: not this pass
+        ev[s] = e < 0 ? (e0 == 0 && n < cend ? -1 : -2) : (e >= e0 && e < e0 + EW ? e - e0 : -2);
     }
 #pragma unroll
     for (int s = 0; s < kSteps; ++s) {
@@ -244,7 +255,7 @@ __global__ __launch_bounds__(kThreads) void route_scatter_kernel(
             if (lane == leader) next[el] = first + __popcll(same);
             todo &= ~same;
         }
-        if (n < cend) s_reverse[n] = pos;
+        if (e >= -1 && n < cend) s_reverse[n] = pos;
         if (valid) {
             s_scatter[pos] = (int32_t)n;
             x_gather[pos] = (int32_t)(n / K);
@@ -258,7 +269,7 @@ __global__ __launch_bounds__(kThreads) void route_scatter_kernel(
 extern "C" int64_t mts_moe_route_workspace_bytes(int64_t T, int K, int E) {
     int64_t TK = T * K;
     int64_t n_chunks = (TK + kChunk - 1) / kChunk;
-    return n_chunks * E * (int64_t)sizeof(int32_t);
+    return n_chunks * (E < MTS_MAX_EXPERTS ? E : MTS_MAX_EXPERTS) * (int64_t)sizeof(int32_t);   // one window of experts at a time
 }
 
 namespace {
@@ -273,16 +284,19 @@ int route_launch(const int32_t* top_k_index, int64_t T, int K, int E, int block_
     const int64_t TK = T * K;
     const int64_t n_chunks = (TK + kChunk - 1) / kChunk;
     const int grid = (int)((n_chunks + kWaves - 1) / kWaves);
-    const size_t lds = (size_t)kWaves * E * sizeof(int32_t);
-    route_hist_kernel<<<grid, kThreads, lds, s>>>(top_k_index, TK, E, cnt);
-    MTS_CHECK_LAUNCH();
-    route_scan_kernel<<<1, 1024, 0, s>>>(cnt, n_chunks, E, TK, block_m, counts, expert_start,
-                                         tile_row_start, tile_expert, tile_count);
-    MTS_CHECK_LAUNCH();
-    if (!permute) return MTS_OK;
-    route_scatter_kernel<<<grid, kThreads, lds, s>>>(top_k_index, TK, K, E, kChunk, cnt, expert_start,
-                                                     s_scatter, s_reverse, x_gather);
-    MTS_CHECK_LAUNCH();
+    for (int e0 = 0; e0 < E; e0 += MTS_MAX_EXPERTS) {   // one pass per window of experts
+        const int EW = E - e0 < MTS_MAX_EXPERTS ? E - e0 : MTS_MAX_EXPERTS;
+        const size_t lds = (size_t)kWaves * EW * sizeof(int32_t);
+        route_hist_kernel<<<grid, kThreads, lds, s>>>(top_k_index, TK, E, e0, EW, cnt);
+        MTS_CHECK_LAUNCH();
+        route_scan_kernel<<<1, 1024, 0, s>>>(cnt, n_chunks, EW, TK, block_m, counts + e0, expert_start + e0,
+                                             tile_row_start, tile_expert, tile_count, e0);
+        MTS_CHECK_LAUNCH();
+        if (!permute) continue;
+        route_scatter_kernel<<<grid, kThreads, lds, s>>>(top_k_index, TK, K, E, e0, EW, kChunk, cnt, expert_start + e0,
+                                                         s_scatter, s_reverse, x_gather);
+        MTS_CHECK_LAUNCH();
+    }
     return MTS_OK;
 }
 
@@ -295,7 +309,7 @@ int route_check(const int32_t* top_k_index, int64_t T, int K, int E, int block_m
     const bool permute = s_scatter || s_reverse || x_gather;
     if (!top_k_index || !counts || !expert_start) return MTS_ERR_NULL;
     if (permute && (!s_scatter || !s_reverse || !x_gather)) return MTS_ERR_NULL;
-    if (T <= 0 || K < 1 || E < 1 || E > MTS_MAX_EXPERTS || block_m < 1 ||
+    if (T <= 0 || K < 1 || E < 1 || E > MTS_MAX_MOE_EXPERTS || block_m < 1 ||
         T * (int64_t)K > 0x7fffffffLL)
         return MTS_ERR_SHAPE;
     return MTS_OK;
@@ -388,7 +402,7 @@ extern "C" int mts_moe_head_fwd(const void* x, const float* w_r, int64_t T, int 
     MTS_CHECK_LAUNCH();
     const int grid = (int)((n_chunks + kWaves - 1) / kWaves);
     const size_t lds = (size_t)kWaves * E * sizeof(int32_t);
-    route_scatter_kernel<<<grid, kThreads, lds, s>>>(indices, T * (int64_t)K, K, E, (int)(rows_per_chunk * K), cnt,
+    route_scatter_kernel<<<grid, kThreads, lds, s>>>(indices, T * (int64_t)K, K, E, 0, E, (int)(rows_per_chunk * K), cnt,
                                                      expert_start, s_scatter, s_reverse, x_gather);
     MTS_CHECK_LAUNCH();
     return MTS_OK;

@@ -15,7 +15,7 @@ import torch
 
 from minitrain_amd import _lib
 
-_MAX_EXPERTS = 1024
+_MAX_EXPERTS = 65534   # MTS_MAX_MOE_EXPERTS
 BLOCK_M_TOKEN = 64
 
 
@@ -54,11 +54,9 @@ def expert_contract(x, gate_up_proj, down_proj):
          "gate_up_proj is [E,2I,H] and down_proj [E,H,I] for x [T,H]"),
         (gate_up_proj.dtype in param_dtypes and down_proj.dtype in param_dtypes,
          "expert parameters in the activation dtype or fp32 (any of fp32/bf16/fp16 under fp32 activations)"),
-        (H % (4 if wide else 8) == 0, "hidden size a multiple of 8 (4 for fp32 activations)"),
         # rows of x and of dO are gathered from anywhere through 32-bit offsets; the [T*K, ...] intermediates are
         # addressed tile by tile and may be larger
         (wide or (T * H * 2 < 2**31 and 2 * I * H * 2 < 2**31), "16-bit activations and one expert's weights smaller than 2 GiB each"),
-        (wide or I % 8 == 0, "expert width a multiple of 8 for 16-bit activations"),
     ]
 
 
@@ -72,7 +70,7 @@ def routing_contract(x, gate_up_proj, top_k_index, top_k_weights):
         (top_k_index.is_cuda and top_k_weights.is_cuda and top_k_index.device == x.device == top_k_weights.device,
          "routing tensors on the activations' GPU"),
         (top_k_weights.shape == top_k_index.shape and top_k_index.shape[0] == x.shape[0], "top_k_index and top_k_weights are [T,K]"),
-        (0 < K <= min(gate_up_proj.shape[0], 32768), "1 <= K <= number of experts"),
+        (0 < K <= min(gate_up_proj.shape[0], 32768), "1 <= K <= number of experts (at most 32768)"),
         (x.shape[0] * K < 2**31, "fewer than 2^31 routes"),
         (top_k_index.dtype == torch.int32, "int32 expert indices"),
         (top_k_weights.dtype == x.dtype, "routing weights in the activation dtype"),
@@ -482,8 +480,39 @@ class _FusedMoEFunction(torch.autograd.Function):
         return dx, dw1, dw2, None, ds
 
 
+def _width_granule(dtype: torch.dtype) -> int:
+    """The kernels move 16 bytes per lane: rows must be a whole number of 16-byte chunks."""
+    return 4 if dtype == torch.float32 else 8
+
+
+def needs_padding(x, gate_up_proj) -> bool:
+    g = _width_granule(x.dtype)
+    return x.shape[1] % g != 0 or (x.dtype != torch.float32 and (gate_up_proj.shape[1] // 2) % g != 0)
+
+
+def _padded_operands(x, gate_up_proj, down_proj):
+    """Zero-padded copies whose widths are whole 16-byte chunks: H -> H8 everywhere, I -> I8 with the gate
+    rows at 0.. and the up rows at I8...  Zero columns and rows contribute nothing to any product, so the
+    operator's result on the padded operands, cut back to H columns, is the result on the originals; the
+    copies are made with differentiable torch ops, so the gradients come back cut to size as well."""
+    g = _width_granule(x.dtype)
+    E, two_i, H = gate_up_proj.shape
+    I = two_i // 2
+    H8 = -(-H // g) * g
+    I8 = I if x.dtype == torch.float32 else -(-I // g) * g
+    pad = torch.nn.functional.pad
+    gate, up = gate_up_proj[:, :I], gate_up_proj[:, I:]
+    w1 = torch.cat([pad(gate, (0, H8 - H, 0, I8 - I)), pad(up, (0, H8 - H, 0, I8 - I))], dim=1)
+    return pad(x, (0, H8 - H)), w1, pad(down_proj, (0, I8 - I, 0, H8 - H))
+
+
 def fused_moe(x, gate_up_proj, down_proj, top_k_index, top_k_weights):
     missed = fused_moe_violation(x, gate_up_proj, down_proj, top_k_index, top_k_weights)
     if missed is not None:
         raise RuntimeError(f"Unsupported tensor contract for hip fused MoE: it requires {missed}")
+    if needs_padding(x, gate_up_proj):
+        # widths that are not whole 16-byte chunks (legal in the reference, minitrain/kernels/triton/fused_moe.py:55-70)
+        H = x.shape[1]
+        xp, w1p, w2p = _padded_operands(x, gate_up_proj, down_proj)
+        return _FusedMoEFunction.apply(xp, w1p, w2p, top_k_index, top_k_weights)[:, :H]
     return _FusedMoEFunction.apply(x, gate_up_proj, down_proj, top_k_index, top_k_weights)

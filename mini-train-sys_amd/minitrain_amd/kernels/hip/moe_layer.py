@@ -14,7 +14,7 @@ offers it (``ops.moe_layer``) and the configuration allows it.
 import torch
 
 from minitrain_amd import _lib
-from minitrain_amd.kernels.hip.fused_moe import expert_contract, first_violation, moe_backward, moe_forward
+from minitrain_amd.kernels.hip.fused_moe import expert_contract, first_violation, moe_backward, moe_forward, needs_padding
 from minitrain_amd.kernels.hip.router import _MAX_TOP_K, is_router_logits_supported
 
 
@@ -30,6 +30,7 @@ def moe_layer_violation(x, router_weight, gate_up_proj, down_proj, top_k: int):
         (is_router_logits_supported(x, router_weight),
          "an fp32 router weight on the same GPU, at most 16 experts and a hidden size of at most 1024"),
         (1 <= top_k <= min(E, _MAX_TOP_K), f"1 <= top_k <= min(E, {_MAX_TOP_K})"),
+        (not needs_padding(x, gate_up_proj), "hidden and expert widths that are whole 16-byte chunks"),
         (x.shape[0] * top_k < 2**31, "fewer than 2^31 routes"),
     ])
 

@@ -41,6 +41,15 @@ def test_fp16_activations(T, H, E, I, K):
     _compare(routed_case(60 + T, T, H, E, I, K, dtype=torch.float16))
 
 
+@pytest.mark.parametrize("T,H,E,I,K,dtype", [(300, 100, 4, 52, 2, torch.bfloat16), (65, 36, 3, 20, 1, torch.float16),
+                                             (200, 50, 4, 30, 2, torch.float32), (257, 64, 8, 100, 2, torch.bfloat16)])
+def test_widths_that_are_not_whole_16_byte_chunks(T, H, E, I, K, dtype):
+    """H or I not a multiple of 8 (4 for fp32) is legal in the reference (triton/fused_moe.py:55-70); the
+    operator pads the operands with zeros, which changes no product, and cuts results and gradients back."""
+    print(f"moe odd widths T={T} H={H} E={E} I={I} K={K} {dtype}", flush=True)
+    _compare(routed_case(120 + T, T, H, E, I, K, dtype=dtype), tol=1e-5 if dtype == torch.float32 else BF16_TOL)
+
+
 def test_fp16_activations_fp32_master_weights():
     print("moe fp16 with fp32 weights", flush=True)
     case = routed_case(61, 300, 128, 4, 192, 2, dtype=torch.float16)
@@ -291,7 +300,7 @@ def test_unweighted_post_act_path(monkeypatch):
         assert torch.equal(a[1][3], b[1][3])   # dS does not depend on where the weight is applied
 
 
-@pytest.mark.parametrize("T,H,E,I,skew", [(600, 64, 130, 64, 0.0), (900, 64, 130, 64, 0.6)])
+@pytest.mark.parametrize("T,H,E,I,skew", [(600, 64, 130, 64, 0.0), (900, 64, 130, 64, 0.6), (400, 64, 1500, 32, 0.0)])
 def test_more_experts_than_a_wave_holds(T, H, E, I, skew):
     """E > 64: the tile and unit lookups of the GEMM kernels take more than one round of 64 experts
     (with skew, row chunks of an over-full expert add workspace slots to the lookup)."""
