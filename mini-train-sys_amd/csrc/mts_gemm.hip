@@ -545,7 +545,7 @@ constexpr int kXcds = 8;
 // ballot picks the first expert whose offset range contains the tile (63 experts per
 // round; more experts take more rounds).
 template <int BM>
-__device__ __forceinline__ bool locate_rows_tile(const RowsParams& p, int b, int& e, int& row0, int& rend, int& ntile) {
+__device__ __forceinline__ bool find_rows_tile(const RowsParams& p, int b, int& e, int& row0, int& rend, int& ntile) {
     const int xcd = b % kXcds, j = b / kXcds;
     const int lane = threadIdx.x % MTS_WAVE;
     int tile = xcd + kXcds * (j / p.n_tiles);
@@ -585,6 +585,20 @@ __device__ __forceinline__ bool locate_rows_tile(const RowsParams& p, int b, int
         seen += __shfl(incl, MTS_WAVE - 1, MTS_WAVE);
     }
     return false;
+}
+
+// The answer is the same in every lane, and the compiler is told so behind the search loop: descriptors
+// and LDS addresses built from these values then stay in scalar registers (a buffer instruction whose
+// descriptor sits in vector registers is wrapped in a loop over its distinct values).
+template <int BM>
+__device__ __forceinline__ bool locate_rows_tile(const RowsParams& p, int b, int& e, int& row0, int& rend, int& ntile) {
+    int fe = 0, frow0 = 0, frend = 0, fn = 0;
+    const bool found = find_rows_tile<BM>(p, b, fe, frow0, frend, fn);
+    e = __builtin_amdgcn_readfirstlane(fe);
+    row0 = __builtin_amdgcn_readfirstlane(frow0);
+    rend = __builtin_amdgcn_readfirstlane(frend);
+    ntile = __builtin_amdgcn_readfirstlane(fn);
+    return __builtin_amdgcn_readfirstlane((int)found) != 0;
 }
 
 // ---------------------------------------------------------------------------

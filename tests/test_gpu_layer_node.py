@@ -105,7 +105,8 @@ def _separate_grads(ops, case, K, normalize, dtype, fp32_params):
 @pytest.mark.parametrize("T,H,E,I,K,dtype,fp32_params,normalize", [
     (512, 128, 8, 256, 2, torch.bfloat16, False, True), (2048, 768, 8, 1024, 2, torch.bfloat16, True, True),
     (33, 64, 4, 64, 1, torch.float16, False, True), (700, 72, 3, 40, 2, torch.bfloat16, False, False),
-    (300, 64, 16, 96, 4, torch.float32, False, True), (1, 64, 4, 64, 2, torch.bfloat16, False, True)])
+    (300, 64, 16, 96, 4, torch.float32, False, True), (1, 64, 4, 64, 2, torch.bfloat16, False, True),
+    (200, 64, 8, 64, 5, torch.bfloat16, False, True)])
 def test_layer_node_equals_the_separate_operators_and_the_oracle(T, H, E, I, K, dtype, fp32_params, normalize):
     print(f"layer node T={T} H={H} E={E} I={I} K={K} {dtype} fp32_params={fp32_params} normalize={normalize}", flush=True)
     ops = hip_backend()
