@@ -1547,10 +1547,10 @@ enum Kind { K_GATEUP = 0, K_DOWN, K_DY1, K_DX, K_DW2, K_DW1, K_COUNT };
 const char* const kKindEnv[K_COUNT] = {"MTS_TILE_GATEUP", "MTS_TILE_DOWN", "MTS_TILE_DY1",
                                        "MTS_TILE_DX",     "MTS_TILE_DW2",  "MTS_TILE_DW1"};
 // rows_gemm: 0 StagedSmall, 1 RingTwoPerCu, 2 WsLarge;  dw_gemm: 0 StagedSmall, 2 DwWsLarge.
-// Defaults are the fastest measured on the 24576-token, 768/1024, 8-expert layer: dY1, whose
-// epilogue is as long as its main loop, gains more from two co-resident blocks, everything
-// else from specialised waves (gate/up since its epilogue arithmetic got cheaper).
-const int kDefaultTile[K_COUNT] = {2, 2, 1, 2, 2, 2};
+// Defaults are the fastest measured on the 24576-token, 768/1024, 8-expert layer: the two GEMMs with
+// the heavy epilogues (gate/up + SwiGLU, dO*W2 + SwiGLU backward) gain more from two co-resident
+// 4-wave blocks per CU, the others from specialised waves.
+const int kDefaultTile[K_COUNT] = {1, 2, 1, 2, 2, 2};
 
 // tile shape per GEMM; the environment overrides exist for tuning runs only
 int tile_choice(int kind) {
