@@ -1552,6 +1552,8 @@ const char* const kKindEnv[K_COUNT] = {"MTS_TILE_GATEUP", "MTS_TILE_DOWN", "MTS_
 // 4-wave blocks per CU, the others from specialised waves.
 const int kDefaultTile[K_COUNT] = {1, 2, 1, 2, 2, 2};
 
+bool tile_forced(int kind) { return getenv(kKindEnv[kind]) != nullptr; }
+
 // tile shape per GEMM; the environment overrides exist for tuning runs only
 int tile_choice(int kind) {
     static int choice[K_COUNT] = {-1, -1, -1, -1, -1, -1};
@@ -1583,21 +1585,25 @@ int64_t m_tiles(int64_t TK, int E) {
     return a < TK ? a : TK;
 }
 
-// MTS_XCD_RANGES=0 selects the round-robin deal of m-tiles to XCDs (tuning runs only)
-int xcd_ranges_choice() {
-    static int choice = -1;
-    if (choice < 0) {
+// Contiguous ranges of m-tiles per XCD pay off while one expert's weight matrix stays resident in an
+// XCD's 4 MiB L2 next to the streaming operands; larger weights are better streamed by all XCDs at the
+// same time (round-robin deal: one fetch from HBM, the other seven from the Infinity Cache).
+// MTS_XCD_RANGES=0/1 forces one or the other (tuning runs only).
+int xcd_ranges_choice(int64_t expert_weight_bytes) {
+    static int forced = -2;
+    if (forced == -2) {
         const char* s = getenv("MTS_XCD_RANGES");
-        choice = (s && atoi(s) == 0) ? 0 : 1;
+        forced = s ? (atoi(s) != 0) : -1;
     }
-    return choice;
+    if (forced >= 0) return forced;
+    return expert_weight_bytes <= (4 << 20) ? 1 : 0;
 }
 
 template <class T, int EPI>
 dim3 rows_grid(RowsParams& p, int64_t TK) {
     const int per_block = (EPI == EPI_SWIGLU) ? T::BN / 2 : T::BN;
     p.n_tiles = (p.N + per_block - 1) / per_block;
-    p.xcd_ranges = xcd_ranges_choice();
+    p.xcd_ranges = xcd_ranges_choice((int64_t)p.b_rows * p.Kdim * (int64_t)sizeof(bf16_t));
     const int64_t m_groups = (m_tiles<T>(TK, p.E) + kXcds - 1) / kXcds;
     return dim3((unsigned)(m_groups * kXcds * p.n_tiles));
 }
@@ -1610,6 +1616,9 @@ bool rows_kmajor_ok(int kind, int Kdim) { return tile_choice(kind) >= 1 && Kdim 
 template <int EPI>
 int launch_rows_any(int kind, RowsParams p, int64_t TK, hipStream_t s, bool b_kmajor = false) {
     int choice = tile_choice(kind);
+    // gate/up: two co-resident ring blocks per CU win while the SwiGLU epilogue is a large part of a tile
+    // (short reductions); long reductions are better off with specialised waves
+    if (kind == K_GATEUP && !tile_forced(kind) && p.Kdim > 1024) choice = 2;
     // the ring kernels need whole k-tiles; other shapes use the staged kernel
     if (choice >= 1 && p.Kdim % 64 != 0) choice = 0;
     if (b_kmajor && (choice == 0 || EPI == EPI_SWIGLU)) return MTS_ERR_SHAPE;

@@ -65,7 +65,7 @@ class MoeRanges:
         return t
 
 
-def run(layers=12, batch=24, seq=1024, vocab=50257, steps=5, warmup=2, seed=4, fused_loss=False) -> dict:
+def run(layers=12, batch=24, seq=1024, vocab=50257, steps=5, warmup=5, seed=4, fused_loss=False) -> dict:
     """Builds the decoder, trains ``warmup + steps`` steps on one synthetic batch and returns the record."""
     torch.manual_seed(seed)
     cfg = ModelConfig(vocab_size=vocab, seq_len=seq, n_layers=layers, n_heads=12, hidden_size=768,
@@ -110,7 +110,8 @@ def main():
     ap.add_argument("--seq", type=int, default=1024)
     ap.add_argument("--vocab", type=int, default=50257)
     ap.add_argument("--steps", type=int, default=5)
-    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--warmup", type=int, default=5,
+                    help="untimed steps; the caching allocator settles within the first four (one of them stalls ~70 ms)")
     ap.add_argument("--seed", type=int, default=4)
     ap.add_argument("--fused-loss", action="store_true")
     args = ap.parse_args()
