@@ -45,8 +45,8 @@ RIDGE_FLOP_PER_BYTE = PEAK_BF16_TFLOPS * 1e12 / (PEAK_HBM_GBS * 1e9)   # 312.5: 
 # line names the file that holds the runs' commands and tables.
 TRAFFIC_SOURCE = "profiles/moe_layer_24x1024_hbm_traffic.txt"
 MEASURED_TRAFFIC_BYTES = {
-    "fwd_gateup_swiglu": 694.8e6, "fwd_down": 303.4e6, "bwd_dy1": 710.5e6, "bwd_joint": 1115.7e6,
-    "combine": 115.2e6, "dx_combine": 114.4e6,
+    "fwd_gateup_swiglu": 656.9e6, "fwd_down": 223.9e6, "bwd_dy1": 531.2e6, "bwd_joint": 971.4e6,
+    "combine": 114.6e6, "dx_combine": 152.4e6,
 }
 
 WORKLOAD = dict(name="moe_layer_24x1024_d768_e8_top2_ff1024_bf16", seed=1, T=24576, H=768, E=8, K=2, I=1024)
@@ -226,6 +226,39 @@ def stage_breakdown(layer, steps):
     return rows
 
 
+def mfma_sustained(blocks=512, rounds=2500, repeats=3):
+    """What the matrix pipes sustain on registers alone (no LDS, no memory): the library's probe kernel,
+    timed with events on the launching stream.  Operands that toggle from instruction to instruction cost
+    clock on this power-limited chip, so the rate on pseudo-random registers is the practical ceiling the
+    GEMM figures are read against; the nominal peak stays the denominator of every `frac`."""
+    import ctypes
+
+    from minitrain_amd import _lib
+
+    lib = _lib.load()
+    sink = torch.empty(lib.mts_probe_mfma_sink_bytes(blocks), dtype=torch.uint8, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    flops = ctypes.c_double(0.0)
+    out = {}
+    for name, random_operands in (("random_operands", 1), ("constant_operands", 0)):
+        best = None
+        for it in range(1 + repeats):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            rc = lib.mts_probe_mfma_rate(random_operands, blocks, rounds, sink.data_ptr(), sink.numel(), ctypes.addressof(flops), st)
+            e1.record()
+            if rc != 0:
+                raise RuntimeError(f"mts_probe_mfma_rate returned {rc}")
+            torch.cuda.synchronize()
+            if it:
+                ms = e0.elapsed_time(e1)
+                best = ms if best is None else min(best, ms)
+        out[name + "_tflops"] = round(flops.value / (best * 1e-3) / 1e12, 1)
+    out.update(peak=PEAK_BF16_TFLOPS, unit="TFLOP/s", frac_of_peak=round(out["random_operands_tflops"] / PEAK_BF16_TFLOPS, 4),
+               kernel="register-only bf16 32x32x16 MFMA loop, 512 blocks of 4 waves, best of 3 launches of ~8 ms")
+    return out
+
+
 def cpu_baseline(budget_s=20.0):
     """The oracle's restatement of the reference's PyTorch path (input-dtype arithmetic,
     autograd backward) on the host cores, on the first ``sample`` tokens of the workload."""
@@ -263,6 +296,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-breakdown", action="store_true")
+    ap.add_argument("--no-mfma-probe", action="store_true", help="skip the register-only MFMA rate probe")
     ap.add_argument("--no-settle", action="store_true", help="skip the untimed clock-settling steps before the warm-up")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 256 MiB -> 256 MiB elementwise copy (the known-size kernel that "
@@ -328,6 +362,11 @@ def main():
         result["combine_roofline"] = {"bound": "hbm", "achieved": round(c_ach, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                                       "frac": round(c_ach / PEAK_HBM_GBS, 4), "sum_ms": round(c_ms, 4)}
         result["kernel_sum_ms"] = round(sum(r["avg_ms"] for r in rows), 4)
+    if not args.no_mfma_probe:
+        result["mfma_sustained"] = mfma_sustained()
+        if "gemm_roofline" in result:
+            result["gemm_roofline"]["frac_of_sustained"] = round(
+                result["gemm_roofline"]["achieved"] / result["mfma_sustained"]["random_operands_tflops"], 4)
     if args.copy_probe:
         src = torch.ones(64 * 2**20, dtype=torch.float32, device="cuda")
         dst = torch.empty_like(src)

@@ -49,6 +49,8 @@ SIGNATURES = {
     "mts_moe_head_bwd_workspace_bytes": (_l, [_l, _i, _i]),
     "mts_moe_head_bwd": (_i, [_p] * 11 + [_l, _i, _i, _i, _i, _i, _p, _p, _p, _l, _p]),
     "mts_moe_ds_partials": (_i, [_i]),
+    "mts_probe_mfma_sink_bytes": (_l, [_i]),
+    "mts_probe_mfma_rate": (_i, [_i, _i, _i, _p, _l, _p, _p]),
     "mts_moe_bwd_weights_as_stored": (_i, [_i, _i, _i]),
     "mts_moe_bwd_dy1": (_i, [_p, _p, _i, _p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p, _p, _p, _p]),
     "mts_moe_bwd_ds": (_i, [_p, _p, _l, _i, _i, _p, _p]),

@@ -19,7 +19,7 @@ CSRC = os.path.join(os.path.dirname(PKG_DIR), "csrc")
 INCLUDE = os.path.join(os.path.dirname(os.path.dirname(PKG_DIR)), "include")
 LIB_DIR = os.path.join(PKG_DIR, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libmts_moe.so")
-SOURCES = ("mts_router.hip", "mts_router_linear.hip", "mts_route.hip", "mts_capacity.hip", "mts_combine.hip", "mts_gemm.hip", "mts_gemm_f16.hip", "mts_gemm_f32.hip")
+SOURCES = ("mts_router.hip", "mts_router_linear.hip", "mts_route.hip", "mts_capacity.hip", "mts_combine.hip", "mts_gemm.hip", "mts_gemm_f16.hip", "mts_gemm_f32.hip", "mts_probe.hip")
 
 FLAGS = [
     "-O3",

@@ -7,11 +7,15 @@ import re
 import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-HEADER = os.path.join(ROOT, "include", "mts_moe.h")
+HEADERS = [os.path.join(ROOT, "include", name) for name in ("mts_moe.h", "mts_probe.h")]
+
+
+def test_every_public_header_is_covered():
+    assert sorted(os.listdir(os.path.join(ROOT, "include"))) == sorted(os.path.basename(h) for h in HEADERS)
 
 
 def _declared():
-    text = open(HEADER).read()
+    text = "".join(open(h).read() for h in HEADERS)
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(mts_[a-z0-9_]+)\s*\(", text)))
 
@@ -31,7 +35,7 @@ def test_library_exports_every_declared_symbol():
         pytest.fail(f"{_lib.LIB_PATH} not built: run `python -c 'import __graft_entry__ as g; g.build()'`")
     lib = _lib.load()
     for name in _declared():
-        assert hasattr(lib, name), f"{name} is declared in mts_moe.h but not exported"
+        assert hasattr(lib, name), f"{name} is declared in include/ but not exported"
         assert name in _lib.SIGNATURES, f"{name} has no ctypes prototype"
     assert lib.mts_version() == 2
     assert lib.mts_error_string(0) == b"ok"
@@ -77,6 +81,11 @@ def test_contract_violations_are_reported_before_any_launch():
     assert joint(*(ok_args[:14] + [_lib.MTS_F32] + ok_args[15:])) == -3                      # activations must be 16-bit
     assert joint(*(ok_args[:12] + [72, 40] + ok_args[14:])) == SHAPE                          # 2I = 80 has no whole k-tile
     assert joint(*(ok_args[:20] + [fake, 16] + ok_args[22:])) == WORKSPACE
+    # the MFMA rate probe: sink pointer, launch size, sink size
+    assert lib.mts_probe_mfma_sink_bytes(512) == 512 * 256 * 4
+    assert lib.mts_probe_mfma_rate(1, 512, 100, None, 1 << 20, None, None) == NULL
+    assert lib.mts_probe_mfma_rate(1, 0, 100, fake, 1 << 20, None, None) == SHAPE
+    assert lib.mts_probe_mfma_rate(1, 512, 100, fake, 16, None, None) == WORKSPACE
     # unknown element type
     assert lib.mts_moe_combine(fake, None, None, fake, 8, 2, 64, 7, fake, None) == -3
 

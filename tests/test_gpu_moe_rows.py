@@ -58,3 +58,28 @@ def test_decoder_step_at_the_real_size():
     assert 0.0 < rec["moe_share_of_step"] < 1.0 and rec["moe_ms_per_step"] > 0
     assert rec["value"] > 0 and rec["config"]["layers"] == 12
     torch.cuda.empty_cache()
+
+
+def test_mfma_rate_probe_reports_a_plausible_rate():
+    """The register-only MFMA loop the benchmark line quotes as `mfma_sustained`: every thread's sum is
+    finite, the reported FLOPs match the launch, and the rate lies between a tenth of the nominal bf16 peak
+    and the peak itself (2.5 PFLOP/s); constant operands are not slower than toggling ones by more than noise."""
+    print("mfma rate probe", flush=True)
+    import sys
+    from pathlib import Path
+
+    sys.path.insert(0, str(Path(__file__).resolve().parents[1]))
+    import bench
+
+    rec = bench.mfma_sustained(blocks=512, rounds=500, repeats=2)
+    assert rec["peak"] == 2500.0 and rec["unit"] == "TFLOP/s"
+    for key in ("random_operands_tflops", "constant_operands_tflops"):
+        assert 250.0 < rec[key] <= 2500.0, rec
+    assert rec["constant_operands_tflops"] >= 0.9 * rec["random_operands_tflops"], rec
+    from minitrain_amd import _lib
+
+    lib = _lib.load()
+    sink = torch.full((64 * 256,), float("nan"), device="cuda")
+    assert lib.mts_probe_mfma_rate(1, 64, 4, sink.data_ptr(), sink.numel() * 4, None, torch.cuda.current_stream().cuda_stream) == 0
+    torch.cuda.synchronize()
+    assert torch.isfinite(sink).all() and sink.abs().max() > 0
