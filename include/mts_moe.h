@@ -95,7 +95,7 @@ int mts_router_bwd(const float* logits, const float* weights, const int32_t* ind
  * (minitrain/model/moe_router.py:64-76: `hidden_states.float()` followed by
  * `F.linear(router_input, weight.float())`): logits[t,e] = sum_h float(x[t,h]) * w_r[e,h],
  * fp32 products and sums, x [T,H] read in act_dtype (no fp32 copy), w_r [E,H] f32.
- * E <= 16, H a multiple of 4 and at most 1024.                                 */
+ * E <= 16, H a multiple of 4 and at most 4096, E * H <= 32768 (W_r sits in LDS).   */
 int mts_router_logits_fwd(const void* x, const float* w_r, int64_t T, int H, int E,
                           int act_dtype, float* logits, void* stream);
 
@@ -114,7 +114,7 @@ int mts_router_logits_bwd(const float* dlogits, const void* x, const float* w_r,
  * registers, the routes per expert it counts per block are the chunk histogram of the
  * routing metadata, and one block reduces the statistics and scans the counts.  Outputs as in
  * those three calls (logits [T,E] f32 are written for the backward pass; weights_act,
- * load_balance and load_stats may be NULL).  E <= 16, H a multiple of 4 and at most 1024,
+ * load_balance and load_stats may be NULL).  E <= 16, H a multiple of 4 and at most 4096, E * H <= 32768,
  * K <= min(E, MTS_MAX_TOP_K).  The statistics are summed in a fixed order of their own: they agree
  * with mts_router_fwd to rounding, indices and the permutation agree exactly.              */
 int64_t mts_moe_head_workspace_bytes(int64_t T, int K, int E);

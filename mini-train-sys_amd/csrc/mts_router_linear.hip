@@ -86,147 +86,34 @@ __device__ __forceinline__ void reduce_scatter(float (&v)[NV], int lane, int& id
 // One wave computes kRows rows: a lane owns 4 consecutive columns of every 256-column slab,
 // the weights sit in LDS (loaded once per block), and the E partial dot products of a row are
 // summed across the wave with a fixed shuffle tree.
-template <typename XT, int EP, int PASSES>
-__global__ __launch_bounds__(kFwdThreads) void router_logits_fwd_kernel(const XT* __restrict__ x,
-                                                                         const float* __restrict__ w, int64_t T,
-                                                                         int H, int E, float* __restrict__ logits) {
-    extern __shared__ __attribute__((aligned(16))) float w_lds[];   // [E][H]
-#pragma unroll 8
-    for (int i = threadIdx.x * 4; i < E * H; i += kFwdThreads * 4)
-        *reinterpret_cast<f32x4*>(w_lds + i) = *reinterpret_cast<const f32x4*>(w + i);
-    const int lane = threadIdx.x % MTS_WAVE;
-    const int64_t wave0 = (int64_t)blockIdx.x * (kFwdThreads / MTS_WAVE) + threadIdx.x / MTS_WAVE;
-    const int64_t stride = (int64_t)gridDim.x * (kFwdThreads / MTS_WAVE) * kRows;
+// CHUNKED (rows wider than PASSES slabs): the columns are taken in chunks of PASSES slabs, the
+// loads of the next chunk (of the same rows, or the first one of the next row group) in flight
+// behind the arithmetic of the current one, and the partial dot products stay in registers
+// until the last chunk of the row group.
+template <typename XT, int PASSES>
+struct RowGroupLoader {
     typedef typename RawVec<XT>::type raw_t;
-    // the loads of the next row group are issued before the arithmetic of the current one
-    raw_t cur[PASSES][kRows], nxt[PASSES][kRows];
-    auto load_group = [&](raw_t (&dst)[PASSES][kRows], int64_t r0) {
+    // rows r0..r0+kRows-1 (those below `end`), columns of chunk `ch`
+    static __device__ __forceinline__ void load(raw_t (&dst)[PASSES][kRows], const XT* __restrict__ x, int64_t r0,
+                                                int64_t end, int ch, int H, int lane) {
 #pragma unroll
         for (int ps = 0; ps < PASSES; ++ps) {
-            const int c = lane * 4 + ps * MTS_WAVE * 4;
-#pragma unroll
-            for (int r = 0; r < kRows; ++r) {
-                const bool ok = c < H && r0 + r < T;
-                dst[ps][r] = load_raw(x + (ok ? (r0 + r) * H + c : 0));   // a masked lane reads element 0; its weights are skipped
-            }
-        }
-    };
-    int64_t r0 = wave0 * kRows;
-    if (r0 < T) load_group(cur, r0);
-    __syncthreads();
-    for (; r0 < T; r0 += stride) {
-        if (r0 + stride < T) load_group(nxt, r0 + stride);
-        float acc[kRows][EP];
-#pragma unroll
-        for (int r = 0; r < kRows; ++r)
-#pragma unroll
-            for (int e = 0; e < EP; ++e) acc[r][e] = 0.f;
-#pragma unroll
-        for (int ps = 0; ps < PASSES; ++ps) {
-            const int c = lane * 4 + ps * MTS_WAVE * 4;
-            if (c < H) {
-                f32x4 xv[kRows];
-#pragma unroll
-                for (int r = 0; r < kRows; ++r) {
-                    const f32x4 z = {0.f, 0.f, 0.f, 0.f};
-                    xv[r] = r0 + r < T ? widen(cur[ps][r]) : z;
-                }
-#pragma unroll
-                for (int e = 0; e < EP; ++e) {
-                    const f32x4 wv = *reinterpret_cast<const f32x4*>(w_lds + (e < E ? e : 0) * H + c);
-#pragma unroll
-                    for (int r = 0; r < kRows; ++r)
-                        acc[r][e] += xv[r][0] * wv[0] + xv[r][1] * wv[1] + xv[r][2] * wv[2] + xv[r][3] * wv[3];
-                }
-            }
-        }
-#pragma unroll
-        for (int ps = 0; ps < PASSES; ++ps)
-#pragma unroll
-            for (int r = 0; r < kRows; ++r) cur[ps][r] = nxt[ps][r];
-        // Sum over the 64 lanes of kRows*EP values: at every step a lane hands half of its
-        // values to the partner lane and adds the partner's copy of the half it keeps, so the
-        // count halves with the lane distance (fixed order: bit-stable).  With kRows*EP == 32
-        // one value is left after the distance-2 step, shared by a lane pair.
-        static_assert(kRows * EP == 32 || kRows * EP == 64, "reduction layout");
-        constexpr int NV = kRows * EP;
-        float v[NV];
-#pragma unroll
-        for (int r = 0; r < kRows; ++r)
-#pragma unroll
-            for (int e = 0; e < EP; ++e) v[r * EP + e] = acc[r][e];
-        int idx = 0;   // index of the value this lane ends up with, built from its lane bits
-        reduce_scatter<NV, NV, 32>(v, lane, idx);
-        const float mine = v[0];
-        const int r = idx / EP, e = idx % EP;
-        const bool writer = NV == 64 ? true : (lane & 1) == 0;
-        if (writer && e < E && r0 + r < T) logits[(r0 + r) * E + e] = mine;
-    }
-}
-
-// ---------------------------------------------------------------------------
-// The router projection chained to the post-process.  The block takes a contiguous range of
-// rows, a wave a contiguous part of it; the 4 rows x E logits a wave has just summed sit one per
-// lane (pair), so lanes 0..3 collect a row each with cross-lane reads and run the post-process
-// on it (softmax, top-k on the logits, weights) without the logits making a round trip through
-// memory; the logits are still written, for the backward pass.  Per block: the sums of the
-// statistics (fixed order) and the routes per expert, which are at the same time the chunk
-// histogram of the routing metadata (chunk = the entries of the block's rows).
-// ---------------------------------------------------------------------------
-template <typename XT, int EP, int PASSES>
-__global__ __launch_bounds__(kFwdThreads) void router_head_kernel(
-    const XT* __restrict__ x, const float* __restrict__ w, int64_t T, int H, int E, int K, int normalize,
-    int rows_per_wave, float* __restrict__ logits, float* __restrict__ weights, int32_t* __restrict__ indices,
-    void* __restrict__ weights_act, int act_dtype, float* __restrict__ partial, int32_t* __restrict__ cnt) {
-    using namespace mts_router;
-    extern __shared__ __attribute__((aligned(16))) float w_lds[];   // [E][H]
-#pragma unroll 8
-    for (int i = threadIdx.x * 4; i < E * H; i += kFwdThreads * 4)
-        *reinterpret_cast<f32x4*>(w_lds + i) = *reinterpret_cast<const f32x4*>(w + i);
-    constexpr int WAVES = kFwdThreads / MTS_WAVE;
-    const int lane = threadIdx.x % MTS_WAVE, wave = threadIdx.x / MTS_WAVE;
-    const int64_t beg = ((int64_t)blockIdx.x * WAVES + wave) * rows_per_wave;
-    const int64_t end = beg + rows_per_wave < T ? beg + rows_per_wave : T;
-    typedef typename RawVec<XT>::type raw_t;
-    raw_t cur[PASSES][kRows], nxt[PASSES][kRows];
-    auto load_group = [&](raw_t (&dst)[PASSES][kRows], int64_t r0) {
-#pragma unroll
-        for (int ps = 0; ps < PASSES; ++ps) {
-            const int c = lane * 4 + ps * MTS_WAVE * 4;
+            const int c = lane * 4 + (ch * PASSES + ps) * MTS_WAVE * 4;
 #pragma unroll
             for (int r = 0; r < kRows; ++r) {
                 const bool ok = c < H && r0 + r < end;
                 dst[ps][r] = load_raw(x + (ok ? (r0 + r) * H + c : 0));   // a masked lane reads element 0; its weights are skipped
             }
         }
-    };
-    if (beg < end) load_group(cur, beg);
-    __syncthreads();
-
-    // The logits of up to 64 rows are parked in LDS (row stride EP + 1: a lane per row reads without
-    // bank conflicts); then lane L runs the post-process of row L, so a wave pays for the post-process
-    // once per 64 rows, not once per group of kRows.
-    constexpr int LROW = EP + 1;
-    __shared__ float parked[WAVES][MTS_WAVE * LROW];
-    float* mine_rows = parked[wave];
-    float psum[EP], zsum = 0.f, hsum = 0.f;   // statistics of the rows this lane post-processes
-    int csum[EP];
-#pragma unroll
-    for (int e = 0; e < EP; ++e) {
-        psum[e] = 0.f;
-        csum[e] = 0;
     }
-    int64_t pass_base = beg;
-    for (int64_t r0 = beg; r0 < end; r0 += kRows) {
-        if (r0 + kRows < end) load_group(nxt, r0 + kRows);
-        float acc[kRows][EP];
-#pragma unroll
-        for (int r = 0; r < kRows; ++r)
-#pragma unroll
-            for (int e = 0; e < EP; ++e) acc[r][e] = 0.f;
+    // acc[r][e] += the chunk's share of <x[r0+r], w[e]>
+    template <int EP>
+    static __device__ __forceinline__ void accumulate(float (&acc)[kRows][EP], const raw_t (&cur)[PASSES][kRows],
+                                                      const float* w_lds, int64_t r0, int64_t end, int ch, int H, int E,
+                                                      int lane) {
 #pragma unroll
         for (int ps = 0; ps < PASSES; ++ps) {
-            const int c = lane * 4 + ps * MTS_WAVE * 4;
+            const int c = lane * 4 + (ch * PASSES + ps) * MTS_WAVE * 4;
             if (c < H) {
                 f32x4 xv[kRows];
 #pragma unroll
@@ -243,10 +130,135 @@ __global__ __launch_bounds__(kFwdThreads) void router_head_kernel(
                 }
             }
         }
+    }
+};
+
+template <typename XT, int EP, int PASSES, bool CHUNKED = false>
+__global__ __launch_bounds__(kFwdThreads) void router_logits_fwd_kernel(const XT* __restrict__ x,
+                                                                         const float* __restrict__ w, int64_t T,
+                                                                         int H, int E, int n_chunks,
+                                                                         float* __restrict__ logits) {
+    extern __shared__ __attribute__((aligned(16))) float w_lds[];   // [E][H]
+#pragma unroll 8
+    for (int i = threadIdx.x * 4; i < E * H; i += kFwdThreads * 4)
+        *reinterpret_cast<f32x4*>(w_lds + i) = *reinterpret_cast<const f32x4*>(w + i);
+    const int lane = threadIdx.x % MTS_WAVE;
+    const int nch = CHUNKED ? n_chunks : 1;
+    const int64_t wave0 = (int64_t)blockIdx.x * (kFwdThreads / MTS_WAVE) + threadIdx.x / MTS_WAVE;
+    const int64_t stride = (int64_t)gridDim.x * (kFwdThreads / MTS_WAVE) * kRows;
+    typedef RowGroupLoader<XT, PASSES> Loader;
+    typename Loader::raw_t cur[PASSES][kRows], nxt[PASSES][kRows];
+    int64_t r0 = wave0 * kRows;
+    int ch = 0;
+    if (r0 < T) Loader::load(cur, x, r0, T, 0, H, lane);
+    __syncthreads();
+    float acc[kRows][EP];
+    while (r0 < T) {
+        const bool last = ch + 1 == nch;
+        const int64_t nr0 = last ? r0 + stride : r0;
+        const int nc = last ? 0 : ch + 1;
+        if (nr0 < T) Loader::load(nxt, x, nr0, T, nc, H, lane);
+        if (ch == 0) {
+#pragma unroll
+            for (int r = 0; r < kRows; ++r)
+#pragma unroll
+                for (int e = 0; e < EP; ++e) acc[r][e] = 0.f;
+        }
+        Loader::template accumulate<EP>(acc, cur, w_lds, r0, T, ch, H, E, lane);
 #pragma unroll
         for (int ps = 0; ps < PASSES; ++ps)
 #pragma unroll
             for (int r = 0; r < kRows; ++r) cur[ps][r] = nxt[ps][r];
+        if (last) {
+            // Sum over the 64 lanes of kRows*EP values: at every step a lane hands half of its
+            // values to the partner lane and adds the partner's copy of the half it keeps, so the
+            // count halves with the lane distance (fixed order: bit-stable).  With kRows*EP == 32
+            // one value is left after the distance-2 step, shared by a lane pair.
+            static_assert(kRows * EP == 32 || kRows * EP == 64, "reduction layout");
+            constexpr int NV = kRows * EP;
+            float v[NV];
+#pragma unroll
+            for (int r = 0; r < kRows; ++r)
+#pragma unroll
+                for (int e = 0; e < EP; ++e) v[r * EP + e] = acc[r][e];
+            int idx = 0;   // index of the value this lane ends up with, built from its lane bits
+            reduce_scatter<NV, NV, 32>(v, lane, idx);
+            const float mine = v[0];
+            const int r = idx / EP, e = idx % EP;
+            const bool writer = NV == 64 ? true : (lane & 1) == 0;
+            if (writer && e < E && r0 + r < T) logits[(r0 + r) * E + e] = mine;
+        }
+        r0 = nr0;
+        ch = nc;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// The router projection chained to the post-process.  The block takes a contiguous range of
+// rows, a wave a contiguous part of it; the 4 rows x E logits a wave has just summed sit one per
+// lane (pair), so lanes 0..3 collect a row each with cross-lane reads and run the post-process
+// on it (softmax, top-k on the logits, weights) without the logits making a round trip through
+// memory; the logits are still written, for the backward pass.  Per block: the sums of the
+// statistics (fixed order) and the routes per expert, which are at the same time the chunk
+// histogram of the routing metadata (chunk = the entries of the block's rows).
+// ---------------------------------------------------------------------------
+template <typename XT, int EP, int PASSES, bool CHUNKED = false>
+__global__ __launch_bounds__(kFwdThreads) void router_head_kernel(
+    const XT* __restrict__ x, const float* __restrict__ w, int64_t T, int H, int E, int K, int normalize,
+    int rows_per_wave, int n_chunks, float* __restrict__ logits, float* __restrict__ weights, int32_t* __restrict__ indices,
+    void* __restrict__ weights_act, int act_dtype, float* __restrict__ partial, int32_t* __restrict__ cnt) {
+    using namespace mts_router;
+    extern __shared__ __attribute__((aligned(16))) float w_lds[];   // [E][H]
+#pragma unroll 8
+    for (int i = threadIdx.x * 4; i < E * H; i += kFwdThreads * 4)
+        *reinterpret_cast<f32x4*>(w_lds + i) = *reinterpret_cast<const f32x4*>(w + i);
+    constexpr int WAVES = kFwdThreads / MTS_WAVE;
+    const int lane = threadIdx.x % MTS_WAVE, wave = threadIdx.x / MTS_WAVE;
+    const int nch = CHUNKED ? n_chunks : 1;
+    const int64_t beg = ((int64_t)blockIdx.x * WAVES + wave) * rows_per_wave;
+    const int64_t end = beg + rows_per_wave < T ? beg + rows_per_wave : T;
+    typedef RowGroupLoader<XT, PASSES> Loader;
+    typename Loader::raw_t cur[PASSES][kRows], nxt[PASSES][kRows];
+    if (beg < end) Loader::load(cur, x, beg, end, 0, H, lane);
+    __syncthreads();
+
+    // The logits of up to 64 rows are parked in LDS (row stride EP + 1: a lane per row reads without
+    // bank conflicts); then lane L runs the post-process of row L, so a wave pays for the post-process
+    // once per 64 rows, not once per group of kRows.
+    constexpr int LROW = EP + 1;
+    __shared__ float parked[WAVES][MTS_WAVE * LROW];
+    float* mine_rows = parked[wave];
+    float psum[EP], zsum = 0.f, hsum = 0.f;   // statistics of the rows this lane post-processes
+    int csum[EP];
+#pragma unroll
+    for (int e = 0; e < EP; ++e) {
+        psum[e] = 0.f;
+        csum[e] = 0;
+    }
+    int64_t pass_base = beg;
+    int64_t r0 = beg;
+    int ch = 0;
+    float acc[kRows][EP];
+    while (r0 < end) {
+        const bool last = ch + 1 == nch;
+        const int64_t nr0 = last ? r0 + kRows : r0;
+        const int nc = last ? 0 : ch + 1;
+        if (nr0 < end) Loader::load(nxt, x, nr0, end, nc, H, lane);
+        if (ch == 0) {
+#pragma unroll
+            for (int r = 0; r < kRows; ++r)
+#pragma unroll
+                for (int e = 0; e < EP; ++e) acc[r][e] = 0.f;
+        }
+        Loader::template accumulate<EP>(acc, cur, w_lds, r0, end, ch, H, E, lane);
+#pragma unroll
+        for (int ps = 0; ps < PASSES; ++ps)
+#pragma unroll
+            for (int r = 0; r < kRows; ++r) cur[ps][r] = nxt[ps][r];
+        const int64_t g0 = r0;   // the row group whose dot products are complete when `last`
+        r0 = nr0;
+        ch = nc;
+        if (!last) continue;
         static_assert(kRows * EP == 32 || kRows * EP == 64, "reduction layout");
         constexpr int NV = kRows * EP;
         float v[NV];
@@ -256,14 +268,14 @@ __global__ __launch_bounds__(kFwdThreads) void router_head_kernel(
             for (int e = 0; e < EP; ++e) v[r * EP + e] = acc[r][e];
         int idx = 0;
         reduce_scatter<NV, NV, 32>(v, lane, idx);
-        const float mine = v[0];   // value `idx` of the group: row r0 + idx / EP, expert idx % EP
+        const float mine = v[0];   // value `idx` of the group: row g0 + idx / EP, expert idx % EP
         {
             const int r = idx / EP, e = idx % EP;
             const bool writer = NV == 64 ? true : (lane & 1) == 0;
-            if (writer && e < E && r0 + r < end) logits[(r0 + r) * E + e] = mine;
-            if (writer) mine_rows[(int)(r0 - pass_base + r) * LROW + e] = e < E ? mine : -INFINITY;
+            if (writer && e < E && g0 + r < end) logits[(g0 + r) * E + e] = mine;
+            if (writer) mine_rows[(int)(g0 - pass_base + r) * LROW + e] = e < E ? mine : -INFINITY;
         }
-        const int64_t parked_to = r0 + kRows < end ? r0 + kRows : end;
+        const int64_t parked_to = g0 + kRows < end ? g0 + kRows : end;
         if (parked_to - pass_base < MTS_WAVE && parked_to < end) continue;   // wave-uniform: park more rows first
         __builtin_amdgcn_wave_barrier();
         const int64_t row = pass_base + lane;
@@ -350,6 +362,8 @@ __global__ __launch_bounds__(kFwdThreads) void router_head_kernel(
 // A block holds `groups` sets of column threads; each set takes a contiguous share of the block's
 // rows, and the sets' dW_r sums are added through LDS in set order before the block writes its
 // one partial: a quarter of the partials for the same number of waves in flight.
+// Rows wider than a block has column threads for are cut into column ranges (blockIdx.y); a CHAIN
+// block of every range forms the logit gradients of its rows again.
 constexpr int bwd_max_threads(int EP) { return EP <= 8 ? 768 : 384; }   // 16 experts need twice the registers
 
 // What the backward kernel needs to form the logit gradients itself (CHAIN): the saved outputs of
@@ -376,9 +390,10 @@ __global__ __launch_bounds__(bwd_max_threads(EP)) void router_logits_bwd_kernel(
                                                                  const XT* __restrict__ x,
                                                                  const float* __restrict__ w, int64_t T, int H,
                                                                  int E, int rows_per_block, int groups,
-                                                                 XT* __restrict__ dx, float* __restrict__ part,
+                                                                 int cols_per_block, XT* __restrict__ dx,
+                                                                 float* __restrict__ part,
                                                                  RouterGradIn rg = RouterGradIn()) {
-    extern __shared__ __attribute__((aligned(16))) float set_sum[];   // [E][H]
+    extern __shared__ __attribute__((aligned(16))) float set_sum[];   // [E][cols_per_block]
     __shared__ __attribute__((aligned(16))) float dl_lds[CHAIN ? kChainRows * EP : 4];
     if constexpr (CHAIN) {
         using namespace mts_router;
@@ -414,8 +429,9 @@ __global__ __launch_bounds__(bwd_max_threads(EP)) void router_logits_bwd_kernel(
     }
     const int col_threads = blockDim.x / groups;
     const int grp = threadIdx.x / col_threads;
-    const int c = (threadIdx.x % col_threads) * 4;
-    const bool active = c < H;
+    const int cl = (threadIdx.x % col_threads) * 4;   // column within the block's range (blockIdx.y picks the range)
+    const int c = blockIdx.y * cols_per_block + cl;
+    const bool active = cl < cols_per_block && c < H;
     typedef typename RawVec<XT>::type raw_t;
     f32x4 wv[EP], acc[EP];
 #pragma unroll
@@ -488,13 +504,13 @@ __global__ __launch_bounds__(bwd_max_threads(EP)) void router_logits_bwd_kernel(
         if (grp == r && active) {
 #pragma unroll
             for (int e = 0; e < EP; ++e)
-                if (e < E) *reinterpret_cast<f32x4*>(set_sum + e * H + c) = acc[e];
+                if (e < E) *reinterpret_cast<f32x4*>(set_sum + e * cols_per_block + cl) = acc[e];
         }
         __syncthreads();
         if (grp == 0 && active) {
 #pragma unroll
             for (int e = 0; e < EP; ++e)
-                if (e < E) acc[e] += *reinterpret_cast<const f32x4*>(set_sum + e * H + c);
+                if (e < E) acc[e] += *reinterpret_cast<const f32x4*>(set_sum + e * cols_per_block + cl);
         }
         __syncthreads();
     }
@@ -529,19 +545,46 @@ __global__ __launch_bounds__(256) void router_dw_reduce_kernel(const float* __re
 }
 
 constexpr int kMaxE = 16;
-constexpr int kMaxH = 1024;   // E*H floats of weights fit the 64 KiB of LDS a block may use by default
+constexpr int kMaxH = 4096;
+constexpr int kChunkCols = 4 * MTS_WAVE * 4;        // columns a wave of the forward kernels holds in registers at a time
+constexpr size_t kMaxWeightLds = 128 * 1024;        // the forward kernels keep all of W_r [E][H] fp32 in LDS
 constexpr int kBwdBlocks = 1024;
 constexpr int kHeadMaxBlocks = MTS_HEAD_MAX_CHUNKS;   // blocks of the chained forward kernel = chunks of the routing metadata
 
 int check(const void* x, const float* w, int64_t T, int H, int E, int act_dtype) {
     if (!x || !w) return MTS_ERR_NULL;
     if (T <= 0 || E < 1 || E > kMaxE || H < 4 || H % 4 || H > kMaxH) return MTS_ERR_SHAPE;
+    if ((size_t)E * H * sizeof(float) > kMaxWeightLds) return MTS_ERR_SHAPE;   // 4096 columns for 8 experts, 2048 for 16
     if (act_dtype != MTS_BF16 && act_dtype != MTS_F16 && act_dtype != MTS_F32) return MTS_ERR_DTYPE;
     if (!mts_aligned16(w) || (reinterpret_cast<uintptr_t>(x) & 15u)) return MTS_ERR_ALIGN;
     return MTS_OK;
 }
 
 int bwd_blocks(int64_t T) { return (int)(T < kBwdBlocks ? T : kBwdBlocks); }
+
+// a kernel whose dynamic LDS, together with `fixed` bytes of static LDS, passes the default limit of
+// 64 KiB per block has to say so before the launch
+template <typename Kernel>
+hipError_t allow_lds(Kernel kernel, size_t bytes, size_t fixed = 0) {
+    if (bytes + fixed <= 64 * 1024) return hipSuccess;
+    return hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+}
+
+// Block shape of the backward kernel: column ranges (grid.y), column threads per range, row sets per block.
+struct BwdShape {
+    int ranges, cols_per_block, groups, threads;
+};
+BwdShape bwd_shape(int H, int E) {
+    const int max_threads = bwd_max_threads(E <= 8 ? 8 : 16);
+    const int all_threads = ((H / 4 + MTS_WAVE - 1) / MTS_WAVE) * MTS_WAVE;   // one thread per 4 columns
+    BwdShape b;
+    b.ranges = (all_threads + max_threads - 1) / max_threads;
+    const int col_threads = ((all_threads / MTS_WAVE + b.ranges - 1) / b.ranges) * MTS_WAVE;
+    b.cols_per_block = b.ranges == 1 ? H : col_threads * 4;
+    b.groups = max_threads / col_threads < 4 ? max_threads / col_threads : 4;
+    b.threads = b.groups * col_threads;
+    return b;
+}
 
 }  // namespace
 
@@ -556,15 +599,20 @@ extern "C" int mts_router_logits_fwd(const void* x, const float* w_r, int64_t T,
     if (blocks > 256 * 2) blocks = 256 * 2;
     const dim3 grid((unsigned)blocks);
     const size_t lds = (size_t)E * H * sizeof(float);
-    const int passes = (H + MTS_WAVE * 4 - 1) / (MTS_WAVE * 4);   // 1..4 since H <= 1024
-#define MTS_FWD(XT, EP, PS) \
-    router_logits_fwd_kernel<XT, EP, PS><<<grid, kFwdThreads, lds, s>>>((const XT*)x, w_r, T, H, E, logits)
-#define MTS_FWD_PASSES(XT, EP)                   \
-    do {                                         \
-        if (passes == 1) MTS_FWD(XT, EP, 1);     \
-        else if (passes == 2) MTS_FWD(XT, EP, 2); \
-        else if (passes == 3) MTS_FWD(XT, EP, 3); \
-        else MTS_FWD(XT, EP, 4);                 \
+    const int passes = (H + MTS_WAVE * 4 - 1) / (MTS_WAVE * 4);   // 256-column slabs per row
+    const int n_chunks = (H + kChunkCols - 1) / kChunkCols;
+#define MTS_FWD(XT, EP, PS, CH)                                                                                       \
+    do {                                                                                                              \
+        if (allow_lds(router_logits_fwd_kernel<XT, EP, PS, CH>, lds) != hipSuccess) return MTS_ERR_SHAPE;             \
+        router_logits_fwd_kernel<XT, EP, PS, CH><<<grid, kFwdThreads, lds, s>>>((const XT*)x, w_r, T, H, E, n_chunks, logits); \
+    } while (0)
+#define MTS_FWD_PASSES(XT, EP)                          \
+    do {                                                \
+        if (passes == 1) MTS_FWD(XT, EP, 1, false);     \
+        else if (passes == 2) MTS_FWD(XT, EP, 2, false); \
+        else if (passes == 3) MTS_FWD(XT, EP, 3, false); \
+        else if (passes == 4) MTS_FWD(XT, EP, 4, false); \
+        else MTS_FWD(XT, EP, 4, true);                  \
     } while (0)
     if (act_dtype == MTS_BF16) {
         if (E <= 8) MTS_FWD_PASSES(bf16_t, 8);
@@ -606,16 +654,22 @@ int mts_launch_router_head(const void* x, const float* w_r, int64_t T, int H, in
     const dim3 grid((unsigned)blocks);
     const size_t lds = (size_t)E * H * sizeof(float);
     const int passes = (H + MTS_WAVE * 4 - 1) / (MTS_WAVE * 4);
+    const int n_chunks = (H + kChunkCols - 1) / kChunkCols;
     const int wa_dtype = act_dtype == MTS_F16 ? MTS_F16 : MTS_BF16;   // fp32 activations carry no weights_act (checked by the caller)
-#define MTS_HEAD(XT, EP, PS)                                                                                         \
-    router_head_kernel<XT, EP, PS><<<grid, kFwdThreads, lds, s>>>((const XT*)x, w_r, T, H, E, K, normalize, rows_per_wave, \
-                                                                  logits, weights, indices, weights_act, wa_dtype, partial, cnt)
-#define MTS_HEAD_PASSES(XT, EP)                    \
-    do {                                           \
-        if (passes == 1) MTS_HEAD(XT, EP, 1);      \
-        else if (passes == 2) MTS_HEAD(XT, EP, 2); \
-        else if (passes == 3) MTS_HEAD(XT, EP, 3); \
-        else MTS_HEAD(XT, EP, 4);                  \
+#define MTS_HEAD(XT, EP, PS, CH)                                                                                      \
+    do {                                                                                                              \
+        if (allow_lds(router_head_kernel<XT, EP, PS, CH>, lds, 16 * 1024) != hipSuccess) return MTS_ERR_SHAPE;                   \
+        router_head_kernel<XT, EP, PS, CH><<<grid, kFwdThreads, lds, s>>>((const XT*)x, w_r, T, H, E, K, normalize,   \
+                                                                          rows_per_wave, n_chunks, logits, weights, indices, \
+                                                                          weights_act, wa_dtype, partial, cnt);       \
+    } while (0)
+#define MTS_HEAD_PASSES(XT, EP)                           \
+    do {                                                  \
+        if (passes == 1) MTS_HEAD(XT, EP, 1, false);      \
+        else if (passes == 2) MTS_HEAD(XT, EP, 2, false); \
+        else if (passes == 3) MTS_HEAD(XT, EP, 3, false); \
+        else if (passes == 4) MTS_HEAD(XT, EP, 4, false); \
+        else MTS_HEAD(XT, EP, 4, true);                   \
     } while (0)
     if (act_dtype == MTS_BF16) {
         if (E <= 8) MTS_HEAD_PASSES(bf16_t, 8);
@@ -647,24 +701,26 @@ extern "C" int mts_router_logits_bwd(const float* dlogits, const void* x, const 
     if (workspace_bytes < mts_router_logits_bwd_workspace_bytes(T, H, E)) return MTS_ERR_WORKSPACE;
     if (!mts_aligned16(workspace) || !mts_aligned16(d_w_r) || (reinterpret_cast<uintptr_t>(dx) & 15u)) return MTS_ERR_ALIGN;
     hipStream_t s = (hipStream_t)stream;
-    const int col_threads = ((H / 4 + MTS_WAVE - 1) / MTS_WAVE) * MTS_WAVE;   // one thread per 4 columns
-    const int max_threads = bwd_max_threads(E <= 8 ? 8 : 16);
-    const int groups = max_threads / col_threads < 4 ? (max_threads / col_threads < 1 ? 1 : max_threads / col_threads) : 4;   // row sets per block
-    const int threads = groups * col_threads;
+    const BwdShape shape = bwd_shape(H, E);
+    const int groups = shape.groups, threads = shape.threads;
     int nb = (bwd_blocks(T) + groups - 1) / groups;
     const int rows_per_block = (int)((T + nb - 1) / nb);
     nb = (int)((T + rows_per_block - 1) / rows_per_block);   // every block has at least one row
-    const size_t lds = (size_t)E * H * sizeof(float);
+    const dim3 grid((unsigned)nb, (unsigned)shape.ranges);
+    const size_t lds = (size_t)E * shape.cols_per_block * sizeof(float);
     float* part = (float*)workspace;
     const bool vec_dl = mts_aligned16(dlogits);
 #define MTS_BWD(XT, EP)                                                                                    \
     do {                                                                                                   \
+        if (allow_lds(router_logits_bwd_kernel<XT, EP, true>, lds, 1024) != hipSuccess ||                  \
+            allow_lds(router_logits_bwd_kernel<XT, EP, false>, lds, 1024) != hipSuccess)                   \
+            return MTS_ERR_SHAPE;                                                                          \
         if (E == EP && vec_dl)                                                                             \
-            router_logits_bwd_kernel<XT, EP, true><<<nb, threads, lds, s>>>(dlogits, (const XT*)x, w_r, T, H, E, \
-                                                                            rows_per_block, groups, (XT*)dx, part); \
+            router_logits_bwd_kernel<XT, EP, true><<<grid, threads, lds, s>>>(dlogits, (const XT*)x, w_r, T, H, E, \
+                                                                              rows_per_block, groups, shape.cols_per_block, (XT*)dx, part); \
         else                                                                                               \
-            router_logits_bwd_kernel<XT, EP, false><<<nb, threads, lds, s>>>(dlogits, (const XT*)x, w_r, T, H, E, \
-                                                                             rows_per_block, groups, (XT*)dx, part); \
+            router_logits_bwd_kernel<XT, EP, false><<<grid, threads, lds, s>>>(dlogits, (const XT*)x, w_r, T, H, E, \
+                                                                               rows_per_block, groups, shape.cols_per_block, (XT*)dx, part); \
     } while (0)
     if (act_dtype == MTS_BF16) {
         if (E <= 8) MTS_BWD(bf16_t, 8);
@@ -717,20 +773,24 @@ extern "C" int mts_moe_head_bwd(const void* x, const float* w_r, const float* lo
     if (!mts_aligned16(workspace) || !mts_aligned16(d_w_r) || !mts_aligned16(dx) || (E == 8 && !mts_aligned16(logits)))
         return MTS_ERR_ALIGN;
     hipStream_t s = (hipStream_t)stream;
-    const int col_threads = ((H / 4 + MTS_WAVE - 1) / MTS_WAVE) * MTS_WAVE;
-    const int max_threads = bwd_max_threads(E <= 8 ? 8 : 16);
-    const int groups = max_threads / col_threads < 4 ? (max_threads / col_threads < 1 ? 1 : max_threads / col_threads) : 4;
-    const int threads = groups * col_threads;
+    const BwdShape shape = bwd_shape(H, E);
+    const int groups = shape.groups, threads = shape.threads;
     int nb = (int)chain_blocks(T, groups);
     const int rows_per_block = (int)((T + nb - 1) / nb);
     nb = (int)((T + rows_per_block - 1) / rows_per_block);
-    const size_t lds = (size_t)E * H * sizeof(float);
+    const dim3 grid((unsigned)nb, (unsigned)shape.ranges);
+    const size_t lds = (size_t)E * shape.cols_per_block * sizeof(float);
     float* part = (float*)workspace;
     RouterGradIn rg = {logits, weights, indices, counts, g_weights, g_weights_act, g_prob_mean, g_z_loss, g_load_balance,
                        act_dtype, K, normalize};
 #define MTS_CHAIN(XT, EP)                                                                                        \
-    router_logits_bwd_kernel<XT, EP, false, true><<<nb, threads, lds, s>>>(nullptr, (const XT*)x, w_r, T, H, E,    \
-                                                                            rows_per_block, groups, (XT*)dx, part, rg)
+    do {                                                                                                         \
+        if (allow_lds(router_logits_bwd_kernel<XT, EP, false, true>, lds, kChainRows * EP * sizeof(float)) != hipSuccess) \
+            return MTS_ERR_SHAPE;                                                                                \
+        router_logits_bwd_kernel<XT, EP, false, true><<<grid, threads, lds, s>>>(nullptr, (const XT*)x, w_r, T, H, E, \
+                                                                                  rows_per_block, groups,          \
+                                                                                  shape.cols_per_block, (XT*)dx, part, rg); \
+    } while (0)
     if (act_dtype == MTS_BF16) {
         if (E <= 8) MTS_CHAIN(bf16_t, 8);
         else MTS_CHAIN(bf16_t, 16);

@@ -28,7 +28,7 @@ def moe_layer_violation(x, router_weight, gate_up_proj, down_proj, top_k: int):
         (torch.is_tensor(router_weight) and router_weight.ndim == 2 and router_weight.shape[0] == E,
          "router weight is [E,H]"),
         (is_router_logits_supported(x, router_weight),
-         "an fp32 router weight on the same GPU, at most 16 experts and a hidden size of at most 1024"),
+         "an fp32 router weight on the same GPU, at most 16 experts and a hidden size of at most 4096 (E * H <= 32768)"),
         (1 <= top_k <= min(E, _MAX_TOP_K), f"1 <= top_k <= min(E, {_MAX_TOP_K})"),
         (not needs_padding(x, gate_up_proj), "hidden and expert widths that are whole 16-byte chunks"),
         (x.shape[0] * top_k < 2**31, "fewer than 2^31 routes"),

@@ -14,6 +14,7 @@ from minitrain_amd.model.ops import RouterPostprocessOutput
 
 _MAX_EXPERTS = 1024
 _MAX_TOP_K = 8
+_ROUTER_WEIGHT_LDS_BYTES = 128 * 1024   # the projection kernels keep W_r [E,H] fp32 in LDS: H <= 4096 for 8 experts, 2048 for 16
 
 
 def is_router_postprocess_supported(logits: torch.Tensor, top_k: int, normalize: bool) -> bool:
@@ -141,7 +142,8 @@ def is_router_logits_supported(hidden_states: torch.Tensor, weight: torch.Tensor
         and hidden_states.shape[1] == weight.shape[1]
         and weight.shape[0] <= 16
         and hidden_states.shape[1] % 4 == 0
-        and hidden_states.shape[1] <= 1024
+        and hidden_states.shape[1] <= 4096
+        and weight.shape[0] * weight.shape[1] * 4 <= _ROUTER_WEIGHT_LDS_BYTES
     )
 
 
@@ -196,6 +198,6 @@ def router_logits(hidden_states: torch.Tensor, weight: torch.Tensor) -> torch.Te
     if not is_router_logits_supported(hidden_states, weight):
         raise RuntimeError(
             "hip router_logits requires 2D bf16/fp32 activations and a 2D fp32 weight on the GPU with "
-            "at most 16 experts and a hidden size that is a multiple of 4 and at most 1024"
+            "at most 16 experts and a hidden size that is a multiple of 4 and at most 4096 (E * H <= 32768)"
         )
     return _RouterLogitsFunction.apply(hidden_states, weight)

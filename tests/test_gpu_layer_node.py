@@ -41,7 +41,9 @@ def _head(lib, x, w_r, K, normalize):
 @pytest.mark.parametrize("T,H,E,K,dtype,normalize", [
     (24576, 768, 8, 2, torch.bfloat16, True), (1, 64, 4, 1, torch.bfloat16, True), (5, 128, 8, 2, torch.float16, False),
     (257, 1024, 16, 4, torch.bfloat16, True), (3000, 192, 3, 3, torch.float32, True), (2047, 72, 12, 8, torch.float16, True),
-    (98304, 768, 8, 2, torch.bfloat16, True), (700, 256, 16, 1, torch.float32, False)])
+    (98304, 768, 8, 2, torch.bfloat16, True), (700, 256, 16, 1, torch.float32, False),
+    # rows wider than a wave holds in registers: column chunks forward, column ranges backward
+    (4096, 4096, 8, 2, torch.bfloat16, True), (333, 2048, 16, 2, torch.float16, True), (130, 1280, 5, 2, torch.float32, True)])
 def test_chained_head_equals_the_three_operators(T, H, E, K, dtype, normalize):
     print(f"head T={T} H={H} E={E} K={K} {dtype} normalize={normalize}", flush=True)
     from minitrain_amd import _lib
@@ -106,7 +108,7 @@ def _separate_grads(ops, case, K, normalize, dtype, fp32_params):
     (512, 128, 8, 256, 2, torch.bfloat16, False, True), (2048, 768, 8, 1024, 2, torch.bfloat16, True, True),
     (33, 64, 4, 64, 1, torch.float16, False, True), (700, 72, 3, 40, 2, torch.bfloat16, False, False),
     (300, 64, 16, 96, 4, torch.float32, False, True), (1, 64, 4, 64, 2, torch.bfloat16, False, True),
-    (200, 64, 8, 64, 5, torch.bfloat16, False, True)])
+    (200, 64, 8, 64, 5, torch.bfloat16, False, True), (300, 2048, 8, 128, 2, torch.bfloat16, False, True)])
 def test_layer_node_equals_the_separate_operators_and_the_oracle(T, H, E, I, K, dtype, fp32_params, normalize):
     print(f"layer node T={T} H={H} E={E} I={I} K={K} {dtype} fp32_params={fp32_params} normalize={normalize}", flush=True)
     ops = hip_backend()

@@ -30,7 +30,8 @@ def _case(T, H, E, dtype, seed):
     return x, w, g
 
 
-@pytest.mark.parametrize("T,H,E", [(1, 64, 4), (5, 64, 3), (257, 768, 8), (1000, 1024, 16), (4096, 768, 8), (24576, 768, 8)])
+@pytest.mark.parametrize("T,H,E", [(1, 64, 4), (5, 64, 3), (257, 768, 8), (1000, 1024, 16), (4096, 768, 8), (24576, 768, 8),
+                                   (300, 4096, 8), (1000, 2048, 16), (513, 1280, 8), (100, 3072, 5), (64, 2052, 8)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 def test_router_logits_forward_backward(T, H, E, dtype):
     ops = hip_backend()
@@ -71,8 +72,11 @@ def test_router_logits_is_deterministic_and_matches_torch_path():
 
 def test_router_logits_unsupported_contract_returns_none():
     ops = hip_backend()
-    x = torch.randn(8, 2048, device="cuda", dtype=torch.bfloat16)     # hidden size above the kernel's range
-    w = torch.randn(8, 2048, device="cuda")
+    x = torch.randn(8, 8192, device="cuda", dtype=torch.bfloat16)     # hidden size above the kernel's range
+    w = torch.randn(8, 8192, device="cuda")
+    assert ops.router_logits(x, w) is None
+    x = torch.randn(8, 4096, device="cuda", dtype=torch.bfloat16)     # 16 x 4096 fp32 weights do not fit the LDS
+    w = torch.randn(16, 4096, device="cuda")
     assert ops.router_logits(x, w) is None
     x = torch.randn(8, 64, device="cuda", dtype=torch.float64)        # unsupported activation dtype
     assert ops.router_logits(x, torch.randn(8, 64, device="cuda")) is None
