@@ -107,12 +107,13 @@ int mts_router_logits_bwd(const float* dlogits, const void* x, const float* w_r,
                           int H, int E, int act_dtype, void* dx, float* d_w_r,
                           void* workspace, int64_t workspace_bytes, void* stream);
 
-/* ---- the layer's head in three launches -------------------------------------
+/* ---- the layer's head in two launches ---------------------------------------
  * mts_router_logits_fwd + mts_router_fwd + mts_moe_route as one chain (router projection,
  * post-process and routing metadata of minitrain/model/moe_router.py:64-90 and
  * triton/fused_moe.py:74-154): the post-process runs on the logits while they are still in
  * registers, the routes per expert it counts per block are the chunk histogram of the
- * routing metadata, and one block reduces the statistics and scans the counts.  Outputs as in
+ * routing metadata; in the second launch every scatter block adds up those counts itself and
+ * one more block reduces the statistics.  Outputs as in
  * those three calls (logits [T,E] f32 are written for the backward pass; weights_act,
  * load_balance and load_stats may be NULL).  E <= 16, H a multiple of 4 and at most 4096, E * H <= 32768,
  * K <= min(E, MTS_MAX_TOP_K).  The statistics are summed in a fixed order of their own: they agree

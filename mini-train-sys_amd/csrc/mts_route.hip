@@ -20,6 +20,7 @@
 
 namespace {
 
+typedef __attribute__((ext_vector_type(4))) int32_t i32x4;
 constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / MTS_WAVE;
 constexpr int kChunk = 256;   // entries per wave
@@ -140,104 +141,28 @@ __global__ __launch_bounds__(1024) void route_scan_kernel(
     route_scan_block(cnt, n_chunks, E, block_m, counts, expert_start, tile_row_start, tile_expert, tile_count, e0);
 }
 
-// One block after the kernel that chains the router projection to the post-process: the scan over
-// that kernel's per-block route counts (the chunks of the scatter that follows) and the reduction
-// of its per-block statistics.  The E per-expert scans over the chunks and the E + 2 column sums of
-// the statistics are independent jobs spread over the 16 waves, every job with all its loads issued
-// up front (at most kFinishChunks chunks: 8 per lane); one barrier later a few waves finish up.
-constexpr int kFinishChunks = MTS_HEAD_MAX_CHUNKS;
-constexpr int kFinishMaxE = 64;
-__global__ __launch_bounds__(1024) void head_finish_kernel(
-    const float* __restrict__ partial, int32_t* __restrict__ cnt, int n_chunks, int E, float inv_t,
-    float inv_routes, float* __restrict__ prob_mean, float* __restrict__ z_loss, float* __restrict__ entropy,
-    int32_t* __restrict__ counts, float* __restrict__ load_balance, float* __restrict__ load_stats,
-    int32_t* __restrict__ expert_start) {
-    __shared__ mts_router::StatsShared sh;
-    __shared__ float col_mean[kFinishMaxE + 2];
-    __shared__ int32_t total[kFinishMaxE];
-    constexpr int NW = 1024 / MTS_WAVE, PER_LANE = kFinishChunks / MTS_WAVE;
-    const int wave = threadIdx.x / MTS_WAVE, lane = threadIdx.x % MTS_WAVE;
-    for (int job = wave; job < 2 * E + 2; job += NW) {
-        if (job < E + 2) {   // a column of the statistics
-            float v[PER_LANE];
-#pragma unroll
-            for (int q = 0; q < PER_LANE; ++q) {
-                const int b = q * MTS_WAVE + lane;
-                v[q] = b < n_chunks ? partial[(int64_t)b * (E + 2) + job] : 0.f;
-            }
-            float sum = 0.f;
-#pragma unroll
-            for (int q = 0; q < PER_LANE; ++q) sum += v[q];
-            sum = wave_sum(sum) * inv_t;
-            if (lane == 0) col_mean[job] = sum;
-        } else {             // an expert's routes per chunk -> routes in earlier chunks
-            const int e = job - (E + 2);
-            int32_t v[PER_LANE];
-#pragma unroll
-            for (int q = 0; q < PER_LANE; ++q) {
-                const int c = q * MTS_WAVE + lane;
-                v[q] = c < n_chunks ? cnt[(int64_t)c * E + e] : 0;
-            }
-            int32_t carry = 0;
-#pragma unroll
-            for (int q = 0; q < PER_LANE; ++q) {
-                int32_t incl = v[q];
-#pragma unroll
-                for (int o = 1; o < MTS_WAVE; o <<= 1) {
-                    const int32_t up = __shfl_up(incl, o, MTS_WAVE);
-                    if (lane >= o) incl += up;
-                }
-                const int c = q * MTS_WAVE + lane;
-                if (c < n_chunks) cnt[(int64_t)c * E + e] = carry + incl - v[q];
-                carry += __shfl(incl, MTS_WAVE - 1, MTS_WAVE);
-            }
-            if (lane == 0) total[e] = carry;
-        }
-    }
-    __syncthreads();
-    if (threadIdx.x < E + 2)
-        mts_router::stats_column(sh, threadIdx.x, col_mean[threadIdx.x], threadIdx.x < E ? total[threadIdx.x] : 0, E,
-                                 inv_routes, prob_mean, z_loss, entropy, counts);
-    if (wave == NW - 1) {   // exclusive scan of the routes per expert (E <= 64: one lane per expert)
-        const int32_t v = lane < E ? total[lane] : 0;
-        int32_t incl = v;
-#pragma unroll
-        for (int o = 1; o < MTS_WAVE; o <<= 1) {
-            const int32_t up = __shfl_up(incl, o, MTS_WAVE);
-            if (lane >= o) incl += up;
-        }
-        if (lane < E) expert_start[lane] = incl - v;
-        if (lane == E - 1) expert_start[E] = incl;
-    }
-    __syncthreads();
-    mts_router::stats_finalize(sh, wave, 1, 2, E, load_balance, load_stats);
-}
-
-// chunk_len entries per wave (a multiple of 64 is not required); the chunks are the ones the
-// counters in cnt were taken over
-// E: all experts; [e0, e0 + EW): the window of this pass (cnt is [chunk][EW], expert_start points at expert e0)
-__global__ __launch_bounds__(kThreads) void route_scatter_kernel(
-    const int32_t* __restrict__ idx, int64_t TK, int K, int E, int e0, int EW, int chunk_len,
-    const int32_t* __restrict__ cnt, const int32_t* __restrict__ expert_start, int32_t* __restrict__ s_scatter,
-    int32_t* __restrict__ s_reverse, int32_t* __restrict__ x_gather) {
-    extern __shared__ int32_t lds[];  // [kWaves][E] next free row per expert
-    const int wave = threadIdx.x / MTS_WAVE, lane = threadIdx.x % MTS_WAVE;
-    const int64_t chunk = (int64_t)blockIdx.x * kWaves + wave;
-    const int64_t cbeg = chunk * chunk_len;
-    if (cbeg >= TK) return;  // whole wave leaves; no block barrier below
-    const int64_t cend = cbeg + chunk_len < TK ? cbeg + chunk_len : TK;
-    volatile int32_t* next = lds + wave * EW;
-    for (int e = lane; e < EW; e += MTS_WAVE) next[e] = expert_start[e] + cnt[chunk * EW + e];
-    const uint64_t lt = lanemask_lt();
-  for (int64_t base = cbeg; base < cend; base += kChunk) {   // kSteps x 64 entries at a time
-    int ev[kSteps];
+// The stable scatter of one chunk (entries [cbeg, cend)) by one wave; next[e] is the next free row
+// of window expert e for this chunk (LDS, private to the wave).
+// E: all experts; [e0, e0 + EW): the window of this pass.
+// scatter_load fetches the window-relative expert ids of kSteps x 64 entries starting at `base`
+// (-1: dropped route, whose -1 goes to s_reverse in the first pass; -2: not this pass);
+// scatter_place ranks and writes them.
+__device__ __forceinline__ void scatter_load(int (&ev)[kSteps], const int32_t* __restrict__ idx, int E, int e0, int EW,
+                                             int64_t base, int64_t cend) {
+    const int lane = threadIdx.x % MTS_WAVE;
 #pragma unroll
     for (int s = 0; s < kSteps; ++s) {  // these loads are in flight together
         const int64_t n = base + s * MTS_WAVE + lane;
         const int e = n < cend ? clamp_expert(idx[n], E) : -1;
-        // window-relative id; -1: dropped route (its -1 goes to s_reverse in the first pass), -2: not this pass
         ev[s] = e < 0 ? (e0 == 0 && n < cend ? -1 : -2) : (e >= e0 && e < e0 + EW ? e - e0 : -2);
     }
+}
+
+__device__ __forceinline__ void scatter_place(const int (&ev)[kSteps], int K, int64_t base, int64_t cend,
+                                              volatile int32_t* next, int32_t* __restrict__ s_scatter,
+                                              int32_t* __restrict__ s_reverse, int32_t* __restrict__ x_gather) {
+    const int lane = threadIdx.x % MTS_WAVE;
+    const uint64_t lt = lanemask_lt();
 #pragma unroll
     for (int s = 0; s < kSteps; ++s) {
         const int64_t n = base + s * MTS_WAVE + lane;
@@ -261,7 +186,203 @@ __global__ __launch_bounds__(kThreads) void route_scatter_kernel(
             x_gather[pos] = (int32_t)(n / K);
         }
     }
-  }
+}
+
+// `first` holds the ids of the chunk's first kSteps x 64 entries already (scatter_load at cbeg)
+__device__ __forceinline__ void scatter_chunk(int (&first)[kSteps], const int32_t* __restrict__ idx, int K, int E, int e0,
+                                              int EW, int64_t cbeg, int64_t cend, volatile int32_t* next,
+                                              int32_t* __restrict__ s_scatter, int32_t* __restrict__ s_reverse,
+                                              int32_t* __restrict__ x_gather) {
+    scatter_place(first, K, cbeg, cend, next, s_scatter, s_reverse, x_gather);
+    for (int64_t base = cbeg + kChunk; base < cend; base += kChunk) {
+        int ev[kSteps];
+        scatter_load(ev, idx, E, e0, EW, base, cend);
+        scatter_place(ev, K, base, cend, next, s_scatter, s_reverse, x_gather);
+    }
+}
+
+// chunk_len entries per wave (a multiple of 64 is not required); the chunks are the ones the
+// counters in cnt were taken over
+// E: all experts; [e0, e0 + EW): the window of this pass (cnt is [chunk][EW], expert_start points at expert e0)
+__global__ __launch_bounds__(kThreads) void route_scatter_kernel(
+    const int32_t* __restrict__ idx, int64_t TK, int K, int E, int e0, int EW, int chunk_len,
+    const int32_t* __restrict__ cnt, const int32_t* __restrict__ expert_start, int32_t* __restrict__ s_scatter,
+    int32_t* __restrict__ s_reverse, int32_t* __restrict__ x_gather) {
+    extern __shared__ int32_t lds[];  // [kWaves][E] next free row per expert
+    const int wave = threadIdx.x / MTS_WAVE, lane = threadIdx.x % MTS_WAVE;
+    const int64_t chunk = (int64_t)blockIdx.x * kWaves + wave;
+    const int64_t cbeg = chunk * chunk_len;
+    if (cbeg >= TK) return;  // whole wave leaves; no block barrier below
+    const int64_t cend = cbeg + chunk_len < TK ? cbeg + chunk_len : TK;
+    int first[kSteps];
+    scatter_load(first, idx, E, e0, EW, cbeg, cend);   // in flight with the counter loads below
+    volatile int32_t* next = lds + wave * EW;
+    for (int e = lane; e < EW; e += MTS_WAVE) next[e] = expert_start[e] + cnt[chunk * EW + e];
+    scatter_chunk(first, idx, K, E, e0, EW, cbeg, cend, next, s_scatter, s_reverse, x_gather);
+}
+
+// The launch behind the kernel that chains the router projection to the post-process.  Its last block
+// reduces that kernel's per-block statistics and route counts (expert totals, expert_start, the
+// load-balancing term and the load metrics); every other block scatters four chunks, one per wave,
+// and does not wait for the last block: the block adds up the route counts of ALL chunks itself (at most
+// kFinishChunks x kFinishMaxE counters, read from L2) to get the experts' first rows and the rows the
+// chunks before its own take.  One launch and one dependent round trip less than scan-then-scatter.
+constexpr int kFinishChunks = MTS_HEAD_MAX_CHUNKS;
+constexpr int kFinishMaxE = 16;
+__global__ __launch_bounds__(kThreads) void head_scatter_kernel(
+    const float* __restrict__ partial, const int32_t* __restrict__ cnt, int n_chunks, int E, float inv_t,
+    float inv_routes, float* __restrict__ prob_mean, float* __restrict__ z_loss, float* __restrict__ entropy,
+    int32_t* __restrict__ counts, float* __restrict__ load_balance, float* __restrict__ load_stats,
+    int32_t* __restrict__ expert_start, const int32_t* __restrict__ idx, int64_t TK, int K, int chunk_len,
+    int32_t* __restrict__ s_scatter, int32_t* __restrict__ s_reverse, int32_t* __restrict__ x_gather) {
+    const int wave = threadIdx.x / MTS_WAVE, lane = threadIdx.x % MTS_WAVE;
+    if (blockIdx.x + 1 < gridDim.x) {
+        __shared__ int32_t next_rows[kWaves][kFinishMaxE];
+        __shared__ int32_t sums[kWaves][2 * kFinishMaxE];
+        static_assert(kFinishChunks == 2 * kThreads, "two chunks per thread");
+        const int chunk0 = blockIdx.x * kWaves;   // the block's first chunk; wave w scatters chunk0 + w
+        const int64_t cbeg = (int64_t)(chunk0 + wave) * chunk_len;
+        const int64_t cend = cbeg + chunk_len < TK ? cbeg + chunk_len : TK;
+        int first_ids[kSteps];
+        if (cbeg < TK) scatter_load(first_ids, idx, E, 0, E, cbeg, cend);   // in flight with the counter loads below
+        // routes per expert: over all chunks, and over the chunks before the block's first one
+        int32_t total[kFinishMaxE], before[kFinishMaxE];
+#pragma unroll
+        for (int e = 0; e < kFinishMaxE; ++e) total[e] = before[e] = 0;
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            const int c = q * kThreads + threadIdx.x;
+            if (E == 8) {   // a row is two aligned 16-byte loads
+                i32x4 lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
+                if (c < n_chunks) {
+                    lo = *reinterpret_cast<const i32x4*>(cnt + (int64_t)c * 8);
+                    hi = *reinterpret_cast<const i32x4*>(cnt + (int64_t)c * 8 + 4);
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    total[e] += lo[e];
+                    total[e + 4] += hi[e];
+                    before[e] += c < chunk0 ? lo[e] : 0;
+                    before[e + 4] += c < chunk0 ? hi[e] : 0;
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < kFinishMaxE; ++e) {
+                    const int32_t v = (c < n_chunks && e < E) ? cnt[(int64_t)c * E + e] : 0;
+                    total[e] += v;
+                    before[e] += c < chunk0 ? v : 0;
+                }
+            }
+        }
+        // the counts of the block's own chunks before this wave's (at most kWaves - 1 rows), one expert per lane
+        int32_t own = 0;
+        for (int i = 0; i < wave; ++i)
+            if (lane < E && chunk0 + i < n_chunks) own += cnt[(int64_t)(chunk0 + i) * E + lane];
+#pragma unroll
+        for (int e = 0; e < kFinishMaxE; ++e) {
+            if (e < E) {   // block-uniform
+                int32_t t = total[e], b = before[e];
+#pragma unroll
+                for (int o = 32; o > 0; o >>= 1) {
+                    t += __shfl_xor(t, o, MTS_WAVE);
+                    b += __shfl_xor(b, o, MTS_WAVE);
+                }
+                if (lane == 0) {
+                    sums[wave][e] = t;
+                    sums[wave][kFinishMaxE + e] = b;
+                }
+            }
+        }
+        __syncthreads();
+        if (cbeg >= TK) return;  // whole wave leaves; no block barrier below
+        // lane e: the expert's first row = the totals of the experts before it, + its routes in earlier chunks
+        int32_t t = 0, bsum = 0;
+        if (lane < E) {
+#pragma unroll
+            for (int w = 0; w < kWaves; ++w) {
+                t += sums[w][lane];
+                bsum += sums[w][kFinishMaxE + lane];
+            }
+        }
+        int32_t incl = t;
+#pragma unroll
+        for (int o = 1; o < kFinishMaxE; o <<= 1) {
+            const int32_t up = __shfl_up(incl, o, MTS_WAVE);
+            if (lane >= o) incl += up;
+        }
+        volatile int32_t* next = next_rows[wave];
+        if (lane < E) next[lane] = incl - t + bsum + own;
+        scatter_chunk(first_ids, idx, K, E, 0, E, cbeg, cend, next, s_scatter, s_reverse, x_gather);
+        return;
+    }
+    // the last block: thread t holds chunks t and t + kThreads of every column
+    __shared__ mts_router::StatsShared sh;
+    __shared__ float col_part[kWaves][kFinishMaxE + 2];
+    __shared__ int32_t tot_part[kWaves][kFinishMaxE];
+    __shared__ int32_t total_s[kFinishMaxE];
+    float colv[kFinishMaxE + 2];
+    int32_t totv[kFinishMaxE];
+#pragma unroll
+    for (int j = 0; j < kFinishMaxE + 2; ++j) {
+        float v = 0.f;
+        if (j < E + 2) {
+            const int c0 = threadIdx.x, c1 = threadIdx.x + kThreads;
+            const float a = c0 < n_chunks ? partial[(int64_t)c0 * (E + 2) + j] : 0.f;
+            const float b = c1 < n_chunks ? partial[(int64_t)c1 * (E + 2) + j] : 0.f;
+            v = a + b;
+        }
+        colv[j] = v;
+    }
+#pragma unroll
+    for (int e = 0; e < kFinishMaxE; ++e) {
+        int32_t v = 0;
+        if (e < E) {
+            const int c0 = threadIdx.x, c1 = threadIdx.x + kThreads;
+            v = (c0 < n_chunks ? cnt[(int64_t)c0 * E + e] : 0) + (c1 < n_chunks ? cnt[(int64_t)c1 * E + e] : 0);
+        }
+        totv[e] = v;
+    }
+#pragma unroll
+    for (int j = 0; j < kFinishMaxE + 2; ++j) {
+        if (j < E + 2) {   // block-uniform
+            const float v = wave_sum(colv[j]);
+            if (lane == 0) col_part[wave][j] = v;
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < kFinishMaxE; ++e) {
+        if (e < E) {
+            int32_t v = totv[e];
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, MTS_WAVE);
+            if (lane == 0) tot_part[wave][e] = v;
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x < E + 2) {
+        float v = 0.f;
+        int32_t c = 0;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) {
+            v += col_part[w][threadIdx.x];
+            if (threadIdx.x < E) c += tot_part[w][threadIdx.x];
+        }
+        if (threadIdx.x < E) total_s[threadIdx.x] = c;
+        mts_router::stats_column(sh, threadIdx.x, v * inv_t, c, E, inv_routes, prob_mean, z_loss, entropy, counts);
+    }
+    __syncthreads();
+    if (wave == kWaves - 1) {   // exclusive scan of the routes per expert: one lane per expert
+        const int32_t v = lane < E ? total_s[lane] : 0;
+        int32_t incl = v;
+#pragma unroll
+        for (int o = 1; o < MTS_WAVE; o <<= 1) {
+            const int32_t up = __shfl_up(incl, o, MTS_WAVE);
+            if (lane >= o) incl += up;
+        }
+        if (lane < E) expert_start[lane] = incl - v;
+        if (lane == E - 1) expert_start[E] = incl;
+    }
+    mts_router::stats_finalize(sh, wave, 0, 1, E, load_balance, load_stats);
 }
 
 }  // namespace
@@ -397,13 +518,11 @@ extern "C" int mts_moe_head_fwd(const void* x, const float* w_r, int64_t T, int 
     const int64_t rows_per_chunk = (int64_t)rows_per_wave * 4;
     const int64_t n_chunks = (T + rows_per_chunk - 1) / rows_per_chunk;
     if (n_chunks > kFinishChunks || E > kFinishMaxE) return MTS_ERR_SHAPE;   // cannot happen: the geometry caps the chunks, the projection E
-    head_finish_kernel<<<1, 1024, 0, s>>>(partial, cnt, (int)n_chunks, E, 1.0f / (float)T, 1.0f / ((float)T * (float)K),
-                                          prob_mean, z_loss, entropy, counts, load_balance, load_stats, expert_start);
-    MTS_CHECK_LAUNCH();
-    const int grid = (int)((n_chunks + kWaves - 1) / kWaves);
-    const size_t lds = (size_t)kWaves * E * sizeof(int32_t);
-    route_scatter_kernel<<<grid, kThreads, lds, s>>>(indices, T * (int64_t)K, K, E, 0, E, (int)(rows_per_chunk * K), cnt,
-                                                     expert_start, s_scatter, s_reverse, x_gather);
+    const int grid = (int)((n_chunks + kWaves - 1) / kWaves) + 1;   // scatter blocks, then the block that reduces
+    head_scatter_kernel<<<grid, kThreads, 0, s>>>(partial, cnt, (int)n_chunks, E, 1.0f / (float)T,
+                                                  1.0f / ((float)T * (float)K), prob_mean, z_loss, entropy, counts,
+                                                  load_balance, load_stats, expert_start, indices, T * (int64_t)K, K,
+                                                  (int)(rows_per_chunk * K), s_scatter, s_reverse, x_gather);
     MTS_CHECK_LAUNCH();
     return MTS_OK;
 }

@@ -5,7 +5,7 @@ The reference composes the layer from three autograd nodes (minitrain/model/moe_
 minitrain/model/blocks.py:86-102): ``F.linear`` for the router logits, ``router_postprocess`` and
 ``fused_moe``.  The activations feed two of them, so autograd sums two gradients for ``x`` with one more
 kernel, and every node boundary is a launch boundary.  Here the forward pass starts with the chained
-head (three launches: projection + post-process, statistics + scan, scatter) and the backward pass
+head (two launches: projection + post-process, then scatter + statistics) and the backward pass
 forms the router's gradient before the dX combine, which adds it to the experts' gradient in the same
 pass.  Same arithmetic as the separate operators; it is an extension the MoE block uses when the backend
 offers it (``ops.moe_layer``) and the configuration allows it.
