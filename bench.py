@@ -45,7 +45,7 @@ RIDGE_FLOP_PER_BYTE = PEAK_BF16_TFLOPS * 1e12 / (PEAK_HBM_GBS * 1e9)   # 312.5: 
 # line names the file that holds the runs' commands and tables.
 TRAFFIC_SOURCE = "profiles/moe_layer_24x1024_hbm_traffic.txt"
 MEASURED_TRAFFIC_BYTES = {
-    "fwd_gateup_swiglu": 656.9e6, "fwd_down": 223.9e6, "bwd_dy1": 531.2e6, "bwd_joint": 971.4e6,
+    "fwd_gateup_swiglu": 654.7e6, "fwd_down": 223.9e6, "bwd_dy1": 530.9e6, "bwd_joint": 972.2e6,
     "combine": 114.6e6, "dx_combine": 152.4e6,
 }
 
@@ -198,20 +198,26 @@ def stage_breakdown(layer, steps):
         ("dx_combine", 1.0 * TK * H, rows_h + 2 * T * H * esz + TK * 4,
          lambda: lib.mts_moe_combine(p(dxe), None, p(dx_r), p(sr), T, K, H, B, p(dx), st)),
     ]
-    ev = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in stages] for _ in range(steps)]
-    for it in range(2 + steps):
-        for j, (name, _, _, fn) in enumerate(stages):
-            if it >= 2:
-                ev[it - 2][j][0].record()
-            rc = fn()
-            if it >= 2:
-                ev[it - 2][j][1].record()
-            if rc != 0:
-                raise RuntimeError(f"{name} returned {rc}")
+    # One stage is bracketed per pass over the whole sequence, so the other stages of that pass run
+    # back to back as they do in the layer step and the chip is in the state it has there.
+    elapsed = [[] for _ in stages]
+    for j in range(len(stages)):
+        for it in range(1 + steps):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            for i, (name, _, _, fn) in enumerate(stages):
+                if i == j:
+                    e0.record()
+                rc = fn()
+                if i == j:
+                    e1.record()
+                if rc != 0:
+                    raise RuntimeError(f"{name} returned {rc}")
+            if it:
+                elapsed[j].append((e0, e1))
     torch.cuda.synchronize()
     rows = []
     for j, (name, flops, nbytes, _) in enumerate(stages):
-        ms = float(np.mean([ev[i][j][0].elapsed_time(ev[i][j][1]) for i in range(steps)]))
+        ms = float(np.mean([a.elapsed_time(b) for a, b in elapsed[j]]))
         intensity = flops / nbytes
         bound = "mfma" if intensity >= RIDGE_FLOP_PER_BYTE else "hbm"
         tflops, gbs = flops / (ms * 1e-3) / 1e12, nbytes / (ms * 1e-3) / 1e9
