@@ -131,3 +131,19 @@ def test_bench_refuses_more_than_one_gpu_and_a_missing_gpu():
         one = subprocess.run([sys.executable, bench, "--steps", "1", "--warmup", "0"], capture_output=True, text=True,
                              timeout=300)
         assert one.returncode == 2 and "needs a GPU" in one.stderr and one.stdout.strip() == ""
+
+
+def test_bench_names_a_committed_file_for_its_counter_derived_traffic():
+    """`roofline.traffic` in the bench line is not measured live: the line names the file that holds the
+    counter runs it comes from, and every stage with such a figure appears in that file."""
+    import sys
+
+    sys.path.insert(0, ROOT)
+    import bench
+
+    path = os.path.join(ROOT, bench.TRAFFIC_SOURCE)
+    assert os.path.isfile(path)
+    text = open(path).read()
+    assert "FETCH_SIZE" in text and "WRITE_SIZE" in text
+    for stage in bench.MEASURED_TRAFFIC_BYTES:
+        assert stage in text, stage

@@ -83,3 +83,43 @@ def test_mfma_rate_probe_reports_a_plausible_rate():
     assert lib.mts_probe_mfma_rate(1, 64, 4, sink.data_ptr(), sink.numel() * 4, None, torch.cuda.current_stream().cuda_stream) == 0
     torch.cuda.synchronize()
     assert torch.isfinite(sink).all() and sink.abs().max() > 0
+
+
+def test_bench_line_carries_the_contract():
+    """`python bench.py` prints one JSON line with the metric of the baseline, the roofline of the dominant
+    kernel (algorithmic bytes beside the counter-derived traffic and the file that holds the counter runs)
+    and the CPU baseline; the fractions follow from the figures in the line."""
+    print("bench line", flush=True)
+    import json
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    root = Path(__file__).resolve().parents[1]
+    run = subprocess.run([sys.executable, str(root / "bench.py"), "--steps", "3", "--warmup", "1"], capture_output=True,
+                         text=True, timeout=600, cwd=str(root))
+    assert run.returncode == 0, run.stderr[-2000:]
+    lines = [l for l in run.stdout.splitlines() if l.startswith("{")]
+    assert len(lines) == 1
+    rec = json.loads(lines[0])
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+                "vs_baseline", "dtype", "data", "config", "roofline", "cpu_baseline"):
+        assert key in rec, key
+    assert rec["n_gpus"] == 1 and rec["steps"] == 3 and rec["warmup"] == 1 and rec["unit"] == "tokens/s"
+    assert rec["dtype"] == "bf16" and rec["data"] == "synthetic" and rec["vs_baseline"] is None
+    assert rec["config"]["workload"] == "moe_layer_24x1024_d768_e8_top2_ff1024_bf16" and "model" not in rec["config"]
+    assert math.isclose(rec["value"], 24576 / (rec["ms_per_step"] * 1e-3), rel_tol=1e-3)
+    roof = rec["roofline"]
+    assert roof["bound"] in ("hbm", "mfma") and roof["unit"] in ("GB/s", "TFLOP/s")
+    assert math.isclose(roof["frac"], roof["achieved"] / roof["peak"], rel_tol=1e-3)
+    assert roof["bound"] == ("mfma" if roof["intensity_flop_per_byte"] >= roof["ridge_flop_per_byte"] else "hbm")
+    assert roof["traffic"] >= roof["algorithmic_bytes"] > 0 and roof["traffic_source"].startswith("profiles/")
+    assert roof["avg_ms"] < rec["ms_per_step"]
+    for stage in rec["kernels"]:
+        assert stage["bound"] == ("mfma" if stage["intensity_flop_per_byte"] >= roof["ridge_flop_per_byte"] else "hbm"), stage
+        assert 0 < stage["frac_mfma"] < 1 and 0 < stage["frac_hbm"] < 1
+    assert sum(s["avg_ms"] for s in rec["kernels"]) < 1.25 * rec["ms_per_step"]
+    cpu = rec["cpu_baseline"]
+    assert cpu["kind"] == "port" and cpu["unit"] == "tokens/s" and cpu["cores"] >= 1 and cpu["value"] > 0 and cpu["sample"]
+    assert rec["value"] > 20 * cpu["value"]
+    assert 0.3 < rec["mfma_sustained"]["frac_of_peak"] < 1.0
