@@ -301,6 +301,40 @@ def test_unweighted_post_act_path(monkeypatch):
         assert torch.equal(a[1][3], b[1][3])   # dS does not depend on where the weight is applied
 
 
+def test_full_size_invariants():
+    """Properties that hold at any size, checked at the benchmark size without a CPU checker.
+    A row of the expert GEMMs does not depend on which rows share its tile, so permuting the tokens
+    permutes the output, dX and dS bit for bit (the weight gradients add the same terms in another
+    order); scaling the routing weights by two scales everything but dS by exactly two (a power of two
+    commutes with every rounding on the way); renaming the experts changes nothing but the order of the
+    weight gradients' leading dimension."""
+    print("moe invariants at 24576 tokens", flush=True)
+    T, H, E, I, K = 24576, 768, 8, 1024, 2
+    case = routed_case(1, T, H, E, I, K)
+    x, w1, w2, idx, w, g = (case[k] for k in ("x", "w1", "w2", "idx", "w", "g"))
+    out, (dx, dw1, dw2, ds) = hip_moe_grads(x, w1, w2, idx, w, g)
+    gen = torch.Generator().manual_seed(5)
+
+    perm = torch.randperm(T, generator=gen)
+    out_p, (dx_p, dw1_p, dw2_p, ds_p) = hip_moe_grads(x[perm], w1, w2, idx[perm], w[perm], g[perm])
+    dev_perm = perm.cuda()
+    assert torch.equal(out_p, out[dev_perm]) and torch.equal(dx_p, dx[dev_perm]) and torch.equal(ds_p, ds[dev_perm])
+    assert_close_scaled(dw1_p, dw1, 5e-3, "dW1 under a token permutation")   # one bf16 rounding of another fp32 sum
+    assert_close_scaled(dw2_p, dw2, 5e-3, "dW2 under a token permutation")
+
+    out_2, (dx_2, dw1_2, dw2_2, ds_2) = hip_moe_grads(x, w1, w2, idx, w * 2, g)
+    for name, a, b in (("out", out_2, out), ("dx", dx_2, dx), ("dW1", dw1_2, dw1), ("dW2", dw2_2, dw2)):
+        assert torch.equal(a.float(), b.float() * 2), name
+    assert torch.equal(ds_2, ds)
+
+    sigma = torch.randperm(E, generator=gen)          # new expert j holds the weights of old expert sigma[j]
+    inverse = torch.empty_like(sigma)
+    inverse[sigma] = torch.arange(E)
+    out_r, (dx_r, dw1_r, dw2_r, ds_r) = hip_moe_grads(x, w1[sigma], w2[sigma], inverse[idx.long()].to(idx.dtype), w, g)
+    assert torch.equal(out_r, out) and torch.equal(dx_r, dx) and torch.equal(ds_r, ds)
+    assert torch.equal(dw1_r, dw1[sigma.cuda()]) and torch.equal(dw2_r, dw2[sigma.cuda()])
+
+
 @pytest.mark.parametrize("T,H,E,I,skew", [(600, 64, 130, 64, 0.0), (900, 64, 130, 64, 0.6), (400, 64, 1500, 32, 0.0)])
 def test_more_experts_than_a_wave_holds(T, H, E, I, skew):
     """E > 64: the tile and unit lookups of the GEMM kernels take more than one round of 64 experts
