@@ -1480,6 +1480,10 @@ __global__ __launch_bounds__(T::NT) void dw_gemm_ws_kernel(DwParams p) {
 // the compiled tile shapes
 typedef Tile<128, 128, 2, 2> StagedSmall;                 // 4 waves of 64x64, any K that is a multiple of 8
 typedef RingTile<256, 128, 2, 2, 32, 3, 2> RingTwoPerCu;  // 4 waves of 128x64, 3 x 24 KiB stages, two blocks per CU
+// 4 waves of 96x64, 2 x 20 KiB stages, three blocks per CU (at most 168 registers per lane): while one block
+// is in its epilogue two others are in their k-loops, and a block that waits for its one tile in flight
+// has two neighbours to cover for it
+typedef RingTile<192, 128, 2, 2, 32, 2, 3> RingThreePerCu;
 typedef WsTile<256, 256, 2, 4, 32, 4, 4, 3> WsLarge;      // 8 consumer waves of 128x64 + 4 producers, 4 x 32 KiB stages
 typedef DwWsTile<256, 256, 2, 4, 32, 4, 4> DwWsLarge;     // same shape for the weight-gradient GEMMs
 
@@ -1546,11 +1550,12 @@ __global__ __launch_bounds__(WsLarge::NT, WsLarge::WAVES_PER_EU) void bwd_joint_
 enum Kind { K_GATEUP = 0, K_DOWN, K_DY1, K_DX, K_DW2, K_DW1, K_COUNT };
 const char* const kKindEnv[K_COUNT] = {"MTS_TILE_GATEUP", "MTS_TILE_DOWN", "MTS_TILE_DY1",
                                        "MTS_TILE_DX",     "MTS_TILE_DW2",  "MTS_TILE_DW1"};
-// rows_gemm: 0 StagedSmall, 1 RingTwoPerCu, 2 WsLarge;  dw_gemm: 0 StagedSmall, 2 DwWsLarge.
+// rows_gemm: 0 StagedSmall, 1 RingTwoPerCu, 2 WsLarge, 3 RingThreePerCu (dY1 without the weighted_act output
+// only);  dw_gemm: 0 StagedSmall, 2 DwWsLarge.
 // Defaults are the fastest measured on the 24576-token, 768/1024, 8-expert layer: the two GEMMs with
-// the heavy epilogues (gate/up + SwiGLU, dO*W2 + SwiGLU backward) gain more from two co-resident
-// 4-wave blocks per CU, the others from specialised waves.
-const int kDefaultTile[K_COUNT] = {1, 2, 1, 2, 2, 2};
+// the heavy epilogues (gate/up + SwiGLU, dO*W2 + SwiGLU backward) gain more from co-resident
+// 4-wave blocks, two per CU for gate/up and three for dY1, the others from specialised waves.
+const int kDefaultTile[K_COUNT] = {1, 2, 3, 2, 2, 2};
 
 bool tile_forced(int kind) { return getenv(kKindEnv[kind]) != nullptr; }
 
@@ -1561,7 +1566,7 @@ int tile_choice(int kind) {
         int c = kDefaultTile[kind];
         const char* s = getenv(kKindEnv[kind]);
         if (s) c = atoi(s);
-        choice[kind] = (c >= 0 && c <= 2) ? c : kDefaultTile[kind];
+        choice[kind] = (c >= 0 && c <= (kind == K_DY1 ? 3 : 2)) ? c : kDefaultTile[kind];
     }
     return choice[kind];
 }
@@ -1619,10 +1624,17 @@ int launch_rows_any(int kind, RowsParams p, int64_t TK, hipStream_t s, bool b_km
     // gate/up: two co-resident ring blocks per CU win while the SwiGLU epilogue is a large part of a tile
     // (short reductions); long reductions are better off with specialised waves
     if (kind == K_GATEUP && !tile_forced(kind) && p.Kdim > 1024) choice = 2;
+    // three blocks per CU hold two stages each: for short reductions, and for the epilogue that fits beside them
+    if (choice == 3 && (EPI != EPI_DY1N || !b_kmajor || (!tile_forced(kind) && p.Kdim > 1024))) choice = 1;
     // the ring kernels need whole k-tiles; other shapes use the staged kernel
     if (choice >= 1 && p.Kdim % 64 != 0) choice = 0;
     if (b_kmajor && (choice == 0 || EPI == EPI_SWIGLU)) return MTS_ERR_SHAPE;
-    if (choice == 1) {
+    if (choice == 3) {
+        if constexpr (EPI == EPI_DY1N) {
+            const dim3 grid = rows_grid<RingThreePerCu, EPI>(p, TK);
+            rows_gemm_ring_kernel<RingThreePerCu, EPI, true><<<grid, RingThreePerCu::NT, 0, s>>>(p);
+        }
+    } else if (choice == 1) {
         const dim3 grid = rows_grid<RingTwoPerCu, EPI>(p, TK);
         if constexpr (EPI != EPI_SWIGLU) {
             if (b_kmajor) rows_gemm_ring_kernel<RingTwoPerCu, EPI, true><<<grid, RingTwoPerCu::NT, 0, s>>>(p);
