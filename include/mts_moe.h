@@ -309,6 +309,32 @@ int mts_moe_bwd_joint(const void* d_out, const void* weighted_act, const void* d
                       void* d_weights, void* workspace1, int64_t workspace1_bytes,
                       void* workspace2, int64_t workspace2_bytes, void* stream);
 
+/* mts_moe_bwd_joint with the router's backward in the same launch: what mts_moe_head_bwd computes
+ * (the autograd backward of minitrain/model/moe_router.py:64-90 given the routing-weight gradient
+ * and the loss-term gradients), by the same per-block arithmetic and with bit-identical results,
+ * as trailing blocks of the joint launch.  They form the routing-weight gradient from ds_partial
+ * themselves, so they depend on nothing the launch writes, and run on the CUs that the last
+ * round of dX tiles leaves idle; one small launch then sums the per-block partials of d_w_r.
+ * w_r [E,H] f32, logits [T,E] f32, weights [T,K] f32, indices [T,K], counts [E] (needed with
+ * g_load_balance), g_prob_mean [E] / g_z_loss / g_load_balance (each may be NULL: zero);
+ * outputs dx_router [T,H] in act_dtype and d_w_r [E,H] f32; router_workspace as for
+ * mts_moe_head_bwd (mts_moe_head_bwd_workspace_bytes).  mts_moe_bwd_joint_router_supported()
+ * says whether the shapes allow it (those of mts_moe_bwd_joint, E <= 8, H a multiple of 4 whose
+ * dW_r sums fit the block's LDS).                                                       */
+int mts_moe_bwd_joint_router_supported(int act_dtype, int64_t T, int H, int I, int E);
+int mts_moe_bwd_joint_router(const void* d_out, const void* weighted_act, const void* d_pre_act,
+                             const void* x, const void* w1, const int32_t* x_gather,
+                             const int32_t* expert_start, const int32_t* s_reverse,
+                             const float* ds_partial, int64_t T, int K, int E, int H, int I,
+                             int act_dtype, int grad_dtype, void* dx_expanded, void* d_w1, void* d_w2,
+                             void* d_weights, void* workspace1, int64_t workspace1_bytes,
+                             void* workspace2, int64_t workspace2_bytes, const float* w_r,
+                             const float* logits, const float* weights, const int32_t* indices,
+                             const int32_t* counts, const float* g_prob_mean, const float* g_z_loss,
+                             const float* g_load_balance, int normalize, void* dx_router,
+                             float* d_w_r, void* router_workspace, int64_t router_workspace_bytes,
+                             void* stream);
+
 #ifdef __cplusplus
 }
 #endif

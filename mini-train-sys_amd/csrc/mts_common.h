@@ -66,6 +66,16 @@ int mts_moe_bwd_joint_f16(const void* d_out, const void* weighted_act, const voi
                           int act_dtype, int grad_dtype, void* dx_expanded, void* d_w1, void* d_w2, void* d_weights,
                           void* workspace1, int64_t workspace1_bytes, void* workspace2, int64_t workspace2_bytes,
                           void* stream);
+int mts_moe_bwd_joint_router_f16(const void* d_out, const void* weighted_act, const void* d_pre_act, const void* x,
+                                 const void* w1, const int32_t* x_gather, const int32_t* expert_start,
+                                 const int32_t* s_reverse, const float* ds_partial, int64_t T, int K, int E, int H,
+                                 int I, int act_dtype, int grad_dtype, void* dx_expanded, void* d_w1, void* d_w2,
+                                 void* d_weights, void* workspace1, int64_t workspace1_bytes, void* workspace2,
+                                 int64_t workspace2_bytes, const float* w_r, const float* logits,
+                                 const float* weights, const int32_t* indices, const int32_t* counts,
+                                 const float* g_prob_mean, const float* g_z_loss, const float* g_load_balance,
+                                 int normalize, void* dx_router, float* d_w_r, void* router_workspace,
+                                 int64_t router_workspace_bytes, void* stream);
 }
 
 // fp32 GEMM launchers (mts_gemm_f32.hip); epi: 0 plain, 1 SwiGLU, 2 dO*W2 with SwiGLU backward
@@ -78,6 +88,15 @@ int mts_f32_dw(const float* P, const int32_t* p_gather, const float* Q, const in
 
 // chained router forward (mts_router_linear.hip), launched by mts_moe_head_fwd (mts_route.hip)
 #define MTS_HEAD_MAX_CHUNKS 512
+// Launch shape of the chained router backward (mts_router_linear.hip): row blocks x column ranges, the threads
+// a block needs (groups sets of col_threads) and its dynamic LDS; contract checks of that path; the reduction
+// of its per-block dW_r partials.
+struct MtsRouterBwdShape {
+    int row_blocks, rows_per_block, groups, col_threads, cols_per_block, ranges;
+};
+int mts_router_bwd_check(const void* x, const float* w_r, int64_t T, int H, int E, int act_dtype);
+void mts_router_bwd_shape(int64_t T, int H, int E, MtsRouterBwdShape* shape);
+int mts_launch_router_dw_reduce(const float* part, int row_blocks, int64_t EH, float* d_w_r, hipStream_t s);
 void mts_router_head_geometry(int64_t T, int* blocks, int* rows_per_wave);
 int mts_launch_router_head(const void* x, const float* w_r, int64_t T, int H, int E, int K, int normalize, int act_dtype,
                            float* logits, float* weights, int32_t* indices, void* weights_act, float* partial,

@@ -26,6 +26,7 @@
 //   A/B fragment: row (l % 32) of the 32-row operand, k = 8*(l/32) .. 8*(l/32)+7
 //   C fragment:   element i (0..15) is row 8*(i/4) + 4*(l/32) + (i%4), column l % 32
 #include "mts_common.h"
+#include "mts_router_bwd_block.h"
 
 #include <stdlib.h>
 
@@ -1098,12 +1099,17 @@ __global__ __launch_bounds__(256) void dw_chunk_sum_kernel(DwParams p) {
     dw_chunk_sum_expert<BM, BN, OutT>(p, blockIdx.y);
 }
 
-// the same for two GEMMs over the same experts in one launch: blockIdx.y < E is the first's expert
+// the same for two GEMMs over the same experts in one launch: blockIdx.y < E is the first's expert; rows of
+// blocks past the second's experts sum the per-block partials of the router's weight gradient, where the
+// router's backward was part of the launch before (r_part != NULL)
 template <int BM, int BN, typename OutT>
-__global__ __launch_bounds__(256) void dw_chunk_sum_pair_kernel(DwParams a, DwParams b) {
+__global__ __launch_bounds__(256) void dw_chunk_sum_pair_kernel(DwParams a, DwParams b, const float* r_part, int r_blocks,
+                                                                int64_t r_EH, float* r_dw) {
+    static_assert(mts_rl::kReduceThreads == 256, "one block shape");
     const int e = blockIdx.y;
     if (e < a.E) dw_chunk_sum_expert<BM, BN, OutT>(a, e);
-    else dw_chunk_sum_expert<BM, BN, OutT>(b, e - a.E);
+    else if (e < a.E + b.E) dw_chunk_sum_expert<BM, BN, OutT>(b, e - a.E);
+    else mts_rl::router_dw_reduce_block(r_part, r_blocks, r_EH, r_dw, (int64_t)(e - a.E - b.E) * gridDim.x + blockIdx.x);
 }
 
 // Stages a [64 k][64 m] block per wave-item: lane = (kgrp = lane%8, mc = lane/8) loads
@@ -1497,6 +1503,7 @@ typedef DwWsTile<256, 256, 2, 4, 32, 4, 4> DwWsLarge;     // same shape for the 
 // Every part starts at a multiple of the XCD count, so block % 8 is still the part's own
 // XCD index.
 // ---------------------------------------------------------------------------
+constexpr int kJointRouterExperts = 8;   // the router blocks of the joint launch are compiled for up to 8 experts
 struct BwdJointParams {
     DwParams dw1, dw2;
     RowsParams dx;
@@ -1506,6 +1513,19 @@ struct BwdJointParams {
     bf16_t* d_weights;             // [entries]
     int np;
     int64_t entries;
+    int n_ds;                      // blocks that reduce dS
+    // The router's backward behind the dS blocks (n_router = 0: not part of this launch): the blocks of the
+    // chained projection backward, which form the routing-weight gradient from ds_part themselves.  They
+    // depend on nothing this launch writes and take the CUs that the last round of dX tiles leaves idle.
+    int n_router, router_row_blocks;
+    const bf16_t* rx;              // activations [T, H]
+    const float* rw;               // router weight [E, H]
+    int64_t rT;
+    int rH, rE, r_rows_per_block, r_groups, r_cols_per_block, r_col_threads;
+    bf16_t* r_dx;                  // the router's share of dx [T, H]
+    float* r_part;                 // [router_row_blocks][E][H] partial dW_r
+    float* r_dw;                   // dW_r [E][H]: summed from r_part by the launch that follows (host side only)
+    mts_rl::RouterGradIn rg;
 };
 
 template <typename OutT>
@@ -1531,15 +1551,26 @@ __global__ __launch_bounds__(WsLarge::NT, WsLarge::WAVES_PER_EU) void bwd_joint_
         return;
     }
     b -= q.n_dx;
-    const int nb = (int)gridDim.x - q.n_dw1 - q.n_dw2 - q.n_dx;
-    for (int64_t n = (int64_t)b * WsLarge::NT + threadIdx.x; n < q.entries; n += (int64_t)nb * WsLarge::NT) {
-        const int32_t r = q.s_reverse[n];
-        float v = 0.f;
-        if (r >= 0) {
-            const float* part = q.ds_part + (int64_t)r * q.np;
-            for (int j = 0; j < q.np; ++j) v += part[j];
+    if (b < q.n_ds) {
+        for (int64_t n = (int64_t)b * WsLarge::NT + threadIdx.x; n < q.entries; n += (int64_t)q.n_ds * WsLarge::NT) {
+            const int32_t r = q.s_reverse[n];
+            float v = 0.f;
+            if (r >= 0) {
+                const float* part = q.ds_part + (int64_t)r * q.np;
+                for (int j = 0; j < q.np; ++j) v += part[j];
+            }
+            q.d_weights[n] = (bf16_t)v;
         }
-        q.d_weights[n] = (bf16_t)v;
+        return;
+    }
+    b -= q.n_ds;
+    if (b < q.n_router) {
+        constexpr int EP = kJointRouterExperts;
+        float* set_sum = reinterpret_cast<float*>(smem);                       // [E][cols_per_block]
+        float* dl_lds = set_sum + q.rE * q.r_cols_per_block;                    // [kChainRows][EP]
+        mts_rl::router_logits_bwd_block<bf16_t, EP, false, true>(
+            nullptr, q.rx, q.rw, q.rT, q.rH, q.rE, q.r_rows_per_block, q.r_groups, q.r_cols_per_block, q.r_dx, q.r_part,
+            q.rg, b % q.router_row_blocks, b / q.router_row_blocks, q.r_col_threads, set_sum, dl_lds);
     }
 }
 
@@ -1735,20 +1766,29 @@ int launch_bwd_joint(BwdJointParams q, int E, int grad_dtype, void* ws1, int64_t
     q.n_dw2 = (int)dw_grid<T>(q.dw2, E, q.dw2.part ? 2 * E : E).x;
     q.n_dx = (int)rows_grid<WsLarge, EPI_PLAIN>(q.dx, q.dx.TK).x;
     const int64_t want = (q.entries + WsLarge::NT * 4 - 1) / (WsLarge::NT * 4);
-    const int n_ds = (int)(want < 64 ? want : 64);
-    const dim3 grid((unsigned)(q.n_dw1 + q.n_dw2 + q.n_dx + n_ds));
+    q.n_ds = (int)(want < 64 ? want : 64);
+    const dim3 grid((unsigned)(q.n_dw1 + q.n_dw2 + q.n_dx + q.n_ds + q.n_router));
     if (grad_dtype == MTS_GEMM_DTYPE) bwd_joint_kernel<bf16_t><<<grid, WsLarge::NT, 0, s>>>(q);
     else bwd_joint_kernel<float><<<grid, WsLarge::NT, 0, s>>>(q);
     MTS_CHECK_LAUNCH();
     if (q.dw1.part && q.dw2.part && 2 * E <= 65535) {
         const int t = q.dw1.tiles_per_expert > q.dw2.tiles_per_expert ? q.dw1.tiles_per_expert : q.dw2.tiles_per_expert;
         const int64_t want = ((int64_t)t * (T::BM * T::BN / 4) + 255) / 256;
-        const dim3 sum_grid((unsigned)(want < 256 ? want : 256), (unsigned)(2 * E));
-        if (grad_dtype == MTS_GEMM_DTYPE) dw_chunk_sum_pair_kernel<T::BM, T::BN, bf16_t><<<sum_grid, 256, 0, s>>>(q.dw1, q.dw2);
-        else dw_chunk_sum_pair_kernel<T::BM, T::BN, float><<<sum_grid, 256, 0, s>>>(q.dw1, q.dw2);
+        const unsigned gx = (unsigned)(want < 256 ? want : 256);
+        // the sum of the router's dW_r partials rides along as extra rows of blocks
+        const int64_t r_EH = (int64_t)q.rE * q.rH;
+        const int64_t r_jobs = q.n_router ? (r_EH + mts_rl::kReduceCols - 1) / mts_rl::kReduceCols : 0;
+        const dim3 sum_grid(gx, (unsigned)(2 * E + (r_jobs + gx - 1) / gx));
+        if (grad_dtype == MTS_GEMM_DTYPE)
+            dw_chunk_sum_pair_kernel<T::BM, T::BN, bf16_t><<<sum_grid, 256, 0, s>>>(q.dw1, q.dw2, q.r_part, q.router_row_blocks, r_EH, q.r_dw);
+        else
+            dw_chunk_sum_pair_kernel<T::BM, T::BN, float><<<sum_grid, 256, 0, s>>>(q.dw1, q.dw2, q.r_part, q.router_row_blocks, r_EH, q.r_dw);
     } else {   // one of the two, or more experts than a grid holds in y twice over
         if (q.dw1.part) launch_dw_chunk_sum(q.dw1, E, grad_dtype, s);
         if (q.dw2.part) launch_dw_chunk_sum(q.dw2, E, grad_dtype, s);
+        MTS_CHECK_LAUNCH();
+        if (q.n_router) return mts_launch_router_dw_reduce(q.r_part, q.router_row_blocks, (int64_t)q.rE * q.rH, q.r_dw, s);
+        return MTS_OK;
     }
     MTS_CHECK_LAUNCH();
     return MTS_OK;
@@ -1943,6 +1983,48 @@ extern "C" int mts_moe_bwd_joint_supported(int act_dtype, int H, int I) {
 }
 #endif
 
+namespace {
+// argument checks of the joint launch and its parameter block (without the router's part)
+int fill_bwd_joint(BwdJointParams& q, const void* d_out, const void* weighted_act, const void* d_pre_act, const void* x,
+                   const void* w1, const int32_t* x_gather, const int32_t* expert_start, const int32_t* s_reverse,
+                   const float* ds_partial, int64_t T, int K, int E, int H, int I, int act_dtype, void* dx_expanded,
+                   void* d_w1, void* d_w2, void* d_weights) {
+    if (!d_out || !weighted_act || !d_pre_act || !x || !w1 || !x_gather || !expert_start || !s_reverse || !ds_partial ||
+        !dx_expanded || !d_w1 || !d_w2 || !d_weights)
+        return MTS_ERR_NULL;
+    if (act_dtype != MTS_GEMM_DTYPE) return MTS_ERR_DTYPE;
+    if (T <= 0 || K < 1) return MTS_ERR_SHAPE;
+    const int64_t TK = T * K;
+    int rc = check_common(TK, E, H, I, T);
+    if (rc) return rc;
+    if (!bwd_joint_ok(H, I)) return MTS_ERR_SHAPE;
+    if (!mts_aligned16(d_out) || !mts_aligned16(weighted_act) || !mts_aligned16(d_pre_act) || !mts_aligned16(x) ||
+        !mts_aligned16(w1) || !mts_aligned16(dx_expanded) || !mts_aligned16(d_w1) || !mts_aligned16(d_w2))
+        return MTS_ERR_ALIGN;
+    q.dw1.P = (const bf16_t*)d_pre_act; q.dw1.p_rows = TK; q.dw1.p_gather = nullptr;
+    q.dw1.Q = (const bf16_t*)x; q.dw1.q_rows = T; q.dw1.q_gather = x_gather;
+    q.dw1.M = 2 * I; q.dw1.N = H; q.dw1.TK = TK; q.dw1.expert_start = expert_start; q.dw1.C = d_w1;
+    q.dw2.P = (const bf16_t*)d_out; q.dw2.p_rows = T; q.dw2.p_gather = x_gather;
+    q.dw2.Q = (const bf16_t*)weighted_act; q.dw2.q_rows = TK; q.dw2.q_gather = nullptr;
+    q.dw2.M = H; q.dw2.N = I; q.dw2.TK = TK; q.dw2.expert_start = expert_start; q.dw2.C = d_w2;
+    q.dx.A = (const bf16_t*)d_pre_act; q.dx.a_rows = TK; q.dx.lda = 2 * I; q.dx.a_gather = nullptr;
+    q.dx.B = (const bf16_t*)w1; q.dx.b_rows = H;
+    q.dx.N = H; q.dx.Kdim = 2 * I; q.dx.expert_start = expert_start; q.dx.E = E;
+    q.dx.C = (bf16_t*)dx_expanded; q.dx.TK = TK;
+    q.ds_part = ds_partial; q.s_reverse = s_reverse; q.d_weights = (bf16_t*)d_weights; q.np = dy1_partials(I); q.entries = TK;
+    return MTS_OK;
+}
+
+// can the router's backward ride in the joint launch?  Its blocks are compiled for up to kJointRouterExperts
+// experts, need no more threads than a block of the launch has, and keep E x cols floats of dW_r sums and the
+// logit gradients of their rows in the block's LDS
+bool joint_router_ok(int H, int E, const MtsRouterBwdShape& g) {
+    constexpr size_t lds_bytes = (size_t)ws_lds_elems<WsLarge, EPI_PLAIN>() * sizeof(bf16_t);
+    const size_t need = ((size_t)E * g.cols_per_block + (size_t)mts_rl::kChainRows * kJointRouterExperts) * sizeof(float);
+    return E <= kJointRouterExperts && g.groups * g.col_threads <= WsLarge::NT && need <= lds_bytes && H % 4 == 0;
+}
+}  // namespace
+
 extern "C" int MTS_GEMM_ENTRY(mts_moe_bwd_joint)(const void* d_out, const void* weighted_act, const void* d_pre_act,
                                                  const void* x, const void* w1, const int32_t* x_gather,
                                                  const int32_t* expert_start, const int32_t* s_reverse,
@@ -1956,29 +2038,61 @@ extern "C" int MTS_GEMM_ENTRY(mts_moe_bwd_joint)(const void* d_out, const void* 
                                      ds_partial, T, K, E, H, I, act_dtype, grad_dtype, dx_expanded, d_w1, d_w2, d_weights,
                                      workspace1, workspace1_bytes, workspace2, workspace2_bytes, stream);
 #endif
-    if (!d_out || !weighted_act || !d_pre_act || !x || !w1 || !x_gather || !expert_start || !s_reverse || !ds_partial ||
-        !dx_expanded || !d_w1 || !d_w2 || !d_weights)
-        return MTS_ERR_NULL;
-    if (act_dtype != MTS_GEMM_DTYPE) return MTS_ERR_DTYPE;
-    if (T <= 0 || K < 1) return MTS_ERR_SHAPE;
-    const int64_t TK = T * K;
-    int rc = check_common(TK, E, H, I, T);
-    if (rc) return rc;
-    if (!bwd_joint_ok(H, I)) return MTS_ERR_SHAPE;
-    if (!mts_aligned16(d_out) || !mts_aligned16(weighted_act) || !mts_aligned16(d_pre_act) || !mts_aligned16(x) ||
-        !mts_aligned16(w1) || !mts_aligned16(dx_expanded) || !mts_aligned16(d_w1) || !mts_aligned16(d_w2))
-        return MTS_ERR_ALIGN;
     BwdJointParams q = {};
-    q.dw1.P = (const bf16_t*)d_pre_act; q.dw1.p_rows = TK; q.dw1.p_gather = nullptr;
-    q.dw1.Q = (const bf16_t*)x; q.dw1.q_rows = T; q.dw1.q_gather = x_gather;
-    q.dw1.M = 2 * I; q.dw1.N = H; q.dw1.TK = TK; q.dw1.expert_start = expert_start; q.dw1.C = d_w1;
-    q.dw2.P = (const bf16_t*)d_out; q.dw2.p_rows = T; q.dw2.p_gather = x_gather;
-    q.dw2.Q = (const bf16_t*)weighted_act; q.dw2.q_rows = TK; q.dw2.q_gather = nullptr;
-    q.dw2.M = H; q.dw2.N = I; q.dw2.TK = TK; q.dw2.expert_start = expert_start; q.dw2.C = d_w2;
-    q.dx.A = (const bf16_t*)d_pre_act; q.dx.a_rows = TK; q.dx.lda = 2 * I; q.dx.a_gather = nullptr;
-    q.dx.B = (const bf16_t*)w1; q.dx.b_rows = H;
-    q.dx.N = H; q.dx.Kdim = 2 * I; q.dx.expert_start = expert_start; q.dx.E = E;
-    q.dx.C = (bf16_t*)dx_expanded; q.dx.TK = TK;
-    q.ds_part = ds_partial; q.s_reverse = s_reverse; q.d_weights = (bf16_t*)d_weights; q.np = dy1_partials(I); q.entries = TK;
+    const int rc = fill_bwd_joint(q, d_out, weighted_act, d_pre_act, x, w1, x_gather, expert_start, s_reverse, ds_partial, T,
+                                  K, E, H, I, act_dtype, dx_expanded, d_w1, d_w2, d_weights);
+    if (rc) return rc;
+    return launch_bwd_joint(q, E, grad_dtype, workspace1, workspace1_bytes, workspace2, workspace2_bytes, (hipStream_t)stream);
+}
+
+#ifndef MTS_GEMM_F16
+extern "C" int mts_moe_bwd_joint_router_supported(int act_dtype, int64_t T, int H, int I, int E) {
+    if (!mts_moe_bwd_joint_supported(act_dtype, H, I) || T <= 0 || H < 4 || H % 4 || E < 1 || E > kJointRouterExperts) return 0;
+    MtsRouterBwdShape g;
+    mts_router_bwd_shape(T, H, E, &g);
+    return joint_router_ok(H, E, g) ? 1 : 0;
+}
+#endif
+
+extern "C" int MTS_GEMM_ENTRY(mts_moe_bwd_joint_router)(
+    const void* d_out, const void* weighted_act, const void* d_pre_act, const void* x, const void* w1,
+    const int32_t* x_gather, const int32_t* expert_start, const int32_t* s_reverse, const float* ds_partial, int64_t T,
+    int K, int E, int H, int I, int act_dtype, int grad_dtype, void* dx_expanded, void* d_w1, void* d_w2, void* d_weights,
+    void* workspace1, int64_t workspace1_bytes, void* workspace2, int64_t workspace2_bytes, const float* w_r,
+    const float* logits, const float* weights, const int32_t* indices, const int32_t* counts, const float* g_prob_mean,
+    const float* g_z_loss, const float* g_load_balance, int normalize, void* dx_router, float* d_w_r,
+    void* router_workspace, int64_t router_workspace_bytes, void* stream) {
+#ifndef MTS_GEMM_F16
+    if (act_dtype == MTS_F16)
+        return mts_moe_bwd_joint_router_f16(d_out, weighted_act, d_pre_act, x, w1, x_gather, expert_start, s_reverse,
+                                            ds_partial, T, K, E, H, I, act_dtype, grad_dtype, dx_expanded, d_w1, d_w2,
+                                            d_weights, workspace1, workspace1_bytes, workspace2, workspace2_bytes, w_r, logits,
+                                            weights, indices, counts, g_prob_mean, g_z_loss, g_load_balance, normalize,
+                                            dx_router, d_w_r, router_workspace, router_workspace_bytes, stream);
+#endif
+    BwdJointParams q = {};
+    int rc = fill_bwd_joint(q, d_out, weighted_act, d_pre_act, x, w1, x_gather, expert_start, s_reverse, ds_partial, T, K, E,
+                            H, I, act_dtype, dx_expanded, d_w1, d_w2, d_weights);
+    if (rc) return rc;
+    rc = mts_router_bwd_check(x, w_r, T, H, E, act_dtype);
+    if (rc) return rc;
+    if (!logits || !weights || !indices || !dx_router || !d_w_r || !router_workspace) return MTS_ERR_NULL;
+    if (g_load_balance && !counts) return MTS_ERR_NULL;
+    if (K > E || K > MTS_MAX_TOP_K) return MTS_ERR_SHAPE;
+    MtsRouterBwdShape g;
+    mts_router_bwd_shape(T, H, E, &g);
+    if (!joint_router_ok(H, E, g)) return MTS_ERR_SHAPE;
+    if (router_workspace_bytes < (int64_t)g.row_blocks * E * H * (int64_t)sizeof(float)) return MTS_ERR_WORKSPACE;
+    if (!mts_aligned16(router_workspace) || !mts_aligned16(d_w_r) || !mts_aligned16(dx_router) ||
+        (E == 8 && !mts_aligned16(logits)))
+        return MTS_ERR_ALIGN;
+    q.n_router = g.row_blocks * g.ranges;
+    q.router_row_blocks = g.row_blocks;
+    q.rx = (const bf16_t*)x; q.rw = w_r; q.rT = T; q.rH = H; q.rE = E;
+    q.r_rows_per_block = g.rows_per_block; q.r_groups = g.groups; q.r_cols_per_block = g.cols_per_block;
+    q.r_col_threads = g.col_threads;
+    q.r_dx = (bf16_t*)dx_router; q.r_part = (float*)router_workspace; q.r_dw = d_w_r;
+    q.rg = {logits, weights, indices, counts, nullptr, nullptr, g_prob_mean, g_z_loss, g_load_balance, act_dtype, K, normalize,
+            ds_partial, s_reverse, q.np};
     return launch_bwd_joint(q, E, grad_dtype, workspace1, workspace1_bytes, workspace2, workspace2_bytes, (hipStream_t)stream);
 }

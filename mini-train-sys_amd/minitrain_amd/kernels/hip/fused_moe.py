@@ -168,6 +168,8 @@ def expert_counts(topk_indices: torch.Tensor, E: int) -> torch.Tensor:
 _OVERLAP = os.environ.get("MTS_NO_OVERLAP", "0") != "1"
 # MTS_NO_JOINT_BWD=1 launches dW2, dW1 and dX separately (on the side streams) even where one launch could hold them
 _JOINT = os.environ.get("MTS_NO_JOINT_BWD", "0") != "1"
+# MTS_NO_TAIL_IN_JOINT=1 keeps the router's backward of the layer node in launches of its own
+_TAIL_IN_JOINT = os.environ.get("MTS_NO_TAIL_IN_JOINT", "0") != "1"
 # MTS_WEIGHTED_POST=0: the forward pass writes the unweighted activation and dY1 writes s * a again (tuning runs only)
 _WEIGHTED_POST = os.environ.get("MTS_WEIGHTED_POST", "1") != "0"
 _SIDE_STREAMS: dict = {}
@@ -277,13 +279,26 @@ def moe_forward(x, gate_up_proj, down_proj, weights_flat, routing):
     return out, tensors, state
 
 
-def moe_backward(tensors, state, dO, needs, x_addend=None):
+class RouterTail:
+    """What the router's backward needs besides ``dS`` (saved router tensors and the gradients of the
+    router's loss terms); ``moe_backward`` fills ``dx_r`` / ``dw_r`` when that backward ran inside the
+    launch of the expert GEMMs' backward."""
+
+    def __init__(self, router_weight, logits, weights, indices, counts, g_prob_mean, g_z_loss, g_load_balance, normalize):
+        self.router_weight, self.logits, self.weights, self.indices, self.counts = router_weight, logits, weights, indices, counts
+        self.g_prob_mean, self.g_z_loss, self.g_load_balance, self.normalize = g_prob_mean, g_z_loss, g_load_balance, normalize
+        self.dx_r = self.dw_r = None
+
+
+def moe_backward(tensors, state, dO, needs, x_addend=None, router_tail=None):
     """``(dx, dW1, dW2, dS)`` for ``needs = (x, W1, W2, S)``.
 
     ``x_addend``: called with ``dS`` (on the caller's stream) once it exists and before the dX combine;
     what it returns ([T,H], activation dtype, or None) is added to ``dx`` inside the combine kernel.
     It is how a caller that owns another path from ``x`` to the loss (the router) avoids a separate
-    sum of the two gradients."""
+    sum of the two gradients.  ``router_tail``: the router's side of that path; where the one-launch
+    backward applies and the library can hold the router's backward in it, its outputs are stored in
+    the object before ``x_addend`` is called."""
     lib = _lib.load()
     (x, gate_up_proj, down_proj, pre_act, weights_flat, expert_start, x_gather, s_scatter, s_reverse) = tensors[:9]
     T, K, E, H, I = state.dims
@@ -376,15 +391,30 @@ def moe_backward(tensors, state, dO, needs, x_addend=None):
         dgate_up_proj, ddown_proj = torch.empty_like(gate_up_proj), torch.empty_like(down_proj)
         d_weights = torch.empty(T, K, dtype=weights_flat.dtype, device=dev)
         dx_expanded = torch.empty(TK, H, dtype=x.dtype, device=dev)
-        _lib.check(
-            lib.mts_moe_bwd_joint(
-                dO.data_ptr(), weighted_act.data_ptr(), d_pre_act.data_ptr(), x.data_ptr(), w1_bwd.data_ptr(),
-                x_gather.data_ptr(), expert_start.data_ptr(), s_reverse.data_ptr(), ds_part.data_ptr(), T, K, E, H, I,
-                act, _lib.dtype_code(gate_up_proj.dtype), dx_expanded.data_ptr(), dgate_up_proj.data_ptr(),
-                ddown_proj.data_ptr(), d_weights.data_ptr(), ws1_ptr, ws1_bytes, ws2_ptr, ws2_bytes, stream,
-            ),
-            "mts_moe_bwd_joint",
+        joint_args = (
+            dO.data_ptr(), weighted_act.data_ptr(), d_pre_act.data_ptr(), x.data_ptr(), w1_bwd.data_ptr(),
+            x_gather.data_ptr(), expert_start.data_ptr(), s_reverse.data_ptr(), ds_part.data_ptr(), T, K, E, H, I,
+            act, _lib.dtype_code(gate_up_proj.dtype), dx_expanded.data_ptr(), dgate_up_proj.data_ptr(),
+            ddown_proj.data_ptr(), d_weights.data_ptr(), ws1_ptr, ws1_bytes, ws2_ptr, ws2_bytes,
         )
+        rt = router_tail
+        if rt is not None and _TAIL_IN_JOINT and lib.mts_moe_bwd_joint_router_supported(act, T, H, I, E):
+            # the router's backward as trailing blocks of the same launch: it needs nothing the launch writes
+            dx_r, dw_r = torch.empty_like(x), torch.empty_like(rt.router_weight)
+            rws_bytes = lib.mts_moe_head_bwd_workspace_bytes(T, H, E)
+            rws = torch.empty(rws_bytes, dtype=torch.uint8, device=dev)
+            _lib.check(
+                lib.mts_moe_bwd_joint_router(
+                    *joint_args, rt.router_weight.data_ptr(), rt.logits.data_ptr(), rt.weights.data_ptr(),
+                    rt.indices.data_ptr(), _lib.ptr(rt.counts), _lib.ptr(rt.g_prob_mean), _lib.ptr(rt.g_z_loss),
+                    _lib.ptr(rt.g_load_balance), int(rt.normalize), dx_r.data_ptr(), dw_r.data_ptr(), rws.data_ptr(),
+                    rws_bytes, stream,
+                ),
+                "mts_moe_bwd_joint_router",
+            )
+            rt.dx_r, rt.dw_r = dx_r, dw_r
+        else:
+            _lib.check(lib.mts_moe_bwd_joint(*joint_args, stream), "mts_moe_bwd_joint")
         return combine_dx(dx_expanded, d_weights), dgate_up_proj, ddown_proj, d_weights
 
     if need_w1 and need_w2:

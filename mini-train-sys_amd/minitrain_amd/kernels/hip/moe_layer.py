@@ -14,7 +14,8 @@ offers it (``ops.moe_layer``) and the configuration allows it.
 import torch
 
 from minitrain_amd import _lib
-from minitrain_amd.kernels.hip.fused_moe import expert_contract, first_violation, moe_backward, moe_forward, needs_padding
+from minitrain_amd.kernels.hip.fused_moe import (RouterTail, expert_contract, first_violation, moe_backward, moe_forward,
+                                                 needs_padding)
 from minitrain_amd.kernels.hip.router import _MAX_TOP_K, is_router_logits_supported
 
 
@@ -102,8 +103,13 @@ class _MoELayerFunction(torch.autograd.Function):
 
         g_lb, g_z, g_p = f32(g_load_balance), f32(g_z_loss), f32(g_prob_mean)
 
+        tail = RouterTail(router_weight, logits, weights, indices, counts, g_p, g_z, g_lb, normalize)
+
         def router_gradient(d_weights):
             """dS and the loss terms of the router -> the router's share of dx, and dW_r."""
+            if tail.dx_r is not None:   # already formed inside the launch of the experts' backward
+                got["dx_r"], got["dw_r"] = tail.dx_r, tail.dw_r
+                return tail.dx_r
             dx_r = torch.empty_like(x)
             dw_r = torch.empty_like(router_weight)
             ws_bytes = lib.mts_moe_head_bwd_workspace_bytes(T, H, E)
@@ -127,7 +133,8 @@ class _MoELayerFunction(torch.autograd.Function):
             return (dx if need_x else None), (got.get("dw_r") if need_wr else None), None, None, None, None
         wants_router = need_x or need_wr
         dx, dw1, dw2, ds = moe_backward(tensors, ctx.state, g_out.contiguous(), (need_x, need_w1, need_w2, wants_router),
-                                        x_addend=router_gradient if wants_router else None)
+                                        x_addend=router_gradient if wants_router else None,
+                                        router_tail=tail if wants_router else None)
         if wants_router and "dw_r" not in got:   # x needs no gradient: the combine, and with it the callback, was skipped
             router_gradient(ds)
         return dx, (got.get("dw_r") if need_wr else None), dw1, dw2, None, None

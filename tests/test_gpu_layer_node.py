@@ -143,6 +143,32 @@ def test_layer_node_equals_the_separate_operators_and_the_oracle(T, H, E, I, K, 
         assert_close_scaled(got, want, 1e-4 if dtype == torch.float32 else gate, name)
 
 
+@pytest.mark.parametrize("T,H,E,I,K,dtype,fp32_params", [
+    (24576, 768, 8, 1024, 2, torch.bfloat16, False), (700, 128, 5, 128, 2, torch.float16, False),
+    (1, 64, 4, 64, 2, torch.bfloat16, False), (2500, 1024, 8, 192, 3, torch.bfloat16, True)])
+def test_router_backward_inside_the_joint_launch_equals_its_own_launches(T, H, E, I, K, dtype, fp32_params, monkeypatch):
+    """With every gradient wanted and at most 8 experts the router's backward rides in the launch of
+    dW1 + dW2 + dX as trailing blocks that form dS from the partial row sums themselves: the same
+    arithmetic block for block, so every gradient equals the separate launches' bit for bit."""
+    print(f"router backward in the joint launch T={T} H={H} E={E} I={I} K={K} {dtype} fp32_params={fp32_params}", flush=True)
+    import importlib
+
+    from minitrain_amd import _lib
+
+    F = importlib.import_module("minitrain_amd.kernels.hip.fused_moe")
+    assert _lib.load().mts_moe_bwd_joint_router_supported(_lib.dtype_code(dtype), T, H, I, E) == 1
+    ops = hip_backend()
+    x, w_r, w1, w2, g = O.make_inputs(900 + T, T, H, E, I)
+    case = dict(x=x, w_r=w_r, w1=w1, w2=w2, g=g)
+    monkeypatch.setattr(F, "_JOINT", True)
+    monkeypatch.setattr(F, "_TAIL_IN_JOINT", True)
+    inside = _layer_grads(ops, case, K, True, dtype, fp32_params)[1]
+    monkeypatch.setattr(F, "_TAIL_IN_JOINT", False)
+    apart = _layer_grads(ops, case, K, True, dtype, fp32_params)[1]
+    for name, a, b in zip(("dx", "dW_r", "dW1", "dW2"), inside, apart):
+        assert a.dtype == b.dtype and torch.equal(a, b), name
+
+
 def test_layer_node_partial_gradients():
     """Only the router's loss terms reach the layer; and activations that need no gradient."""
     print("layer node partial gradients", flush=True)
