@@ -45,7 +45,7 @@ RIDGE_FLOP_PER_BYTE = PEAK_BF16_TFLOPS * 1e12 / (PEAK_HBM_GBS * 1e9)   # 312.5: 
 # line names the file that holds the runs' commands and tables.
 TRAFFIC_SOURCE = "profiles/moe_layer_24x1024_hbm_traffic.txt"
 MEASURED_TRAFFIC_BYTES = {
-    "fwd_gateup_swiglu": 650.2e6, "fwd_down": 223.9e6, "bwd_dy1": 534.8e6, "bwd_joint": 972.4e6,
+    "fwd_gateup_swiglu": 653.5e6, "fwd_down": 223.7e6, "bwd_dy1": 535.3e6, "bwd_joint": 1057.6e6,
     "combine": 114.6e6, "dx_combine": 152.4e6,
 }
 
@@ -188,13 +188,15 @@ def stage_breakdown(layer, steps):
          lambda: lib.mts_moe_combine(p(y), None, None, p(sr), T, K, H, B, p(out), st)),
         ("bwd_dy1", unit, rows_h + w2_b + 2 * rows_i + 2 * rows_i + TK * npart * 4 + TK * (4 + 4 + esz),
          lambda: lib.mts_moe_bwd_dy1(p(g), p(w2), 1, p(pre), p(r_wa), p(xg), p(ss), p(es), T, K, E, H, I, B, p(dpre), None, p(dsp), st)),
-        # dW1, dW2, dX and the dS reduction: one launch (plus the chunk sum), as the operator issues them
-        ("bwd_joint", 5 * unit, 2 * (2 * rows_i) + 2 * rows_h + rows_i + w1_b + rows_h + w1_b + w2_b + TK * npart * 4,
-         lambda: lib.mts_moe_bwd_joint(p(g), p(post), p(dpre), p(x), p(w1), p(xg), p(es), p(sr), p(dsp), T, K, E, H, I, B, B,
-                                       p(dxe), p(dw1), p(dw2), p(dwts), p(dws1), dws1.numel(), p(dws2), dws2.numel(), st)),
-        ("head_bwd", 4.0 * T * H * E, 2 * T * H * esz + T * E * 4 + T * K * (4 + 4 + esz) + 2 * E * H * 4,
-         lambda: lib.mts_moe_head_bwd(p(x), p(w_r), p(logits), p(r_w), p(r_i), p(cnt), None, p(dwts), p(gp), p(gz), p(gz), T, H, E, K,
-                                      1, B, p(dx_r), p(dw_r), p(bws), bws.numel(), st)),
+        # dW1, dW2, dX, the dS reduction and the router's backward (its blocks trail the dX tiles): one launch, plus
+        # one small launch for the chunk sum and the dW_r partial sum, as the layer node issues them
+        ("bwd_joint", 5 * unit + 4.0 * T * H * E,
+         2 * (2 * rows_i) + 2 * rows_h + rows_i + w1_b + rows_h + w1_b + w2_b + 2 * TK * npart * 4
+         + 2 * T * H * esz + T * E * 4 + T * K * (4 + 4) + 2 * E * H * 4,
+         lambda: lib.mts_moe_bwd_joint_router(p(g), p(post), p(dpre), p(x), p(w1), p(xg), p(es), p(sr), p(dsp), T, K, E, H, I, B, B,
+                                              p(dxe), p(dw1), p(dw2), p(dwts), p(dws1), dws1.numel(), p(dws2), dws2.numel(),
+                                              p(w_r), p(logits), p(r_w), p(r_i), p(cnt), p(gp), p(gz), p(gz), 1, p(dx_r), p(dw_r),
+                                              p(bws), bws.numel(), st)),
         ("dx_combine", 1.0 * TK * H, rows_h + 2 * T * H * esz + TK * 4,
          lambda: lib.mts_moe_combine(p(dxe), None, p(dx_r), p(sr), T, K, H, B, p(dx), st)),
     ]
