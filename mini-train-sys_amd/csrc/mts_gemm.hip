@@ -1655,14 +1655,17 @@ int xcd_ranges_choice(int64_t expert_weight_bytes) {
     return expert_weight_bytes <= kL2Bytes ? 1 : 0;
 }
 
-// MTS_NO_TILE_ORDER=1 switches the n-tile groups and the reversed walks of the range mapping off (comparisons)
-bool tile_order_enabled() {
-    static int on = -1;
-    if (on < 0) {
-        const char* s = getenv("MTS_NO_TILE_ORDER");
-        on = (s && atoi(s) != 0) ? 0 : 1;
+// MTS_NO_TILE_ORDER=1 switches the n-tile groups and the reversed walks of the range mapping off; MTS_TILE_ORDER
+// picks them one by one (bit 0: groups, 1: down reversed, 2: dY1 reversed, 3: dX reversed).  For comparisons.
+enum { ORDER_GROUPS = 1, ORDER_DOWN = 2, ORDER_DY1 = 4, ORDER_DX = 8, ORDER_ALL = 15 };
+int tile_order_mask() {
+    static int mask = -1;
+    if (mask < 0) {
+        const char* off = getenv("MTS_NO_TILE_ORDER");
+        const char* pick = getenv("MTS_TILE_ORDER");
+        mask = (off && atoi(off) != 0) ? 0 : (pick ? atoi(pick) & ORDER_ALL : ORDER_ALL);
     }
-    return on != 0;
+    return mask;
 }
 
 template <class T, int EPI>
@@ -1672,7 +1675,7 @@ dim3 rows_grid(RowsParams& p, int64_t TK) {
     const int64_t weight_bytes = (int64_t)p.b_rows * p.Kdim * (int64_t)sizeof(bf16_t);
     p.xcd_ranges = xcd_ranges_choice(weight_bytes);
     p.n_groups = 1;
-    if (p.xcd_ranges && tile_order_enabled())
+    if (p.xcd_ranges && (tile_order_mask() & ORDER_GROUPS))
         while (weight_bytes / p.n_groups > kL2Bytes / 2 && p.n_tiles % (2 * p.n_groups) == 0 && p.n_tiles / (2 * p.n_groups) >= 4)
             p.n_groups *= 2;
     const int64_t m_groups = (m_tiles<T>(TK, p.E) + kXcds - 1) / kXcds;
@@ -1686,7 +1689,8 @@ bool rows_kmajor_ok(int kind, int Kdim) { return tile_choice(kind) >= 1 && Kdim 
 // only the ring and specialised kernels read it that way
 template <int EPI>
 int launch_rows_any(int kind, RowsParams p, int64_t TK, hipStream_t s, bool b_kmajor = false) {
-    p.reverse = tile_order_enabled() && (kind == K_DOWN || kind == K_DX || kind == K_DY1);
+    p.reverse = ((kind == K_DOWN && (tile_order_mask() & ORDER_DOWN)) || (kind == K_DY1 && (tile_order_mask() & ORDER_DY1)) ||
+                 (kind == K_DX && (tile_order_mask() & ORDER_DX))) ? 1 : 0;
     int choice = tile_choice(kind);
     // gate/up: two co-resident ring blocks per CU win while the SwiGLU epilogue is a large part of a tile
     // (short reductions); long reductions are better off with specialised waves
@@ -1800,7 +1804,7 @@ int launch_bwd_joint(BwdJointParams q, int E, int grad_dtype, void* ws1, int64_t
     }
     q.n_dw1 = (int)dw_grid<T>(q.dw1, E, q.dw1.part ? 2 * E : E).x;
     q.n_dw2 = (int)dw_grid<T>(q.dw2, E, q.dw2.part ? 2 * E : E).x;
-    q.dx.reverse = tile_order_enabled();
+    q.dx.reverse = (tile_order_mask() & ORDER_DX) ? 1 : 0;
     q.n_dx = (int)rows_grid<WsLarge, EPI_PLAIN>(q.dx, q.dx.TK).x;
     const int64_t want = (q.entries + WsLarge::NT * 4 - 1) / (WsLarge::NT * 4);
     q.n_ds = (int)(want < 64 ? want : 64);
