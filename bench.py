@@ -45,7 +45,7 @@ RIDGE_FLOP_PER_BYTE = PEAK_BF16_TFLOPS * 1e12 / (PEAK_HBM_GBS * 1e9)   # 312.5: 
 # line names the file that holds the runs' commands and tables.
 TRAFFIC_SOURCE = "profiles/moe_layer_24x1024_hbm_traffic.txt"
 MEASURED_TRAFFIC_BYTES = {
-    "fwd_gateup_swiglu": 653.5e6, "fwd_down": 223.7e6, "bwd_dy1": 535.3e6, "bwd_joint": 1057.6e6,
+    "fwd_gateup_swiglu": 581.6e6, "fwd_down": 223.8e6, "bwd_dy1": 537.5e6, "bwd_joint": 1057.6e6,
     "combine": 114.6e6, "dx_combine": 152.4e6,
 }
 
