@@ -189,16 +189,15 @@ def stage_breakdown(layer, steps):
         ("bwd_dy1", unit, rows_h + w2_b + 2 * rows_i + 2 * rows_i + TK * npart * 4 + TK * (4 + 4 + esz),
          lambda: lib.mts_moe_bwd_dy1(p(g), p(w2), 1, p(pre), p(r_wa), p(xg), p(ss), p(es), T, K, E, H, I, B, p(dpre), None, p(dsp), st)),
         # dW1, dW2, dX, the dS reduction and the router's backward (its blocks trail the dX tiles): one launch, plus
-        # one small launch for the chunk sum and the dW_r partial sum, as the layer node issues them
-        ("bwd_joint", 5 * unit + 4.0 * T * H * E,
+        # one small launch for the chunk sum, the dW_r partial sum and the dX combine, as the layer node issues them
+        ("bwd_joint", 5 * unit + 4.0 * T * H * E + 1.0 * TK * H,
          2 * (2 * rows_i) + 2 * rows_h + rows_i + w1_b + rows_h + w1_b + w2_b + 2 * TK * npart * 4
-         + 2 * T * H * esz + T * E * 4 + T * K * (4 + 4) + 2 * E * H * 4,
+         + 2 * T * H * esz + T * E * 4 + T * K * (4 + 4) + 2 * E * H * 4
+         + rows_h + 2 * T * H * esz + TK * 4,
          lambda: lib.mts_moe_bwd_joint_router(p(g), p(post), p(dpre), p(x), p(w1), p(xg), p(es), p(sr), p(dsp), T, K, E, H, I, B, B,
                                               p(dxe), p(dw1), p(dw2), p(dwts), p(dws1), dws1.numel(), p(dws2), dws2.numel(),
-                                              p(w_r), p(logits), p(r_w), p(r_i), p(cnt), p(gp), p(gz), p(gz), 1, p(dx_r), p(dw_r),
+                                              p(w_r), p(logits), p(r_w), p(r_i), p(cnt), p(gp), p(gz), p(gz), 1, p(dx_r), p(dx), p(dw_r),
                                               p(bws), bws.numel(), st)),
-        ("dx_combine", 1.0 * TK * H, rows_h + 2 * T * H * esz + TK * 4,
-         lambda: lib.mts_moe_combine(p(dxe), None, p(dx_r), p(sr), T, K, H, B, p(dx), st)),
     ]
     # One stage is bracketed per pass over the whole sequence, so the other stages of that pass run
     # back to back as they do in the layer step and the chip is in the state it has there.
@@ -364,7 +363,7 @@ def main():
         g_ach = sum(r["flops"] for r in gemm_rows) / (g_ms * 1e-3) / 1e12
         result["gemm_roofline"] = {"bound": "mfma", "achieved": round(g_ach, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                                    "frac": round(g_ach / PEAK_BF16_TFLOPS, 4), "sum_ms": round(g_ms, 4)}
-        c_rows = [r for r in rows if r["stage"] in ("combine", "dx_combine")]
+        c_rows = [r for r in rows if r["stage"] == "combine"]
         c_ms = sum(r["avg_ms"] for r in c_rows)
         c_ach = sum(r["algorithmic_bytes"] for r in c_rows) / (c_ms * 1e-3) / 1e9
         result["combine_roofline"] = {"bound": "hbm", "achieved": round(c_ach, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",

@@ -318,7 +318,9 @@ int mts_moe_bwd_joint(const void* d_out, const void* weighted_act, const void* d
  * w_r [E,H] f32, logits [T,E] f32, weights [T,K] f32, indices [T,K], counts [E] (needed with
  * g_load_balance), g_prob_mean [E] / g_z_loss / g_load_balance (each may be NULL: zero);
  * outputs dx_router [T,H] in act_dtype and d_w_r [E,H] f32; router_workspace as for
- * mts_moe_head_bwd (mts_moe_head_bwd_workspace_bytes).  mts_moe_bwd_joint_router_supported()
+ * mts_moe_head_bwd (mts_moe_head_bwd_workspace_bytes).  dx (may be NULL): the layer's gradient
+ * of x [T,H], i.e. mts_moe_combine(dx_expanded, NULL, dx_router, s_reverse, ...) as part of
+ * the launch of partial sums (two routes per token) or as one more launch behind it.  mts_moe_bwd_joint_router_supported()
  * says whether the shapes allow it (those of mts_moe_bwd_joint, E <= 8, H a multiple of 4 whose
  * dW_r sums fit the block's LDS).                                                       */
 int mts_moe_bwd_joint_router_supported(int act_dtype, int64_t T, int H, int I, int E);
@@ -331,7 +333,7 @@ int mts_moe_bwd_joint_router(const void* d_out, const void* weighted_act, const 
                              void* workspace2, int64_t workspace2_bytes, const float* w_r,
                              const float* logits, const float* weights, const int32_t* indices,
                              const int32_t* counts, const float* g_prob_mean, const float* g_z_loss,
-                             const float* g_load_balance, int normalize, void* dx_router,
+                             const float* g_load_balance, int normalize, void* dx_router, void* dx,
                              float* d_w_r, void* router_workspace, int64_t router_workspace_bytes,
                              void* stream);
 

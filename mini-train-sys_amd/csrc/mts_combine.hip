@@ -2,76 +2,22 @@
 // expert rows (combine), the routing-weight gradient reduction and the staging
 // (cast / transpose) of expert weights to bf16.
 #include "mts_common.h"
+#include "mts_combine_block.h"
 
 namespace {
 
 constexpr int kThreads = 256;
 
 // ---- combine -------------------------------------------------------------
-// One thread produces 8 consecutive columns (16 bytes of bf16) of one token:
-// K row loads of 16 bytes each, fp32 accumulation, one rounding.  A thread works on
-// UN outputs at a time (token t, t + T/UN, ...) and issues all their index, weight
-// and row loads before the first use, to keep enough bytes in flight per CU.
-// A negative s_rev entry is a dropped route: it contributes nothing, whatever its weight.
-// ET is the 16-bit element type (bf16 or fp16).
-template <typename ET>
-struct Vec8;
-template <>
-struct Vec8<bf16_t> {
-    typedef bf16x8 type;
-};
-template <>
-struct Vec8<mts_f16_t> {
-    typedef mts_f16x8 type;
-};
+// the stand-alone launch of the block function in mts_combine_block.h
+using mts_cb::Vec8;
 
 template <typename ET, int KK, int UN>
 __global__ __launch_bounds__(kThreads) void combine_bf16_kernel(
     const ET* __restrict__ y, const ET* __restrict__ w, const ET* __restrict__ addend,
     const int32_t* __restrict__ s_rev, int64_t T, int K, int H, ET* __restrict__ out) {
-    typedef typename Vec8<ET>::type bf16x8;   // the build's 8-element vector
-    const int vec_per_row = H / 8;
-    const int64_t chunk = (T + UN - 1) / UN;           // tokens per unrolled slice
-    const int64_t total = chunk * (int64_t)vec_per_row;
-    for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total;
-         i += (int64_t)gridDim.x * kThreads) {
-        const int64_t t0 = i / vec_per_row;
-        const int c = (int)(i - t0 * vec_per_row);
-        bf16x8 v[UN][KK], add[UN];
-        float s[UN][KK];
-#pragma unroll
-        for (int u = 0; u < UN; ++u) {
-            const int64_t t = t0 + u * chunk;
-            add[u] = (addend && t < T) ? *reinterpret_cast<const bf16x8*>(addend + t * H + c * 8) : bf16x8{};
-#pragma unroll
-            for (int k = 0; k < KK; ++k) {
-                const bool in = t < T && k < K;
-                const int32_t r = in ? s_rev[t * K + k] : -1;
-                const bool ok = r >= 0;
-                const int64_t row = ok ? r : 0;
-                const float wt = in ? (w ? (float)w[t * K + k] : 1.0f) : 0.f;
-                s[u][k] = ok ? wt : 0.f;
-                v[u][k] = *reinterpret_cast<const bf16x8*>(y + row * H + c * 8);
-                if (!ok) v[u][k] = bf16x8{};   // row 0 may hold anything
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < UN; ++u) {
-            const int64_t t = t0 + u * chunk;
-            if (t >= T) continue;
-            float acc[8];
-#pragma unroll
-            for (int j = 0; j < 8; ++j) acc[j] = (float)add[u][j];
-#pragma unroll
-            for (int k = 0; k < KK; ++k)
-#pragma unroll
-                for (int j = 0; j < 8; ++j) acc[j] += s[u][k] * (float)v[u][k][j];
-            bf16x8 o;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) o[j] = (ET)acc[j];
-            *reinterpret_cast<bf16x8*>(out + t * H + c * 8) = o;
-        }
-    }
+    static_assert(kThreads == mts_cb::kCombineThreads, "one block shape");
+    mts_cb::combine_rows_block<ET, KK, UN>(y, w, addend, s_rev, T, K, H, out, blockIdx.x, gridDim.x);
 }
 
 // any K: the routes of a token are visited in a loop

@@ -74,7 +74,7 @@ int mts_moe_bwd_joint_router_f16(const void* d_out, const void* weighted_act, co
                                  int64_t workspace2_bytes, const float* w_r, const float* logits,
                                  const float* weights, const int32_t* indices, const int32_t* counts,
                                  const float* g_prob_mean, const float* g_z_loss, const float* g_load_balance,
-                                 int normalize, void* dx_router, float* d_w_r, void* router_workspace,
+                                 int normalize, void* dx_router, void* dx, float* d_w_r, void* router_workspace,
                                  int64_t router_workspace_bytes, void* stream);
 }
 

@@ -27,6 +27,7 @@
 //   C fragment:   element i (0..15) is row 8*(i/4) + 4*(l/32) + (i%4), column l % 32
 #include "mts_common.h"
 #include "mts_router_bwd_block.h"
+#include "mts_combine_block.h"
 
 #include <stdlib.h>
 
@@ -1118,17 +1119,38 @@ __global__ __launch_bounds__(256) void dw_chunk_sum_kernel(DwParams p) {
     dw_chunk_sum_expert<BM, BN, OutT>(p, blockIdx.y);
 }
 
-// the same for two GEMMs over the same experts in one launch: blockIdx.y < E is the first's expert; rows of
-// blocks past the second's experts sum the per-block partials of the router's weight gradient, where the
-// router's backward was part of the launch before (r_part != NULL)
+// What follows the joint backward launch of the layer node besides the chunk sums: the sum of the router's
+// dW_r partials and the dX combine (which adds the router's share of dx), as further rows of blocks.
+struct TailJobs {
+    const float* r_part;    // [r_blocks][r_EH] partial dW_r (NULL: none)
+    int r_blocks;
+    int64_t r_EH;
+    float* r_dw;
+    int r_rows;             // rows of blocks (blockIdx.y) that sum dW_r
+    const bf16_t* c_y;      // dx_expanded [T*2, H] (NULL: no combine)
+    const bf16_t* c_addend; // [T, H]
+    const int32_t* c_srev;
+    int64_t c_T;
+    int c_H;
+    bf16_t* c_out;          // dx [T, H]
+    int c_rows;             // rows of blocks that combine
+};
+
+// the same for two GEMMs over the same experts in one launch: blockIdx.y < E is the first's expert; the rows of
+// blocks past the second's experts take the jobs in `t`
 template <int BM, int BN, typename OutT>
-__global__ __launch_bounds__(256) void dw_chunk_sum_pair_kernel(DwParams a, DwParams b, const float* r_part, int r_blocks,
-                                                                int64_t r_EH, float* r_dw) {
-    static_assert(mts_rl::kReduceThreads == 256, "one block shape");
-    const int e = blockIdx.y;
-    if (e < a.E) dw_chunk_sum_expert<BM, BN, OutT>(a, e);
-    else if (e < a.E + b.E) dw_chunk_sum_expert<BM, BN, OutT>(b, e - a.E);
-    else mts_rl::router_dw_reduce_block(r_part, r_blocks, r_EH, r_dw, (int64_t)(e - a.E - b.E) * gridDim.x + blockIdx.x);
+__global__ __launch_bounds__(256) void dw_chunk_sum_pair_kernel(DwParams a, DwParams b, TailJobs t) {
+    static_assert(mts_rl::kReduceThreads == 256 && mts_cb::kCombineThreads == 256, "one block shape");
+    int e = blockIdx.y;
+    if (e < a.E) return dw_chunk_sum_expert<BM, BN, OutT>(a, e);
+    e -= a.E;
+    if (e < b.E) return dw_chunk_sum_expert<BM, BN, OutT>(b, e);
+    e -= b.E;
+    if (e < t.r_rows) return mts_rl::router_dw_reduce_block(t.r_part, t.r_blocks, t.r_EH, t.r_dw, (int64_t)e * gridDim.x + blockIdx.x);
+    e -= t.r_rows;
+    // two routes per token: the combine of the layer's dX (plain sum of the two expert rows plus the addend)
+    mts_cb::combine_rows_block<bf16_t, 2, 2>(t.c_y, (const bf16_t*)nullptr, t.c_addend, t.c_srev, t.c_T, 2, t.c_H, t.c_out,
+                                             (int64_t)e * gridDim.x + blockIdx.x, (int64_t)t.c_rows * gridDim.x);
 }
 
 // Stages a [64 k][64 m] block per wave-item: lane = (kgrp = lane%8, mc = lane/8) loads
@@ -1544,6 +1566,8 @@ struct BwdJointParams {
     bf16_t* r_dx;                  // the router's share of dx [T, H]
     float* r_part;                 // [router_row_blocks][E][H] partial dW_r
     float* r_dw;                   // dW_r [E][H]: summed from r_part by the launch that follows (host side only)
+    bf16_t* c_out;                 // dx [T][H]: the dX combine in the launch that follows (host side only; NULL: not asked for)
+    int c_K;
     mts_rl::RouterGradIn rg;
 };
 
@@ -1788,6 +1812,10 @@ bool bwd_joint_ok(int H, int I) {
            H % 8 == 0;
 }
 
+// the dX combine rides in the launch of the partial sums when the layer has two routes per token (the block
+// function is compiled for that) and whole 16-byte chunks per row
+bool combine_in_tail(const BwdJointParams& q) { return q.c_out && q.n_router && q.c_K == 2 && q.rH % 8 == 0; }
+
 int launch_bwd_joint(BwdJointParams q, int E, int grad_dtype, void* ws1, int64_t ws1_bytes, void* ws2, int64_t ws2_bytes,
                      hipStream_t s) {
     typedef DwWsLarge T;
@@ -1816,22 +1844,37 @@ int launch_bwd_joint(BwdJointParams q, int E, int grad_dtype, void* ws1, int64_t
         const int t = q.dw1.tiles_per_expert > q.dw2.tiles_per_expert ? q.dw1.tiles_per_expert : q.dw2.tiles_per_expert;
         const int64_t want = ((int64_t)t * (T::BM * T::BN / 4) + 255) / 256;
         const unsigned gx = (unsigned)(want < 256 ? want : 256);
-        // the sum of the router's dW_r partials rides along as extra rows of blocks
-        const int64_t r_EH = (int64_t)q.rE * q.rH;
-        const int64_t r_jobs = q.n_router ? (r_EH + mts_rl::kReduceCols - 1) / mts_rl::kReduceCols : 0;
-        const dim3 sum_grid(gx, (unsigned)(2 * E + (r_jobs + gx - 1) / gx));
-        if (grad_dtype == MTS_GEMM_DTYPE)
-            dw_chunk_sum_pair_kernel<T::BM, T::BN, bf16_t><<<sum_grid, 256, 0, s>>>(q.dw1, q.dw2, q.r_part, q.router_row_blocks, r_EH, q.r_dw);
-        else
-            dw_chunk_sum_pair_kernel<T::BM, T::BN, float><<<sum_grid, 256, 0, s>>>(q.dw1, q.dw2, q.r_part, q.router_row_blocks, r_EH, q.r_dw);
+        // the sum of the router's dW_r partials and the dX combine ride along as extra rows of blocks
+        TailJobs jobs = {};
+        if (q.n_router) {
+            jobs.r_part = q.r_part; jobs.r_blocks = q.router_row_blocks; jobs.r_EH = (int64_t)q.rE * q.rH; jobs.r_dw = q.r_dw;
+            jobs.r_rows = (int)(((jobs.r_EH + mts_rl::kReduceCols - 1) / mts_rl::kReduceCols + gx - 1) / gx);
+        }
+        const bool combined = combine_in_tail(q);
+        if (combined) {
+            jobs.c_y = q.dx.C; jobs.c_addend = q.r_dx; jobs.c_srev = q.s_reverse; jobs.c_T = q.rT; jobs.c_H = q.rH;
+            jobs.c_out = q.c_out;
+            const int64_t items = ((q.rT + 1) / 2) * (int64_t)(q.rH / 8);   // 16 bytes of output for two tokens each
+            const int64_t rows = ((items + 255) / 256 + gx - 1) / gx;
+            jobs.c_rows = (int)(rows < 32 ? rows : 32);
+        }
+        const dim3 sum_grid(gx, (unsigned)(2 * E + jobs.r_rows + jobs.c_rows));
+        if (grad_dtype == MTS_GEMM_DTYPE) dw_chunk_sum_pair_kernel<T::BM, T::BN, bf16_t><<<sum_grid, 256, 0, s>>>(q.dw1, q.dw2, jobs);
+        else dw_chunk_sum_pair_kernel<T::BM, T::BN, float><<<sum_grid, 256, 0, s>>>(q.dw1, q.dw2, jobs);
+        MTS_CHECK_LAUNCH();
+        if (combined) return MTS_OK;
     } else {   // one of the two, or more experts than a grid holds in y twice over
         if (q.dw1.part) launch_dw_chunk_sum(q.dw1, E, grad_dtype, s);
         if (q.dw2.part) launch_dw_chunk_sum(q.dw2, E, grad_dtype, s);
         MTS_CHECK_LAUNCH();
-        if (q.n_router) return mts_launch_router_dw_reduce(q.r_part, q.router_row_blocks, (int64_t)q.rE * q.rH, q.r_dw, s);
-        return MTS_OK;
+        if (q.n_router) {
+            const int rc = mts_launch_router_dw_reduce(q.r_part, q.router_row_blocks, (int64_t)q.rE * q.rH, q.r_dw, s);
+            if (rc) return rc;
+        }
     }
-    MTS_CHECK_LAUNCH();
+    // the dX combine, where it was asked for and did not ride in the launch above
+    if (q.c_out)
+        return mts_moe_combine(q.dx.C, nullptr, q.r_dx, q.s_reverse, q.rT, q.c_K, q.rH, MTS_GEMM_DTYPE, q.c_out, (void*)s);
     return MTS_OK;
 }
 
@@ -2101,7 +2144,7 @@ extern "C" int MTS_GEMM_ENTRY(mts_moe_bwd_joint_router)(
     int K, int E, int H, int I, int act_dtype, int grad_dtype, void* dx_expanded, void* d_w1, void* d_w2, void* d_weights,
     void* workspace1, int64_t workspace1_bytes, void* workspace2, int64_t workspace2_bytes, const float* w_r,
     const float* logits, const float* weights, const int32_t* indices, const int32_t* counts, const float* g_prob_mean,
-    const float* g_z_loss, const float* g_load_balance, int normalize, void* dx_router, float* d_w_r,
+    const float* g_z_loss, const float* g_load_balance, int normalize, void* dx_router, void* dx, float* d_w_r,
     void* router_workspace, int64_t router_workspace_bytes, void* stream) {
 #ifndef MTS_GEMM_F16
     if (act_dtype == MTS_F16)
@@ -2109,7 +2152,7 @@ extern "C" int MTS_GEMM_ENTRY(mts_moe_bwd_joint_router)(
                                             ds_partial, T, K, E, H, I, act_dtype, grad_dtype, dx_expanded, d_w1, d_w2,
                                             d_weights, workspace1, workspace1_bytes, workspace2, workspace2_bytes, w_r, logits,
                                             weights, indices, counts, g_prob_mean, g_z_loss, g_load_balance, normalize,
-                                            dx_router, d_w_r, router_workspace, router_workspace_bytes, stream);
+                                            dx_router, dx, d_w_r, router_workspace, router_workspace_bytes, stream);
 #endif
     BwdJointParams q = {};
     int rc = fill_bwd_joint(q, d_out, weighted_act, d_pre_act, x, w1, x_gather, expert_start, s_reverse, ds_partial, T, K, E,
@@ -2124,7 +2167,7 @@ extern "C" int MTS_GEMM_ENTRY(mts_moe_bwd_joint_router)(
     mts_router_bwd_shape(T, H, E, &g);
     if (!joint_router_ok(H, E, g)) return MTS_ERR_SHAPE;
     if (router_workspace_bytes < (int64_t)g.row_blocks * E * H * (int64_t)sizeof(float)) return MTS_ERR_WORKSPACE;
-    if (!mts_aligned16(router_workspace) || !mts_aligned16(d_w_r) || !mts_aligned16(dx_router) ||
+    if (!mts_aligned16(router_workspace) || !mts_aligned16(d_w_r) || !mts_aligned16(dx_router) || !mts_aligned16(dx) ||
         (E == 8 && !mts_aligned16(logits)))
         return MTS_ERR_ALIGN;
     q.n_router = g.row_blocks * g.ranges;
@@ -2133,6 +2176,7 @@ extern "C" int MTS_GEMM_ENTRY(mts_moe_bwd_joint_router)(
     q.r_rows_per_block = g.rows_per_block; q.r_groups = g.groups; q.r_cols_per_block = g.cols_per_block;
     q.r_col_threads = g.col_threads;
     q.r_dx = (bf16_t*)dx_router; q.r_part = (float*)router_workspace; q.r_dw = d_w_r;
+    q.c_out = (bf16_t*)dx; q.c_K = K;
     q.rg = {logits, weights, indices, counts, nullptr, nullptr, g_prob_mean, g_z_loss, g_load_balance, act_dtype, K, normalize,
             ds_partial, s_reverse, q.np};
     return launch_bwd_joint(q, E, grad_dtype, workspace1, workspace1_bytes, workspace2, workspace2_bytes, (hipStream_t)stream);

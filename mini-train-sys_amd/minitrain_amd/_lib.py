@@ -62,7 +62,7 @@ SIGNATURES = {
     "mts_moe_bwd_joint": (_i, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _i, _p, _p, _p, _p, _p, _l, _p, _l, _p]),
     "mts_moe_bwd_joint_router_supported": (_i, [_i, _l, _i, _i, _i]),
     "mts_moe_bwd_joint_router": (_i, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _i, _p, _p, _p, _p, _p, _l, _p, _l]
-                                 + [_p] * 8 + [_i, _p, _p, _p, _l, _p]),
+                                 + [_p] * 8 + [_i, _p, _p, _p, _p, _l, _p]),
 }
 
 _lib = None

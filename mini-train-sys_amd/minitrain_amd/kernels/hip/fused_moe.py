@@ -170,6 +170,8 @@ _OVERLAP = os.environ.get("MTS_NO_OVERLAP", "0") != "1"
 _JOINT = os.environ.get("MTS_NO_JOINT_BWD", "0") != "1"
 # MTS_NO_TAIL_IN_JOINT=1 keeps the router's backward of the layer node in launches of its own
 _TAIL_IN_JOINT = os.environ.get("MTS_NO_TAIL_IN_JOINT", "0") != "1"
+# MTS_NO_COMBINE_IN_TAIL=1 keeps the dX combine behind that launch in a launch of its own
+_COMBINE_IN_TAIL = os.environ.get("MTS_NO_COMBINE_IN_TAIL", "0") != "1"
 # MTS_WEIGHTED_POST=0: the forward pass writes the unweighted activation and dY1 writes s * a again (tuning runs only)
 _WEIGHTED_POST = os.environ.get("MTS_WEIGHTED_POST", "1") != "0"
 _SIDE_STREAMS: dict = {}
@@ -401,20 +403,25 @@ def moe_backward(tensors, state, dO, needs, x_addend=None, router_tail=None):
         if rt is not None and _TAIL_IN_JOINT and lib.mts_moe_bwd_joint_router_supported(act, T, H, I, E):
             # the router's backward as trailing blocks of the same launch: it needs nothing the launch writes
             dx_r, dw_r = torch.empty_like(x), torch.empty_like(rt.router_weight)
+            dx = torch.empty_like(x) if _COMBINE_IN_TAIL else None
             rws_bytes = lib.mts_moe_head_bwd_workspace_bytes(T, H, E)
             rws = torch.empty(rws_bytes, dtype=torch.uint8, device=dev)
             _lib.check(
                 lib.mts_moe_bwd_joint_router(
                     *joint_args, rt.router_weight.data_ptr(), rt.logits.data_ptr(), rt.weights.data_ptr(),
                     rt.indices.data_ptr(), _lib.ptr(rt.counts), _lib.ptr(rt.g_prob_mean), _lib.ptr(rt.g_z_loss),
-                    _lib.ptr(rt.g_load_balance), int(rt.normalize), dx_r.data_ptr(), dw_r.data_ptr(), rws.data_ptr(),
-                    rws_bytes, stream,
+                    _lib.ptr(rt.g_load_balance), int(rt.normalize), dx_r.data_ptr(), _lib.ptr(dx), dw_r.data_ptr(),
+                    rws.data_ptr(), rws_bytes, stream,
                 ),
                 "mts_moe_bwd_joint_router",
             )
             rt.dx_r, rt.dw_r = dx_r, dw_r
-        else:
-            _lib.check(lib.mts_moe_bwd_joint(*joint_args, stream), "mts_moe_bwd_joint")
+            if dx is None:
+                return combine_dx(dx_expanded, d_weights), dgate_up_proj, ddown_proj, d_weights
+            if x_addend is not None:
+                x_addend(d_weights)   # lets the caller pick the router's outputs up; the combine has been launched
+            return dx, dgate_up_proj, ddown_proj, d_weights
+        _lib.check(lib.mts_moe_bwd_joint(*joint_args, stream), "mts_moe_bwd_joint")
         return combine_dx(dx_expanded, d_weights), dgate_up_proj, ddown_proj, d_weights
 
     if need_w1 and need_w2:

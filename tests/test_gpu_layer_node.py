@@ -144,7 +144,7 @@ def test_layer_node_equals_the_separate_operators_and_the_oracle(T, H, E, I, K, 
 
 
 @pytest.mark.parametrize("T,H,E,I,K,dtype,fp32_params", [
-    (24576, 768, 8, 1024, 2, torch.bfloat16, False), (700, 128, 5, 128, 2, torch.float16, False),
+    (24576, 768, 8, 1024, 2, torch.bfloat16, False), (701, 128, 5, 128, 2, torch.float16, False),
     (1, 64, 4, 64, 2, torch.bfloat16, False), (2500, 1024, 8, 192, 3, torch.bfloat16, True)])
 def test_router_backward_inside_the_joint_launch_equals_its_own_launches(T, H, E, I, K, dtype, fp32_params, monkeypatch):
     """With every gradient wanted and at most 8 experts the router's backward rides in the launch of
@@ -162,11 +162,15 @@ def test_router_backward_inside_the_joint_launch_equals_its_own_launches(T, H, E
     case = dict(x=x, w_r=w_r, w1=w1, w2=w2, g=g)
     monkeypatch.setattr(F, "_JOINT", True)
     monkeypatch.setattr(F, "_TAIL_IN_JOINT", True)
-    inside = _layer_grads(ops, case, K, True, dtype, fp32_params)[1]
+    monkeypatch.setattr(F, "_COMBINE_IN_TAIL", True)   # the dX combine too (inside the library: with the partial sums
+    inside = _layer_grads(ops, case, K, True, dtype, fp32_params)[1]   # for two routes per token, else one more launch)
+    monkeypatch.setattr(F, "_COMBINE_IN_TAIL", False)
+    own_combine = _layer_grads(ops, case, K, True, dtype, fp32_params)[1]
     monkeypatch.setattr(F, "_TAIL_IN_JOINT", False)
     apart = _layer_grads(ops, case, K, True, dtype, fp32_params)[1]
-    for name, a, b in zip(("dx", "dW_r", "dW1", "dW2"), inside, apart):
-        assert a.dtype == b.dtype and torch.equal(a, b), name
+    for other in (own_combine, apart):
+        for name, a, b in zip(("dx", "dW_r", "dW1", "dW2"), inside, other):
+            assert a.dtype == b.dtype and torch.equal(a, b), name
 
 
 def test_layer_node_partial_gradients():
