@@ -1626,10 +1626,13 @@ const char* const kKindEnv[K_COUNT] = {"MTS_TILE_GATEUP", "MTS_TILE_DOWN", "MTS_
                                        "MTS_TILE_DX",     "MTS_TILE_DW2",  "MTS_TILE_DW1"};
 // rows_gemm: 0 StagedSmall, 1 RingTwoPerCu, 2 WsLarge, 3 RingThreePerCu (dY1 without the weighted_act output
 // only);  dw_gemm: 0 StagedSmall, 2 DwWsLarge.
-// Defaults are the fastest measured on the 24576-token, 768/1024, 8-expert layer: the two GEMMs with
-// the heavy epilogues (gate/up + SwiGLU, dO*W2 + SwiGLU backward) gain more from co-resident
-// 4-wave blocks, two per CU for gate/up and three for dY1, the others from specialised waves.
-const int kDefaultTile[K_COUNT] = {1, 2, 3, 2, 2, 2};
+// Defaults are the choices with the shortest LAYER STEP measured on the 24576-token, 768/1024, 8-expert layer.
+// The chip runs this step against its power limit, so a kernel's own duration is not the whole story: what
+// it leaves of the power budget shows in the kernels around it.  Gate/up on 256x256 tiles with specialised
+// waves moves a third less data from L2 to LDS per FLOP than on two co-resident 256x128 ring blocks and makes
+// the step 2-3.5 % shorter, although the kernel alone is at best as fast; dO*W2 with the SwiGLU backward in
+// its epilogue is better off with three co-resident 4-wave blocks per CU.
+const int kDefaultTile[K_COUNT] = {2, 2, 3, 2, 2, 2};
 
 bool tile_forced(int kind) { return getenv(kKindEnv[kind]) != nullptr; }
 
@@ -1716,9 +1719,6 @@ int launch_rows_any(int kind, RowsParams p, int64_t TK, hipStream_t s, bool b_km
     p.reverse = ((kind == K_DOWN && (tile_order_mask() & ORDER_DOWN)) || (kind == K_DY1 && (tile_order_mask() & ORDER_DY1)) ||
                  (kind == K_DX && (tile_order_mask() & ORDER_DX))) ? 1 : 0;
     int choice = tile_choice(kind);
-    // gate/up: two co-resident ring blocks per CU win while the SwiGLU epilogue is a large part of a tile
-    // (short reductions); long reductions are better off with specialised waves
-    if (kind == K_GATEUP && !tile_forced(kind) && p.Kdim > 1024) choice = 2;
     // three blocks per CU hold two stages each: for short reductions, and for the epilogue that fits beside them
     if (choice == 3 && (EPI != EPI_DY1N || !b_kmajor || (!tile_forced(kind) && p.Kdim > 1024))) choice = 1;
     // the ring kernels need whole k-tiles; other shapes use the staged kernel
