@@ -233,11 +233,12 @@ def stage_breakdown(layer, steps):
     return rows
 
 
-def mfma_sustained(blocks=512, rounds=2500, repeats=3):
-    """What the matrix pipes sustain on registers alone (no LDS, no memory): the library's probe kernel,
-    timed with events on the launching stream.  Operands that toggle from instruction to instruction cost
-    clock on this power-limited chip, so the rate on pseudo-random registers is the practical ceiling the
-    GEMM figures are read against; the nominal peak stays the denominator of every `frac`."""
+def mfma_sustained(blocks=512, rounds=1000, launches=40, lead=10):
+    """What the matrix pipes sustain on registers alone (no LDS, no memory): the library's probe kernel
+    (two blocks of four waves per CU), launched back to back for ~100 ms and timed with events on the
+    launching stream over the launches behind the first `lead` ones, so that the clocks are where the
+    power governor leaves them under continuous load.  The rate on pseudo-random registers is the ceiling
+    the GEMM figures are read against; the nominal peak stays the denominator of every `frac`."""
     import ctypes
 
     from minitrain_amd import _lib
@@ -248,21 +249,19 @@ def mfma_sustained(blocks=512, rounds=2500, repeats=3):
     flops = ctypes.c_double(0.0)
     out = {}
     for name, random_operands in (("random_operands", 1), ("constant_operands", 0)):
-        best = None
-        for it in range(1 + repeats):
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for it in range(launches):
+            if it == lead:
+                e0.record()
             rc = lib.mts_probe_mfma_rate(random_operands, blocks, rounds, sink.data_ptr(), sink.numel(), ctypes.addressof(flops), st)
-            e1.record()
             if rc != 0:
                 raise RuntimeError(f"mts_probe_mfma_rate returned {rc}")
-            torch.cuda.synchronize()
-            if it:
-                ms = e0.elapsed_time(e1)
-                best = ms if best is None else min(best, ms)
-        out[name + "_tflops"] = round(flops.value / (best * 1e-3) / 1e12, 1)
+        e1.record()
+        torch.cuda.synchronize()
+        out[name + "_tflops"] = round(flops.value * (launches - lead) / (e0.elapsed_time(e1) * 1e-3) / 1e12, 1)
     out.update(peak=PEAK_BF16_TFLOPS, unit="TFLOP/s", frac_of_peak=round(out["random_operands_tflops"] / PEAK_BF16_TFLOPS, 4),
-               kernel="register-only bf16 32x32x16 MFMA loop, 512 blocks of 4 waves, best of 3 launches of ~8 ms")
+               kernel=f"register-only bf16 32x32x16 MFMA loop, {blocks} blocks of 4 waves (two per CU), {launches} launches back to back, "
+                      f"the last {launches - lead} timed")
     return out
 
 

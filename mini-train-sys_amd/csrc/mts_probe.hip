@@ -1,9 +1,9 @@
 // Measurement aid, not part of the operator boundary: what the matrix pipes of the GPU sustain with
 // nothing else going on.  A register-only loop of bf16 32x32x16 MFMAs (no LDS, no memory traffic), two
 // 256-thread blocks per CU, eight independent accumulators per wave.  With `random_operands` the A and B
-// registers are eight pseudo-random sets rotated from instruction to instruction, otherwise constants:
-// under MFMA load the chip is power-limited and operands that toggle cost clock, so the two rates differ,
-// and the expert-GEMM figures of the benchmark are printed next to the first.
+// registers hold pseudo-random values, otherwise constants: operands that toggle cost power, and under
+// continuous MFMA load the power governor sets the clock, so the two rates differ; the expert-GEMM figures
+// of the benchmark are printed next to the first.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -22,16 +22,19 @@ __device__ __forceinline__ uint32_t lcg(uint32_t& s) {
     return s;
 }
 
-template <bool RANDOM>
-__global__ __launch_bounds__(kThreads) void mfma_rate_kernel(float* sink, int rounds) {
+// Two blocks per CU (two waves per SIMD), so that the matrix pipe never waits for one wave's issue.  The
+// operands are selected at run time, which keeps both variants in vector registers (constants known at
+// compile time would be held in scalar registers and spill from there).  Consecutive MFMAs use the
+// operands the way a 4x2 register tile of a GEMM does: the A fragment stays for two instructions.
+__global__ __launch_bounds__(kThreads, 2) void mfma_rate_kernel(float* sink, int rounds, int random) {
     bf16x8 a[kSets], b[kSets];
     uint32_t s = threadIdx.x * 2654435761u + blockIdx.x * 97u + 12345u;
     for (int n = 0; n < kSets; ++n)
         for (int i = 0; i < 8; ++i) {
-            const float va = RANDOM ? ((int)(lcg(s) >> 8) % 2001 - 1000) * 0.001f : 0.5f;
-            const float vb = RANDOM ? ((int)(lcg(s) >> 8) % 2001 - 1000) * 0.00002f : 0.01f;
-            a[n][i] = (__bf16)va;
-            b[n][i] = (__bf16)vb;
+            const float ra = ((int)(lcg(s) >> 8) % 2001 - 1000) * 0.001f;
+            const float rb = ((int)(lcg(s) >> 8) % 2001 - 1000) * 0.00002f;
+            a[n][i] = (__bf16)(random ? ra : 0.5f);
+            b[n][i] = (__bf16)(random ? rb : 0.01f);
         }
     f32x16 acc[kSets];
     for (int j = 0; j < kSets; ++j)
@@ -41,7 +44,8 @@ __global__ __launch_bounds__(kThreads) void mfma_rate_kernel(float* sink, int ro
         for (int r = 0; r < kSets; ++r)
 #pragma unroll
             for (int j = 0; j < kSets; ++j)
-                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[(j + 3 * r) & 7], b[(j + r) & 7], acc[j], 0, 0, 0);
+                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[(j / 2 + 4 * (r & 1)) & 7], b[(j % 2 + 2 * (r & 3)) & 7],
+                                                                 acc[j], 0, 0, 0);
     }
     float total = 0.f;
     for (int j = 0; j < kSets; ++j)
@@ -59,10 +63,7 @@ extern "C" int mts_probe_mfma_rate(int random_operands, int blocks, int rounds, 
     if (blocks <= 0 || blocks > 65535 || rounds <= 0 || rounds > (1 << 20)) return MTS_ERR_SHAPE;
     if (sink_bytes < mts_probe_mfma_sink_bytes(blocks)) return MTS_ERR_WORKSPACE;
     if (flops) *flops = (double)blocks * (kThreads / 64) * rounds * (kSets * kSets) * (2.0 * 32 * 32 * 16);
-    if (random_operands)
-        mfma_rate_kernel<true><<<blocks, kThreads, 0, (hipStream_t)stream>>>((float*)sink, rounds);
-    else
-        mfma_rate_kernel<false><<<blocks, kThreads, 0, (hipStream_t)stream>>>((float*)sink, rounds);
+    mfma_rate_kernel<<<blocks, kThreads, 0, (hipStream_t)stream>>>((float*)sink, rounds, random_operands != 0);
     MTS_CHECK_LAUNCH();
     return MTS_OK;
 }

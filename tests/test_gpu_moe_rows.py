@@ -62,7 +62,7 @@ def test_decoder_step_at_the_real_size():
 
 def test_mfma_rate_probe_reports_a_plausible_rate():
     """The register-only MFMA loop the benchmark line quotes as `mfma_sustained`: every thread's sum is
-    finite, the reported FLOPs match the launch, and the rate lies between a tenth of the nominal bf16 peak
+    finite, the reported FLOPs match the launch, and the rate lies between a fifth of the nominal bf16 peak
     and the peak itself (2.5 PFLOP/s); constant operands are not slower than toggling ones by more than noise."""
     print("mfma rate probe", flush=True)
     import sys
@@ -71,10 +71,10 @@ def test_mfma_rate_probe_reports_a_plausible_rate():
     sys.path.insert(0, str(Path(__file__).resolve().parents[1]))
     import bench
 
-    rec = bench.mfma_sustained(blocks=512, rounds=500, repeats=2)
+    rec = bench.mfma_sustained(blocks=512, rounds=200, launches=12, lead=4)
     assert rec["peak"] == 2500.0 and rec["unit"] == "TFLOP/s"
     for key in ("random_operands_tflops", "constant_operands_tflops"):
-        assert 250.0 < rec[key] <= 2500.0, rec
+        assert 500.0 < rec[key] <= 2500.0, rec
     assert rec["constant_operands_tflops"] >= 0.9 * rec["random_operands_tflops"], rec
     from minitrain_amd import _lib
 
