@@ -45,8 +45,9 @@ RIDGE_FLOP_PER_BYTE = PEAK_BF16_TFLOPS * 1e12 / (PEAK_HBM_GBS * 1e9)   # 312.5: 
 # line names the file that holds the runs' commands and tables.
 TRAFFIC_SOURCE = "profiles/moe_layer_24x1024_hbm_traffic.txt"
 MEASURED_TRAFFIC_BYTES = {
-    "fwd_gateup_swiglu": 581.6e6, "fwd_down": 223.8e6, "bwd_dy1": 537.5e6, "bwd_joint": 1057.6e6,
-    "combine": 114.6e6, "dx_combine": 152.4e6,
+    "fwd_gateup_swiglu": 551.9e6, "fwd_down": 223.8e6, "bwd_dy1": 537.6e6,
+    "bwd_joint": 1221.7e6,   # the joint launch (1056.5) and the launch of partial sums with the dX combine behind it (165.2)
+    "combine": 114.6e6,
 }
 
 WORKLOAD = dict(name="moe_layer_24x1024_d768_e8_top2_ff1024_bf16", seed=1, T=24576, H=768, E=8, K=2, I=1024)
