@@ -296,16 +296,20 @@ struct FragPipe {
     // MFMAs of k-step `ks` (weight fragment first); behind them, the fragments of k-step `nks`
     // of the stage at `next` are read: the weight fragments up front into the other buffer, each
     // activation fragment as soon as its MFMAs are issued
+    // READ = false: the MFMAs only (the last k-step of a buffer whose successor is not visible yet)
+    template <bool READ = true>
     __device__ __forceinline__ void step(int ks, f32x16 (&acc)[T::MF][T::NF], const bf16_t* next, int nks) {
         const int coff = chunk_off(nks), buf = ks & 1;
+        if constexpr (READ) {
 #pragma unroll
-        for (int nf = 0; nf < T::NF; ++nf) b[buf ^ 1][nf] = read_b(next, nf, nks, coff);
+            for (int nf = 0; nf < T::NF; ++nf) b[buf ^ 1][nf] = read_b(next, nf, nks, coff);
+        }
 #pragma unroll
         for (int mf = 0; mf < T::MF; ++mf) {
 #pragma unroll
             for (int nf = 0; nf < T::NF; ++nf)
                 acc[mf][nf] = MTS_MFMA_32x32x16(b[buf][nf], a[mf], acc[mf][nf], 0, 0, 0);
-            a[mf] = *reinterpret_cast<const bf16x8*>(next + a_off + mf * 32 * ROWLEN + coff);
+            if constexpr (READ) a[mf] = *reinterpret_cast<const bf16x8*>(next + a_off + mf * 32 * ROWLEN + coff);
         }
     }
 };
@@ -866,7 +870,7 @@ struct WsTile {
     static_assert(BKS == 32 || BKS == 64, "LDS rows are 64 or 128 bytes");
     static_assert(WM % 32 == 0 && WN % 64 == 0, "wave tile must hold whole 32x32 fragments");
     static_assert(A_INSTR * RPI * PRODUCERS == BM && B_INSTR * RPI * PRODUCERS == BN, "loader split");
-    static_assert(STAGES == 4 && (A_INSTR + B_INSTR) * 2 <= 63, "the producer waits are written for a 4-stage ring");
+    static_assert((STAGES == 4 || STAGES == 2) && (A_INSTR + B_INSTR) * 2 <= 63, "the producer waits are written for a 4-stage ring and for two buffers");
     static_assert(LDS_ELEMS * 2 <= 160 * 1024, "LDS capacity");
 };
 
@@ -940,6 +944,18 @@ __device__ __forceinline__ void rows_gemm_ws_block(const RowsParams& p, bf16_t* 
             for (int j = 0; j < T::B_INSTR; ++j)
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_b, MTS_LDS_PTR(sb + j * 512), 16, (int)voff_b[j], soff_b, 0, 0);
         };
+        if constexpr (S == 2) {
+            // Two buffers of 64-wide k-tiles (a row contributes a whole 128-byte line per load): barrier kt says
+            // that tile kt has landed and that tile kt-1 has been consumed, whose buffer then takes tile kt+1.
+            issue(0, 0);
+            for (int kt = 0; kt < nk; ++kt) {
+                wait_vmcnt<0>();
+                __builtin_amdgcn_s_barrier();
+                if (kt + 1 < nk) issue((kt + 1) & 1, kt + 1);
+            }
+            __builtin_amdgcn_s_barrier();       // matches the consumers' barrier behind the last tile
+            return;
+        }
         // Barrier kt tells the consumers that tiles kt and kt+1 have landed (they read the first
         // fragments of tile kt+1 behind the last MFMAs of tile kt) and tells the producers that
         // every consumer is done with tile kt-1, whose stage then takes tile kt-1+S.
@@ -967,6 +983,19 @@ __device__ __forceinline__ void rows_gemm_ws_block(const RowsParams& p, bf16_t* 
     FragPipe<T, SWIGLU, T::BKS, BKM> pipe;
     pipe.init(wm, wn);
     constexpr int KSTEPS = T::BKS / 16;
+    if constexpr (S == 2) {
+        for (int kt = 0; kt < nk; ++kt) {
+            __builtin_amdgcn_s_barrier();   // tile kt is visible
+            const bf16_t* cur = smem + (kt & 1) * T::STAGE;
+            pipe.prime(cur);
+#pragma unroll
+            for (int ks = 0; ks < KSTEPS - 1; ++ks) pipe.step(ks, acc, cur, ks + 1);
+            pipe.template step<false>(KSTEPS - 1, acc, cur, 0);
+        }
+        __builtin_amdgcn_s_barrier();       // every wave is done with the buffers before the epilogue reuses them
+        rows_epilogue<T, EPI>(p, acc, smem, row0, rend, n0, wm, wn);
+        return;
+    }
     __builtin_amdgcn_s_barrier();   // tiles 0 and 1 are visible
     pipe.prime(smem);
     int stage = 0;
@@ -1532,6 +1561,7 @@ typedef RingTile<256, 128, 2, 2, 32, 3, 2> RingTwoPerCu;  // 4 waves of 128x64, 
 // has two neighbours to cover for it
 typedef RingTile<192, 128, 2, 2, 32, 2, 3> RingThreePerCu;
 typedef WsTile<256, 256, 2, 4, 32, 4, 4, 3> WsLarge;      // 8 consumer waves of 128x64 + 4 producers, 4 x 32 KiB stages
+typedef WsTile<256, 256, 2, 4, 64, 2, 4, 3> WsWide;       // the same waves on two buffers of 64-wide k-tiles (whole cache lines per row)
 typedef DwWsTile<256, 256, 2, 4, 32, 4, 4> DwWsLarge;     // same shape for the weight-gradient GEMMs
 
 // ---------------------------------------------------------------------------
@@ -1625,14 +1655,18 @@ enum Kind { K_GATEUP = 0, K_DOWN, K_DY1, K_DX, K_DW2, K_DW1, K_COUNT };
 const char* const kKindEnv[K_COUNT] = {"MTS_TILE_GATEUP", "MTS_TILE_DOWN", "MTS_TILE_DY1",
                                        "MTS_TILE_DX",     "MTS_TILE_DW2",  "MTS_TILE_DW1"};
 // rows_gemm: 0 StagedSmall, 1 RingTwoPerCu, 2 WsLarge, 3 RingThreePerCu (dY1 without the weighted_act output
-// only);  dw_gemm: 0 StagedSmall, 2 DwWsLarge.
+// only), 4 WsWide (row-major weights, no SwiGLU backward: gate/up and down; the others fall back to 2);
+// dw_gemm: 0 StagedSmall, 2 DwWsLarge.
 // Defaults are the choices with the shortest LAYER STEP measured on the 24576-token, 768/1024, 8-expert layer.
 // The chip runs this step against its power limit, so a kernel's own duration is not the whole story: what
 // it leaves of the power budget shows in the kernels around it.  Gate/up on 256x256 tiles with specialised
 // waves moves a third less data from L2 to LDS per FLOP than on two co-resident 256x128 ring blocks and makes
 // the step 2-3.5 % shorter, although the kernel alone is at best as fast; dO*W2 with the SwiGLU backward in
-// its epilogue is better off with three co-resident 4-wave blocks per CU.
-const int kDefaultTile[K_COUNT] = {2, 2, 3, 2, 2, 2};
+// its epilogue is better off with three co-resident 4-wave blocks per CU.  The forward GEMMs take their
+// k-tiles 64 wide (two buffers instead of four stages, the same time for a tile to land): a row then contributes
+// a whole 128-byte line per load instruction, which the CU's vector cache serves at twice the rate of two
+// half lines (gate/up -2.4 %, down -1 %).
+const int kDefaultTile[K_COUNT] = {4, 4, 3, 2, 2, 2};
 
 bool tile_forced(int kind) { return getenv(kKindEnv[kind]) != nullptr; }
 
@@ -1643,7 +1677,7 @@ int tile_choice(int kind) {
         int c = kDefaultTile[kind];
         const char* s = getenv(kKindEnv[kind]);
         if (s) c = atoi(s);
-        choice[kind] = (c >= 0 && c <= (kind == K_DY1 ? 3 : 2)) ? c : kDefaultTile[kind];
+        choice[kind] = (c >= 0 && c <= 4) ? c : kDefaultTile[kind];
     }
     return choice[kind];
 }
@@ -1721,6 +1755,8 @@ int launch_rows_any(int kind, RowsParams p, int64_t TK, hipStream_t s, bool b_km
     int choice = tile_choice(kind);
     // three blocks per CU hold two stages each: for short reductions, and for the epilogue that fits beside them
     if (choice == 3 && (EPI != EPI_DY1N || !b_kmajor || (!tile_forced(kind) && p.Kdim > 1024))) choice = 1;
+    // the 64-wide variant exists for the forward GEMMs with row-major weights
+    if (choice == 4 && (b_kmajor || epi_is_dy1(EPI))) choice = 2;
     // the ring kernels need whole k-tiles; other shapes use the staged kernel
     if (choice >= 1 && p.Kdim % 64 != 0) choice = 0;
     if (b_kmajor && (choice == 0 || EPI == EPI_SWIGLU)) return MTS_ERR_SHAPE;
@@ -1736,6 +1772,11 @@ int launch_rows_any(int kind, RowsParams p, int64_t TK, hipStream_t s, bool b_km
             else rows_gemm_ring_kernel<RingTwoPerCu, EPI><<<grid, RingTwoPerCu::NT, 0, s>>>(p);
         } else {
             rows_gemm_ring_kernel<RingTwoPerCu, EPI><<<grid, RingTwoPerCu::NT, 0, s>>>(p);
+        }
+    } else if (choice == 4) {
+        if constexpr (!epi_is_dy1(EPI)) {
+            const dim3 grid = rows_grid<WsWide, EPI>(p, TK);
+            rows_gemm_ws_kernel<WsWide, EPI><<<grid, WsWide::NT, 0, s>>>(p);
         }
     } else if (choice == 2) {
         const dim3 grid = rows_grid<WsLarge, EPI>(p, TK);
