@@ -1601,10 +1601,11 @@ struct BwdJointParams {
     mts_rl::RouterGradIn rg;
 };
 
+typedef WsWide JointDxTile;   // dX reads d_pre_act row-major: whole lines per row with 64-wide k-tiles
 template <typename OutT>
 __global__ __launch_bounds__(WsLarge::NT, WsLarge::WAVES_PER_EU) void bwd_joint_kernel(BwdJointParams q) {
-    static_assert(WsLarge::NT == DwWsLarge::NT, "one block shape");
-    constexpr int ROWS_LDS = ws_lds_elems<WsLarge, EPI_PLAIN>();
+    static_assert(WsLarge::NT == DwWsLarge::NT && JointDxTile::NT == WsLarge::NT, "one block shape");
+    constexpr int ROWS_LDS = ws_lds_elems<JointDxTile, EPI_PLAIN>();
     constexpr int LDS_ELEMS = ROWS_LDS > DwWsLarge::LDS_ELEMS ? ROWS_LDS : DwWsLarge::LDS_ELEMS;
     static_assert(LDS_ELEMS * 2 <= 160 * 1024, "LDS capacity");
     __shared__ __attribute__((aligned(1024))) bf16_t smem[LDS_ELEMS];
@@ -1620,7 +1621,7 @@ __global__ __launch_bounds__(WsLarge::NT, WsLarge::WAVES_PER_EU) void bwd_joint_
     }
     b -= q.n_dw2;
     if (b < q.n_dx) {
-        rows_gemm_ws_block<WsLarge, EPI_PLAIN, true>(q.dx, smem, b);   // W1 as stored: [E][2I][H]
+        rows_gemm_ws_block<JointDxTile, EPI_PLAIN, true>(q.dx, smem, b);   // W1 as stored: [E][2I][H]
         return;
     }
     b -= q.n_dx;
@@ -1655,7 +1656,7 @@ enum Kind { K_GATEUP = 0, K_DOWN, K_DY1, K_DX, K_DW2, K_DW1, K_COUNT };
 const char* const kKindEnv[K_COUNT] = {"MTS_TILE_GATEUP", "MTS_TILE_DOWN", "MTS_TILE_DY1",
                                        "MTS_TILE_DX",     "MTS_TILE_DW2",  "MTS_TILE_DW1"};
 // rows_gemm: 0 StagedSmall, 1 RingTwoPerCu, 2 WsLarge, 3 RingThreePerCu (dY1 without the weighted_act output
-// only), 4 WsWide (row-major weights, no SwiGLU backward: gate/up and down; the others fall back to 2);
+// only), 4 WsWide (no SwiGLU backward: gate/up, down and dX; dY1 falls back to 2);
 // dw_gemm: 0 StagedSmall, 2 DwWsLarge.
 // Defaults are the choices with the shortest LAYER STEP measured on the 24576-token, 768/1024, 8-expert layer.
 // The chip runs this step against its power limit, so a kernel's own duration is not the whole story: what
@@ -1665,8 +1666,8 @@ const char* const kKindEnv[K_COUNT] = {"MTS_TILE_GATEUP", "MTS_TILE_DOWN", "MTS_
 // its epilogue is better off with three co-resident 4-wave blocks per CU.  The forward GEMMs take their
 // k-tiles 64 wide (two buffers instead of four stages, the same time for a tile to land): a row then contributes
 // a whole 128-byte line per load instruction, which the CU's vector cache serves at twice the rate of two
-// half lines (gate/up -2.4 %, down -1 %).
-const int kDefaultTile[K_COUNT] = {4, 4, 3, 2, 2, 2};
+// half lines (gate/up -2.4 %, down -1 %); so does dX, inside the joint backward launch and on its own.
+const int kDefaultTile[K_COUNT] = {4, 4, 3, 4, 2, 2};
 
 bool tile_forced(int kind) { return getenv(kKindEnv[kind]) != nullptr; }
 
@@ -1755,8 +1756,8 @@ int launch_rows_any(int kind, RowsParams p, int64_t TK, hipStream_t s, bool b_km
     int choice = tile_choice(kind);
     // three blocks per CU hold two stages each: for short reductions, and for the epilogue that fits beside them
     if (choice == 3 && (EPI != EPI_DY1N || !b_kmajor || (!tile_forced(kind) && p.Kdim > 1024))) choice = 1;
-    // the 64-wide variant exists for the forward GEMMs with row-major weights
-    if (choice == 4 && (b_kmajor || epi_is_dy1(EPI))) choice = 2;
+    // the 64-wide variant exists for the GEMMs with a plain or SwiGLU epilogue
+    if (choice == 4 && epi_is_dy1(EPI)) choice = 2;
     // the ring kernels need whole k-tiles; other shapes use the staged kernel
     if (choice >= 1 && p.Kdim % 64 != 0) choice = 0;
     if (b_kmajor && (choice == 0 || EPI == EPI_SWIGLU)) return MTS_ERR_SHAPE;
@@ -1776,7 +1777,12 @@ int launch_rows_any(int kind, RowsParams p, int64_t TK, hipStream_t s, bool b_km
     } else if (choice == 4) {
         if constexpr (!epi_is_dy1(EPI)) {
             const dim3 grid = rows_grid<WsWide, EPI>(p, TK);
-            rows_gemm_ws_kernel<WsWide, EPI><<<grid, WsWide::NT, 0, s>>>(p);
+            if constexpr (EPI != EPI_SWIGLU) {
+                if (b_kmajor) rows_gemm_ws_kernel<WsWide, EPI, true><<<grid, WsWide::NT, 0, s>>>(p);
+                else rows_gemm_ws_kernel<WsWide, EPI><<<grid, WsWide::NT, 0, s>>>(p);
+            } else {
+                rows_gemm_ws_kernel<WsWide, EPI><<<grid, WsWide::NT, 0, s>>>(p);
+            }
         }
     } else if (choice == 2) {
         const dim3 grid = rows_grid<WsLarge, EPI>(p, TK);
@@ -1849,7 +1855,7 @@ int dy1_partials(int I) { return (I + 63) / 64; }
 
 // can dW1, dW2, dX and the dS reduction go out as one launch for these shapes?
 bool bwd_joint_ok(int H, int I) {
-    return tile_choice(K_DX) == 2 && tile_choice(K_DW1) == 2 && tile_choice(K_DW2) == 2 && rows_kmajor_ok(K_DX, 2 * I) &&
+    return tile_choice(K_DX) >= 2 && tile_choice(K_DW1) == 2 && tile_choice(K_DW2) == 2 && rows_kmajor_ok(K_DX, 2 * I) &&
            H % 8 == 0;
 }
 
@@ -1874,7 +1880,7 @@ int launch_bwd_joint(BwdJointParams q, int E, int grad_dtype, void* ws1, int64_t
     q.n_dw1 = (int)dw_grid<T>(q.dw1, E, q.dw1.part ? 2 * E : E).x;
     q.n_dw2 = (int)dw_grid<T>(q.dw2, E, q.dw2.part ? 2 * E : E).x;
     q.dx.reverse = (tile_order_mask() & ORDER_DX) ? 1 : 0;
-    q.n_dx = (int)rows_grid<WsLarge, EPI_PLAIN>(q.dx, q.dx.TK).x;
+    q.n_dx = (int)rows_grid<JointDxTile, EPI_PLAIN>(q.dx, q.dx.TK).x;
     const int64_t want = (q.entries + WsLarge::NT * 4 - 1) / (WsLarge::NT * 4);
     q.n_ds = (int)(want < 64 ? want : 64);
     const dim3 grid((unsigned)(q.n_dw1 + q.n_dw2 + q.n_dx + q.n_ds + q.n_router));
@@ -2144,7 +2150,7 @@ int fill_bwd_joint(BwdJointParams& q, const void* d_out, const void* weighted_ac
 // experts, need no more threads than a block of the launch has, and keep E x cols floats of dW_r sums and the
 // logit gradients of their rows in the block's LDS
 bool joint_router_ok(int H, int E, const MtsRouterBwdShape& g) {
-    constexpr size_t lds_bytes = (size_t)ws_lds_elems<WsLarge, EPI_PLAIN>() * sizeof(bf16_t);
+    constexpr size_t lds_bytes = (size_t)ws_lds_elems<JointDxTile, EPI_PLAIN>() * sizeof(bf16_t);
     const size_t need = ((size_t)E * g.cols_per_block + (size_t)mts_rl::kChainRows * kJointRouterExperts) * sizeof(float);
     return E <= kJointRouterExperts && g.groups * g.col_threads <= WsLarge::NT && need <= lds_bytes && H % 4 == 0;
 }
