@@ -142,6 +142,8 @@ struct RowsParams {
     int xcd_ranges;            // block -> tile mapping: 1 = every XCD takes a contiguous range of m-tiles
     int n_groups;              // with xcd_ranges: the n-tiles are walked in this many groups, all m-tiles of the range per group
     int reverse;               // with xcd_ranges: the range's m-tiles are walked from the last to the first
+    int tail_slots;            // with xcd_ranges: blocks an XCD runs at a time; when the tiles behind its last whole round
+                               // fill at most half of them, each of those is cut into two tiles of half the height (0: never)
 };
 
 // ---------------------------------------------------------------------------
@@ -560,11 +562,14 @@ constexpr int kXcds = 8;
 // ballot picks the first expert whose offset range contains the tile (63 experts per
 // round; more experts take more rounds).
 template <int BM>
-__device__ __forceinline__ bool find_rows_tile(const RowsParams& p, int b, int& e, int& row0, int& rend, int& ntile) {
-    const int xcd = b % kXcds, j = b / kXcds;
+__device__ __forceinline__ bool find_rows_tile(const RowsParams& p, int b, int& e, int& row0, int& rend, int& ntile, int& parts) {
+    const int xcd = b % kXcds;
+    int j = b / kXcds;
     const int lane = threadIdx.x % MTS_WAVE;
     int tile = xcd + kXcds * (j / p.n_tiles);
     ntile = j % p.n_tiles;
+    parts = 1;      // pieces the tile is cut into: this block computes piece `part`
+    int part = 0;
     if (p.xcd_ranges) {
         // m-tiles of the launch: the first (total % 8) XCDs take one more than the others
         int mine = 0;
@@ -573,6 +578,18 @@ __device__ __forceinline__ bool find_rows_tile(const RowsParams& p, int b, int& 
         for (int o = 32; o > 0; o >>= 1) mine += __shfl_xor(mine, o, MTS_WAVE);
         const int per = mine / kXcds, rem = mine % kXcds;
         const int my = per + (xcd < rem ? 1 : 0);
+        if (p.tail_slots > 0) {
+            // the blocks behind the last whole round of this XCD: two per tile, the upper and the lower half (cutting
+            // into four where a quarter of the slots is filled gains another 0.15 % of the layer step: not done)
+            const int total = my * p.n_tiles, whole = total / p.tail_slots * p.tail_slots;
+            const int cut = 2 * (total - whole) <= p.tail_slots ? 2 : 1;
+            if (cut > 1 && j >= whole) {
+                parts = cut;
+                part = (j - whole) % cut;
+                j = whole + (j - whole) / cut;
+                ntile = j % p.n_tiles;
+            }
+        }
         int k = j / p.n_tiles;
         if (p.n_groups > 1 && my > 0) {
             const int npg = p.n_tiles / p.n_groups;   // n-tiles per group (n_tiles is a multiple of n_groups)
@@ -605,6 +622,11 @@ __device__ __forceinline__ bool find_rows_tile(const RowsParams& p, int b, int& 
             e = e0 + w;
             row0 = __shfl(s0, w, MTS_WAVE) + (tile - first) * BM;
             rend = __shfl(s1, w, MTS_WAVE);
+            if (parts > 1) {
+                row0 += part * (BM / parts);
+                if (row0 + BM / parts < rend) rend = row0 + BM / parts;
+                return row0 < rend;
+            }
             return true;
         }
         seen += __shfl(incl, MTS_WAVE - 1, MTS_WAVE);
@@ -616,14 +638,20 @@ __device__ __forceinline__ bool find_rows_tile(const RowsParams& p, int b, int& 
 // and LDS addresses built from these values then stay in scalar registers (a buffer instruction whose
 // descriptor sits in vector registers is wrapped in a loop over its distinct values).
 template <int BM>
-__device__ __forceinline__ bool locate_rows_tile(const RowsParams& p, int b, int& e, int& row0, int& rend, int& ntile) {
-    int fe = 0, frow0 = 0, frend = 0, fn = 0;
-    const bool found = find_rows_tile<BM>(p, b, fe, frow0, frend, fn);
+__device__ __forceinline__ bool locate_rows_tile(const RowsParams& p, int b, int& e, int& row0, int& rend, int& ntile, int& parts) {
+    int fe = 0, frow0 = 0, frend = 0, fn = 0, fh = 1;
+    const bool found = find_rows_tile<BM>(p, b, fe, frow0, frend, fn, fh);
     e = __builtin_amdgcn_readfirstlane(fe);
     row0 = __builtin_amdgcn_readfirstlane(frow0);
     rend = __builtin_amdgcn_readfirstlane(frend);
     ntile = __builtin_amdgcn_readfirstlane(fn);
+    parts = __builtin_amdgcn_readfirstlane(fh);
     return __builtin_amdgcn_readfirstlane((int)found) != 0;
+}
+template <int BM>
+__device__ __forceinline__ bool locate_rows_tile(const RowsParams& p, int b, int& e, int& row0, int& rend, int& ntile) {
+    int parts;   // a slice of a tile is a tile with fewer rows to a kernel that does not treat it specially
+    return locate_rows_tile<BM>(p, b, e, row0, rend, ntile, parts);
 }
 
 // ---------------------------------------------------------------------------
@@ -879,14 +907,11 @@ constexpr int ws_lds_elems() {
     return T::LDS_ELEMS > EpiShape<T, EPI>::ELEMS ? T::LDS_ELEMS : EpiShape<T, EPI>::ELEMS;
 }
 
-// the work of block `block` of a launch; `smem` holds ws_lds_elems<T, EPI>() elements, 1 KiB aligned
+// one output tile: rows [row0, rend) of expert e (at most T::BM of them), column tile ntile
 template <class T, int EPI, bool BKM>
-__device__ __forceinline__ void rows_gemm_ws_block(const RowsParams& p, bf16_t* smem, int block) {
+__device__ __forceinline__ void rows_gemm_ws_tile(const RowsParams& p, bf16_t* smem, int e, int row0, int rend, int ntile) {
     constexpr bool SWIGLU = (EPI == EPI_SWIGLU);
     constexpr int S = T::STAGES, L = T::A_INSTR + T::B_INSTR;
-
-    int e, row0, rend, ntile;
-    if (!locate_rows_tile<T::BM>(p, block, e, row0, rend, ntile)) return;
     const int n0 = ntile * (SWIGLU ? T::BN / 2 : T::BN);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / MTS_WAVE), lane = threadIdx.x % MTS_WAVE;
     const int nk = p.Kdim / T::BKS;
@@ -1014,11 +1039,25 @@ __device__ __forceinline__ void rows_gemm_ws_block(const RowsParams& p, bf16_t* 
     rows_epilogue<T, EPI>(p, acc, smem, row0, rend, n0, wm, wn);
 }
 
-template <class T, int EPI, bool BKM = false>
+// the work of block `block` of a launch; `smem` holds ws_lds_elems<T, EPI>() elements, 1 KiB aligned.
+// TH (same block shape and columns, half the rows) runs the halves of the tiles that a launch with tail_slots cuts up.
+template <class T, int EPI, bool BKM, class TH = T>
+__device__ __forceinline__ void rows_gemm_ws_block(const RowsParams& p, bf16_t* smem, int block) {
+    static_assert(TH::NT == T::NT && TH::BN == T::BN && (TH::BM == T::BM || 2 * TH::BM == T::BM), "half tile shape");
+    static_assert(ws_lds_elems<TH, EPI>() <= ws_lds_elems<T, EPI>(), "the half tile fits the same LDS");
+    int e, row0, rend, ntile, parts;
+    if (!locate_rows_tile<T::BM>(p, block, e, row0, rend, ntile, parts)) return;
+    if constexpr (TH::BM != T::BM) {
+        if (parts == 2) return rows_gemm_ws_tile<TH, EPI, BKM>(p, smem, e, row0, rend, ntile);
+    }
+    rows_gemm_ws_tile<T, EPI, BKM>(p, smem, e, row0, rend, ntile);
+}
+
+template <class T, int EPI, bool BKM = false, class TH = T>
 __global__ __launch_bounds__(T::NT, T::WAVES_PER_EU) void rows_gemm_ws_kernel(RowsParams p) {
     static_assert(ws_lds_elems<T, EPI>() * 2 <= 160 * 1024, "LDS capacity");
     __shared__ __attribute__((aligned(1024))) bf16_t smem[ws_lds_elems<T, EPI>()];
-    rows_gemm_ws_block<T, EPI, BKM>(p, smem, blockIdx.x);
+    rows_gemm_ws_block<T, EPI, BKM, TH>(p, smem, blockIdx.x);
 }
 
 // ---------------------------------------------------------------------------
@@ -1562,7 +1601,9 @@ typedef RingTile<256, 128, 2, 2, 32, 3, 2> RingTwoPerCu;  // 4 waves of 128x64, 
 typedef RingTile<192, 128, 2, 2, 32, 2, 3> RingThreePerCu;
 typedef WsTile<256, 256, 2, 4, 32, 4, 4, 3> WsLarge;      // 8 consumer waves of 128x64 + 4 producers, 4 x 32 KiB stages
 typedef WsTile<256, 256, 4, 2, 64, 2, 4, 3> WsWideGu;     // gate/up: waves of 64x128, so that a wave stores 64 columns (whole lines) of g, u and a
-typedef WsTile<256, 256, 2, 4, 64, 2, 4, 3> WsWide;       // the same waves on two buffers of 64-wide k-tiles (whole cache lines per row)
+typedef WsTile<256, 256, 2, 4, 64, 2, 4, 3> WsWide;
+typedef WsTile<128, 256, 2, 4, 64, 2, 4, 3> WsWideHalf;    // half-height tiles of the last round: the same waves take 64x64 each,
+typedef WsTile<128, 256, 4, 2, 64, 2, 4, 3> WsWideGuHalf;  // and for gate/up 32x128 each       // the same waves on two buffers of 64-wide k-tiles (whole cache lines per row)
 typedef DwWsTile<256, 256, 2, 4, 32, 4, 4> DwWsLarge;     // same shape for the weight-gradient GEMMs
 
 // ---------------------------------------------------------------------------
@@ -1731,6 +1772,17 @@ int tile_order_mask() {
     return mask;
 }
 
+// MTS_NO_TAIL_SPLIT=1 keeps every tile whole (for comparisons)
+constexpr int kCusPerXcd = 32;
+bool tail_split_on() {
+    static int on = -1;
+    if (on < 0) {
+        const char* s = getenv("MTS_NO_TAIL_SPLIT");
+        on = (s && atoi(s) != 0) ? 0 : 1;
+    }
+    return on != 0;
+}
+
 template <class T, int EPI>
 dim3 rows_grid(RowsParams& p, int64_t TK) {
     const int per_block = (EPI == EPI_SWIGLU) ? T::BN / 2 : T::BN;
@@ -1742,7 +1794,9 @@ dim3 rows_grid(RowsParams& p, int64_t TK) {
         while (weight_bytes / p.n_groups > kL2Bytes / 2 && p.n_tiles % (2 * p.n_groups) == 0 && p.n_tiles / (2 * p.n_groups) >= 4)
             p.n_groups *= 2;
     const int64_t m_groups = (m_tiles<T>(TK, p.E) + kXcds - 1) / kXcds;
-    return dim3((unsigned)(m_groups * kXcds * p.n_tiles));
+    if (!p.xcd_ranges) p.tail_slots = 0;
+    // tiles that are cut in two add at most tail_slots / 2 blocks per XCD
+    return dim3((unsigned)((m_groups * p.n_tiles + p.tail_slots / 2) * kXcds));
 }
 
 // does launch_rows_any take B in the weights' stored layout for this kind and reduction length?
@@ -1777,15 +1831,19 @@ int launch_rows_any(int kind, RowsParams p, int64_t TK, hipStream_t s, bool b_km
         }
     } else if (choice == 4) {
         if constexpr (!epi_is_dy1(EPI)) {
+            // The tiles are few and long: 6.25 (gate/up) and 2.34 (down) per CU at the 24576-token layer.  The ones
+            // behind the last whole round of an XCD's 32 CUs are cut in two where they would leave more than half
+            // of the CUs idle (gate/up -3 %, down -4 %).
+            if (!b_kmajor && tail_split_on()) p.tail_slots = kCusPerXcd;
             const dim3 grid = rows_grid<WsWide, EPI>(p, TK);
             if constexpr (EPI != EPI_SWIGLU) {
                 if (b_kmajor) rows_gemm_ws_kernel<WsWide, EPI, true><<<grid, WsWide::NT, 0, s>>>(p);
-                else rows_gemm_ws_kernel<WsWide, EPI><<<grid, WsWide::NT, 0, s>>>(p);
+                else rows_gemm_ws_kernel<WsWide, EPI, false, WsWideHalf><<<grid, WsWide::NT, 0, s>>>(p);
             } else {
                 // same tile, waves of 64x128: a wave's 32-row slab of g, u and a is 64 columns wide, i.e. whole 128-byte
                 // lines per row and store (with 128x64 waves it is 32 columns: gate/up +2.5 %)
                 static_assert(WsWideGu::BM == WsWide::BM && WsWideGu::BN == WsWide::BN && WsWideGu::NT == WsWide::NT, "same grid");
-                rows_gemm_ws_kernel<WsWideGu, EPI><<<grid, WsWideGu::NT, 0, s>>>(p);
+                rows_gemm_ws_kernel<WsWideGu, EPI, false, WsWideGuHalf><<<grid, WsWideGu::NT, 0, s>>>(p);
             }
         }
     } else if (choice == 2) {
