@@ -287,13 +287,16 @@ struct FragPipe {
     }
     __device__ __forceinline__ int chunk_off(int ks) const { return ((ks * 2 + kb) ^ swz) << 3; }
     // all fragments of k-step 0 of the stage at `tile`
-    __device__ __forceinline__ void prime(const bf16_t* tile) {
+    __device__ __forceinline__ void prime(const bf16_t* tile) { prime(tile, tile); }
+    // the same with the two operands in buffers of their own: tile_b is where a stage would start whose weight tile
+    // is the buffer (the buffer's address minus the size of an activation tile)
+    __device__ __forceinline__ void prime(const bf16_t* tile, const bf16_t* tile_b) {
         const int coff = chunk_off(0);
 #pragma unroll
         for (int mf = 0; mf < T::MF; ++mf)
             a[mf] = *reinterpret_cast<const bf16x8*>(tile + a_off + mf * 32 * ROWLEN + coff);
 #pragma unroll
-        for (int nf = 0; nf < T::NF; ++nf) b[0][nf] = read_b(tile, nf, 0, coff);
+        for (int nf = 0; nf < T::NF; ++nf) b[0][nf] = read_b(tile_b, nf, 0, coff);
     }
     // MFMAs of k-step `ks` (weight fragment first); behind them, the fragments of k-step `nks`
     // of the stage at `next` are read: the weight fragments up front into the other buffer, each
@@ -301,10 +304,14 @@ struct FragPipe {
     // READ = false: the MFMAs only (the last k-step of a buffer whose successor is not visible yet)
     template <bool READ = true>
     __device__ __forceinline__ void step(int ks, f32x16 (&acc)[T::MF][T::NF], const bf16_t* next, int nks) {
+        step<READ>(ks, acc, next, next, nks);
+    }
+    template <bool READ = true>
+    __device__ __forceinline__ void step(int ks, f32x16 (&acc)[T::MF][T::NF], const bf16_t* next, const bf16_t* next_b, int nks) {
         const int coff = chunk_off(nks), buf = ks & 1;
         if constexpr (READ) {
 #pragma unroll
-            for (int nf = 0; nf < T::NF; ++nf) b[buf ^ 1][nf] = read_b(next, nf, nks, coff);
+            for (int nf = 0; nf < T::NF; ++nf) b[buf ^ 1][nf] = read_b(next_b, nf, nks, coff);
         }
 #pragma unroll
         for (int mf = 0; mf < T::MF; ++mf) {
@@ -894,11 +901,13 @@ struct WsTile {
     static constexpr int RPI = MTS_WAVE / CHUNKS;
     static constexpr int A_INSTR = BM / RPI / PRODUCERS, B_INSTR = BN / RPI / PRODUCERS;   // per producer wave
     static constexpr int STAGE = (BM + BN) * BKS;
-    static constexpr int LDS_ELEMS = STAGES * STAGE;
+    // STAGES == 3: three buffers for the activation tile and two for the weight tile (the gathered rows come from
+    // further away than the weights, which mostly sit in the XCD's L2)
+    static constexpr int LDS_ELEMS = STAGES == 3 ? (3 * BM + 2 * BN) * BKS : STAGES * STAGE;
     static_assert(BKS == 32 || BKS == 64, "LDS rows are 64 or 128 bytes");
     static_assert(WM % 32 == 0 && WN % 64 == 0, "wave tile must hold whole 32x32 fragments");
     static_assert(A_INSTR * RPI * PRODUCERS == BM && B_INSTR * RPI * PRODUCERS == BN, "loader split");
-    static_assert((STAGES == 4 || STAGES == 2) && (A_INSTR + B_INSTR) * 2 <= 63, "the producer waits are written for a 4-stage ring and for two buffers");
+    static_assert((STAGES == 4 || STAGES == 2 || STAGES == 3) && (A_INSTR + B_INSTR) * 2 <= 63, "the producer waits are written for a 4-stage ring, for two buffers and for three plus two");
     static_assert(LDS_ELEMS * 2 <= 160 * 1024, "LDS capacity");
 };
 
@@ -969,6 +978,39 @@ __device__ __forceinline__ void rows_gemm_ws_tile(const RowsParams& p, bf16_t* s
             for (int j = 0; j < T::B_INSTR; ++j)
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_b, MTS_LDS_PTR(sb + j * 512), 16, (int)voff_b[j], soff_b, 0, 0);
         };
+        if constexpr (S == 3) {
+            // Three buffers for the activation tile, two for the weight tile.  Barrier kt says that tile kt has landed
+            // and that tile kt-1 has been consumed: its weight buffer then takes tile kt+1 and its activation buffer
+            // tile kt+2, which has two tiles' time to land.  The activation loads of tile kt+1, the youngest in flight,
+            // may still be on their way at barrier kt-1... they are waited for one barrier later.
+            auto issue_a = [&](int buf, int kt) {
+                bf16_t* sa = smem + buf * T::BM * T::BKS + pw * T::A_INSTR * 512;
+#pragma unroll
+                for (int j = 0; j < T::A_INSTR; ++j)
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, MTS_LDS_PTR(sa + j * 512), 16, (int)voff_a[j], kt * T::BKS * 2, 0, 0);
+            };
+            auto issue_b = [&](int buf, int kt) {
+                bf16_t* sb = smem + 3 * T::BM * T::BKS + buf * T::BN * T::BKS + pw * T::B_INSTR * 512;
+                const int soff_b = BKM ? kt * T::BKS * p.N * 2 : kt * T::BKS * 2;   // a k-tile of k-major B is BKS memory rows further
+#pragma unroll
+                for (int j = 0; j < T::B_INSTR; ++j)
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_b, MTS_LDS_PTR(sb + j * 512), 16, (int)voff_b[j], soff_b, 0, 0);
+            };
+            issue_a(0, 0);
+            issue_b(0, 0);
+            if (nk > 1) issue_a(1, 1);
+            int abuf = 2;   // activation buffer of tile kt+2
+            for (int kt = 0; kt < nk; ++kt) {
+                if (kt + 1 < nk) wait_vmcnt<T::A_INSTR>();   // all but the activation tile kt+1
+                else wait_vmcnt<0>();
+                __builtin_amdgcn_s_barrier();
+                if (kt + 1 < nk) issue_b((kt + 1) & 1, kt + 1);
+                if (kt + 2 < nk) issue_a(abuf, kt + 2);
+                abuf = abuf == 2 ? 0 : abuf + 1;
+            }
+            __builtin_amdgcn_s_barrier();       // matches the consumers' barrier behind the last tile
+            return;
+        }
         if constexpr (S == 2) {
             // Two buffers of 64-wide k-tiles (a row contributes a whole 128-byte line per load): barrier kt says
             // that tile kt has landed and that tile kt-1 has been consumed, whose buffer then takes tile kt+1.
@@ -1008,6 +1050,22 @@ __device__ __forceinline__ void rows_gemm_ws_tile(const RowsParams& p, bf16_t* s
     FragPipe<T, SWIGLU, T::BKS, BKM> pipe;
     pipe.init(wm, wn);
     constexpr int KSTEPS = T::BKS / 16;
+    if constexpr (S == 3) {
+        int abuf = 0;
+        for (int kt = 0; kt < nk; ++kt) {
+            __builtin_amdgcn_s_barrier();   // tile kt is visible
+            const bf16_t* cur = smem + abuf * T::BM * T::BKS;
+            const bf16_t* cur_b = smem + 3 * T::BM * T::BKS + (kt & 1) * T::BN * T::BKS - T::BM * T::BKS;
+            abuf = abuf == 2 ? 0 : abuf + 1;
+            pipe.prime(cur, cur_b);
+#pragma unroll
+            for (int ks = 0; ks < KSTEPS - 1; ++ks) pipe.step(ks, acc, cur, cur_b, ks + 1);
+            pipe.template step<false>(KSTEPS - 1, acc, cur, cur_b, 0);
+        }
+        __builtin_amdgcn_s_barrier();       // every wave is done with the buffers before the epilogue reuses them
+        rows_epilogue<T, EPI>(p, acc, smem, row0, rend, n0, wm, wn);
+        return;
+    }
     if constexpr (S == 2) {
         for (int kt = 0; kt < nk; ++kt) {
             __builtin_amdgcn_s_barrier();   // tile kt is visible
@@ -1602,6 +1660,8 @@ typedef RingTile<192, 128, 2, 2, 32, 2, 3> RingThreePerCu;
 typedef WsTile<256, 256, 2, 4, 32, 4, 4, 3> WsLarge;      // 8 consumer waves of 128x64 + 4 producers, 4 x 32 KiB stages
 typedef WsTile<256, 256, 4, 2, 64, 2, 4, 3> WsWideGu;     // gate/up: waves of 64x128, so that a wave stores 64 columns (whole lines) of g, u and a
 typedef WsTile<256, 256, 2, 4, 64, 2, 4, 3> WsWide;
+typedef WsTile<256, 256, 2, 4, 64, 3, 4, 3> WsDeep;        // three activation buffers and two weight buffers: the down projection, whose
+typedef WsTile<128, 256, 2, 4, 64, 3, 4, 3> WsDeepHalf;    // activation rows the launch before it has written (-4 %; nothing for gate/up and dX)
 typedef WsTile<128, 256, 2, 4, 64, 2, 4, 3> WsWideHalf;    // half-height tiles of the last round: the same waves take 64x64 each,
 typedef WsTile<128, 256, 4, 2, 64, 2, 4, 3> WsWideGuHalf;  // and for gate/up 32x128 each       // the same waves on two buffers of 64-wide k-tiles (whole cache lines per row)
 typedef DwWsTile<256, 256, 2, 4, 32, 4, 4> DwWsLarge;     // same shape for the weight-gradient GEMMs
@@ -1643,7 +1703,7 @@ struct BwdJointParams {
     mts_rl::RouterGradIn rg;
 };
 
-typedef WsWide JointDxTile;   // dX reads d_pre_act row-major: whole lines per row with 64-wide k-tiles
+typedef WsWide JointDxTile;   // dX reads d_pre_act row-major: whole lines per row with 64-wide k-tiles (a third buffer gains nothing here)
 template <typename OutT>
 __global__ __launch_bounds__(WsLarge::NT, WsLarge::WAVES_PER_EU) void bwd_joint_kernel(BwdJointParams q) {
     static_assert(WsLarge::NT == DwWsLarge::NT && JointDxTile::NT == WsLarge::NT, "one block shape");
@@ -1838,7 +1898,7 @@ int launch_rows_any(int kind, RowsParams p, int64_t TK, hipStream_t s, bool b_km
             const dim3 grid = rows_grid<WsWide, EPI>(p, TK);
             if constexpr (EPI != EPI_SWIGLU) {
                 if (b_kmajor) rows_gemm_ws_kernel<WsWide, EPI, true><<<grid, WsWide::NT, 0, s>>>(p);
-                else rows_gemm_ws_kernel<WsWide, EPI, false, WsWideHalf><<<grid, WsWide::NT, 0, s>>>(p);
+                else rows_gemm_ws_kernel<WsDeep, EPI, false, WsDeepHalf><<<grid, WsWide::NT, 0, s>>>(p);
             } else {
                 // same tile, waves of 64x128: a wave's 32-row slab of g, u and a is 64 columns wide, i.e. whole 128-byte
                 // lines per row and store (with 128x64 waves it is 32 columns: gate/up +2.5 %)
