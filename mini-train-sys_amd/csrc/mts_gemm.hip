@@ -746,8 +746,10 @@ __global__ __launch_bounds__(T::NT) void rows_gemm_kernel(RowsParams p) {
 // the swizzle is applied on the global side: lane l fetches the chunk that
 // belongs at its landing slot.  Requires Kdim % BKS == 0.
 // ---------------------------------------------------------------------------
-template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int BKS_, int STAGES_, int WAVES_PER_EU_ = 1>
+// A_STAGES_ = STAGES_ + 1: the activation tile has a buffer more than the weight tile (two stages only)
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int BKS_, int STAGES_, int WAVES_PER_EU_ = 1, int A_STAGES_ = STAGES_>
 struct RingTile {
+    static constexpr int A_STAGES = A_STAGES_;
     static constexpr int WAVES_PER_EU = WAVES_PER_EU_;  // register budget: 512 / WAVES_PER_EU per lane
     static constexpr int BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
     static constexpr int BKS = BKS_, STAGES = STAGES_;
@@ -759,11 +761,12 @@ struct RingTile {
     static constexpr int RPI = MTS_WAVE / CHUNKS;   // rows covered by one wave instruction
     static constexpr int A_INSTR = BM / RPI / NWAVES, B_INSTR = BN / RPI / NWAVES;
     static constexpr int STAGE = (BM + BN) * BKS;
-    static constexpr int LDS_ELEMS = STAGES * STAGE;
+    static constexpr int LDS_ELEMS = (A_STAGES * BM + STAGES * BN) * BKS;
     static_assert(BKS == 32 || BKS == 64, "LDS rows are 64 or 128 bytes");
     static_assert(WM % 32 == 0 && WN % 64 == 0, "wave tile must hold whole 32x32 fragments");
     static_assert(A_INSTR * RPI * NWAVES == BM && B_INSTR * RPI * NWAVES == BN, "loader split");
     static_assert(STAGES >= 2 && STAGES <= 4 && (A_INSTR + B_INSTR) * (STAGES - 2) <= 63, "vmcnt range");
+    static_assert(A_STAGES == STAGES || (A_STAGES == 3 && STAGES == 2 && BKS == 32), "the extra activation buffer goes with two stages");
     static_assert(LDS_ELEMS * 2 <= 160 * 1024, "LDS capacity");
 };
 
@@ -854,6 +857,47 @@ __global__ __launch_bounds__(T::NT, T::WAVES_PER_EU) void rows_gemm_ring_kernel(
     zero_acc<T>(acc);
 
     const int nk = p.Kdim / T::BKS;
+    if constexpr (T::A_STAGES == 3 && S == 2) {
+        // The activation tile (rows gathered from anywhere) is fetched two k-tiles ahead into three buffers, the
+        // weight tile one ahead into two.  The weight loads of tile kt+1 are issued in the first k-step of tile kt,
+        // the activation loads of tile kt+2 in the second: the wait in front of a tile then leaves only the youngest
+        // activation loads in flight.
+        static_assert(T::BKS / 16 == 2, "two k-steps per tile");
+        auto issue_a = [&](int buf, int kt) {
+            bf16_t* sa = smem + buf * T::BM * T::BKS + wave * T::A_INSTR * 512;
+            const int soff = kt * T::BKS * 2;
+#pragma unroll
+            for (int j = 0; j < T::A_INSTR; ++j)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, MTS_LDS_PTR(sa + j * 512), 16, (int)voff_a[j], soff, 0, 0);
+        };
+        auto issue_b = [&](int buf, int kt) {
+            bf16_t* sb = smem + 3 * T::BM * T::BKS + buf * T::BN * T::BKS + wave * T::B_INSTR * 512;
+            const int soff_b = BKM ? kt * T::BKS * p.N * 2 : kt * T::BKS * 2;
+#pragma unroll
+            for (int j = 0; j < T::B_INSTR; ++j)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_b, MTS_LDS_PTR(sb + j * 512), 16, (int)voff_b[j], soff_b, 0, 0);
+        };
+        issue_a(0, 0);
+        issue_b(0, 0);
+        if (nk > 1) issue_a(1, 1);
+        int abuf = 0;
+        for (int kt = 0; kt < nk; ++kt) {
+            if (kt + 1 < nk) wait_vmcnt<T::A_INSTR>();
+            else wait_vmcnt<0>();
+            __builtin_amdgcn_s_barrier();   // tile kt has landed for every wave, and every wave is past tile kt-1
+            const bf16_t* ca = smem + abuf * T::BM * T::BKS;
+            const bf16_t* cb = smem + 3 * T::BM * T::BKS + (kt & 1) * T::BN * T::BKS;
+            const int a_next = abuf == 0 ? 2 : abuf - 1;   // buffer of tile kt+2 = buffer of tile kt-1
+            mma_tile<T, SWIGLU, T::BKS, true, BKM>(ca, cb, wm, wn, acc, [&](int ks) {
+                if (ks == 0 && kt + 1 < nk) issue_b((kt + 1) & 1, kt + 1);
+                if (ks == 1 && kt + 2 < nk) issue_a(a_next, kt + 2);
+            });
+            abuf = abuf == 2 ? 0 : abuf + 1;
+        }
+        __builtin_amdgcn_s_barrier();  // every wave is done reading the buffers before they are reused
+        rows_epilogue<T, EPI, true>(p, acc, smem, row0, rend, n0, wm, wn);
+        return;
+    }
 #pragma unroll
     for (int s = 0; s < S - 1; ++s)
         if (s < nk) issue(s, s, 0, 1);
@@ -1656,7 +1700,7 @@ typedef RingTile<256, 128, 2, 2, 32, 3, 2> RingTwoPerCu;  // 4 waves of 128x64, 
 // 4 waves of 96x64, 2 x 20 KiB stages, three blocks per CU (at most 168 registers per lane): while one block
 // is in its epilogue two others are in their k-loops, and a block that waits for its one tile in flight
 // has two neighbours to cover for it
-typedef RingTile<192, 128, 2, 2, 32, 2, 3> RingThreePerCu;
+typedef RingTile<192, 128, 2, 2, 32, 2, 3, 3> RingThreePerCu;   // three activation buffers + two weight buffers: 52 KiB a block
 typedef WsTile<256, 256, 2, 4, 32, 4, 4, 3> WsLarge;      // 8 consumer waves of 128x64 + 4 producers, 4 x 32 KiB stages
 typedef WsTile<256, 256, 4, 2, 64, 2, 4, 3> WsWideGu;     // gate/up: waves of 64x128, so that a wave stores 64 columns (whole lines) of g, u and a
 typedef WsTile<256, 256, 2, 4, 64, 2, 4, 3> WsWide;
