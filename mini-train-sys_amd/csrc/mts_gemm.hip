@@ -1494,7 +1494,8 @@ struct DwWsTile {
     static constexpr int LDS_ELEMS = STAGES * STAGE;
     static_assert(A_INSTR >= 1 && B_INSTR >= 1 && A_INSTR * RPI_A * PRODUCERS == BKS && B_INSTR * RPI_B * PRODUCERS == BKS,
                   "loader split");
-    static_assert(STAGES == 4 && (A_INSTR + B_INSTR) * 2 <= 63, "the producer waits are written for a 4-stage ring");
+    static_assert((STAGES == 4 || STAGES == 2) && (A_INSTR + B_INSTR) * 2 <= 63,
+                  "the producer waits are written for a 4-stage ring and for two buffers");
     static_assert(LDS_ELEMS * 2 <= 160 * 1024, "LDS capacity");
 };
 
@@ -1529,7 +1530,7 @@ __device__ __forceinline__ void dw_gemm_ws_block(const DwParams& p, bf16_t* smem
         const bool gath_p = p.p_gather != nullptr, gath_q = p.q_gather != nullptr;
         constexpr int ROWS_A = T::A_INSTR * T::RPI_A, ROWS_B = T::B_INSTR * T::RPI_B;
         static_assert(T::RPI_A == 2 && T::RPI_B == 2 && T::CPR_A == T::CPR_B, "two rows per wave instruction");
-        static_assert(ROWS_A == 8 && ROWS_B == 8, "index fetch layout: 8 rows per producer wave");
+        static_assert(ROWS_A == ROWS_B && (ROWS_A == 8 || ROWS_A == 16), "index fetch layout: 8 or 16 rows per producer wave");
         const bool upper = lane >= T::CPR_A;
         const uint32_t ld_a = (uint32_t)p.M * 2u, ld_b = (uint32_t)p.N * 2u;   // row pitch in bytes
         uint32_t col_a[T::A_INSTR], col_b[T::B_INSTR], fix_a[T::A_INSTR], fix_b[T::B_INSTR];
@@ -1556,8 +1557,11 @@ __device__ __forceinline__ void dw_gemm_ws_block(const DwParams& p, bf16_t* smem
         const u32x4 rs_gq = scalar_rsrc(p.q_gather, gath_q ? p.TK * 4 : 0);
         i32x4 idx_a[ROWS_A / 4] = {}, idx_b[ROWS_B / 4] = {};
         auto fetch_index = [&](int r0) {
-            if (gath_p) s_buffer_load8(rs_gp, (r0 + pw * ROWS_A) * 4, idx_a[0], idx_a[1]);
-            if (gath_q) s_buffer_load8(rs_gq, (r0 + pw * ROWS_B) * 4, idx_b[0], idx_b[1]);
+#pragma unroll
+            for (int h = 0; h < ROWS_A / 8; ++h) {
+                if (gath_p) s_buffer_load8(rs_gp, (r0 + pw * ROWS_A + 8 * h) * 4, idx_a[2 * h], idx_a[2 * h + 1]);
+                if (gath_q) s_buffer_load8(rs_gq, (r0 + pw * ROWS_B + 8 * h) * 4, idx_b[2 * h], idx_b[2 * h + 1]);
+            }
         };
         auto issue = [&](int stage, int r0) {
             bf16_t* sa = smem + stage * T::STAGE + pw * T::A_INSTR * 512;
@@ -1593,6 +1597,22 @@ __device__ __forceinline__ void dw_gemm_ws_block(const DwParams& p, bf16_t* smem
             }
         };
 
+        if constexpr (S == 2) {
+            // Two buffers of wide tiles: barrier kt tells the consumers that tile kt has landed and
+            // the producers that tile kt-1 is consumed, whose buffer then takes tile kt+1.
+            fetch_index(rbeg);
+            issue(0, rbeg);
+            if (1 < nk) fetch_index(rbeg + T::BKS);
+            for (int kt = 0; kt < nk; ++kt) {
+                wait_vmcnt<0>();
+                __builtin_amdgcn_s_barrier();
+                if (kt + 1 < nk) {
+                    issue((kt + 1) & 1, rbeg + (kt + 1) * T::BKS);
+                    if (kt + 2 < nk) fetch_index(rbeg + (kt + 2) * T::BKS);
+                }
+            }
+            return;
+        }
         // Barrier kt tells the consumers that tiles kt and kt+1 have landed (they read the first
         // fragments of tile kt+1 behind the last MFMAs of tile kt) and tells the producers that
         // every consumer is done with tile kt-1, whose stage then takes tile kt-1+S.
@@ -1643,6 +1663,24 @@ __device__ __forceinline__ void dw_gemm_ws_block(const DwParams& p, bf16_t* smem
             fa[mf] = read_frag_tr<T::BM>(next, nks * 16, wm * T::WM + mf * 32);
         }
     };
+    if constexpr (S == 2) {
+        for (int kt = 0; kt < nk; ++kt) {
+            __builtin_amdgcn_s_barrier();   // tile kt is visible, tile kt-1 may be overwritten
+            const bf16_t* cur = smem + (kt & 1) * T::STAGE;
+#pragma unroll
+            for (int mf = 0; mf < T::MF; ++mf) fa[mf] = read_frag_tr<T::BM>(cur, 0, wm * T::WM + mf * 32);
+#pragma unroll
+            for (int nf = 0; nf < T::NF; ++nf)
+                fb[0][nf] = read_frag_tr<T::BN>(cur + T::BKS * T::BM, 0, wn * T::WN + nf * 32);
+#pragma unroll
+            for (int ks = 0; ks < KSTEPS - 1; ++ks) step(ks, cur, ks + 1);
+#pragma unroll
+            for (int mf = 0; mf < T::MF; ++mf)
+#pragma unroll
+                for (int nf = 0; nf < T::NF; ++nf)
+                    acc[mf][nf] = MTS_MFMA_32x32x16(fa[mf], fb[(KSTEPS - 1) & 1][nf], acc[mf][nf], 0, 0, 0);
+        }
+    } else {
     __builtin_amdgcn_s_barrier();   // tiles 0 and 1 are visible
 #pragma unroll
     for (int mf = 0; mf < T::MF; ++mf) fa[mf] = read_frag_tr<T::BM>(smem, 0, wm * T::WM + mf * 32);
@@ -1658,6 +1696,7 @@ __device__ __forceinline__ void dw_gemm_ws_block(const DwParams& p, bf16_t* smem
         // this reads a stage nobody uses: harmless)
         step(KSTEPS - 1, smem + stage * T::STAGE, 0);
         __builtin_amdgcn_s_barrier();   // tile kt+2 is visible, tile kt may be overwritten
+    }
     }
 
     const int fcol = lane % 32, frow4 = (lane / 32) * 4;
@@ -1709,6 +1748,8 @@ typedef WsTile<128, 256, 2, 4, 64, 3, 4, 3> WsDeepHalf;    // activation rows th
 typedef WsTile<128, 256, 2, 4, 64, 2, 4, 3> WsWideHalf;    // half-height tiles of the last round: the same waves take 64x64 each,
 typedef WsTile<128, 256, 4, 2, 64, 2, 4, 3> WsWideGuHalf;  // and for gate/up 32x128 each       // the same waves on two buffers of 64-wide k-tiles (whole cache lines per row)
 typedef DwWsTile<256, 256, 2, 4, 32, 4, 4> DwWsLarge;     // same shape for the weight-gradient GEMMs
+typedef DwWsTile<256, 256, 2, 4, 64, 2, 4> DwWsWide;      // two buffers of 64 rows: half the barriers per row
+typedef DwWsWide JointDwTile;                             // the weight-gradient tile of the joint backward launch
 
 // ---------------------------------------------------------------------------
 // dW1, dW2, dX and the reduction of the dS partials as one launch.  All four depend on dY1
@@ -1750,19 +1791,19 @@ struct BwdJointParams {
 typedef WsWide JointDxTile;   // dX reads d_pre_act row-major: whole lines per row with 64-wide k-tiles (a third buffer gains nothing here)
 template <typename OutT>
 __global__ __launch_bounds__(WsLarge::NT, WsLarge::WAVES_PER_EU) void bwd_joint_kernel(BwdJointParams q) {
-    static_assert(WsLarge::NT == DwWsLarge::NT && JointDxTile::NT == WsLarge::NT, "one block shape");
+    static_assert(WsLarge::NT == JointDwTile::NT && JointDxTile::NT == WsLarge::NT, "one block shape");
     constexpr int ROWS_LDS = ws_lds_elems<JointDxTile, EPI_PLAIN>();
-    constexpr int LDS_ELEMS = ROWS_LDS > DwWsLarge::LDS_ELEMS ? ROWS_LDS : DwWsLarge::LDS_ELEMS;
+    constexpr int LDS_ELEMS = ROWS_LDS > JointDwTile::LDS_ELEMS ? ROWS_LDS : JointDwTile::LDS_ELEMS;
     static_assert(LDS_ELEMS * 2 <= 160 * 1024, "LDS capacity");
     __shared__ __attribute__((aligned(1024))) bf16_t smem[LDS_ELEMS];
     int b = blockIdx.x;
     if (b < q.n_dw1) {
-        dw_gemm_ws_block<DwWsLarge, OutT>(q.dw1, smem, b);
+        dw_gemm_ws_block<JointDwTile, OutT>(q.dw1, smem, b);
         return;
     }
     b -= q.n_dw1;
     if (b < q.n_dw2) {
-        dw_gemm_ws_block<DwWsLarge, OutT>(q.dw2, smem, b);
+        dw_gemm_ws_block<JointDwTile, OutT>(q.dw2, smem, b);
         return;
     }
     b -= q.n_dw2;
@@ -1803,7 +1844,7 @@ const char* const kKindEnv[K_COUNT] = {"MTS_TILE_GATEUP", "MTS_TILE_DOWN", "MTS_
                                        "MTS_TILE_DX",     "MTS_TILE_DW2",  "MTS_TILE_DW1"};
 // rows_gemm: 0 StagedSmall, 1 RingTwoPerCu, 2 WsLarge, 3 RingThreePerCu (dY1 without the weighted_act output
 // only), 4 WsWide (no SwiGLU backward: gate/up, down and dX; dY1 falls back to 2);
-// dw_gemm: 0 StagedSmall, 2 DwWsLarge.
+// dw_gemm: 0 StagedSmall, 2 DwWsLarge, 4 DwWsWide (the same output tiles, so one workspace layout).
 // Defaults are the choices with the shortest LAYER STEP measured on the 24576-token, 768/1024, 8-expert layer.
 // The chip runs this step against its power limit, so a kernel's own duration is not the whole story: what
 // it leaves of the power budget shows in the kernels around it.  Gate/up on 256x256 tiles with specialised
@@ -1813,7 +1854,9 @@ const char* const kKindEnv[K_COUNT] = {"MTS_TILE_GATEUP", "MTS_TILE_DOWN", "MTS_
 // k-tiles 64 wide (two buffers instead of four stages, the same time for a tile to land): a row then contributes
 // a whole 128-byte line per load instruction, which the CU's vector cache serves at twice the rate of two
 // half lines (gate/up -2.4 %, down -1 %); so does dX, inside the joint backward launch and on its own.
-const int kDefaultTile[K_COUNT] = {4, 4, 3, 4, 2, 2};
+// The weight gradients read whole lines either way (a k-tile is rows of 256 columns); taking 64 rows per
+// tile into two buffers halves their barriers (joint launch -1.7 %).
+const int kDefaultTile[K_COUNT] = {4, 4, 3, 4, 4, 4};
 
 bool tile_forced(int kind) { return getenv(kKindEnv[kind]) != nullptr; }
 
@@ -1994,16 +2037,23 @@ void launch_dw_chunk_sum(const DwParams& p, int E, int grad_dtype, hipStream_t s
 int launch_dw_any(int kind, DwParams p, int E, int grad_dtype, void* workspace, int64_t workspace_bytes,
                   hipStream_t s) {
     if (grad_dtype != MTS_GEMM_DTYPE && grad_dtype != MTS_F32) return MTS_ERR_DTYPE;
-    if (tile_choice(kind) == 2) {
-        typedef DwWsLarge T;
+    const int choice = tile_choice(kind);
+    if (choice == 2 || choice == 4) {
+        typedef DwWsLarge T;   // DwWsWide has the same output tile, grid and block
+        static_assert(DwWsWide::BM == T::BM && DwWsWide::BN == T::BN && DwWsWide::NT == T::NT, "one grid for both");
         if (workspace) {
             if (workspace_bytes < dw_chunk_workspace_bytes(E, p.M, p.N)) return MTS_ERR_WORKSPACE;
             if (!mts_aligned16(workspace)) return MTS_ERR_ALIGN;
             p.part = (float*)workspace;
         }
         const dim3 grid = dw_grid<T>(p, E, p.part ? 2 * E : E);
-        if (grad_dtype == MTS_GEMM_DTYPE) dw_gemm_ws_kernel<T, bf16_t><<<grid, T::NT, 0, s>>>(p);
-        else dw_gemm_ws_kernel<T, float><<<grid, T::NT, 0, s>>>(p);
+        if (choice == 4) {
+            if (grad_dtype == MTS_GEMM_DTYPE) dw_gemm_ws_kernel<DwWsWide, bf16_t><<<grid, T::NT, 0, s>>>(p);
+            else dw_gemm_ws_kernel<DwWsWide, float><<<grid, T::NT, 0, s>>>(p);
+        } else {
+            if (grad_dtype == MTS_GEMM_DTYPE) dw_gemm_ws_kernel<T, bf16_t><<<grid, T::NT, 0, s>>>(p);
+            else dw_gemm_ws_kernel<T, float><<<grid, T::NT, 0, s>>>(p);
+        }
         if (p.part) {
             MTS_CHECK_LAUNCH();
             launch_dw_chunk_sum(p, E, grad_dtype, s);
@@ -2021,7 +2071,7 @@ int dy1_partials(int I) { return (I + 63) / 64; }
 
 // can dW1, dW2, dX and the dS reduction go out as one launch for these shapes?
 bool bwd_joint_ok(int H, int I) {
-    return tile_choice(K_DX) >= 2 && tile_choice(K_DW1) == 2 && tile_choice(K_DW2) == 2 && rows_kmajor_ok(K_DX, 2 * I) &&
+    return tile_choice(K_DX) >= 2 && tile_choice(K_DW1) == 4 && tile_choice(K_DW2) == 4 && rows_kmajor_ok(K_DX, 2 * I) &&
            H % 8 == 0;
 }
 

@@ -24,8 +24,9 @@ CONFIGURATIONS = {
                                               MTS_TILE_DW1="0", MTS_TILE_DW2="0", MTS_NO_JOINT_BWD="1", MTS_NO_OVERLAP="1"),
     "specialised waves for dY1, round-robin tiles": dict(MTS_TILE_DY1="2", MTS_XCD_RANGES="0", MTS_NO_TILE_ORDER="1"),
     "four stages of 32-wide k-tiles, separate launches": dict(MTS_TILE_GATEUP="2", MTS_TILE_DOWN="2", MTS_TILE_DX="2",
-                                                              MTS_NO_JOINT_BWD="1"),
-    "64-wide k-tiles for dX on its own, every tile whole": dict(MTS_NO_JOINT_BWD="1", MTS_NO_TAIL_SPLIT="1"),
+                                                              MTS_TILE_DW1="2", MTS_TILE_DW2="2", MTS_NO_JOINT_BWD="1"),
+    "64-wide k-tiles for dX and the weight gradients on their own, every tile whole": dict(MTS_NO_JOINT_BWD="1",
+                                                                                           MTS_NO_TAIL_SPLIT="1"),
     "ranges per XCD, plain order, tail launches apart": dict(MTS_XCD_RANGES="1", MTS_NO_TILE_ORDER="1",
                                                              MTS_NO_TAIL_IN_JOINT="1"),
 }
