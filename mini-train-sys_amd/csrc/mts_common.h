@@ -97,7 +97,8 @@ struct MtsRouterBwdShape {
 int mts_router_bwd_check(const void* x, const float* w_r, int64_t T, int H, int E, int act_dtype);
 void mts_router_bwd_shape(int64_t T, int H, int E, MtsRouterBwdShape* shape);
 int mts_launch_router_dw_reduce(const float* part, int row_blocks, int64_t EH, float* d_w_r, hipStream_t s);
-void mts_router_head_geometry(int64_t T, int* blocks, int* rows_per_wave);
+int mts_router_head_group(int H, int E, int act_dtype);   // rows a wave of the chained forward kernel finishes together
+void mts_router_head_geometry(int64_t T, int group, int* blocks, int* rows_per_wave);
 int mts_launch_router_head(const void* x, const float* w_r, int64_t T, int H, int E, int K, int normalize, int act_dtype,
                            float* logits, float* weights, int32_t* indices, void* weights_act, float* partial,
                            int32_t* cnt, hipStream_t s);

@@ -514,7 +514,7 @@ extern "C" int mts_moe_head_fwd(const void* x, const float* w_r, int64_t T, int 
                                           partial, cnt, s);
     if (rc) return rc;
     int blocks, rows_per_wave;
-    mts_router_head_geometry(T, &blocks, &rows_per_wave);
+    mts_router_head_geometry(T, mts_router_head_group(H, E, act_dtype), &blocks, &rows_per_wave);
     const int64_t rows_per_chunk = (int64_t)rows_per_wave * 4;
     const int64_t n_chunks = (T + rows_per_chunk - 1) / rows_per_chunk;
     if (n_chunks > kFinishChunks || E > kFinishMaxE) return MTS_ERR_SHAPE;   // cannot happen: the geometry caps the chunks, the projection E

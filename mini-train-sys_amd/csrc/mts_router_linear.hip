@@ -87,6 +87,189 @@ struct RowGroupLoader {
     }
 };
 
+// ---------------------------------------------------------------------------
+// The projection on the matrix pipe (bf16 activations, E <= 8).  An fp32 weight is the exact sum
+// of three bf16 terms (each takes the next 8 bits of the mantissa), a bf16 x times a bf16 term is
+// exact in fp32, so  x . w  =  x . t0 + x . t1 + x . t2  with fp32 accumulation is an fp32 dot
+// product in another order of summation.  The block splits W_r once into LDS, [term][expert][H]
+// bf16 = 24 rows; a wave takes 16 rows of x at a time as the N side of 16x16x32 MFMAs, and the 24
+// weight rows as the M side of two of them per k-step, ordered so that lane (n, q) of the
+// accumulators (row n of x, q = lane / 16) ends up with the three terms of experts 2q and 2q+1:
+//   first MFMA,  M rows 4q .. 4q+3:  (2q, t0) (2q, t1) (2q, t2) (2q+1, t0)
+//   second MFMA, M rows 4q .. 4q+3:  (2q+1, t1) (2q+1, t2) zero zero
+// A lane reads its row of x straight from memory, 16 bytes per k-step: the four lanes of a row
+// read 64 consecutive bytes, 768 columns of it in flight at once.
+// ---------------------------------------------------------------------------
+constexpr int kMmaRows = 16;          // rows of x per wave pass
+constexpr int kMmaSteps = 12;         // k-steps (of 32 columns) per register chunk: two chunks are in flight
+constexpr int kMmaTerms = 3;          // bf16 terms of an fp32 weight
+constexpr int kMmaMaxH = 2048;        // 24 x (H + 32) bf16 of LDS
+constexpr int kStageBatch = 6;        // weight quads a thread has in flight while it splits them
+constexpr uint32_t kOutOfRange = 0x80000000u;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+
+__host__ __device__ inline int mma_lds_stride(int H) { return H + 32; }   // elements: consecutive rows 16 banks apart when H % 128 == 0
+inline size_t mma_lds_bytes(int H) { return (size_t)kMmaTerms * 8 * mma_lds_stride(H) * sizeof(bf16_t); }
+inline bool mma_projection_ok(int H, int E, int act_dtype) {
+    static const bool off = getenv("MTS_NO_MFMA_ROUTER") != nullptr;
+    return !off && act_dtype == MTS_BF16 && E <= 8 && H % 32 == 0 && H <= kMmaMaxH;
+}
+
+// Every thread of the block: W_r [E][H] fp32 -> wb [3][8][stride] bf16 (experts past E are zeros).  The loads of a
+// batch are issued together (`mma_weights_load`), whatever the caller wants in flight behind them next, and the
+// split follows (`mma_weights_split`): returns are in order, so the weights must not queue behind rows of x.
+template <int NT>
+struct MmaWeights {
+    f32x4 v[kStageBatch];
+    __device__ __forceinline__ void load(const float* __restrict__ w, int H, int E, int batch) {
+        const int quads = H / 4;
+#pragma unroll
+        for (int u = 0; u < kStageBatch; ++u) {
+            const int i = threadIdx.x + (batch * kStageBatch + u) * NT;
+            const int e = i / quads, k = (i % quads) * 4;
+            const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+            v[u] = (i < 8 * quads && e < E) ? *reinterpret_cast<const f32x4*>(w + (int64_t)e * H + k) : z;
+        }
+    }
+    __device__ __forceinline__ void split(bf16_t* wb, int H, int batch) const {
+        const int quads = H / 4, stride = mma_lds_stride(H);
+#pragma unroll
+        for (int u = 0; u < kStageBatch; ++u) {
+            const int i = threadIdx.x + (batch * kStageBatch + u) * NT;
+            if (i >= 8 * quads) continue;
+            const int e = i / quads, k = (i % quads) * 4;
+            bf16x4 t0, t1, t2;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const float a = v[u][q];
+                t0[q] = (bf16_t)a;
+                const float r1 = a - (float)t0[q];   // exact
+                t1[q] = (bf16_t)r1;
+                const float r2 = r1 - (float)t1[q];  // exact, 8 bits or fewer are left
+                t2[q] = (bf16_t)r2;
+            }
+            *reinterpret_cast<bf16x4*>(wb + (0 * 8 + e) * stride + k) = t0;
+            *reinterpret_cast<bf16x4*>(wb + (1 * 8 + e) * stride + k) = t1;
+            *reinterpret_cast<bf16x4*>(wb + (2 * 8 + e) * stride + k) = t2;
+        }
+    }
+    static __device__ __forceinline__ int batches(int H) { return (8 * (H / 4) + kStageBatch * NT - 1) / (kStageBatch * NT); }
+};
+
+struct MmaRows {
+    __amdgpu_buffer_rsrc_t rsrc;   // the wave's rows r0 .. min(r0 + 16, end), so that rows past the end read as zeros
+    uint32_t row_off;
+};
+__device__ __forceinline__ MmaRows mma_rows(const bf16_t* x, int64_t r0, int64_t end, int H, int lane) {
+    // r0 and end are the same for the whole wave; say so, a descriptor lives in scalar registers
+    const int64_t first = ((int64_t)__builtin_amdgcn_readfirstlane((int)(r0 >> 32)) << 32) |
+                          (uint32_t)__builtin_amdgcn_readfirstlane((int)r0);
+    const int64_t left = end - r0 < kMmaRows ? end - r0 : kMmaRows;
+    const int rows = __builtin_amdgcn_readfirstlane((int)(left > 0 ? left : 0));
+    MmaRows m;
+    m.rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(x + first * H), 0, rows * H * 2, 0x00020000);
+    m.row_off = (uint32_t)(lane % 16) * (uint32_t)H * 2u;
+    return m;
+}
+// chunk `ch` of the lane's row: k-step j covers columns ch*384 + 32 j .. + 32, this lane's quarter at 8 (lane / 16)
+__device__ __forceinline__ void mma_load_chunk(u32x4 (&dst)[kMmaSteps], const MmaRows& m, int ch, int H, int lane) {
+#pragma unroll
+    for (int j = 0; j < kMmaSteps; ++j) {
+        const int col = (ch * kMmaSteps + j) * 32 + 8 * (lane / 16);
+        dst[j] = __builtin_amdgcn_raw_buffer_load_b128(m.rsrc, (int)(col < H ? m.row_off + (uint32_t)col * 2u : kOutOfRange), 0, 0);
+    }
+}
+// the LDS rows this lane reads as M row lane % 16 of the first and of the second MFMA (nullptr: a row of zeros)
+struct MmaLaneRows {
+    const bf16_t* first;
+    const bf16_t* second;
+};
+__device__ __forceinline__ MmaLaneRows mma_lane_rows(const bf16_t* wb, int H, int lane) {
+    const int stride = mma_lds_stride(H), m = lane % 16, q = m / 4, i = m % 4, k0 = 8 * (lane / 16);
+    MmaLaneRows r;
+    const int e1 = i == 3 ? 2 * q + 1 : 2 * q, t1 = i == 3 ? 0 : i;
+    r.first = wb + (t1 * 8 + e1) * stride + k0;
+    r.second = i < 2 ? wb + ((i + 1) * 8 + 2 * q + 1) * stride + k0 : nullptr;
+    return r;
+}
+__device__ __forceinline__ void mma_chunk(f32x4 (&acc)[2][2], const u32x4 (&cur)[kMmaSteps], const MmaLaneRows& rows, int ch,
+                                          int H) {
+#pragma unroll
+    for (int j = 0; j < kMmaSteps; ++j) {
+        const int col = (ch * kMmaSteps + j) * 32;
+        if (col < H) {   // wave-uniform
+            const bf16x8 a1 = *reinterpret_cast<const bf16x8*>(rows.first + col);
+            bf16x8 a2 = {};
+            if (rows.second) a2 = *reinterpret_cast<const bf16x8*>(rows.second + col);
+            const bf16x8 b = __builtin_bit_cast(bf16x8, cur[j]);
+            acc[j & 1][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, b, acc[j & 1][0], 0, 0, 0);
+            acc[j & 1][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a2, b, acc[j & 1][1], 0, 0, 0);
+        }
+    }
+}
+// Chunk number p of the wave's stream of chunks, counted from chunk 0 of the rows at r0: the wave's row groups lie
+// `step` rows apart and have nch chunks each.  Nothing is loaded past `end`.
+__device__ __forceinline__ void mma_prefetch(u32x4 (&dst)[kMmaSteps], const bf16_t* x, int64_t r0, int64_t step, int64_t end,
+                                             int H, int nch, int p, int lane) {
+    const int64_t rb = r0 + (p / nch) * step;
+    if (rb < end) mma_load_chunk(dst, mma_rows(x, rb, end, H, lane), p % nch, H, lane);
+}
+__device__ __forceinline__ int mma_chunks(int H) { return (H + kMmaSteps * 32 - 1) / (kMmaSteps * 32); }
+// logits of experts 2 (lane / 16) and 2 (lane / 16) + 1 of row r0 + lane % 16.  On entry `cur` and `nxt` hold chunks
+// 0 and 1 of the stream that starts at r0, on return those of the stream that starts at r0 + step.
+__device__ __forceinline__ void mma_project(float (&out)[2], u32x4 (&cur)[kMmaSteps], u32x4 (&nxt)[kMmaSteps], const bf16_t* x,
+                                            int64_t r0, int64_t step, int64_t end, int H, const bf16_t* wb, int lane) {
+    const int nch = mma_chunks(H);
+    const MmaLaneRows lrows = mma_lane_rows(wb, H, lane);
+    f32x4 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[0][0][i] = acc[0][1][i] = acc[1][0][i] = acc[1][1][i] = 0.f;
+    for (int ch = 0; ch < nch; ++ch) {
+        mma_chunk(acc, cur, lrows, ch, H);
+#pragma unroll
+        for (int j = 0; j < kMmaSteps; ++j) cur[j] = nxt[j];
+        mma_prefetch(nxt, x, r0, step, end, H, nch, ch + 2, lane);
+    }
+    // accumulator element i of lane (n, q): M row 4q + i
+    const f32x4 one = acc[0][0] + acc[1][0], two = acc[0][1] + acc[1][1];
+    out[0] = (one[2] + one[1]) + one[0];   // small terms first
+    out[1] = (two[1] + two[0]) + one[3];
+}
+
+// logits only: a wave takes every (waves)th group of 16 rows
+__global__ __launch_bounds__(kFwdThreads) void router_logits_mma_kernel(const bf16_t* __restrict__ x,
+                                                                         const float* __restrict__ w, int64_t T, int H,
+                                                                         int E, float* __restrict__ logits) {
+    extern __shared__ __attribute__((aligned(16))) float w_lds[];
+    bf16_t* wb = reinterpret_cast<bf16_t*>(w_lds);
+    const int lane = threadIdx.x % MTS_WAVE;
+    const int64_t stride = (int64_t)gridDim.x * (kFwdThreads / MTS_WAVE) * kMmaRows;
+    int64_t r0 = ((int64_t)blockIdx.x * (kFwdThreads / MTS_WAVE) + threadIdx.x / MTS_WAVE) * kMmaRows;
+    u32x4 cur[kMmaSteps], nxt[kMmaSteps];
+    MmaWeights<kFwdThreads> stage;
+    stage.load(w, H, E, 0);
+    mma_prefetch(cur, x, r0, stride, T, H, mma_chunks(H), 0, lane);
+    mma_prefetch(nxt, x, r0, stride, T, H, mma_chunks(H), 1, lane);
+    stage.split(wb, H, 0);
+    for (int b = 1; b < stage.batches(H); ++b) {
+        stage.load(w, H, E, b);
+        stage.split(wb, H, b);
+    }
+    __syncthreads();
+    for (; r0 < T; r0 += stride) {
+        float lg[2];
+        mma_project(lg, cur, nxt, x, r0, stride, T, H, wb, lane);
+        const int64_t row = r0 + lane % 16;
+        if (row < T) {
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                const int e = 2 * (lane / 16) + q;
+                if (e < E) logits[row * E + e] = lg[q];
+            }
+        }
+    }
+}
+
 template <typename XT, int EP, int PASSES, bool CHUNKED = false>
 __global__ __launch_bounds__(kFwdThreads) void router_logits_fwd_kernel(const XT* __restrict__ x,
                                                                          const float* __restrict__ w, int64_t T,
@@ -156,24 +339,40 @@ __global__ __launch_bounds__(kFwdThreads) void router_logits_fwd_kernel(const XT
 // statistics (fixed order) and the routes per expert, which are at the same time the chunk
 // histogram of the routing metadata (chunk = the entries of the block's rows).
 // ---------------------------------------------------------------------------
-template <typename XT, int EP, int PASSES, bool CHUNKED = false>
-__global__ __launch_bounds__(kFwdThreads) void router_head_kernel(
+template <typename XT, int EP, int PASSES, bool CHUNKED = false, bool MMA = false>
+__global__ __launch_bounds__(kFwdThreads, MMA ? 2 : 1) void router_head_kernel(
     const XT* __restrict__ x, const float* __restrict__ w, int64_t T, int H, int E, int K, int normalize,
     int rows_per_wave, int n_chunks, float* __restrict__ logits, float* __restrict__ weights, int32_t* __restrict__ indices,
     void* __restrict__ weights_act, int act_dtype, float* __restrict__ partial, int32_t* __restrict__ cnt) {
     using namespace mts_router;
-    extern __shared__ __attribute__((aligned(16))) float w_lds[];   // [E][H]
-#pragma unroll 8
-    for (int i = threadIdx.x * 4; i < E * H; i += kFwdThreads * 4)
-        *reinterpret_cast<f32x4*>(w_lds + i) = *reinterpret_cast<const f32x4*>(w + i);
+    static_assert(!MMA || (EP == 8 && sizeof(XT) == 2 && !CHUNKED), "the matrix-pipe projection: bf16 rows, up to 8 experts");
+    extern __shared__ __attribute__((aligned(16))) float w_lds[];   // [E][H] fp32, or the bf16 terms of the matrix-pipe path
     constexpr int WAVES = kFwdThreads / MTS_WAVE;
+    constexpr int GROUP = MMA ? kMmaRows : kRows;   // rows whose logits are complete together
     const int lane = threadIdx.x % MTS_WAVE, wave = threadIdx.x / MTS_WAVE;
     const int nch = CHUNKED ? n_chunks : 1;
     const int64_t beg = ((int64_t)blockIdx.x * WAVES + wave) * rows_per_wave;
     const int64_t end = beg + rows_per_wave < T ? beg + rows_per_wave : T;
     typedef RowGroupLoader<XT, PASSES> Loader;
     typename Loader::raw_t cur[PASSES][kRows], nxt[PASSES][kRows];
-    if (beg < end) Loader::load(cur, x, beg, end, 0, H, lane);
+    u32x4 mcur[MMA ? kMmaSteps : 1], mnxt[MMA ? kMmaSteps : 1];
+    if constexpr (MMA) {
+        // the first rows are on their way while the block splits the weights
+        MmaWeights<kFwdThreads> stage;
+        stage.load(w, H, E, 0);
+        mma_prefetch(mcur, reinterpret_cast<const bf16_t*>(x), beg, kMmaRows, end, H, mma_chunks(H), 0, lane);
+        mma_prefetch(mnxt, reinterpret_cast<const bf16_t*>(x), beg, kMmaRows, end, H, mma_chunks(H), 1, lane);
+        stage.split(reinterpret_cast<bf16_t*>(w_lds), H, 0);
+        for (int b = 1; b < stage.batches(H); ++b) {
+            stage.load(w, H, E, b);
+            stage.split(reinterpret_cast<bf16_t*>(w_lds), H, b);
+        }
+    } else {
+#pragma unroll 8
+        for (int i = threadIdx.x * 4; i < E * H; i += kFwdThreads * 4)
+            *reinterpret_cast<f32x4*>(w_lds + i) = *reinterpret_cast<const f32x4*>(w + i);
+        if (beg < end) Loader::load(cur, x, beg, end, 0, H, lane);
+    }
     __syncthreads();
 
     // The logits of up to 64 rows are parked in LDS (row stride EP + 1: a lane per row reads without
@@ -194,6 +393,21 @@ __global__ __launch_bounds__(kFwdThreads) void router_head_kernel(
     int ch = 0;
     float acc[kRows][EP];
     while (r0 < end) {
+        int64_t g0;   // the row group whose dot products are complete
+        if constexpr (MMA) {
+            float lg[2];
+            mma_project(lg, mcur, mnxt, reinterpret_cast<const bf16_t*>(x), r0, kMmaRows, end, H,
+                        reinterpret_cast<const bf16_t*>(w_lds), lane);
+            g0 = r0;
+            r0 += kMmaRows;
+            const int r = lane % 16;
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                const int e = 2 * (lane / 16) + q;
+                if (e < E && g0 + r < end) logits[(g0 + r) * E + e] = lg[q];
+                mine_rows[(int)(g0 - pass_base + r) * LROW + e] = e < E ? lg[q] : -INFINITY;
+            }
+        } else {
         const bool last = ch + 1 == nch;
         const int64_t nr0 = last ? r0 + kRows : r0;
         const int nc = last ? 0 : ch + 1;
@@ -209,7 +423,7 @@ __global__ __launch_bounds__(kFwdThreads) void router_head_kernel(
         for (int ps = 0; ps < PASSES; ++ps)
 #pragma unroll
             for (int r = 0; r < kRows; ++r) cur[ps][r] = nxt[ps][r];
-        const int64_t g0 = r0;   // the row group whose dot products are complete when `last`
+        g0 = r0;   // complete when `last`
         r0 = nr0;
         ch = nc;
         if (!last) continue;
@@ -229,7 +443,8 @@ __global__ __launch_bounds__(kFwdThreads) void router_head_kernel(
             if (writer && e < E && g0 + r < end) logits[(g0 + r) * E + e] = mine;
             if (writer) mine_rows[(int)(g0 - pass_base + r) * LROW + e] = e < E ? mine : -INFINITY;
         }
-        const int64_t parked_to = g0 + kRows < end ? g0 + kRows : end;
+        }
+        const int64_t parked_to = g0 + GROUP < end ? g0 + GROUP : end;
         if (parked_to - pass_base < MTS_WAVE && parked_to < end) continue;   // wave-uniform: park more rows first
         __builtin_amdgcn_wave_barrier();
         const int64_t row = pass_base + lane;
@@ -388,6 +603,15 @@ extern "C" int mts_router_logits_fwd(const void* x, const float* w_r, int64_t T,
     if (rc != MTS_OK) return rc;
     if (!logits) return MTS_ERR_NULL;
     hipStream_t s = (hipStream_t)stream;
+    if (mma_projection_ok(H, E, act_dtype)) {
+        int64_t nb = ((T + kMmaRows - 1) / kMmaRows + 3) / 4;
+        if (nb > 256 * 2) nb = 256 * 2;
+        const size_t bytes = mma_lds_bytes(H);
+        if (allow_lds(router_logits_mma_kernel, bytes) != hipSuccess) return MTS_ERR_SHAPE;
+        router_logits_mma_kernel<<<dim3((unsigned)nb), kFwdThreads, bytes, s>>>((const bf16_t*)x, w_r, T, H, E, logits);
+        MTS_CHECK_LAUNCH();
+        return MTS_OK;
+    }
     const int64_t groups = (T + kRows - 1) / kRows;
     int64_t blocks = (groups + 3) / 4;
     if (blocks > 256 * 2) blocks = 256 * 2;
@@ -426,12 +650,14 @@ extern "C" int mts_router_logits_fwd(const void* x, const float* w_r, int64_t T,
 
 // Geometry of the chained forward kernel: blocks, rows per wave (a multiple of kRows); a block's
 // rows are one chunk of the routing metadata.
-void mts_router_head_geometry(int64_t T, int* blocks, int* rows_per_wave) {
-    const int64_t groups = (T + kRows - 1) / kRows;
+int mts_router_head_group(int H, int E, int act_dtype) { return mma_projection_ok(H, E, act_dtype) ? kMmaRows : kRows; }
+
+void mts_router_head_geometry(int64_t T, int group, int* blocks, int* rows_per_wave) {
+    const int64_t groups = (T + group - 1) / group;
     int64_t b = (groups + 3) / 4;
     if (b > kHeadMaxBlocks) b = kHeadMaxBlocks;
     const int64_t waves = b * (kFwdThreads / MTS_WAVE);
-    const int64_t per_wave = ((T + waves - 1) / waves + kRows - 1) / kRows * kRows;
+    const int64_t per_wave = ((T + waves - 1) / waves + group - 1) / group * group;
     *blocks = (int)b;
     *rows_per_wave = (int)per_wave;
 }
@@ -444,8 +670,17 @@ int mts_launch_router_head(const void* x, const float* w_r, int64_t T, int H, in
     if (!logits || !weights || !indices || !partial || !cnt) return MTS_ERR_NULL;
     if (K < 1 || K > E || K > MTS_MAX_TOP_K) return MTS_ERR_SHAPE;
     int blocks, rows_per_wave;
-    mts_router_head_geometry(T, &blocks, &rows_per_wave);
+    mts_router_head_geometry(T, mts_router_head_group(H, E, act_dtype), &blocks, &rows_per_wave);
     const dim3 grid((unsigned)blocks);
+    if (mma_projection_ok(H, E, act_dtype)) {
+        const size_t bytes = mma_lds_bytes(H);
+        if (allow_lds(router_head_kernel<bf16_t, 8, 1, false, true>, bytes, 16 * 1024) != hipSuccess) return MTS_ERR_SHAPE;
+        router_head_kernel<bf16_t, 8, 1, false, true><<<grid, kFwdThreads, bytes, s>>>(
+            (const bf16_t*)x, w_r, T, H, E, K, normalize, rows_per_wave, 1, logits, weights, indices, weights_act, MTS_BF16,
+            partial, cnt);
+        MTS_CHECK_LAUNCH();
+        return MTS_OK;
+    }
     const size_t lds = (size_t)E * H * sizeof(float);
     const int passes = (H + MTS_WAVE * 4 - 1) / (MTS_WAVE * 4);
     const int n_chunks = (H + kChunkCols - 1) / kChunkCols;

@@ -27,6 +27,7 @@ CONFIGURATIONS = {
                                                               MTS_TILE_DW1="2", MTS_TILE_DW2="2", MTS_NO_JOINT_BWD="1"),
     "64-wide k-tiles for dX and the weight gradients on their own, every tile whole": dict(MTS_NO_JOINT_BWD="1",
                                                                                            MTS_NO_TAIL_SPLIT="1"),
+    "router projection on the vector pipe": dict(MTS_NO_MFMA_ROUTER="1"),
     "ranges per XCD, plain order, tail launches apart": dict(MTS_XCD_RANGES="1", MTS_NO_TILE_ORDER="1",
                                                              MTS_NO_TAIL_IN_JOINT="1"),
 }
