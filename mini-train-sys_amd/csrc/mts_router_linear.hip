@@ -98,7 +98,7 @@ struct RowGroupLoader {
 //   first MFMA,  M rows 4q .. 4q+3:  (2q, t0) (2q, t1) (2q, t2) (2q+1, t0)
 //   second MFMA, M rows 4q .. 4q+3:  (2q+1, t1) (2q+1, t2) zero zero
 // A lane reads its row of x straight from memory, 16 bytes per k-step: the four lanes of a row
-// read 64 consecutive bytes, 768 columns of it in flight at once.
+// read a 128-byte line in two k-steps, 768 columns of it in flight at once.
 // ---------------------------------------------------------------------------
 constexpr int kMmaRows = 16;          // rows of x per wave pass
 constexpr int kMmaSteps = 12;         // k-steps (of 32 columns) per register chunk: two chunks are in flight
@@ -112,7 +112,7 @@ __host__ __device__ inline int mma_lds_stride(int H) { return H + 32; }   // ele
 inline size_t mma_lds_bytes(int H) { return (size_t)kMmaTerms * 8 * mma_lds_stride(H) * sizeof(bf16_t); }
 inline bool mma_projection_ok(int H, int E, int act_dtype) {
     static const bool off = getenv("MTS_NO_MFMA_ROUTER") != nullptr;
-    return !off && act_dtype == MTS_BF16 && E <= 8 && H % 32 == 0 && H <= kMmaMaxH;
+    return !off && act_dtype == MTS_BF16 && E <= 8 && H % 64 == 0 && H <= kMmaMaxH;
 }
 
 // Every thread of the block: W_r [E][H] fp32 -> wb [3][8][stride] bf16 (experts past E are zeros).  The loads of a
@@ -156,6 +156,11 @@ struct MmaWeights {
     static __device__ __forceinline__ int batches(int H) { return (8 * (H / 4) + kStageBatch * NT - 1) / (kStageBatch * NT); }
 };
 
+// First column of the 8 that quarter q (= lane / 16) of a row contributes to k-step `step`.  Which 32 columns
+// make up a k-step is free as long as both operands agree: two consecutive k-steps share 64 columns and a
+// quarter's two pieces are adjacent, so the four lanes of a row ask for a whole 128-byte line in two loads.
+__device__ __forceinline__ int mma_col(int step, int q) { return 64 * (step / 2) + 16 * q + 8 * (step % 2); }
+
 struct MmaRows {
     __amdgpu_buffer_rsrc_t rsrc;   // the wave's rows r0 .. min(r0 + 16, end), so that rows past the end read as zeros
     uint32_t row_off;
@@ -171,11 +176,11 @@ __device__ __forceinline__ MmaRows mma_rows(const bf16_t* x, int64_t r0, int64_t
     m.row_off = (uint32_t)(lane % 16) * (uint32_t)H * 2u;
     return m;
 }
-// chunk `ch` of the lane's row: k-step j covers columns ch*384 + 32 j .. + 32, this lane's quarter at 8 (lane / 16)
+// chunk `ch` of the lane's row: k-steps ch*12 .. ch*12 + 11, see mma_col
 __device__ __forceinline__ void mma_load_chunk(u32x4 (&dst)[kMmaSteps], const MmaRows& m, int ch, int H, int lane) {
 #pragma unroll
     for (int j = 0; j < kMmaSteps; ++j) {
-        const int col = (ch * kMmaSteps + j) * 32 + 8 * (lane / 16);
+        const int col = mma_col(ch * kMmaSteps + j, lane / 16);
         dst[j] = __builtin_amdgcn_raw_buffer_load_b128(m.rsrc, (int)(col < H ? m.row_off + (uint32_t)col * 2u : kOutOfRange), 0, 0);
     }
 }
@@ -185,7 +190,7 @@ struct MmaLaneRows {
     const bf16_t* second;
 };
 __device__ __forceinline__ MmaLaneRows mma_lane_rows(const bf16_t* wb, int H, int lane) {
-    const int stride = mma_lds_stride(H), m = lane % 16, q = m / 4, i = m % 4, k0 = 8 * (lane / 16);
+    const int stride = mma_lds_stride(H), m = lane % 16, q = m / 4, i = m % 4, k0 = 16 * (lane / 16);
     MmaLaneRows r;
     const int e1 = i == 3 ? 2 * q + 1 : 2 * q, t1 = i == 3 ? 0 : i;
     r.first = wb + (t1 * 8 + e1) * stride + k0;
@@ -196,8 +201,8 @@ __device__ __forceinline__ void mma_chunk(f32x4 (&acc)[2][2], const u32x4 (&cur)
                                           int H) {
 #pragma unroll
     for (int j = 0; j < kMmaSteps; ++j) {
-        const int col = (ch * kMmaSteps + j) * 32;
-        if (col < H) {   // wave-uniform
+        const int col = mma_col(ch * kMmaSteps + j, 0);   // the lane's quarter is part of its row pointers
+        if (col < H) {   // wave-uniform: H is a multiple of 64
             const bf16x8 a1 = *reinterpret_cast<const bf16x8*>(rows.first + col);
             bf16x8 a2 = {};
             if (rows.second) a2 = *reinterpret_cast<const bf16x8*>(rows.second + col);

@@ -32,7 +32,7 @@ def _case(T, H, E, dtype, seed):
 
 @pytest.mark.parametrize("T,H,E", [(1, 64, 4), (5, 64, 3), (257, 768, 8), (1000, 1024, 16), (4096, 768, 8), (24576, 768, 8),
                                    (300, 4096, 8), (1000, 2048, 16), (513, 1280, 8), (100, 3072, 5), (64, 2052, 8),
-                                   # bf16 rows, up to 8 experts, H % 32 == 0 and H <= 2048: the projection on the matrix pipe;
+                                   # bf16 rows, up to 8 experts, H % 64 == 0 and H <= 2048: the projection on the matrix pipe;
                                    # several register chunks per row, more groups of 16 rows than waves
                                    (40000, 1024, 7), (333, 2048, 8)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
