@@ -92,7 +92,7 @@ struct RowGroupLoader {
 // of three bf16 terms (each takes the next 8 bits of the mantissa), a bf16 x times a bf16 term is
 // exact in fp32, so  x . w  =  x . t0 + x . t1 + x . t2  with fp32 accumulation is an fp32 dot
 // product in another order of summation.  The block splits W_r once into LDS, [term][expert][H]
-// bf16 = 24 rows; a wave takes 16 rows of x at a time as the N side of 16x16x32 MFMAs, and the 24
+// bf16 = 24 rows (and one of zeros); a wave takes 16 rows of x at a time as the N side of 16x16x32 MFMAs, and the 24
 // weight rows as the M side of two of them per k-step, ordered so that lane (n, q) of the
 // accumulators (row n of x, q = lane / 16) ends up with the three terms of experts 2q and 2q+1:
 //   first MFMA,  M rows 4q .. 4q+3:  (2q, t0) (2q, t1) (2q, t2) (2q+1, t0)
@@ -103,19 +103,19 @@ struct RowGroupLoader {
 constexpr int kMmaRows = 16;          // rows of x per wave pass
 constexpr int kMmaSteps = 12;         // k-steps (of 32 columns) per register chunk: two chunks are in flight
 constexpr int kMmaTerms = 3;          // bf16 terms of an fp32 weight
-constexpr int kMmaMaxH = 2048;        // 24 x (H + 32) bf16 of LDS
+constexpr int kMmaMaxH = 2048;        // 25 x (H + 32) bf16 of LDS
 constexpr int kStageBatch = 6;        // weight quads a thread has in flight while it splits them
 constexpr uint32_t kOutOfRange = 0x80000000u;
 typedef __attribute__((ext_vector_type(2))) float f32x2;
 
 __host__ __device__ inline int mma_lds_stride(int H) { return H + 32; }   // elements: consecutive rows 16 banks apart when H % 128 == 0
-inline size_t mma_lds_bytes(int H) { return (size_t)kMmaTerms * 8 * mma_lds_stride(H) * sizeof(bf16_t); }
+inline size_t mma_lds_bytes(int H) { return (size_t)(kMmaTerms * 8 + 1) * mma_lds_stride(H) * sizeof(bf16_t); }   // + a row of zeros
 inline bool mma_projection_ok(int H, int E, int act_dtype) {
     static const bool off = getenv("MTS_NO_MFMA_ROUTER") != nullptr;
     return !off && act_dtype == MTS_BF16 && E <= 8 && H % 64 == 0 && H <= kMmaMaxH;
 }
 
-// Every thread of the block: W_r [E][H] fp32 -> wb [3][8][stride] bf16 (experts past E are zeros).  The loads of a
+// Every thread of the block: W_r [E][H] fp32 -> wb [3][8][stride] bf16 (experts past E are zeros), then a row of zeros.  The loads of a
 // batch are issued together (`mma_weights_load`), whatever the caller wants in flight behind them next, and the
 // split follows (`mma_weights_split`): returns are in order, so the weights must not queue behind rows of x.
 template <int NT>
@@ -133,6 +133,10 @@ struct MmaWeights {
     }
     __device__ __forceinline__ void split(bf16_t* wb, int H, int batch) const {
         const int quads = H / 4, stride = mma_lds_stride(H);
+        if (batch == 0) {   // the row of zeros that stands in for the M rows no term maps to
+            const bf16x4 z = {};
+            for (int k = threadIdx.x * 4; k < H; k += NT * 4) *reinterpret_cast<bf16x4*>(wb + kMmaTerms * 8 * stride + k) = z;
+        }
 #pragma unroll
         for (int u = 0; u < kStageBatch; ++u) {
             const int i = threadIdx.x + (batch * kStageBatch + u) * NT;
@@ -184,7 +188,7 @@ __device__ __forceinline__ void mma_load_chunk(u32x4 (&dst)[kMmaSteps], const Mm
         dst[j] = __builtin_amdgcn_raw_buffer_load_b128(m.rsrc, (int)(col < H ? m.row_off + (uint32_t)col * 2u : kOutOfRange), 0, 0);
     }
 }
-// the LDS rows this lane reads as M row lane % 16 of the first and of the second MFMA (nullptr: a row of zeros)
+// the LDS rows this lane reads as M row lane % 16 of the first and of the second MFMA
 struct MmaLaneRows {
     const bf16_t* first;
     const bf16_t* second;
@@ -194,23 +198,28 @@ __device__ __forceinline__ MmaLaneRows mma_lane_rows(const bf16_t* wb, int H, in
     MmaLaneRows r;
     const int e1 = i == 3 ? 2 * q + 1 : 2 * q, t1 = i == 3 ? 0 : i;
     r.first = wb + (t1 * 8 + e1) * stride + k0;
-    r.second = i < 2 ? wb + ((i + 1) * 8 + 2 * q + 1) * stride + k0 : nullptr;
+    r.second = wb + (i < 2 ? (i + 1) * 8 + 2 * q + 1 : kMmaTerms * 8) * stride + k0;   // row 24 holds zeros
     return r;
 }
-__device__ __forceinline__ void mma_chunk(f32x4 (&acc)[2][2], const u32x4 (&cur)[kMmaSteps], const MmaLaneRows& rows, int ch,
-                                          int H) {
+template <bool WHOLE>   // WHOLE: all k-steps of the chunk lie inside the row, no test per step (the fragment reads can then run ahead)
+__device__ __forceinline__ void mma_chunk_steps(f32x4 (&acc)[2][2], const u32x4 (&cur)[kMmaSteps], const MmaLaneRows& rows,
+                                                int ch, int H) {
 #pragma unroll
     for (int j = 0; j < kMmaSteps; ++j) {
         const int col = mma_col(ch * kMmaSteps + j, 0);   // the lane's quarter is part of its row pointers
-        if (col < H) {   // wave-uniform: H is a multiple of 64
+        if (WHOLE || col < H) {   // wave-uniform: H is a multiple of 64
             const bf16x8 a1 = *reinterpret_cast<const bf16x8*>(rows.first + col);
-            bf16x8 a2 = {};
-            if (rows.second) a2 = *reinterpret_cast<const bf16x8*>(rows.second + col);
+            const bf16x8 a2 = *reinterpret_cast<const bf16x8*>(rows.second + col);
             const bf16x8 b = __builtin_bit_cast(bf16x8, cur[j]);
             acc[j & 1][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, b, acc[j & 1][0], 0, 0, 0);
             acc[j & 1][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a2, b, acc[j & 1][1], 0, 0, 0);
         }
     }
+}
+__device__ __forceinline__ void mma_chunk(f32x4 (&acc)[2][2], const u32x4 (&cur)[kMmaSteps], const MmaLaneRows& rows, int ch,
+                                          int H) {
+    if ((ch + 1) * kMmaSteps * 32 <= H) mma_chunk_steps<true>(acc, cur, rows, ch, H);
+    else mma_chunk_steps<false>(acc, cur, rows, ch, H);
 }
 // Chunk number p of the wave's stream of chunks, counted from chunk 0 of the rows at r0: the wave's row groups lie
 // `step` rows apart and have nch chunks each.  Nothing is loaded past `end`.
