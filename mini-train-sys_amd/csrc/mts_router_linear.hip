@@ -1,7 +1,8 @@
 // Router projection around the post-process kernels: logits = float(x) W_r^T in fp32 and its
 // backward (dx in the activation dtype, dW_r in fp32).  x is read in its own dtype, so no fp32
 // copy of the activations is made; every sum runs in a fixed order (no float atomics).
-// All three kernels are VALU/HBM bound: 2*T*H*E FLOP forward, twice that backward.
+// 2*T*H*E FLOP forward, twice that backward: the backward kernels and the forward ones for fp16 / fp32 rows
+// run them on the vector pipe; bf16 rows with up to 8 experts take the forward product to the matrix pipe.
 #include "mts_common.h"
 #include "mts_router_row.h"
 #include "mts_router_bwd_block.h"
