@@ -25,6 +25,7 @@ constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / MTS_WAVE;
 constexpr int kChunk = 256;   // entries per wave
 constexpr int kSteps = kChunk / MTS_WAVE;
+constexpr int kFewExperts = 8;   // windows up to this many experts are ranked with one ballot per expert
 
 // Expert ids >= E are a caller error; they are clamped so that no address derived from
 // them can leave the output arrays.  Negative ids (dropped routes) stay negative.
@@ -158,11 +159,41 @@ __device__ __forceinline__ void scatter_load(int (&ev)[kSteps], const int32_t* _
     }
 }
 
-__device__ __forceinline__ void scatter_place(const int (&ev)[kSteps], int K, int64_t base, int64_t cend,
+__device__ __forceinline__ void scatter_place(const int (&ev)[kSteps], int K, int EW, int64_t base, int64_t cend,
                                               volatile int32_t* next, int32_t* __restrict__ s_scatter,
                                               int32_t* __restrict__ s_reverse, int32_t* __restrict__ x_gather) {
     const int lane = threadIdx.x % MTS_WAVE;
     const uint64_t lt = lanemask_lt();
+    if (EW <= kFewExperts) {   // wave-uniform
+        // A window of few experts: one ballot per expert ranks the 64 entries of a step, and the next free rows
+        // stay in registers from step to step (the same positions as the loop over the experts present below:
+        // entries of one expert in lane order).
+        int32_t nx[kFewExperts];
+#pragma unroll
+        for (int x = 0; x < kFewExperts; ++x) nx[x] = x < EW ? next[x] : 0;
+#pragma unroll
+        for (int s = 0; s < kSteps; ++s) {
+            const int64_t n = base + s * MTS_WAVE + lane;
+            if (base + s * MTS_WAVE >= cend) break;   // wave-uniform
+            const int e = ev[s];
+            int pos = -1;
+#pragma unroll
+            for (int x = 0; x < kFewExperts; ++x) {
+                const uint64_t same = __ballot(e == x);
+                if (e == x) pos = nx[x] + __popcll(same & lt);
+                nx[x] += __popcll(same);
+            }
+            if (e >= -1 && n < cend) s_reverse[n] = pos;
+            if (e >= 0) {
+                s_scatter[pos] = (int32_t)n;
+                x_gather[pos] = (int32_t)(n / K);
+            }
+        }
+#pragma unroll
+        for (int x = 0; x < kFewExperts; ++x)
+            if (lane == x && x < EW) next[x] = nx[x];
+        return;
+    }
 #pragma unroll
     for (int s = 0; s < kSteps; ++s) {
         const int64_t n = base + s * MTS_WAVE + lane;
@@ -193,11 +224,11 @@ __device__ __forceinline__ void scatter_chunk(int (&first)[kSteps], const int32_
                                               int EW, int64_t cbeg, int64_t cend, volatile int32_t* next,
                                               int32_t* __restrict__ s_scatter, int32_t* __restrict__ s_reverse,
                                               int32_t* __restrict__ x_gather) {
-    scatter_place(first, K, cbeg, cend, next, s_scatter, s_reverse, x_gather);
+    scatter_place(first, K, EW, cbeg, cend, next, s_scatter, s_reverse, x_gather);
     for (int64_t base = cbeg + kChunk; base < cend; base += kChunk) {
         int ev[kSteps];
         scatter_load(ev, idx, E, e0, EW, base, cend);
-        scatter_place(ev, K, base, cend, next, s_scatter, s_reverse, x_gather);
+        scatter_place(ev, K, EW, base, cend, next, s_scatter, s_reverse, x_gather);
     }
 }
 
@@ -315,60 +346,44 @@ __global__ __launch_bounds__(kThreads) void head_scatter_kernel(
         scatter_chunk(first_ids, idx, K, E, 0, E, cbeg, cend, next, s_scatter, s_reverse, x_gather);
         return;
     }
-    // the last block: thread t holds chunks t and t + kThreads of every column
+    // the last block: wave w sums columns w, w + kWaves, ... of the partials (and, for an expert's column, its
+    // route counts); a lane takes chunks lane, lane + 64, ..., all of them requested before the first sum
     __shared__ mts_router::StatsShared sh;
-    __shared__ float col_part[kWaves][kFinishMaxE + 2];
-    __shared__ int32_t tot_part[kWaves][kFinishMaxE];
     __shared__ int32_t total_s[kFinishMaxE];
-    float colv[kFinishMaxE + 2];
-    int32_t totv[kFinishMaxE];
+    static_assert(kFinishChunks % MTS_WAVE == 0, "whole rounds of lanes over the chunks");
+    constexpr int ROUNDS = kFinishChunks / MTS_WAVE;
+    constexpr int COLS = (kFinishMaxE + 2 + kWaves - 1) / kWaves;   // columns per wave, at most
+    float colv[COLS][ROUNDS];
+    int32_t totv[COLS][ROUNDS];
 #pragma unroll
-    for (int j = 0; j < kFinishMaxE + 2; ++j) {
-        float v = 0.f;
-        if (j < E + 2) {
-            const int c0 = threadIdx.x, c1 = threadIdx.x + kThreads;
-            const float a = c0 < n_chunks ? partial[(int64_t)c0 * (E + 2) + j] : 0.f;
-            const float b = c1 < n_chunks ? partial[(int64_t)c1 * (E + 2) + j] : 0.f;
-            v = a + b;
-        }
-        colv[j] = v;
-    }
+    for (int q = 0; q < COLS; ++q) {
+        const int i = wave + q * kWaves;
 #pragma unroll
-    for (int e = 0; e < kFinishMaxE; ++e) {
-        int32_t v = 0;
-        if (e < E) {
-            const int c0 = threadIdx.x, c1 = threadIdx.x + kThreads;
-            v = (c0 < n_chunks ? cnt[(int64_t)c0 * E + e] : 0) + (c1 < n_chunks ? cnt[(int64_t)c1 * E + e] : 0);
-        }
-        totv[e] = v;
-    }
-#pragma unroll
-    for (int j = 0; j < kFinishMaxE + 2; ++j) {
-        if (j < E + 2) {   // block-uniform
-            const float v = wave_sum(colv[j]);
-            if (lane == 0) col_part[wave][j] = v;
+        for (int u = 0; u < ROUNDS; ++u) {
+            const int c = lane + u * MTS_WAVE;
+            colv[q][u] = (i < E + 2 && c < n_chunks) ? partial[(int64_t)c * (E + 2) + i] : 0.f;
+            totv[q][u] = (i < E && c < n_chunks) ? cnt[(int64_t)c * E + i] : 0;
         }
     }
 #pragma unroll
-    for (int e = 0; e < kFinishMaxE; ++e) {
-        if (e < E) {
-            int32_t v = totv[e];
+    for (int q = 0; q < COLS; ++q) {
+        const int i = wave + q * kWaves;
+        if (i < E + 2) {   // wave-uniform
+            float v = 0.f;
+            int32_t c = 0;
 #pragma unroll
-            for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, MTS_WAVE);
-            if (lane == 0) tot_part[wave][e] = v;
-        }
-    }
-    __syncthreads();
-    if (threadIdx.x < E + 2) {
-        float v = 0.f;
-        int32_t c = 0;
+            for (int u = 0; u < ROUNDS; ++u) {
+                v += colv[q][u];
+                c += totv[q][u];
+            }
+            v = wave_sum(v);
 #pragma unroll
-        for (int w = 0; w < kWaves; ++w) {
-            v += col_part[w][threadIdx.x];
-            if (threadIdx.x < E) c += tot_part[w][threadIdx.x];
+            for (int o = 32; o > 0; o >>= 1) c += __shfl_xor(c, o, MTS_WAVE);
+            if (lane == 0) {
+                if (i < E) total_s[i] = c;
+                mts_router::stats_column(sh, i, v * inv_t, c, E, inv_routes, prob_mean, z_loss, entropy, counts);
+            }
         }
-        if (threadIdx.x < E) total_s[threadIdx.x] = c;
-        mts_router::stats_column(sh, threadIdx.x, v * inv_t, c, E, inv_routes, prob_mean, z_loss, entropy, counts);
     }
     __syncthreads();
     if (wave == kWaves - 1) {   // exclusive scan of the routes per expert: one lane per expert
