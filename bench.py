@@ -45,8 +45,8 @@ RIDGE_FLOP_PER_BYTE = PEAK_BF16_TFLOPS * 1e12 / (PEAK_HBM_GBS * 1e9)   # 312.5: 
 # line names the file that holds the runs' commands and tables.
 TRAFFIC_SOURCE = "profiles/moe_layer_24x1024_hbm_traffic.txt"
 MEASURED_TRAFFIC_BYTES = {
-    "fwd_gateup_swiglu": 546.9e6, "fwd_down": 224.1e6, "bwd_dy1": 540.3e6,
-    "bwd_joint": 1228.4e6,   # the joint launch (1063.3) and the launch of partial sums with the dX combine behind it (165.1)
+    "fwd_gateup_swiglu": 546.9e6, "fwd_down": 224.1e6, "bwd_dy1": 539.7e6,
+    "bwd_joint": 1232.3e6,   # the joint launch (1067.2) and the launch of partial sums with the dX combine behind it (165.1)
     "combine": 114.6e6,
 }
 
