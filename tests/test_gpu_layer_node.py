@@ -43,7 +43,9 @@ def _head(lib, x, w_r, K, normalize):
     (257, 1024, 16, 4, torch.bfloat16, True), (3000, 192, 3, 3, torch.float32, True), (2047, 72, 12, 8, torch.float16, True),
     (98304, 768, 8, 2, torch.bfloat16, True), (700, 256, 16, 1, torch.float32, False),
     # rows wider than a wave holds in registers: column chunks forward, column ranges backward
-    (4096, 4096, 8, 2, torch.bfloat16, True), (333, 2048, 16, 2, torch.float16, True), (130, 1280, 5, 2, torch.float32, True)])
+    (4096, 4096, 8, 2, torch.bfloat16, True), (333, 2048, 16, 2, torch.float16, True), (130, 1280, 5, 2, torch.float32, True),
+    # the widest rows the matrix-pipe projection takes (several register chunks per row, 104 KiB of weight terms in LDS)
+    (300, 2048, 8, 2, torch.bfloat16, True), (1000, 1280, 6, 3, torch.bfloat16, False)])
 def test_chained_head_equals_the_three_operators(T, H, E, K, dtype, normalize):
     print(f"head T={T} H={H} E={E} K={K} {dtype} normalize={normalize}", flush=True)
     from minitrain_amd import _lib
