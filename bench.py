@@ -13,6 +13,10 @@ One JSON line is printed.  Besides the whole-layer tokens/s it carries
   * ``roofline``: the same figures for the stage that takes the most time;
   * ``gemm_roofline`` / ``combine_roofline``: all expert GEMMs together against the
     dense bf16 MFMA peak, and the combine kernels against peak HBM bandwidth;
+  * ``configs``: the other benchmark workloads, each a short run of its own: the headline layer through the
+    unchanged two-method operator protocol (no extension hooks), the 98304-token batch with its peak
+    allocation, Zipf-imbalanced routing with exact ties, and the 12-layer decoder's training step with the
+    MoE share of it;
   * ``cpu_baseline``: the CPU restatement of the reference's PyTorch path timed on
     the host cores of the same box on a bounded sample of the same workload.
 """
@@ -65,10 +69,19 @@ def make_inputs(seed, T, H, E, I):
 
 
 class Layer:
-    """The layer as the MoE block runs it, with leaves that collect gradients."""
+    """The layer as the MoE block runs it, with leaves that collect gradients.
 
-    def __init__(self, ops, x, w_r, w1, w2, g, K):
+    ``protocol_only``: the step goes through the two methods of the reference's operator protocol alone
+    (`router_postprocess`, `fused_moe`) with `F.linear` for the logits, `torch.bincount` for the route counts
+    and autograd's own sum of the two gradients of `x`, i.e. what an unmodified `minitrain/model` MoE block
+    costs (minitrain/model/moe_router.py:63-144, blocks.py:86-102); none of the backend's extension hooks
+    (`moe_layer`, `router_logits`, the counts and casts inside the post-process) is used.
+    ``logit_transform``: applied to the logits before the post-process (the imbalanced-routing workload);
+    it takes the layer off the one-node path, which forms the logits itself."""
+
+    def __init__(self, ops, x, w_r, w1, w2, g, K, protocol_only=False, logit_transform=None):
         self.ops, self.K = ops, K
+        self.protocol_only, self.logit_transform = protocol_only, logit_transform
         self.x = x.cuda().bfloat16().requires_grad_(True)
         self.w_r = w_r.cuda().requires_grad_(True)
         self.w1 = w1.cuda().bfloat16().requires_grad_(True)
@@ -78,30 +91,36 @@ class Layer:
         self.seed_aux = torch.tensor(0.01, device="cuda")    # router_aux_loss_coef (minitrain/model/config.py:20)
         self.seed_z = torch.tensor(0.001, device="cuda")     # router_z_loss_coef (config.py:21)
 
+    def hook(self, name):
+        return None if self.protocol_only else getattr(self.ops, name, None)
+
     def step(self):
         for t in (self.x, self.w_r, self.w1, self.w2):
             t.grad = None
         # as the MoE block does: a backend that offers the whole layer as one node is asked first
-        layer = getattr(self.ops, "moe_layer", None)
+        layer = self.hook("moe_layer") if self.logit_transform is None else None
         whole = layer(self.x, self.w_r, self.w1, self.w2, self.K, normalize=True) if layer is not None else None
         if whole is not None:
             out, aux, z_loss = whole[:3]
             torch.autograd.backward([out, aux, z_loss], [self.g, self.seed_aux, self.seed_z])
             return out
-        fused = getattr(self.ops, "router_logits", None)
+        fused = self.hook("router_logits")
         logits = fused(self.x, self.w_r) if fused is not None else None
         if logits is None:
             logits = F.linear(self.x.float(), self.w_r)
+        if self.logit_transform is not None:
+            logits = self.logit_transform(logits)
         # as the router module does: the backend may hand back the weights in the activation dtype itself
-        extra = {"weights_dtype": self.x.dtype} if getattr(self.ops, "casts_router_weights", False) else {}
+        extra = {"weights_dtype": self.x.dtype} if self.hook("casts_router_weights") else {}
         route = self.ops.router_postprocess(logits, self.K, normalize=True, **extra)
-        aux = getattr(route, "load_balance_loss", None)
+        aux = None if self.protocol_only else getattr(route, "load_balance_loss", None)
         if aux is None:
             counts = torch.bincount(route.expert_indices.flatten().long(), minlength=self.E)
             aux = self.E * torch.sum(counts.float() / route.expert_indices.numel() * route.probability_per_expert)
-        weights = getattr(route, "expert_weights_cast", None)
+        weights = None if self.protocol_only else getattr(route, "expert_weights_cast", None)
         if weights is None:
             weights = route.expert_weights.to(self.x.dtype)
+        self.last_indices = route.expert_indices
         out = self.ops.fused_moe(self.x, self.w1, self.w2, route.expert_indices, weights)
         # loss = sum(out * G) + 0.01 * aux + 0.001 * z: its gradient enters as the three seeds G, 0.01 and
         # 0.001, so the scalar itself (a few 5 us element-wise launches on 0-dim tensors) is not formed
@@ -266,6 +285,87 @@ def mfma_sustained(blocks=512, rounds=1000, launches=40, lead=10):
     return out
 
 
+def zipf_ties_transform(T, E, seed, s=1.2, tie_fraction=0.01):
+    """The imbalanced-routing workload: log p_e is added to the logits, p_e ~ rank^-s over the experts, and on a
+    seeded `tie_fraction` of the tokens two or three logits are overwritten with one value above the row's
+    maximum (exact ties for rank 1/2, for rank 2/3 behind a clear winner, and three-way, in turn)."""
+    rank = np.arange(1, E + 1, dtype=np.float64) ** (-s)
+    bias = torch.from_numpy(np.log(rank / rank.sum()).astype(np.float32)).cuda()
+    rng = np.random.Generator(np.random.Philox(seed + 1000))
+    rows = rng.choice(T, size=max(1, int(round(tie_fraction * T))), replace=False)
+    mask = np.zeros((T, E), dtype=bool)
+    lift = np.zeros((T, E), dtype=np.float32)
+    for j, t in enumerate(rows):
+        cols = rng.choice(E, size=3, replace=False)
+        kind = j % 3
+        picked = cols[:2] if kind == 0 else cols
+        mask[t, picked] = True
+        lift[t, picked] = 1.0
+        if kind == 1:
+            lift[t, cols[0]] = 2.0
+    mask, lift = torch.from_numpy(mask).cuda(), torch.from_numpy(lift).cuda()
+
+    def transform(logits):
+        biased = logits + bias
+        top = biased.detach().amax(dim=1, keepdim=True)
+        return torch.where(mask, top + lift, biased)
+
+    transform.tied_tokens = int(len(rows))
+    return transform
+
+
+def run_config(ops, seed, T, steps, warmup, **layer_kwargs):
+    """tokens/s and peak allocation of one more workload of the same layer shape."""
+    w = WORKLOAD
+    transform = layer_kwargs.pop("transform_factory", None)
+    if transform is not None:
+        layer_kwargs["logit_transform"] = transform(T, w["E"], seed)
+    layer = Layer(ops, *make_inputs(seed, T, w["H"], w["E"], w["I"]), w["K"], **layer_kwargs)
+    torch.cuda.synchronize()
+    resident = torch.cuda.memory_allocated()
+    settle(layer, seconds=0.2, at_least=10)
+    torch.cuda.reset_peak_memory_stats()
+    sec = time_layer(layer, steps, warmup)
+    rec = {"tokens": T, "seed": seed, "ms_per_step": round(sec * 1e3, 4), "tokens_per_s": round(T / sec, 1),
+           "layer_gemm_tflops": round(18.0 * T * w["K"] * w["H"] * w["I"] / sec / 1e12, 2),
+           "peak_hbm_allocated_mb": round(torch.cuda.max_memory_allocated() / 2**20, 1),
+           "resident_inputs_mb": round(resident / 2**20, 1)}
+    idx = getattr(layer, "last_indices", None)
+    if idx is not None and transform is not None:
+        counts = torch.bincount(idx.flatten().long(), minlength=w["E"]).float()
+        rec["top_expert_share"] = round(float(counts.max() / counts.sum()), 4)
+        rec["tied_tokens"] = layer.logit_transform.tied_tokens
+    del layer
+    torch.cuda.empty_cache()
+    return rec
+
+
+def other_configs(ops, steps, warmup):
+    """The benchmark workloads besides the headline one, each a short run of its own: the headline layer through
+    the unchanged operator protocol, the 98304-token batch with its peak allocation, imbalanced routing with
+    exact ties, and the 12-layer decoder's training step with the MoE share of it."""
+    w = WORKLOAD
+    out = {}
+    out["layer_24x1024_protocol_only"] = dict(
+        run_config(ops, w["seed"], w["T"], steps, warmup, protocol_only=True),
+        path="F.linear + OpsBackend.router_postprocess + torch.bincount + OpsBackend.fused_moe, autograd sums dx; no extension hooks")
+    out["layer_96x1024"] = dict(run_config(ops, 2, 98304, max(3, steps // 2), max(1, warmup // 2)), path="one autograd node (as the headline)")
+    out["layer_24x1024_zipf_ties"] = dict(
+        run_config(ops, 3, w["T"], steps, warmup, transform_factory=zipf_ties_transform),
+        path="router_logits hook + bias and ties (torch) + router_postprocess + fused_moe")
+    from minitrain_amd.train.bench_step import run as decoder_step
+
+    rec = decoder_step(steps=5, warmup=4)
+    out["decoder_12layer_24x1024"] = {
+        "tokens_per_s": round(rec["value"], 1), "ms_per_step": round(rec["ms_per_step"], 3),
+        "moe_ms_per_step": round(rec["moe_ms_per_step"], 3), "moe_share_of_step": round(rec["moe_share_of_step"], 4),
+        "parameters": rec["parameters"], "peak_hbm_allocated_mb": round(rec["peak_allocated_gib"] * 1024, 1),
+        "ms_per_step_mean": round(rec["ms_per_step_mean"], 3), "timing": "median of the timed steps (each ends with the host reading the loss)",
+        "steps": 5, "warmup": 4, "dtype": "bf16 autocast, fp32 parameters, AdamW", "seed": 4}
+    torch.cuda.empty_cache()
+    return out
+
+
 def cpu_baseline(budget_s=20.0):
     """The oracle's restatement of the reference's PyTorch path (input-dtype arithmetic,
     autograd backward) on the host cores, on the first ``sample`` tokens of the workload."""
@@ -304,6 +404,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-breakdown", action="store_true")
     ap.add_argument("--no-mfma-probe", action="store_true", help="skip the register-only MFMA rate probe")
+    ap.add_argument("--no-configs", action="store_true", help="skip the workloads besides the headline one (`configs` in the line)")
     ap.add_argument("--no-settle", action="store_true", help="skip the untimed clock-settling steps before the warm-up")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 256 MiB -> 256 MiB elementwise copy (the known-size kernel that "
@@ -381,6 +482,10 @@ def main():
             torch.mul(src, 1.0, out=dst)
         torch.cuda.synchronize()
         result["copy_probe_bytes_each_way"] = src.numel() * 4
+    if not args.no_configs:
+        del layer
+        torch.cuda.empty_cache()
+        result["configs"] = other_configs(ops, max(5, min(args.steps, 20)), max(2, min(args.warmup, 5)))
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline()
     print(json.dumps(result))

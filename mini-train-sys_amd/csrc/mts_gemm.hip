@@ -28,6 +28,7 @@
 #include "mts_common.h"
 #include "mts_router_bwd_block.h"
 #include "mts_combine_block.h"
+#include "mts_tuning.h"
 
 #include <stdlib.h>
 
@@ -1839,9 +1840,9 @@ __global__ __launch_bounds__(WsLarge::NT, WsLarge::WAVES_PER_EU) void bwd_joint_
 // host side
 // ---------------------------------------------------------------------------
 
-enum Kind { K_GATEUP = 0, K_DOWN, K_DY1, K_DX, K_DW2, K_DW1, K_COUNT };
-const char* const kKindEnv[K_COUNT] = {"MTS_TILE_GATEUP", "MTS_TILE_DOWN", "MTS_TILE_DY1",
-                                       "MTS_TILE_DX",     "MTS_TILE_DW2",  "MTS_TILE_DW1"};
+typedef MtsGemmKind Kind;
+constexpr Kind K_GATEUP = MTS_K_GATEUP, K_DOWN = MTS_K_DOWN, K_DY1 = MTS_K_DY1, K_DX = MTS_K_DX, K_DW2 = MTS_K_DW2, K_DW1 = MTS_K_DW1;
+constexpr int K_COUNT = MTS_K_COUNT;
 // rows_gemm: 0 StagedSmall, 1 RingTwoPerCu, 2 WsLarge, 3 RingThreePerCu (dY1 without the weighted_act output
 // only), 4 WsWide (no SwiGLU backward: gate/up, down and dX; dY1 falls back to 2);
 // dw_gemm: 0 StagedSmall, 2 DwWsLarge, 4 DwWsWide (the same output tiles, so one workspace layout).
@@ -1858,19 +1859,9 @@ const char* const kKindEnv[K_COUNT] = {"MTS_TILE_GATEUP", "MTS_TILE_DOWN", "MTS_
 // tile into two buffers halves their barriers (joint launch -1.7 %).
 const int kDefaultTile[K_COUNT] = {4, 4, 3, 4, 4, 4};
 
-bool tile_forced(int kind) { return getenv(kKindEnv[kind]) != nullptr; }
-
-// tile shape per GEMM; the environment overrides exist for tuning runs only
-int tile_choice(int kind) {
-    static int choice[K_COUNT] = {-1, -1, -1, -1, -1, -1};
-    if (choice[kind] < 0) {
-        int c = kDefaultTile[kind];
-        const char* s = getenv(kKindEnv[kind]);
-        if (s) c = atoi(s);
-        choice[kind] = (c >= 0 && c <= 4) ? c : kDefaultTile[kind];
-    }
-    return choice[kind];
-}
+// a tile family forced for a comparison run (mts_tuning.h), else the default
+bool tile_forced(int kind) { return mts_tuning().tile[kind] >= 0; }
+int tile_choice(int kind) { return tile_forced(kind) ? mts_tuning().tile[kind] : kDefaultTile[kind]; }
 
 // `gathered_rows`: rows of the [T,H] operand that is read through the token gather (0: none).  Lane
 // offsets are 32-bit: one expert's weights and an operand whose rows are gathered from anywhere must
@@ -1894,41 +1885,20 @@ int64_t m_tiles(int64_t TK, int E) {
 // Contiguous ranges of m-tiles per XCD pay off while one expert's weight matrix stays resident in an
 // XCD's 4 MiB L2 next to the streaming operands; larger weights are better streamed by all XCDs at the
 // same time (round-robin deal: one fetch from HBM, the other seven from the Infinity Cache).
-// MTS_XCD_RANGES=0/1 forces one or the other (tuning runs only).
+// A comparison run can force one or the other (mts_tuning.h).
 constexpr int64_t kL2Bytes = 4 << 20;   // per XCD
 int xcd_ranges_choice(int64_t expert_weight_bytes) {
-    static int forced = -2;
-    if (forced == -2) {
-        const char* s = getenv("MTS_XCD_RANGES");
-        forced = s ? (atoi(s) != 0) : -1;
-    }
+    const int forced = mts_tuning().xcd_ranges;
     if (forced >= 0) return forced;
     return expert_weight_bytes <= kL2Bytes ? 1 : 0;
 }
 
-// MTS_NO_TILE_ORDER=1 switches the n-tile groups and the reversed walks of the range mapping off; MTS_TILE_ORDER
-// picks them one by one (bit 0: groups, 1: down reversed, 2: dY1 reversed, 3: dX reversed).  For comparisons.
+// the n-tile groups and the reversed walks of the range mapping, which a comparison run can switch off one by one
 enum { ORDER_GROUPS = 1, ORDER_DOWN = 2, ORDER_DY1 = 4, ORDER_DX = 8, ORDER_ALL = 15 };
-int tile_order_mask() {
-    static int mask = -1;
-    if (mask < 0) {
-        const char* off = getenv("MTS_NO_TILE_ORDER");
-        const char* pick = getenv("MTS_TILE_ORDER");
-        mask = (off && atoi(off) != 0) ? 0 : (pick ? atoi(pick) & ORDER_ALL : ORDER_ALL);
-    }
-    return mask;
-}
+int tile_order_mask() { return mts_tuning().tile_order_mask; }
 
-// MTS_NO_TAIL_SPLIT=1 keeps every tile whole (for comparisons)
 constexpr int kCusPerXcd = 32;
-bool tail_split_on() {
-    static int on = -1;
-    if (on < 0) {
-        const char* s = getenv("MTS_NO_TAIL_SPLIT");
-        on = (s && atoi(s) != 0) ? 0 : 1;
-    }
-    return on != 0;
-}
+bool tail_split_on() { return mts_tuning().tail_split; }
 
 template <class T, int EPI>
 dim3 rows_grid(RowsParams& p, int64_t TK) {
@@ -2095,6 +2065,12 @@ int launch_bwd_joint(BwdJointParams q, int E, int grad_dtype, void* ws1, int64_t
     }
     q.n_dw1 = (int)dw_grid<T>(q.dw1, E, q.dw1.part ? 2 * E : E).x;
     q.n_dw2 = (int)dw_grid<T>(q.dw2, E, q.dw2.part ? 2 * E : E).x;
+    const bool own_dw2 = q.dw2.C != nullptr;
+    if (!own_dw2) {
+        q.n_dw2 = 0;
+        q.dw2.E = 0;
+        q.dw2.part = nullptr;
+    }
     q.dx.reverse = (tile_order_mask() & ORDER_DX) ? 1 : 0;
     q.n_dx = (int)rows_grid<JointDxTile, EPI_PLAIN>(q.dx, q.dx.TK).x;
     const int64_t want = (q.entries + WsLarge::NT * 4 - 1) / (WsLarge::NT * 4);
@@ -2103,7 +2079,7 @@ int launch_bwd_joint(BwdJointParams q, int E, int grad_dtype, void* ws1, int64_t
     if (grad_dtype == MTS_GEMM_DTYPE) bwd_joint_kernel<bf16_t><<<grid, WsLarge::NT, 0, s>>>(q);
     else bwd_joint_kernel<float><<<grid, WsLarge::NT, 0, s>>>(q);
     MTS_CHECK_LAUNCH();
-    if (q.dw1.part && q.dw2.part && 2 * E <= 65535) {
+    if (q.dw1.part && (q.dw2.part || !own_dw2) && 2 * E <= 65535) {
         const int t = q.dw1.tiles_per_expert > q.dw2.tiles_per_expert ? q.dw1.tiles_per_expert : q.dw2.tiles_per_expert;
         const int64_t want = ((int64_t)t * (T::BM * T::BN / 4) + 255) / 256;
         const unsigned gx = (unsigned)(want < 256 ? want : 256);
@@ -2121,7 +2097,7 @@ int launch_bwd_joint(BwdJointParams q, int E, int grad_dtype, void* ws1, int64_t
             const int64_t rows = ((items + 255) / 256 + gx - 1) / gx;
             jobs.c_rows = (int)(rows < 32 ? rows : 32);
         }
-        const dim3 sum_grid(gx, (unsigned)(2 * E + jobs.r_rows + jobs.c_rows));
+        const dim3 sum_grid(gx, (unsigned)(q.dw1.E + q.dw2.E + jobs.r_rows + jobs.c_rows));
         if (grad_dtype == MTS_GEMM_DTYPE) dw_chunk_sum_pair_kernel<T::BM, T::BN, bf16_t><<<sum_grid, 256, 0, s>>>(q.dw1, q.dw2, jobs);
         else dw_chunk_sum_pair_kernel<T::BM, T::BN, float><<<sum_grid, 256, 0, s>>>(q.dw1, q.dw2, jobs);
         MTS_CHECK_LAUNCH();
@@ -2336,8 +2312,9 @@ int fill_bwd_joint(BwdJointParams& q, const void* d_out, const void* weighted_ac
                    const void* w1, const int32_t* x_gather, const int32_t* expert_start, const int32_t* s_reverse,
                    const float* ds_partial, int64_t T, int K, int E, int H, int I, int act_dtype, void* dx_expanded,
                    void* d_w1, void* d_w2, void* d_weights) {
-    if (!d_out || !weighted_act || !d_pre_act || !x || !w1 || !x_gather || !expert_start || !s_reverse || !ds_partial ||
-        !dx_expanded || !d_w1 || !d_w2 || !d_weights)
+    // d_w2 == NULL: the caller runs dW2 in a launch of its own (next to dO*W2, which it does not depend on)
+    if (!d_out || !d_pre_act || !x || !w1 || !x_gather || !expert_start || !s_reverse || !ds_partial ||
+        !dx_expanded || !d_w1 || !d_weights || (d_w2 && !weighted_act))
         return MTS_ERR_NULL;
     if (act_dtype != MTS_GEMM_DTYPE) return MTS_ERR_DTYPE;
     if (T <= 0 || K < 1) return MTS_ERR_SHAPE;

@@ -6,6 +6,7 @@
 #include "mts_common.h"
 #include "mts_router_row.h"
 #include "mts_router_bwd_block.h"
+#include "mts_tuning.h"
 
 namespace {
 
@@ -112,8 +113,7 @@ typedef __attribute__((ext_vector_type(2))) float f32x2;
 __host__ __device__ inline int mma_lds_stride(int H) { return H + 32; }   // elements: consecutive rows 16 banks apart when H % 128 == 0
 inline size_t mma_lds_bytes(int H) { return (size_t)(kMmaTerms * 8 + 1) * mma_lds_stride(H) * sizeof(bf16_t); }   // + a row of zeros
 inline bool mma_projection_ok(int H, int E, int act_dtype) {
-    static const bool off = getenv("MTS_NO_MFMA_ROUTER") != nullptr;
-    return !off && act_dtype == MTS_BF16 && E <= 8 && H % 64 == 0 && H <= kMmaMaxH;
+    return mts_tuning().mfma_router && act_dtype == MTS_BF16 && E <= 8 && H % 64 == 0 && H <= kMmaMaxH;
 }
 
 // Every thread of the block: W_r [E][H] fp32 -> wb [3][8][stride] bf16 (experts past E are zeros), then a row of zeros.  The loads of a
@@ -147,8 +147,14 @@ struct MmaWeights {
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 const float a = v[u][q];
-                t0[q] = (bf16_t)a;
-                const float r1 = a - (float)t0[q];   // exact
+                bf16_t h = (bf16_t)a;
+                // A NaN or infinite weight is carried by the first term alone (inf - inf would turn an infinite weight
+                // into NaN logits where the fp32 dot product gives inf); a finite weight that rounds up to infinity
+                // is truncated instead, and the terms behind it carry the rest as for every other weight.
+                const bool finite = __builtin_isfinite(a);
+                if (finite && !__builtin_isfinite((float)h)) h = __builtin_bit_cast(bf16_t, (uint16_t)(__float_as_uint(a) >> 16));
+                t0[q] = h;
+                const float r1 = finite ? a - (float)h : 0.f;   // exact
                 t1[q] = (bf16_t)r1;
                 const float r2 = r1 - (float)t1[q];  // exact, 8 bits or fewer are left
                 t2[q] = (bf16_t)r2;

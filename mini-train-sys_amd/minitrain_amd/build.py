@@ -19,7 +19,7 @@ CSRC = os.path.join(os.path.dirname(PKG_DIR), "csrc")
 INCLUDE = os.path.join(os.path.dirname(os.path.dirname(PKG_DIR)), "include")
 LIB_DIR = os.path.join(PKG_DIR, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libmts_moe.so")
-SOURCES = ("mts_router.hip", "mts_router_linear.hip", "mts_route.hip", "mts_capacity.hip", "mts_combine.hip", "mts_gemm.hip", "mts_gemm_f16.hip", "mts_gemm_f32.hip", "mts_probe.hip")
+SOURCES = ("mts_router.hip", "mts_router_linear.hip", "mts_route.hip", "mts_capacity.hip", "mts_combine.hip", "mts_gemm.hip", "mts_gemm_f16.hip", "mts_gemm_f32.hip", "mts_probe.hip", "mts_tuning.hip")
 
 FLAGS = [
     "-O3",
@@ -57,11 +57,19 @@ def build_library(verbose: bool = False, resource_report: bool = False, out: str
             procs.append((obj, subprocess.Popen(base + ["-c", os.path.join(CSRC, src), "-o", obj],
                                                 stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)))
         stderr = ""
+        failure = None
         for obj, proc in procs:
+            if failure is not None:
+                # one compile has failed: the others are ended and reaped before their directory goes away
+                proc.kill()
+                proc.communicate()
+                continue
             _, err = proc.communicate()
             stderr += err
             if proc.returncode != 0:
-                raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{_quiet(err)}")
+                failure = f"hipcc failed ({proc.returncode}):\n{_quiet(err)}"
+        if failure is not None:
+            raise RuntimeError(failure)
         tmp = out + ".tmp"
         link = subprocess.run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *[o for o, _ in procs], "-o", tmp],
                               capture_output=True, text=True)

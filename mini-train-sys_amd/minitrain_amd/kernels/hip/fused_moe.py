@@ -139,6 +139,30 @@ def compute_routing_metadata(topk_indices: torch.Tensor, E: int, block_m_token: 
     )
 
 
+def routing_for_experts(topk_indices: torch.Tensor, E: int):
+    """``(expert_start, x_gather, s_scatter, s_reverse)``: what the operator itself needs of the routing
+    metadata, in one int32 allocation (the tile list of the reference's kernels is not produced)."""
+    lib = _lib.load()
+    T, K = topk_indices.shape
+    TK = T * K
+    dev = topk_indices.device
+    pad = -(-(2 * E + 1) // 4) * 4           # the per-row arrays start on 16-byte boundaries
+    buf = torch.empty(pad + 3 * TK, dtype=torch.int32, device=dev)
+    counts, expert_start = buf[:E], buf[E:2 * E + 1]
+    s_scatter, s_reverse, x_gather = buf[pad:pad + TK], buf[pad + TK:pad + 2 * TK], buf[pad + 2 * TK:]
+    ws_bytes = lib.mts_moe_route_workspace_bytes(T, K, E)
+    ws = torch.empty(max(ws_bytes, 4), dtype=torch.uint8, device=dev)
+    _lib.check(
+        lib.mts_moe_route(
+            topk_indices.data_ptr(), T, K, E, BLOCK_M_TOKEN, counts.data_ptr(), expert_start.data_ptr(),
+            s_scatter.data_ptr(), s_reverse.data_ptr(), x_gather.data_ptr(), None, None, None, ws.data_ptr(), ws_bytes,
+            _lib.stream_of(topk_indices),
+        ),
+        "mts_moe_route",
+    )
+    return expert_start, x_gather, s_scatter, s_reverse
+
+
 def expert_counts(topk_indices: torch.Tensor, E: int) -> torch.Tensor:
     """Routes per expert, int32 ``[E]``: the histogram pass of the routing metadata alone.
 
@@ -497,10 +521,9 @@ class _FusedMoEFunction(torch.autograd.Function):
         T, K = top_k_index.shape
         E = gate_up_proj.shape[0]
         with torch.no_grad():
-            (_, expert_start, x_gather, s_scatter, s_reverse, _, _, _) = compute_routing_metadata(top_k_index, E)
+            routing = routing_for_experts(top_k_index, E)
         weights_flat = top_k_weights.flatten().contiguous()
-        out, tensors, state = moe_forward(x, gate_up_proj, down_proj, weights_flat,
-                                          (expert_start, x_gather, s_scatter, s_reverse))
+        out, tensors, state = moe_forward(x, gate_up_proj, down_proj, weights_flat, routing)
         ctx.save_for_backward(*tensors)
         ctx.state = state
         ctx.mark_non_differentiable(top_k_index)

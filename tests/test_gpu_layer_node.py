@@ -79,6 +79,46 @@ def test_chained_head_equals_the_three_operators(T, H, E, K, dtype, normalize):
     assert torch.equal(got["s_scatter"], ss) and torch.equal(got["s_reverse"], sr) and torch.equal(got["x_gather"], xg)
 
 
+@pytest.mark.parametrize("T,H,E,K,dtype", [
+    (1500, 768, 8, 2, torch.bfloat16),    # projection on the matrix pipe
+    (1500, 256, 8, 3, torch.float16),     # 16-bit rows the matrix-pipe projection does not take: vector pipe
+    (700, 192, 12, 4, torch.float32),     # more than 8 experts: several lanes per row in the post-process
+    (1500, 768, 6, 2, torch.bfloat16)])
+def test_ties_reach_the_chained_head_and_the_layer_node(T, H, E, K, dtype):
+    """Exactly tied logits inside the chained head: experts with identical router rows tie for every
+    token, all-zero tokens tie over all experts.  The lower expert index must win, in the head kernel
+    and in the layer node, on the matrix-pipe and on the vector-pipe projection."""
+    print(f"ties through the head T={T} H={H} E={E} K={K} {dtype}", flush=True)
+    from minitrain_amd import _lib
+
+    lib = _lib.load()
+    x, w_r, w1, w2, _ = O.make_inputs(4100 + T + E, T, H, E, 64)
+    w_r[1] = w_r[0]                      # experts 0 and 1 tie for every token
+    w_r[E - 1] = w_r[2]                  # and so do 2 and the last one
+    x[::7] = 0.0                         # every logit of these tokens is exactly 0
+    x[3::11] = x[3::11].abs()            # some rows where the tied pair is likely to be on top
+    x, w_r = x.to(dtype).cuda(), w_r.cuda()
+    got = _head(lib, x, w_r, K, True)
+    logits = got["logits"]
+    assert torch.equal(logits[:, 0], logits[:, 1]) and torch.equal(logits[:, 2], logits[:, E - 1])   # the ties are real
+    assert bool((logits[::7] == 0).all())
+    ref = O.router_postprocess(logits.cpu(), K, normalize=True)
+    assert torch.equal(got["indices"].cpu(), ref.expert_indices)
+    # lowest index wins: an all-tied row selects experts 0..K-1 in that order, and the second expert of a
+    # tied pair is never selected without the first
+    assert torch.equal(got["indices"][::7].cpu(), torch.arange(K, dtype=torch.int32).expand(len(range(0, T, 7)), K))
+    sel = torch.zeros(T, E, dtype=torch.bool).scatter_(1, ref.expert_indices.long(), True)
+    assert bool((~sel[:, 1] | sel[:, 0]).all()) and bool((~sel[:, E - 1] | sel[:, 2]).all())
+    torch.testing.assert_close(got["weights"].cpu(), ref.expert_weights, rtol=2e-5, atol=2e-5)
+    assert torch.equal(got["counts"].cpu(), torch.bincount(ref.expert_indices.flatten().long(), minlength=E).int())
+    # the layer node routes through the same head
+    ops = hip_backend()
+    pdt = dtype
+    res = ops.moe_layer(x, w_r, w1.to(pdt).cuda(), w2.to(pdt).cuda(), K, normalize=True)
+    assert res is not None
+    assert torch.equal(res[7].cpu(), ref.expert_indices)
+
+
 def _layer_grads(ops, case, K, normalize, dtype, fp32_params):
     pdt = torch.float32 if fp32_params else dtype
     leaves = [case["x"].to(dtype).cuda().requires_grad_(True), case["w_r"].cuda().requires_grad_(True),

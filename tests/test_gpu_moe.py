@@ -254,7 +254,7 @@ def test_full_size_configs(name, seed, T, imbalanced):
         print("peak HBM allocated (MB):", torch.cuda.max_memory_allocated() / 2**20, flush=True)
 
 
-def _expert_weight_gradients_f64(case, e, rows1, rows2):
+def _expert_weight_gradients_f64(case, e, rows1, rows2, wide=None):
     """Rows ``rows1`` of dW1[e] and ``rows2`` of dW2[e] from the definition (minitrain/kernels/torch_ops.py:
     122-150 differentiated by hand), accumulated in float64 on the CPU over the routes of expert ``e``."""
     x, w1, w2, idx, w, g = (case[k] for k in ("x", "w1", "w2", "idx", "w", "g"))
@@ -264,7 +264,8 @@ def _expert_weight_gradients_f64(case, e, rows1, rows2):
     I = W2.shape[1]
     # per-row quantities: float64, or float32 products widened afterwards where the expert holds very many rows
     # (a 768-term dot product in fp32 is good to 1e-6); the sums over the rows below are always float64
-    wide = torch.float64 if len(tok) <= 40000 else torch.float32
+    if wide is None:
+        wide = torch.float64 if len(tok) <= 40000 else torch.float32
     pre = (xe.to(wide) @ W1.to(wide).T).double()
     gate, up = pre[:, :I], pre[:, I:]
     sig = torch.sigmoid(gate)
@@ -384,6 +385,54 @@ def test_intermediates_beyond_2_gib():
     assert_close_scaled(grads[1][E - 1].cpu()[0:2 * I:127], dw1_ref, BF16_TOL, "dW1 slice of the last expert")
     assert_close_scaled(grads[2][E - 1].cpu()[0:H:61], dw2_ref, BF16_TOL, "dW2 slice of the last expert")
     assert all(torch.isfinite(t.float()).all() for t in grads)
+
+
+@pytest.mark.parametrize("T", [512, 8192])
+def test_reference_sweep_sizes(T):
+    """The smallest and a middle size of the reference's operator sweep (benchmarks/operators/moe_runner.py:135-204:
+    512 ... 57 344 tokens at the layer shape) against the whole CPU oracle: at 512 tokens an expert holds fewer
+    rows than one 256-row tile, so every tile of every GEMM is a partial one."""
+    print(f"moe sweep size T={T}", flush=True)
+    _compare(routed_case(20 + T, T, 768, 8, 1024, 2))
+
+
+def test_mixtral_class_widths():
+    """H = 4096, I = 14336 (the reference's `mixtral_7b` benchmark profile, moe_runner.py:53): one expert's weights
+    are 224 MiB, far more than an XCD's L2, so the row-tiled GEMMs deal their tiles round-robin over the XCDs, and
+    the reduction of dO*W2 is longer than the three-blocks-per-CU kernel takes, so it runs on the two-block ring.
+    Checked against the CPU oracle on sampled tokens (forward, dX, dS) and on slices of one expert's dW1 / dW2
+    (float64 sums over the expert's routes), and through the reference's acceptance rule on the whole operator."""
+    print("moe mixtral-class widths", flush=True)
+    T, H, E, I, K = 1024, 4096, 8, 14336, 2
+    gen = torch.Generator(device="cuda").manual_seed(53)
+    rn = lambda *shape, std=1.0: (torch.randn(*shape, generator=gen, device="cuda") * std).bfloat16().cpu()
+    x, w1, w2, g = rn(T, H), rn(E, 2 * I, H, std=0.02), rn(E, H, I, std=0.02), rn(T, H)
+    logits = torch.randn(T, E, generator=gen, device="cuda").cpu()
+    route = O.router_postprocess(logits, K, normalize=True)
+    case = dict(x=x, w1=w1, w2=w2, g=g, idx=route.expert_indices, w=route.expert_weights.bfloat16())
+    out, grads = hip_moe_grads(x, w1, w2, case["idx"], case["w"], g)
+    assert all(torch.isfinite(t.float()).all() for t in (out, *grads))
+    pick = torch.from_numpy(np.random.Generator(np.random.Philox(53)).choice(T, size=48, replace=False))
+    leaves = [t.float().requires_grad_(r) for t, r in ((x[pick], True), (w1, False), (w2, False), (case["w"][pick], True))]
+    ref_out = O.fused_moe(leaves[0], leaves[1], leaves[2], case["idx"][pick], leaves[3])
+    (ref_out * g[pick].float()).sum().backward()
+    assert_close_scaled(out.cpu()[pick], ref_out.detach(), BF16_TOL, "sampled tokens vs CPU oracle")
+    assert_close_scaled(grads[0].cpu()[pick], leaves[0].grad, BF16_TOL, "sampled dX vs CPU oracle")
+    assert_close_scaled(grads[3].cpu()[pick], leaves[3].grad, BF16_TOL, "sampled dS vs CPU oracle")
+    del leaves, ref_out
+    e = 5
+    dw1_ref, dw2_ref = _expert_weight_gradients_f64(case, e, rows1=slice(0, 2 * I, 1409), rows2=slice(0, H, 211), wide=torch.float32)
+    assert_close_scaled(grads[1][e].cpu()[0:2 * I:1409], dw1_ref, BF16_TOL, "dW1 slice of one expert vs float64 CPU sum")
+    assert_close_scaled(grads[2][e].cpu()[0:H:211], dw2_ref, BF16_TOL, "dW2 slice of one expert vs float64 CPU sum")
+    del out, grads
+    torch.cuda.empty_cache()
+    # the reference's gate on the whole operator at this profile (moe_runner.py:176-193)
+    from minitrain_amd.benchmarks.moe_rows import operator_rows
+
+    hip = operator_rows("mixtral", T, iters=2, warmup=1, seed=1, with_torch=False)[0]
+    for side in ("fwd", "bwd"):
+        assert hip[f"{side}_relative_l2"] <= 1e-2 and hip[f"{side}_cosine_similarity"] >= 0.9999, hip
+    torch.cuda.empty_cache()
 
 
 def test_moe_block_end_to_end():

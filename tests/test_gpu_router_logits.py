@@ -86,3 +86,30 @@ def test_router_logits_unsupported_contract_returns_none():
     from minitrain_amd.kernels.hip import router_logits
     with pytest.raises(RuntimeError):
         router_logits(x, torch.randn(8, 64, device="cuda"))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])   # bf16: matrix-pipe projection; fp16: vector pipe
+def test_router_logits_with_weights_that_are_not_finite_or_round_to_infinity(dtype):
+    """An infinite weight gives infinite logits of the product's sign (NaN where the activation is zero), a NaN
+    weight gives NaN, and a finite weight beyond the largest bf16 value stays finite: what the fp32 dot product
+    of the reference (`F.linear(x.float(), w)`) gives, on both projections, and the other experts do not notice."""
+    ops = hip_backend()
+    T, H, E = 600, 256, 8
+    x, w, _ = _case(T, H, E, dtype, seed=77)
+    x[5] = 0.0                                  # 0 * inf
+    w[2, 17] = float("inf")
+    w[4, 200] = float("nan")
+    w[6, 3] = -float("inf")
+    w[1, 9] = 3.4e38                            # finite in fp32, above the largest bf16 value
+    x[:, 9] = x[:, 9] * 1e-3                    # keeps expert 1's logits finite
+    got = ops.router_logits(x.cuda(), w.cuda()).cpu()
+    want = torch.nn.functional.linear(x.float(), w)
+    assert torch.equal(torch.isnan(got), torch.isnan(want))
+    assert torch.equal(torch.isinf(got), torch.isinf(want))
+    inf = torch.isinf(want)
+    assert torch.equal(torch.sign(got[inf]), torch.sign(want[inf]))
+    fin = torch.isfinite(want)
+    assert bool(fin[:, 1].all())
+    ref64 = (x.double()[:, None, :] * w.double()[None, :, :]).nan_to_num(0.0, 0.0, 0.0).sum(-1)
+    for e in (0, 1, 3, 5, 7):
+        assert _scaled_err(got[:, e], ref64[:, e]) <= F32_TOL, e

@@ -29,9 +29,16 @@ def _route(lib, idx, E, static, block_m=64):
     ptrs = [outs[k].data_ptr() for k in ("counts", "expert_start", "s_scatter", "s_reverse", "x_gather",
                                          "tile_row_start", "tile_expert", "tile_count")]
     if static:
+        # two views of "allocates nothing": torch's caching allocator saw no request, and the device's own count
+        # of free bytes (which a raw hipMalloc / hipFree inside the library would move) is where it was
+        torch.cuda.synchronize()
         before = torch.cuda.memory_stats(dev)["allocation.all.allocated"]
+        free_before = torch.cuda.mem_get_info(dev)[0]
         rc = lib.mts_moe_route_static(idx.data_ptr(), T, K, E, block_m, *ptrs, stream)
+        free_during = torch.cuda.mem_get_info(dev)[0]
+        torch.cuda.synchronize()
         assert torch.cuda.memory_stats(dev)["allocation.all.allocated"] == before
+        assert free_during == free_before == torch.cuda.mem_get_info(dev)[0]
     else:
         ws_bytes = lib.mts_moe_route_workspace_bytes(T, K, E)
         ws = torch.empty(max(ws_bytes, 4), dtype=torch.uint8, device=dev)
@@ -57,6 +64,13 @@ def test_static_route_equals_workspace_route_on_consecutive_calls():
     lib = _lib.load()
     # a larger problem first, then smaller ones in the same array (which still holds the larger one's counters)
     cases = [(1, 24576, 2, 8, False), (2, 3000, 3, 64, True), (3, 1, 1, 4, False), (4, 700, 8, 1024, False)]
+    # the first static call on a device looks the array's address up (and may load the code object): made here,
+    # before any call whose free-memory reading is compared
+    _route(lib, _indices(0, 64, 2, 8), 8, static=False)
+    warm = _indices(0, 64, 2, 8)
+    ptr_args = [torch.empty(64 * 2 + 16, dtype=torch.int32, device="cuda") for _ in range(8)]
+    assert lib.mts_moe_route_static(warm.data_ptr(), 64, 2, 8, 64, *[t.data_ptr() for t in ptr_args], _lib.stream_of(warm)) == 0
+    torch.cuda.synchronize()
     for seed, T, K, E, dropped in cases:
         idx = _indices(seed, T, K, E, dropped)
         want = _route(lib, idx, E, static=False)
