@@ -191,6 +191,7 @@ def stage_breakdown(layer, steps):
     gp, gz = torch.randn(E, device=dev), torch.ones((), device=dev)
     bws = torch.empty(lib.mts_moe_head_bwd_workspace_bytes(T, H, E), dtype=torch.uint8, device=dev)
     dx_r, dw_r = torch.empty(T, H, **bf), torch.empty_like(w_r)
+    sched = torch.empty(lib.mts_moe_bwd_schedule_bytes(E) // 4, **i32)   # written by the dO*W2 launch, read by the joint one
 
     unit = 2.0 * TK * H * I                  # FLOPs of one [TK,H] x [H,I] product
     w1_b, w2_b = E * 2 * I * H * esz, E * H * I * esz
@@ -207,7 +208,7 @@ def stage_breakdown(layer, steps):
         ("combine", 1.0 * TK * H, rows_h + T * H * esz + TK * 4,
          lambda: lib.mts_moe_combine(p(y), None, None, p(sr), T, K, H, B, p(out), st)),
         ("bwd_dy1", unit, rows_h + w2_b + 2 * rows_i + 2 * rows_i + TK * npart * 4 + TK * (4 + 4 + esz),
-         lambda: lib.mts_moe_bwd_dy1(p(g), p(w2), 1, p(pre), p(r_wa), p(xg), p(ss), p(es), T, K, E, H, I, B, p(dpre), None, p(dsp), st)),
+         lambda: lib.mts_moe_bwd_dy1(p(g), p(w2), 1, p(pre), p(r_wa), p(xg), p(ss), p(es), T, K, E, H, I, B, p(dpre), None, p(dsp), p(sched), st)),
         # dW1, dW2, dX, the dS reduction and the router's backward (its blocks trail the dX tiles): one launch, plus
         # one small launch for the chunk sum, the dW_r partial sum and the dX combine, as the layer node issues them
         ("bwd_joint", 5 * unit + 4.0 * T * H * E + 1.0 * TK * H,
@@ -217,7 +218,7 @@ def stage_breakdown(layer, steps):
          lambda: lib.mts_moe_bwd_joint_router(p(g), p(post), p(dpre), p(x), p(w1), p(xg), p(es), p(sr), p(dsp), T, K, E, H, I, B, B,
                                               p(dxe), p(dw1), p(dw2), p(dwts), p(dws1), dws1.numel(), p(dws2), dws2.numel(),
                                               p(w_r), p(logits), p(r_w), p(r_i), p(cnt), p(gp), p(gz), p(gz), 1, p(dx_r), p(dx), p(dw_r),
-                                              p(bws), bws.numel(), st)),
+                                              p(bws), bws.numel(), p(sched), st)),
     ]
     # One stage is bracketed per pass over the whole sequence, so the other stages of that pass run
     # back to back as they do in the layer step and the chip is in the state it has there.

@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define MTS_VERSION 2
+#define MTS_VERSION 3
 
 /* element types of activations / weights / weight gradients */
 #define MTS_BF16 0
@@ -243,14 +243,16 @@ int mts_moe_combine(const void* y, const void* weights, const void* addend, cons
  * multiples of 64); otherwise they return MTS_ERR_SHAPE for it.  ds_partial is
  * [TK, mts_moe_ds_partials(I)] f32 scratch reduced by mts_moe_bwd_ds (fixed order, no
  * atomics).  weighted_act may be NULL: it is then not written (the caller holds s*a already,
- * see mts_moe_fwd_gateup_swiglu).                                              */
+ * see mts_moe_fwd_gateup_swiglu).  schedule may be NULL; otherwise (16-bit activations,
+ * mts_moe_bwd_schedule_bytes(E) > 0 bytes, 16-byte aligned) one more block of the launch
+ * writes the schedule of mts_moe_bwd_joint there, see mts_moe_bwd_schedule.            */
 int mts_moe_ds_partials(int I);
 int mts_moe_bwd_weights_as_stored(int act_dtype, int H, int I);
 int mts_moe_bwd_dy1(const void* d_out, const void* w2, int w2_as_stored, const void* pre_act,
                     const void* weights, const int32_t* x_gather, const int32_t* s_scatter,
                     const int32_t* expert_start, int64_t T, int K, int E, int H, int I,
                     int act_dtype, void* d_pre_act, void* weighted_act, float* ds_partial,
-                    void* stream);
+                    int32_t* schedule, void* stream);
 
 /* dS[entry] = sum of the partials of row s_reverse[entry], cast to act_dtype
  * (fused_moe.py:437-443 returns dS as [T,K] in the weights' dtype).          */
@@ -299,15 +301,30 @@ int mts_moe_bwd_dw1(const void* d_pre_act, const void* x, const int32_t* x_gathe
  * weight-gradient tiles, which are the long ones, start first and the dX tiles fill the
  * CUs as they come free.  mts_moe_bwd_joint_supported() says whether the shapes allow it
  * (16-bit activations, 2I a multiple of 64); both weight gradients have grad_dtype.
- * workspace1 / workspace2: as for mts_moe_bwd_dw1 / mts_moe_bwd_dw2 (may be NULL).     */
+ * workspace1 / workspace2: as for mts_moe_bwd_dw1 / mts_moe_bwd_dw2 (may be NULL).
+ * d_w2 == NULL (then weighted_act and workspace2 may be NULL too): dW2 is left to a call of
+ * mts_moe_bwd_dw2, which does not depend on mts_moe_bwd_dy1.
+ *
+ * schedule (may be NULL; no counterpart in the reference, whose launches leave the placement
+ * of blocks to the hardware): all tiles of a weight-gradient unit (an expert, or a row chunk of
+ * an over-full one) run on one XCD, and with uneven routing a round-robin deal of the units
+ * leaves most of the chip waiting for the XCD that drew the longest ones.  The schedule is a
+ * table, written on the GPU from expert_start alone, that deals the units out longest first to
+ * the XCD with the fewest rows so far and splits the dX tiles so that every XCD ends up with the
+ * same work.  It is used when both workspaces are given (it presumes their row chunks) and
+ * changes which block computes a tile, not the tile: results are bit-identical with and without.
+ * mts_moe_bwd_dy1 writes it as a by-product; mts_moe_bwd_schedule does in a launch of its own.
+ * mts_moe_bwd_schedule_bytes(E): bytes of the table, 0 when E is beyond what it covers (32). */
 int mts_moe_bwd_joint_supported(int act_dtype, int H, int I);
+int64_t mts_moe_bwd_schedule_bytes(int E);
+int mts_moe_bwd_schedule(const int32_t* expert_start, int64_t TK, int E, int32_t* schedule, void* stream);
 int mts_moe_bwd_joint(const void* d_out, const void* weighted_act, const void* d_pre_act,
                       const void* x, const void* w1, const int32_t* x_gather,
                       const int32_t* expert_start, const int32_t* s_reverse,
                       const float* ds_partial, int64_t T, int K, int E, int H, int I,
                       int act_dtype, int grad_dtype, void* dx_expanded, void* d_w1, void* d_w2,
                       void* d_weights, void* workspace1, int64_t workspace1_bytes,
-                      void* workspace2, int64_t workspace2_bytes, void* stream);
+                      void* workspace2, int64_t workspace2_bytes, const int32_t* schedule, void* stream);
 
 /* mts_moe_bwd_joint with the router's backward in the same launch: what mts_moe_head_bwd computes
  * (the autograd backward of minitrain/model/moe_router.py:64-90 given the routing-weight gradient
@@ -335,7 +352,7 @@ int mts_moe_bwd_joint_router(const void* d_out, const void* weighted_act, const 
                              const int32_t* counts, const float* g_prob_mean, const float* g_z_loss,
                              const float* g_load_balance, int normalize, void* dx_router, void* dx,
                              float* d_w_r, void* router_workspace, int64_t router_workspace_bytes,
-                             void* stream);
+                             const int32_t* schedule, void* stream);
 
 #ifdef __cplusplus
 }

@@ -51,7 +51,7 @@ int mts_moe_fwd_down_f16(const void* post_act, const void* w2, const int32_t* ex
 int mts_moe_bwd_dy1_f16(const void* d_out, const void* w2, int w2_as_stored, const void* pre_act, const void* weights,
                         const int32_t* x_gather, const int32_t* s_scatter, const int32_t* expert_start, int64_t T,
                         int K, int E, int H, int I, int act_dtype, void* d_pre_act, void* weighted_act,
-                        float* ds_partial, void* stream);
+                        float* ds_partial, int32_t* schedule, void* stream);
 int mts_moe_bwd_dx_f16(const void* d_pre_act, const void* w1, int w1_as_stored, const int32_t* expert_start,
                        int64_t TK, int E, int H, int I, int act_dtype, void* dx_expanded, void* stream);
 int mts_moe_bwd_dw2_f16(const void* d_out, const void* weighted_act, const int32_t* x_gather,
@@ -65,7 +65,7 @@ int mts_moe_bwd_joint_f16(const void* d_out, const void* weighted_act, const voi
                           const int32_t* s_reverse, const float* ds_partial, int64_t T, int K, int E, int H, int I,
                           int act_dtype, int grad_dtype, void* dx_expanded, void* d_w1, void* d_w2, void* d_weights,
                           void* workspace1, int64_t workspace1_bytes, void* workspace2, int64_t workspace2_bytes,
-                          void* stream);
+                          const int32_t* schedule, void* stream);
 int mts_moe_bwd_joint_router_f16(const void* d_out, const void* weighted_act, const void* d_pre_act, const void* x,
                                  const void* w1, const int32_t* x_gather, const int32_t* expert_start,
                                  const int32_t* s_reverse, const float* ds_partial, int64_t T, int K, int E, int H,
@@ -75,7 +75,7 @@ int mts_moe_bwd_joint_router_f16(const void* d_out, const void* weighted_act, co
                                  const float* weights, const int32_t* indices, const int32_t* counts,
                                  const float* g_prob_mean, const float* g_z_loss, const float* g_load_balance,
                                  int normalize, void* dx_router, void* dx, float* d_w_r, void* router_workspace,
-                                 int64_t router_workspace_bytes, void* stream);
+                                 int64_t router_workspace_bytes, const int32_t* schedule, void* stream);
 }
 
 // fp32 GEMM launchers (mts_gemm_f32.hip); epi: 0 plain, 1 SwiGLU, 2 dO*W2 with SwiGLU backward

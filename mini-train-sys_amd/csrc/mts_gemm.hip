@@ -145,7 +145,24 @@ struct RowsParams {
     int reverse;               // with xcd_ranges: the range's m-tiles are walked from the last to the first
     int tail_slots;            // with xcd_ranges: blocks an XCD runs at a time; when the tiles behind its last whole round
                                // fill at most half of them, each of those is cut into two tiles of half the height (0: never)
+    const int32_t* sched;      // with xcd_ranges: the m-tile range of every XCD (first[8], count[8]) from the schedule of the joint
+                               // backward launch, or NULL: equal ranges
+    int32_t* sched_out;        // dO*W2 launch: one more block writes the schedule of the joint backward launch here (NULL: none)
+    int sched_slots, sched_dx_cap;
 };
+
+// the schedule of the joint backward launch (defined with the weight-gradient GEMMs below)
+__device__ __forceinline__ void joint_schedule_wave(const int32_t* __restrict__ expert_start, int E, int slots, int dx_bm,
+                                                    int dx_cap, int32_t* __restrict__ sched);
+constexpr int kSchedDxRows = 256;   // rows of a dX tile of that launch (JointDxTile::BM)
+
+// The last block of a dO*W2 launch that was given a table writes the schedule: it needs nothing but expert_start,
+// and inside this launch it costs no time of its own.
+__device__ __forceinline__ bool schedule_block(const RowsParams& p) {
+    if (p.sched_out == nullptr || blockIdx.x != gridDim.x - 1) return false;
+    if (threadIdx.x < MTS_WAVE) joint_schedule_wave(p.expert_start, p.E, p.sched_slots, kSchedDxRows, p.sched_dx_cap, p.sched_out);
+    return true;
+}
 
 // ---------------------------------------------------------------------------
 // global -> register -> LDS staging of a [ROWS][BK] tile whose rows are K-contiguous
@@ -585,7 +602,7 @@ __device__ __forceinline__ bool find_rows_tile(const RowsParams& p, int b, int& 
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) mine += __shfl_xor(mine, o, MTS_WAVE);
         const int per = mine / kXcds, rem = mine % kXcds;
-        const int my = per + (xcd < rem ? 1 : 0);
+        const int my = p.sched ? p.sched[kXcds + xcd] : per + (xcd < rem ? 1 : 0);
         if (p.tail_slots > 0) {
             // the blocks behind the last whole round of this XCD: two per tile, the upper and the lower half (cutting
             // into four where a quarter of the slots is filled gains another 0.15 % of the layer step: not done)
@@ -609,7 +626,7 @@ __device__ __forceinline__ bool find_rows_tile(const RowsParams& p, int b, int& 
         }
         if (k >= my) return false;
         if (p.reverse) k = my - 1 - k;
-        tile = xcd * per + (xcd < rem ? xcd : rem) + k;
+        tile = (p.sched ? p.sched[xcd] : xcd * per + (xcd < rem ? xcd : rem)) + k;
     }
     int seen = 0;
     for (int e0 = 0; e0 < p.E; e0 += MTS_WAVE) {
@@ -672,6 +689,9 @@ __global__ __launch_bounds__(T::NT) void rows_gemm_kernel(RowsParams p) {
     __shared__ __attribute__((aligned(16))) bf16_t smem[LDS_ELEMS];
     constexpr bool SWIGLU = (EPI == EPI_SWIGLU);
 
+    if constexpr (epi_is_dy1(EPI)) {
+        if (schedule_block(p)) return;
+    }
     int e, row0, rend, ntile;
     if (!locate_rows_tile<T::BM>(p, blockIdx.x, e, row0, rend, ntile)) return;
     const int n0 = ntile * (SWIGLU ? T::BN / 2 : T::BN);  // first output column of this block
@@ -790,6 +810,9 @@ __global__ __launch_bounds__(T::NT, T::WAVES_PER_EU) void rows_gemm_ring_kernel(
     constexpr bool SWIGLU = (EPI == EPI_SWIGLU);
     constexpr int S = T::STAGES, L = T::A_INSTR + T::B_INSTR;
 
+    if constexpr (epi_is_dy1(EPI)) {
+        if (schedule_block(p)) return;
+    }
     int e, row0, rend, ntile;
     if (!locate_rows_tile<T::BM>(p, blockIdx.x, e, row0, rend, ntile)) return;
     const int n0 = ntile * (SWIGLU ? T::BN / 2 : T::BN);
@@ -1160,6 +1183,9 @@ template <class T, int EPI, bool BKM = false, class TH = T>
 __global__ __launch_bounds__(T::NT, T::WAVES_PER_EU) void rows_gemm_ws_kernel(RowsParams p) {
     static_assert(ws_lds_elems<T, EPI>() * 2 <= 160 * 1024, "LDS capacity");
     __shared__ __attribute__((aligned(1024))) bf16_t smem[ws_lds_elems<T, EPI>()];
+    if constexpr (epi_is_dy1(EPI)) {
+        if (schedule_block(p)) return;
+    }
     rows_gemm_ws_block<T, EPI, BKM, TH>(p, smem, blockIdx.x);
 }
 
@@ -1179,6 +1205,8 @@ struct DwParams {
     void* C;  // [E][M][N], bf16 or f32
     float* part;   // fp32 tile partials of experts whose rows are split over several blocks, or null
     int E, n_tiles, tiles_per_expert;  // set by the launcher
+    const int32_t* sched;   // the unit table of the joint backward launch's schedule (which units an XCD runs), or NULL:
+    int sched_slots;        // unit u runs on XCD u % 8; sched_slots: table entries per XCD
 };
 
 // ---------------------------------------------------------------------------
@@ -1196,13 +1224,15 @@ struct DwUnit {
     int slot;            // index of the unit's partial tiles in the workspace, -1: writes C itself
 };
 
-__device__ __forceinline__ int dw_share(const DwParams& p) {
-    const int total = p.expert_start[p.E] - p.expert_start[0];   // the caller may pass a sub-range of the experts
-    return ((total + p.E - 1) / p.E + 31) / 32 * 32;
+__device__ __forceinline__ int dw_share_of(const int32_t* expert_start, int E) {
+    const int total = expert_start[E] - expert_start[0];   // the caller may pass a sub-range of the experts
+    return ((total + E - 1) / E + 31) / 32 * 32;
 }
+__device__ __forceinline__ int dw_share(const DwParams& p) { return dw_share_of(p.expert_start, p.E); }
 
+__device__ __forceinline__ int dw_chunks_cut(int count, int share) { return count > share + share / 4 ? (count + share - 1) / share : 1; }
 __device__ __forceinline__ int dw_chunks(const DwParams& p, int count, int share) {
-    return (p.part != nullptr && count > share + share / 4) ? (count + share - 1) / share : 1;
+    return p.part != nullptr ? dw_chunks_cut(count, share) : 1;
 }
 
 // every lane of the calling wave gets the same answer
@@ -1243,6 +1273,155 @@ __device__ __forceinline__ bool locate_dw_unit(const DwParams& p, int unit, DwUn
         seen_slots += __shfl(sincl, MTS_WAVE - 1, MTS_WAVE);
     }
     return false;
+}
+
+
+// ---------------------------------------------------------------------------
+// Schedule of the joint backward launch under uneven routing.  Block b of a launch runs on XCD b % 8, and
+// the weight-gradient tiles of a unit (an expert, or a row chunk of an over-full one) all run on one XCD.  With
+// the units dealt round-robin an XCD that draws two long units finishes far behind the others (routing in a
+// trained model is uneven: the fullest expert of a layer holds 1.1 to 2 times the balanced share).  One wave
+// works the deal out before the launch: the units go to the XCDs longest first, each to the XCD with the least
+// rows so far (at most `slots` units per XCD, which is what the grid holds), and the dX tiles, which any XCD
+// can run, are split so that weight-gradient and dX work together are the same everywhere: a row costs a
+// weight-gradient unit 6 H I FLOPs (dW1 and dW2) and a dX tile 4 H I.  Which XCD computes a tile has no
+// influence on the tile's value: results are the same as with the round-robin deal, bit for bit.
+// Table (int32): [0,8) first dX m-tile of every XCD, [8,16) its number of m-tiles, [16,24) its number of
+// units, from kSchedUnits on (e, first row, end row, workspace slot) of unit k of XCD x at (x * slots + k) * 4.
+// ---------------------------------------------------------------------------
+constexpr int kSchedCounts = 16, kSchedUnits = 32;
+constexpr int kSchedMaxExperts = 32;          // one unit per lane: 2 E <= 64
+constexpr int64_t kSchedBytes = 4096;         // (32 + 8 * 8 * 4) * 4 bytes are used
+// Called by one whole wave (lane = threadIdx.x % 64); E <= kSchedMaxExperts.  Units are cut as locate_dw_unit cuts
+// them when it has a workspace for the chunk partials.
+__device__ __forceinline__ void joint_schedule_wave(const int32_t* __restrict__ expert_start, int E, int slots, int dx_bm,
+                                                    int dx_cap, int32_t* __restrict__ sched) {
+    const int lane = threadIdx.x % MTS_WAVE;
+    const int share = dw_share_of(expert_start, E);
+    const int s0 = lane < E ? expert_start[lane] : 0, s1 = lane < E ? expert_start[lane + 1] : 0;
+    const int nc = lane < E ? dw_chunks_cut(s1 - s0, share) : 0;
+    const int ns = nc > 1 ? nc : 0;
+    const int nt = (s1 - s0 + dx_bm - 1) / dx_bm;
+    int uincl = nc, sincl = ns, tincl = nt;
+#pragma unroll
+    for (int o = 1; o < MTS_WAVE; o <<= 1) {
+        const int a = __shfl_up(uincl, o, MTS_WAVE), b = __shfl_up(sincl, o, MTS_WAVE), c = __shfl_up(tincl, o, MTS_WAVE);
+        if (lane >= o) {
+            uincl += a;
+            sincl += b;
+            tincl += c;
+        }
+    }
+    const int n_units = __shfl(uincl, MTS_WAVE - 1, MTS_WAVE);
+    const int m_tiles = __shfl(tincl, MTS_WAVE - 1, MTS_WAVE);
+    // lane u < n_units: unit u in expert order
+    int ue = 0, ub = 0, uend = 0, uslot = -1;
+    for (int e = 0; e < E; ++e) {
+        const int n = __shfl(nc, e, MTS_WAVE), off = __shfl(uincl, e, MTS_WAVE) - n;
+        const int b = __shfl(s0, e, MTS_WAVE), en = __shfl(s1, e, MTS_WAVE);
+        const int sl = __shfl(sincl, e, MTS_WAVE) - __shfl(ns, e, MTS_WAVE);
+        if (lane >= off && lane < off + n) {
+            const int c = lane - off;
+            const int per = ((en - b + n - 1) / n + 31) / 32 * 32;
+            const int r0 = b + c * per;
+            ue = e;
+            ub = r0 < en ? r0 : en;
+            uend = r0 + per < en ? r0 + per : en;
+            uslot = n > 1 ? sl + c : -1;
+        }
+    }
+    const int urows = lane < n_units ? uend - ub : 0;
+    int rank = 0;   // position in the order longest first (ties: expert order)
+    for (int v = 0; v < n_units; ++v) {
+        const int rv = __shfl(urows, v, MTS_WAVE);
+        rank += (rv > urows || (rv == urows && v < lane)) ? 1 : 0;
+    }
+    // the rows of the units in that order, one per lane, so that the deal below reads them with a lane index
+    int sorted_rows = 0;
+    for (int v = 0; v < n_units; ++v) {
+        const int rk = __shfl(rank, v, MTS_WAVE), rv = __shfl(urows, v, MTS_WAVE);
+        if (rk == lane) sorted_rows = rv;
+    }
+    int load[kXcds], held[kXcds];
+#pragma unroll
+    for (int x = 0; x < kXcds; ++x) load[x] = held[x] = 0;
+    int my_x = 0, my_k = 0;
+    for (int k = 0; k < n_units; ++k) {
+        const int r = __builtin_amdgcn_readlane(sorted_rows, k);
+        int best = -1, best_load = 0;
+#pragma unroll
+        for (int x = 0; x < kXcds; ++x)
+            if (held[x] < slots && (best < 0 || load[x] < best_load)) {
+                best = x;
+                best_load = load[x];
+            }
+#pragma unroll
+        for (int x = 0; x < kXcds; ++x)
+            if (x == best) {
+                if (rank == k) {
+                    my_x = x;
+                    my_k = held[x];
+                }
+                load[x] += r;
+                held[x] += 1;
+            }
+    }
+    if (lane < n_units) {
+        int32_t* u = sched + kSchedUnits + (my_x * slots + my_k) * 4;
+        u[0] = ue; u[1] = ub; u[2] = uend; u[3] = uslot;
+    }
+    if (lane == 0) {
+        // dX rows an XCD should take: (5 * total / 8 - 3 * its weight-gradient rows) / 2, not below zero; the
+        // m-tiles (in expert order) are cut at the running sums of these wishes, at most dx_cap of them per XCD
+        const float total = (float)(expert_start[E] - expert_start[0]);
+        float want[kXcds], sum = 0.f;
+#pragma unroll
+        for (int x = 0; x < kXcds; ++x) {
+            const float w = 5.f * total - 24.f * (float)load[x];
+            want[x] = w > 0.f ? w : 0.f;
+            sum += want[x];
+        }
+        const float scale = sum > 0.f ? (float)m_tiles * __builtin_amdgcn_rcpf(sum) : 0.f;
+        int count[kXcds];
+        float run = 0.f;
+        int before = 0;
+#pragma unroll
+        for (int x = 0; x < kXcds; ++x) {
+            run += want[x];
+            int upto = sum > 0.f ? (int)(run * scale + 0.5f) : (m_tiles * (x + 1)) / kXcds;
+            upto = upto < before ? before : (upto > m_tiles ? m_tiles : upto);
+            if (x == kXcds - 1) upto = m_tiles;
+            count[x] = upto - before;
+            before = upto;
+        }
+        int carry = 0;   // what an XCD cannot hold moves to the next one, and what is left at the end moves back
+#pragma unroll
+        for (int x = 0; x < kXcds; ++x) {
+            const int c = count[x] + carry;
+            count[x] = c > dx_cap ? dx_cap : c;
+            carry = c - count[x];
+        }
+#pragma unroll
+        for (int x = kXcds - 1; x >= 0; --x) {
+            const int c = count[x] + carry;
+            count[x] = c > dx_cap ? dx_cap : c;
+            carry = c - count[x];
+        }
+        int first = 0;
+#pragma unroll
+        for (int x = 0; x < kXcds; ++x) {
+            sched[x] = first;
+            sched[kXcds + x] = count[x];
+            sched[kSchedCounts + x] = held[x];
+            first += count[x];
+        }
+    }
+}
+
+// the schedule in a launch of its own (for a caller whose dO*W2 GEMM is not this library's)
+__global__ __launch_bounds__(MTS_WAVE) void joint_schedule_kernel(const int32_t* expert_start, int E, int slots, int dx_bm, int dx_cap,
+                                                                    int32_t* sched) {
+    joint_schedule_wave(expert_start, E, slots, dx_bm, dx_cap, sched);
 }
 
 // Adds the chunk partials of the experts that were cut: thread = 4 consecutive columns of a tile row.
@@ -1507,7 +1686,14 @@ __device__ __forceinline__ void dw_gemm_ws_block(const DwParams& p, bf16_t* smem
     // all tiles of a unit (an expert, or a row chunk of an over-full one) run on one XCD
     const int xcd = block % kXcds, jb = block / kXcds;
     DwUnit unit;
-    if (!locate_dw_unit(p, xcd + kXcds * (jb / p.tiles_per_expert), unit)) return;
+    if (p.sched) {
+        const int k = jb / p.tiles_per_expert;
+        if (k >= p.sched[kSchedCounts + xcd]) return;
+        const int32_t* u = p.sched + kSchedUnits + (xcd * p.sched_slots + k) * 4;
+        unit.e = u[0]; unit.rbeg = u[1]; unit.rend = u[2]; unit.slot = u[3];
+    } else if (!locate_dw_unit(p, xcd + kXcds * (jb / p.tiles_per_expert), unit)) {
+        return;
+    }
     const int e = __builtin_amdgcn_readfirstlane(unit.e);
     const int rbeg = __builtin_amdgcn_readfirstlane(unit.rbeg), rend = __builtin_amdgcn_readfirstlane(unit.rend);
     const int slot = __builtin_amdgcn_readfirstlane(unit.slot);
@@ -1789,6 +1975,7 @@ struct BwdJointParams {
     mts_rl::RouterGradIn rg;
 };
 
+static_assert(WsWide::BM == kSchedDxRows, "the schedule counts dX tiles of this height");
 typedef WsWide JointDxTile;   // dX reads d_pre_act row-major: whole lines per row with 64-wide k-tiles (a third buffer gains nothing here)
 template <typename OutT>
 __global__ __launch_bounds__(WsLarge::NT, WsLarge::WAVES_PER_EU) void bwd_joint_kernel(BwdJointParams q) {
@@ -1912,8 +2099,8 @@ dim3 rows_grid(RowsParams& p, int64_t TK) {
             p.n_groups *= 2;
     const int64_t m_groups = (m_tiles<T>(TK, p.E) + kXcds - 1) / kXcds;
     if (!p.xcd_ranges) p.tail_slots = 0;
-    // tiles that are cut in two add at most tail_slots / 2 blocks per XCD
-    return dim3((unsigned)((m_groups * p.n_tiles + p.tail_slots / 2) * kXcds));
+    // tiles that are cut in two add at most tail_slots / 2 blocks per XCD; one more block writes the schedule (dO*W2 only)
+    return dim3((unsigned)((m_groups * p.n_tiles + p.tail_slots / 2) * kXcds + (p.sched_out ? 1 : 0)));
 }
 
 // does launch_rows_any take B in the weights' stored layout for this kind and reduction length?
@@ -2049,8 +2236,17 @@ bool bwd_joint_ok(int H, int I) {
 // function is compiled for that) and whole 16-byte chunks per row
 bool combine_in_tail(const BwdJointParams& q) { return q.c_out && q.n_router && q.c_K == 2 && q.rH % 8 == 0; }
 
+// table entries per XCD and the most dX m-tiles one XCD is given (twice the even share): the dO*W2 launch that writes
+// the table and the joint launch that sizes its grid by it must agree
+void schedule_shape(int64_t TK, int E, int& slots, int& cap) {
+    slots = (2 * E + kXcds - 1) / kXcds;
+    const int64_t upper = m_tiles<WsWide>(TK, E);
+    const int64_t even = (upper + kXcds - 1) / kXcds;
+    cap = (int)(2 * even + 1 < upper ? 2 * even + 1 : upper);
+}
+
 int launch_bwd_joint(BwdJointParams q, int E, int grad_dtype, void* ws1, int64_t ws1_bytes, void* ws2, int64_t ws2_bytes,
-                     hipStream_t s) {
+                     const int32_t* schedule, hipStream_t s) {
     typedef DwWsLarge T;
     if (grad_dtype != MTS_GEMM_DTYPE && grad_dtype != MTS_F32) return MTS_ERR_DTYPE;
     if (ws1) {
@@ -2073,6 +2269,19 @@ int launch_bwd_joint(BwdJointParams q, int E, int grad_dtype, void* ws1, int64_t
     }
     q.dx.reverse = (tile_order_mask() & ORDER_DX) ? 1 : 0;
     q.n_dx = (int)rows_grid<JointDxTile, EPI_PLAIN>(q.dx, q.dx.TK).x;
+    // With both workspaces (row chunks on) and a schedule from the caller (written by the dO*W2 launch), units and dX
+    // tiles go to the XCDs as the table says.
+    if (schedule && own_dw2 && q.dw1.part && q.dw2.part && E <= kSchedMaxExperts && mts_tuning().joint_schedule) {
+        if (!mts_aligned16(schedule)) return MTS_ERR_ALIGN;
+        int slots, cap;
+        schedule_shape(q.dx.TK, E, slots, cap);
+        q.dw1.sched = q.dw2.sched = schedule;
+        q.dw1.sched_slots = q.dw2.sched_slots = slots;
+        if (q.dx.xcd_ranges) {
+            q.dx.sched = schedule;
+            q.n_dx = cap * q.dx.n_tiles * kXcds;
+        }
+    }
     const int64_t want = (q.entries + WsLarge::NT * 4 - 1) / (WsLarge::NT * 4);
     q.n_ds = (int)(want < 64 ? want : 64);
     const dim3 grid((unsigned)(q.n_dw1 + q.n_dw2 + q.n_dx + q.n_ds + q.n_router));
@@ -2187,14 +2396,15 @@ extern "C" int MTS_GEMM_ENTRY(mts_moe_bwd_dy1)(const void* d_out, const void* w2
                                const void* weights, const int32_t* x_gather,
                                const int32_t* s_scatter, const int32_t* expert_start, int64_t T,
                                int K, int E, int H, int I, int act_dtype, void* d_pre_act,
-                               void* weighted_act, float* ds_partial, void* stream) {
+                               void* weighted_act, float* ds_partial, int32_t* schedule, void* stream) {
 #ifndef MTS_GEMM_F16
-    if (act_dtype == MTS_F16) return mts_moe_bwd_dy1_f16(d_out, w2t, w2_as_stored, pre_act, weights, x_gather, s_scatter, expert_start, T, K, E, H, I, act_dtype, d_pre_act, weighted_act, ds_partial, stream);
+    if (act_dtype == MTS_F16) return mts_moe_bwd_dy1_f16(d_out, w2t, w2_as_stored, pre_act, weights, x_gather, s_scatter, expert_start, T, K, E, H, I, act_dtype, d_pre_act, weighted_act, ds_partial, schedule, stream);
 #endif
     if (!d_out || !w2t || !pre_act || !weights || !x_gather || !s_scatter || !expert_start ||
         !d_pre_act || !ds_partial)
         return MTS_ERR_NULL;
     if (T <= 0 || K < 1) return MTS_ERR_SHAPE;
+    if (schedule && (E > kSchedMaxExperts || act_dtype == MTS_F32)) return MTS_ERR_SHAPE;   // see mts_moe_bwd_schedule_bytes
     if (act_dtype == MTS_F32) {
         if (E < 1 || E > MTS_MAX_MOE_EXPERTS || H < 1 || I < 1 || T * K > 0x7fffffffLL || w2_as_stored) return MTS_ERR_SHAPE;
         return mts_f32_rows(2, (const float*)d_out, H, x_gather, (const float*)w2t, I, I, H, expert_start, E, T * K,
@@ -2214,6 +2424,11 @@ extern "C" int MTS_GEMM_ENTRY(mts_moe_bwd_dy1)(const void* d_out, const void* w2
     p.C = (bf16_t*)d_pre_act; p.C2 = (bf16_t*)weighted_act;
     p.pre_act = (const bf16_t*)pre_act; p.route_w = (const bf16_t*)weights;
     p.s_scatter = s_scatter; p.ds_part = ds_partial; p.np = mts_moe_ds_partials(I); p.TK = T * K;
+    if (schedule) {
+        if (!mts_aligned16(schedule)) return MTS_ERR_ALIGN;
+        p.sched_out = schedule;
+        schedule_shape(T * K, E, p.sched_slots, p.sched_dx_cap);
+    }
     if (!weighted_act) return launch_rows_any<EPI_DY1N>(K_DY1, p, T * K, (hipStream_t)stream, w2_as_stored != 0);
     return launch_rows_any<EPI_DY1>(K_DY1, p, T * K, (hipStream_t)stream, w2_as_stored != 0);
 }
@@ -2355,21 +2570,35 @@ extern "C" int MTS_GEMM_ENTRY(mts_moe_bwd_joint)(const void* d_out, const void* 
                                                  const float* ds_partial, int64_t T, int K, int E, int H, int I,
                                                  int act_dtype, int grad_dtype, void* dx_expanded, void* d_w1, void* d_w2,
                                                  void* d_weights, void* workspace1, int64_t workspace1_bytes,
-                                                 void* workspace2, int64_t workspace2_bytes, void* stream) {
+                                                 void* workspace2, int64_t workspace2_bytes, const int32_t* schedule,
+                                                 void* stream) {
 #ifndef MTS_GEMM_F16
     if (act_dtype == MTS_F16)
         return mts_moe_bwd_joint_f16(d_out, weighted_act, d_pre_act, x, w1, x_gather, expert_start, s_reverse,
                                      ds_partial, T, K, E, H, I, act_dtype, grad_dtype, dx_expanded, d_w1, d_w2, d_weights,
-                                     workspace1, workspace1_bytes, workspace2, workspace2_bytes, stream);
+                                     workspace1, workspace1_bytes, workspace2, workspace2_bytes, schedule, stream);
 #endif
     BwdJointParams q = {};
     const int rc = fill_bwd_joint(q, d_out, weighted_act, d_pre_act, x, w1, x_gather, expert_start, s_reverse, ds_partial, T,
                                   K, E, H, I, act_dtype, dx_expanded, d_w1, d_w2, d_weights);
     if (rc) return rc;
-    return launch_bwd_joint(q, E, grad_dtype, workspace1, workspace1_bytes, workspace2, workspace2_bytes, (hipStream_t)stream);
+    return launch_bwd_joint(q, E, grad_dtype, workspace1, workspace1_bytes, workspace2, workspace2_bytes, schedule, (hipStream_t)stream);
 }
 
 #ifndef MTS_GEMM_F16
+extern "C" int64_t mts_moe_bwd_schedule_bytes(int E) { return E >= 1 && E <= kSchedMaxExperts ? kSchedBytes : 0; }
+
+extern "C" int mts_moe_bwd_schedule(const int32_t* expert_start, int64_t TK, int E, int32_t* schedule, void* stream) {
+    if (!expert_start || !schedule) return MTS_ERR_NULL;
+    if (TK <= 0 || TK > 0x7fffffffLL || E < 1 || E > kSchedMaxExperts) return MTS_ERR_SHAPE;
+    if (!mts_aligned16(schedule)) return MTS_ERR_ALIGN;
+    int slots, cap;
+    schedule_shape(TK, E, slots, cap);
+    joint_schedule_kernel<<<1, MTS_WAVE, 0, (hipStream_t)stream>>>(expert_start, E, slots, kSchedDxRows, cap, schedule);
+    MTS_CHECK_LAUNCH();
+    return MTS_OK;
+}
+
 extern "C" int mts_moe_bwd_joint_router_supported(int act_dtype, int64_t T, int H, int I, int E) {
     if (!mts_moe_bwd_joint_supported(act_dtype, H, I) || T <= 0 || H < 4 || H % 4 || E < 1 || E > kJointRouterExperts) return 0;
     MtsRouterBwdShape g;
@@ -2385,14 +2614,14 @@ extern "C" int MTS_GEMM_ENTRY(mts_moe_bwd_joint_router)(
     void* workspace1, int64_t workspace1_bytes, void* workspace2, int64_t workspace2_bytes, const float* w_r,
     const float* logits, const float* weights, const int32_t* indices, const int32_t* counts, const float* g_prob_mean,
     const float* g_z_loss, const float* g_load_balance, int normalize, void* dx_router, void* dx, float* d_w_r,
-    void* router_workspace, int64_t router_workspace_bytes, void* stream) {
+    void* router_workspace, int64_t router_workspace_bytes, const int32_t* schedule, void* stream) {
 #ifndef MTS_GEMM_F16
     if (act_dtype == MTS_F16)
         return mts_moe_bwd_joint_router_f16(d_out, weighted_act, d_pre_act, x, w1, x_gather, expert_start, s_reverse,
                                             ds_partial, T, K, E, H, I, act_dtype, grad_dtype, dx_expanded, d_w1, d_w2,
                                             d_weights, workspace1, workspace1_bytes, workspace2, workspace2_bytes, w_r, logits,
                                             weights, indices, counts, g_prob_mean, g_z_loss, g_load_balance, normalize,
-                                            dx_router, dx, d_w_r, router_workspace, router_workspace_bytes, stream);
+                                            dx_router, dx, d_w_r, router_workspace, router_workspace_bytes, schedule, stream);
 #endif
     BwdJointParams q = {};
     int rc = fill_bwd_joint(q, d_out, weighted_act, d_pre_act, x, w1, x_gather, expert_start, s_reverse, ds_partial, T, K, E,
@@ -2419,5 +2648,5 @@ extern "C" int MTS_GEMM_ENTRY(mts_moe_bwd_joint_router)(
     q.c_out = (bf16_t*)dx; q.c_K = K;
     q.rg = {logits, weights, indices, counts, nullptr, nullptr, g_prob_mean, g_z_loss, g_load_balance, act_dtype, K, normalize,
             ds_partial, s_reverse, q.np};
-    return launch_bwd_joint(q, E, grad_dtype, workspace1, workspace1_bytes, workspace2, workspace2_bytes, (hipStream_t)stream);
+    return launch_bwd_joint(q, E, grad_dtype, workspace1, workspace1_bytes, workspace2, workspace2_bytes, schedule, (hipStream_t)stream);
 }

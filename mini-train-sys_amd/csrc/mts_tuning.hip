@@ -26,6 +26,7 @@ MtsTuning read_environment() {
     t.tail_split = !flag("MTS_NO_TAIL_SPLIT");
     t.mfma_router = !flag("MTS_NO_MFMA_ROUTER");
     t.fused_cast = !flag("MTS_NO_FUSED_CAST");
+    t.joint_schedule = !flag("MTS_NO_JOINT_SCHEDULE");
     return t;
 }
 

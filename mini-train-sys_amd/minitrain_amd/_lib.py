@@ -52,17 +52,19 @@ SIGNATURES = {
     "mts_probe_mfma_sink_bytes": (_l, [_i]),
     "mts_probe_mfma_rate": (_i, [_i, _i, _i, _p, _l, _p, _p]),
     "mts_moe_bwd_weights_as_stored": (_i, [_i, _i, _i]),
-    "mts_moe_bwd_dy1": (_i, [_p, _p, _i, _p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p, _p, _p, _p]),
+    "mts_moe_bwd_dy1": (_i, [_p, _p, _i, _p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p, _p, _p, _p, _p]),
+    "mts_moe_bwd_schedule_bytes": (_l, [_i]),
+    "mts_moe_bwd_schedule": (_i, [_p, _l, _i, _p, _p]),
     "mts_moe_bwd_ds": (_i, [_p, _p, _l, _i, _i, _p, _p]),
     "mts_moe_bwd_dx": (_i, [_p, _p, _i, _p, _l, _i, _i, _i, _i, _p, _p]),
     "mts_moe_bwd_dw_workspace_bytes": (_l, [_i, _i, _i, _i]),
     "mts_moe_bwd_dw2": (_i, [_p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _i, _p, _p, _l, _p]),
     "mts_moe_bwd_dw1": (_i, [_p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _i, _p, _p, _l, _p]),
     "mts_moe_bwd_joint_supported": (_i, [_i, _i, _i]),
-    "mts_moe_bwd_joint": (_i, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _i, _p, _p, _p, _p, _p, _l, _p, _l, _p]),
+    "mts_moe_bwd_joint": (_i, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _i, _p, _p, _p, _p, _p, _l, _p, _l, _p, _p]),
     "mts_moe_bwd_joint_router_supported": (_i, [_i, _l, _i, _i, _i]),
     "mts_moe_bwd_joint_router": (_i, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _i, _p, _p, _p, _p, _p, _l, _p, _l]
-                                 + [_p] * 8 + [_i, _p, _p, _p, _p, _l, _p]),
+                                 + [_p] * 8 + [_i, _p, _p, _p, _p, _l, _p, _p]),
 }
 
 _lib = None

@@ -196,6 +196,8 @@ _JOINT = os.environ.get("MTS_NO_JOINT_BWD", "0") != "1"
 _TAIL_IN_JOINT = os.environ.get("MTS_NO_TAIL_IN_JOINT", "0") != "1"
 # MTS_NO_COMBINE_IN_TAIL=1 keeps the dX combine behind that launch in a launch of its own
 _COMBINE_IN_TAIL = os.environ.get("MTS_NO_COMBINE_IN_TAIL", "0") != "1"
+# MTS_NO_JOINT_SCHEDULE=1: that launch deals its blocks out to the XCDs without looking at the routes per expert
+_SCHEDULE = os.environ.get("MTS_NO_JOINT_SCHEDULE", "0") != "1"
 # MTS_WEIGHTED_POST=0: the forward pass writes the unweighted activation and dY1 writes s * a again (tuning runs only)
 _WEIGHTED_POST = os.environ.get("MTS_WEIGHTED_POST", "1") != "0"
 _SIDE_STREAMS: dict = {}
@@ -383,19 +385,31 @@ def moe_backward(tensors, state, dO, needs, x_addend=None, router_tail=None):
     weighted_act = tensors[9] if state.weighted else torch.empty(TK, I, dtype=x.dtype, device=dev)
     n_part = lib.mts_moe_ds_partials(I)
     ds_part = torch.empty(TK, n_part, dtype=torch.float32, device=dev)
+    # When every gradient is wanted, dW1, dW2, dX and the dS reduction go out as ONE launch whose block
+    # order starts the long weight-gradient tiles first; no side stream is involved.  Which XCD runs which of
+    # its units and dX tiles follows a table that the dO * W2 launch writes on the side (uneven routing).
+    joint = (
+        _JOINT and need_x and need_w1 and need_w2 and need_s and as_stored
+        and gate_up_proj.dtype == down_proj.dtype and bool(lib.mts_moe_bwd_joint_supported(act, H, I))
+    )
+    ws1, ws1_ptr, ws1_bytes = _dw_workspace(lib, 1, E, H, I, x.dtype, dev) if need_w1 else (None, 0, 0)
+    ws2, ws2_ptr, ws2_bytes = _dw_workspace(lib, 2, E, H, I, x.dtype, dev) if need_w2 else (None, 0, 0)
+    schedule = None
+    if joint and _SCHEDULE and ws1 is not None and ws2 is not None:
+        sched_bytes = lib.mts_moe_bwd_schedule_bytes(E)
+        if sched_bytes > 0:
+            schedule = torch.empty(sched_bytes // 4, dtype=torch.int32, device=dev)
     _lib.check(
         lib.mts_moe_bwd_dy1(
             dO.data_ptr(), w2_bwd.data_ptr(), int(as_stored), pre_act.data_ptr(), weights_flat.data_ptr(),
             x_gather.data_ptr(),
             s_scatter.data_ptr(), expert_start.data_ptr(), T, K, E, H, I, act, d_pre_act.data_ptr(),
-            None if state.weighted else weighted_act.data_ptr(), ds_part.data_ptr(), stream,
+            None if state.weighted else weighted_act.data_ptr(), ds_part.data_ptr(), _lib.ptr(schedule), stream,
         ),
         "mts_moe_bwd_dy1",
     )
 
     ddown_proj = None
-    ws1, ws1_ptr, ws1_bytes = _dw_workspace(lib, 1, E, H, I, x.dtype, dev) if need_w1 else (None, 0, 0)
-    ws2, ws2_ptr, ws2_bytes = _dw_workspace(lib, 2, E, H, I, x.dtype, dev) if need_w2 else (None, 0, 0)
 
     def combine_dx(dx_expanded, d_weights):
         addend = x_addend(d_weights) if x_addend is not None else None
@@ -408,12 +422,7 @@ def moe_backward(tensors, state, dO, needs, x_addend=None, router_tail=None):
         )
         return dx
 
-    # When every gradient is wanted, dW1, dW2, dX and the dS reduction go out as ONE launch whose block
-    # order starts the long weight-gradient tiles first; no side stream is involved.
-    if (
-        _JOINT and need_x and need_w1 and need_w2 and need_s and as_stored
-        and gate_up_proj.dtype == down_proj.dtype and lib.mts_moe_bwd_joint_supported(act, H, I)
-    ):
+    if joint:
         dgate_up_proj, ddown_proj = torch.empty_like(gate_up_proj), torch.empty_like(down_proj)
         d_weights = torch.empty(T, K, dtype=weights_flat.dtype, device=dev)
         dx_expanded = torch.empty(TK, H, dtype=x.dtype, device=dev)
@@ -423,6 +432,7 @@ def moe_backward(tensors, state, dO, needs, x_addend=None, router_tail=None):
             act, _lib.dtype_code(gate_up_proj.dtype), dx_expanded.data_ptr(), dgate_up_proj.data_ptr(),
             ddown_proj.data_ptr(), d_weights.data_ptr(), ws1_ptr, ws1_bytes, ws2_ptr, ws2_bytes,
         )
+        sched_ptr = _lib.ptr(schedule)
         rt = router_tail
         if rt is not None and _TAIL_IN_JOINT and lib.mts_moe_bwd_joint_router_supported(act, T, H, I, E):
             # the router's backward as trailing blocks of the same launch: it needs nothing the launch writes
@@ -435,7 +445,7 @@ def moe_backward(tensors, state, dO, needs, x_addend=None, router_tail=None):
                     *joint_args, rt.router_weight.data_ptr(), rt.logits.data_ptr(), rt.weights.data_ptr(),
                     rt.indices.data_ptr(), _lib.ptr(rt.counts), _lib.ptr(rt.g_prob_mean), _lib.ptr(rt.g_z_loss),
                     _lib.ptr(rt.g_load_balance), int(rt.normalize), dx_r.data_ptr(), _lib.ptr(dx), dw_r.data_ptr(),
-                    rws.data_ptr(), rws_bytes, stream,
+                    rws.data_ptr(), rws_bytes, sched_ptr, stream,
                 ),
                 "mts_moe_bwd_joint_router",
             )
@@ -445,7 +455,7 @@ def moe_backward(tensors, state, dO, needs, x_addend=None, router_tail=None):
             if x_addend is not None:
                 x_addend(d_weights)   # lets the caller pick the router's outputs up; the combine has been launched
             return dx, dgate_up_proj, ddown_proj, d_weights
-        _lib.check(lib.mts_moe_bwd_joint(*joint_args, stream), "mts_moe_bwd_joint")
+        _lib.check(lib.mts_moe_bwd_joint(*joint_args, sched_ptr, stream), "mts_moe_bwd_joint")
         return combine_dx(dx_expanded, d_weights), dgate_up_proj, ddown_proj, d_weights
 
     if need_w1 and need_w2:

@@ -37,7 +37,7 @@ def test_library_exports_every_declared_symbol():
     for name in _declared():
         assert hasattr(lib, name), f"{name} is declared in include/ but not exported"
         assert name in _lib.SIGNATURES, f"{name} has no ctypes prototype"
-    assert lib.mts_version() == 2
+    assert lib.mts_version() == 3
     assert lib.mts_error_string(0) == b"ok"
     # argument checks run on the host before any launch: safe without a GPU
     assert lib.mts_router_fwd(None, 4, 8, 2, 1, None, None, None, None, None, None, None, None, None, 0, None, 0, None) == -1
@@ -76,11 +76,23 @@ def test_contract_violations_are_reported_before_any_launch():
     assert lib.mts_moe_bwd_joint_supported(_lib.MTS_F32, 768, 1024) == 0
     assert lib.mts_moe_bwd_joint_supported(_lib.MTS_BF16, 72, 40) == 0
     joint = lambda *a: lib.mts_moe_bwd_joint(*a)
-    ok_args = [fake] * 9 + [256, 2, 4, 64, 128, _lib.MTS_BF16, _lib.MTS_BF16, fake, fake, fake, fake, None, 0, None, 0, None]
+    ok_args = [fake] * 9 + [256, 2, 4, 64, 128, _lib.MTS_BF16, _lib.MTS_BF16, fake, fake, fake, fake, None, 0, None, 0, None, None]
     assert joint(*([None] + ok_args[1:])) == NULL
     assert joint(*(ok_args[:14] + [_lib.MTS_F32] + ok_args[15:])) == -3                      # activations must be 16-bit
     assert joint(*(ok_args[:12] + [72, 40] + ok_args[14:])) == SHAPE                          # 2I = 80 has no whole k-tile
     assert joint(*(ok_args[:20] + [fake, 16] + ok_args[22:])) == WORKSPACE
+    # without d_w2 the joint launch leaves dW2 to a call of its own: weighted_act and the second workspace may be absent
+    # too (the next check that fails is the unsupported width, not a missing pointer)
+    no_dw2 = ok_args[:1] + [None] + ok_args[2:12] + [72, 40] + ok_args[14:18] + [None] + ok_args[19:]
+    assert joint(*no_dw2) == SHAPE
+    # the schedule of the joint launch covers up to 32 experts; dO*W2 refuses to write one beyond that
+    assert lib.mts_moe_bwd_schedule_bytes(8) == 4096 and lib.mts_moe_bwd_schedule_bytes(32) == 4096
+    assert lib.mts_moe_bwd_schedule_bytes(33) == 0 and lib.mts_moe_bwd_schedule_bytes(0) == 0
+    assert lib.mts_moe_bwd_schedule(None, 1024, 8, fake, None) == NULL
+    assert lib.mts_moe_bwd_schedule(fake, 1024, 33, fake, None) == SHAPE
+    assert lib.mts_moe_bwd_schedule(fake, 1024, 8, fake + 4, None) == -5
+    assert lib.mts_moe_bwd_dy1(fake, fake, 1, fake, fake, fake, fake, fake, 256, 2, 40, 64, 128, _lib.MTS_BF16, fake, None, fake,
+                               fake, None) == SHAPE
     # the MFMA rate probe: sink pointer, launch size, sink size
     assert lib.mts_probe_mfma_sink_bytes(512) == 512 * 256 * 4
     assert lib.mts_probe_mfma_rate(1, 512, 100, None, 1 << 20, None, None) == NULL

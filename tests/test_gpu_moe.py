@@ -387,6 +387,118 @@ def test_intermediates_beyond_2_gib():
     assert all(torch.isfinite(t.float()).all() for t in grads)
 
 
+def _skewed_indices(T, E, K, shares, seed):
+    """K distinct experts per token, drawn one after the other with odds proportional to `shares`."""
+    g = torch.Generator().manual_seed(seed)
+    p = torch.tensor(shares, dtype=torch.float64).expand(T, E).clone()
+    cols = []
+    for _ in range(K):
+        c = torch.multinomial(p, 1, generator=g)
+        p.scatter_(1, c, 0.0)
+        cols.append(c)
+    return torch.cat(cols, 1).int()
+
+
+def _read_schedule(table, E):
+    """The used part of a schedule table as Python values: dX ranges and the units of every XCD."""
+    t = table.cpu().tolist()
+    slots = (2 * E + 7) // 8
+    first, count, held = t[0:8], t[8:16], t[16:24]
+    units = [[tuple(t[32 + (x * slots + k) * 4: 32 + (x * slots + k) * 4 + 4]) for k in range(held[x])] for x in range(8)]
+    return first, count, held, units
+
+
+@pytest.mark.parametrize("E,K,shares", [
+    (8, 2, [4862, 12086, 3507, 3153, 6471, 5392, 7811, 5870]),      # routes per expert of a layer of the 12-layer decoder
+    (8, 2, [0.48, 0.2, 0.1, 0.07, 0.05, 0.04, 0.03, 0.03]),          # Zipf-like
+    (8, 2, [1] * 8), (5, 3, [5, 1, 1, 1, 0.2]), (32, 4, [1.0 / (r + 1) for r in range(32)]), (3, 1, [1, 0, 3])])
+def test_joint_launch_schedule(E, K, shares):
+    """The table that deals the joint backward launch's blocks out to the XCDs (written by the dO*W2 launch, or by a
+    launch of its own): every unit is a row range of one expert, the units of an expert tile its rows in order, no
+    XCD holds more units than the grid has room for, the dX m-tiles are split into eight consecutive ranges that
+    cover them all, and the XCD with the most weight-gradient rows gets the fewest dX tiles.  Both ways of writing
+    it give the same table."""
+    print(f"joint launch schedule E={E} K={K}", flush=True)
+    from minitrain_amd import _lib
+    from minitrain_amd.kernels.hip.fused_moe import compute_routing_metadata
+
+    lib = _lib.load()
+    T, H, I = 6000, 128, 128
+    idx = _skewed_indices(T, E, K, shares, 17).cuda()
+    counts, es = compute_routing_metadata(idx, E)[:2]
+    nbytes = lib.mts_moe_bwd_schedule_bytes(E)
+    assert nbytes == 4096
+    own = torch.full((nbytes // 4,), -1, dtype=torch.int32, device="cuda")
+    assert lib.mts_moe_bwd_schedule(es.data_ptr(), T * K, E, own.data_ptr(), _lib.stream_of(own)) == 0
+    first, count, held, units = _read_schedule(own, E)
+    c = counts.cpu().tolist()
+    start = es.cpu().tolist()
+    slots = (2 * E + 7) // 8
+    assert all(h <= slots for h in held)
+    share = (-(-T * K // E) + 31) // 32 * 32
+    by_expert = {}
+    for x in range(8):
+        for (e, rb, re_, slot) in units[x]:
+            assert 0 <= e < E and start[e] <= rb <= re_ <= start[e + 1]
+            by_expert.setdefault(e, []).append((rb, re_, slot))
+    slot_seen = []
+    for e in range(E):
+        parts = sorted(by_expert.get(e, []))
+        assert parts and parts[0][0] == start[e] and parts[-1][1] == start[e + 1]            # every expert is covered ...
+        assert all(a[1] == b[0] for a, b in zip(parts, parts[1:]))                            # ... by consecutive ranges
+        cut = c[e] > share + share // 4
+        assert len(parts) == (-(-c[e] // share) if cut else 1)
+        assert all((p[2] >= 0) == cut for p in parts)
+        slot_seen += [p[2] for p in parts if cut]
+    assert sorted(slot_seen) == list(range(len(slot_seen)))                                     # workspace slots in expert order
+    m_tiles = sum(-(-n // 256) for n in c)
+    assert first[0] == 0 and all(first[x + 1] == first[x] + count[x] for x in range(7)) and first[7] + count[7] == m_tiles
+    loads = [sum(u[1] - u[0] for u in [(rb, re_) for (_, rb, re_, _) in units[x]]) for x in range(8)]
+    if max(loads) > min(loads) and m_tiles >= 16:
+        assert count[loads.index(max(loads))] <= count[loads.index(min(loads))]
+    # the dO*W2 launch writes the same table on the side
+    x = torch.randn(T, H, device="cuda").bfloat16()
+    w2 = (torch.randn(E, H, I, device="cuda") * 0.02).bfloat16()
+    pre = torch.randn(T * K, 2 * I, device="cuda").bfloat16()
+    wts = torch.rand(T * K, device="cuda").bfloat16()
+    _, _, xg, ss, _, _, _, _ = compute_routing_metadata(idx, E)
+    dpre = torch.empty_like(pre)
+    dsp = torch.empty(T * K, lib.mts_moe_ds_partials(I), device="cuda")
+    side = torch.full_like(own, -1)
+    rc = lib.mts_moe_bwd_dy1(x.data_ptr(), w2.data_ptr(), 1, pre.data_ptr(), wts.data_ptr(), xg.data_ptr(), ss.data_ptr(),
+                             es.data_ptr(), T, K, E, H, I, _lib.MTS_BF16, dpre.data_ptr(), None, dsp.data_ptr(), side.data_ptr(),
+                             _lib.stream_of(x))
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert _read_schedule(side, E) == (first, count, held, units)
+
+
+@pytest.mark.parametrize("dtype,fp32_params", [(torch.bfloat16, False), (torch.float16, True)])
+def test_scheduled_joint_launch_equals_the_unscheduled_one(dtype, fp32_params, monkeypatch):
+    """Which XCD computes a tile does not change the tile: with the schedule and without it the operator returns
+    the same gradients bit for bit under skewed routing (where the schedule moves most blocks), and they match the
+    oracle."""
+    print(f"scheduled joint launch {dtype} fp32_params={fp32_params}", flush=True)
+    import importlib
+
+    F = importlib.import_module("minitrain_amd.kernels.hip.fused_moe")
+    T, H, E, I, K = 5000, 256, 8, 512, 2
+    case = routed_case(61, T, H, E, I, K, dtype=dtype, bias=O.zipf_log_bias(E) * 0.5)
+    if fp32_params:
+        case["w1"], case["w2"] = case["w1"].float(), case["w2"].float()
+    args = (case["x"], case["w1"], case["w2"], case["idx"], case["w"], case["g"])
+    monkeypatch.setattr(F, "_JOINT", True)
+    monkeypatch.setattr(F, "_SCHEDULE", True)
+    with_table = hip_moe_grads(*args)
+    monkeypatch.setattr(F, "_SCHEDULE", False)
+    without = hip_moe_grads(*args)
+    assert torch.equal(with_table[0], without[0])
+    for name, a, b in zip(NAMES, with_table[1], without[1]):
+        assert a.dtype == b.dtype and torch.equal(a, b), name
+    monkeypatch.setattr(F, "_SCHEDULE", True)
+    _compare(case)
+
+
 @pytest.mark.parametrize("T", [512, 8192])
 def test_reference_sweep_sizes(T):
     """The smallest and a middle size of the reference's operator sweep (benchmarks/operators/moe_runner.py:135-204:
