@@ -203,6 +203,14 @@ int mts_moe_capacity_mask(const int32_t* top_k_index, const float* top_k_weights
 int mts_moe_stage_weights(const void* src, int src_dtype, void* dst, int dst_dtype, int E,
                           int64_t R, int64_t C, int transpose, void* stream);
 
+/* The same casts for fp32 master weights (the reference's single-GPU training contract,
+ * minitrain/train/trainer.py:95-98: fp32 parameters under bf16 autocast) as ONE launch for both
+ * expert weights: w1 (n1 values) -> w1_out, w2 (n2 values) -> w2_out, both of dst_dtype
+ * (MTS_BF16 or MTS_F16), same layout; n1 and n2 multiples of 8, all pointers 16-byte aligned.
+ * The backward GEMMs read the same copies, so a layer step casts each weight once.        */
+int mts_moe_cast_weights_pair(const float* w1, void* w1_out, int64_t n1, const float* w2,
+                              void* w2_out, int64_t n2, int dst_dtype, void* stream);
+
 /* ---- forward ------------------------------------------------------------
  * Replaces _fused_up_proj_swiglu_kernel (fused_moe_kernels.py:264-367):
  * for every row r (token x_gather[r], expert e): [g;u] = W1[e] x ; a = silu(g)*u.

@@ -242,6 +242,42 @@ extern "C" int mts_moe_stage_weights(const void* src, int src_dtype, void* dst, 
     return MTS_OK;
 }
 
+// fp32 -> 16-bit casts of both expert weights in one launch: a thread turns eight consecutive fp32 values
+// (two 16-byte loads) into one 16-byte store; the first n1 / 8 items belong to the first tensor.
+template <typename DstT>
+__global__ __launch_bounds__(kThreads) void cast_pair_kernel(const float* __restrict__ a, DstT* __restrict__ da, int64_t n1,
+                                                             const float* __restrict__ b, DstT* __restrict__ db, int64_t n2) {
+    typedef typename Vec8<DstT>::type vec8;
+    const int64_t items1 = n1 / 8, items = items1 + n2 / 8;
+    for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < items; i += (int64_t)gridDim.x * kThreads) {
+        const bool first = i < items1;
+        const float* src = (first ? a : b) + (first ? i : i - items1) * 8;
+        DstT* dst = (first ? da : db) + (first ? i : i - items1) * 8;
+        const f32x4 lo = *reinterpret_cast<const f32x4*>(src), hi = *reinterpret_cast<const f32x4*>(src + 4);
+        vec8 v;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            v[j] = (DstT)lo[j];
+            v[4 + j] = (DstT)hi[j];
+        }
+        *reinterpret_cast<vec8*>(dst) = v;
+    }
+}
+
+extern "C" int mts_moe_cast_weights_pair(const float* w1, void* w1_out, int64_t n1, const float* w2, void* w2_out, int64_t n2,
+                                         int dst_dtype, void* stream) {
+    if (!w1 || !w1_out || !w2 || !w2_out) return MTS_ERR_NULL;
+    if (n1 < 8 || n2 < 8 || n1 % 8 || n2 % 8) return MTS_ERR_SHAPE;
+    if (!mts_aligned16(w1) || !mts_aligned16(w1_out) || !mts_aligned16(w2) || !mts_aligned16(w2_out)) return MTS_ERR_ALIGN;
+    const int blocks = grid_1d((n1 + n2) / 8);
+    hipStream_t s = (hipStream_t)stream;
+    if (dst_dtype == MTS_BF16) cast_pair_kernel<bf16_t><<<blocks, kThreads, 0, s>>>(w1, (bf16_t*)w1_out, n1, w2, (bf16_t*)w2_out, n2);
+    else if (dst_dtype == MTS_F16) cast_pair_kernel<mts_f16_t><<<blocks, kThreads, 0, s>>>(w1, (mts_f16_t*)w1_out, n1, w2, (mts_f16_t*)w2_out, n2);
+    else return MTS_ERR_DTYPE;
+    MTS_CHECK_LAUNCH();
+    return MTS_OK;
+}
+
 extern "C" int mts_version(void) { return MTS_VERSION; }
 
 extern "C" const char* mts_error_string(int code) {

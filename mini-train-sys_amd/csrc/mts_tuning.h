@@ -10,7 +10,6 @@
 //   MTS_NO_TAIL_SPLIT = 1         every tile whole (the tiles behind an XCD's last whole round are not cut in two)
 //   MTS_NO_MFMA_ROUTER = 1        router projection on the vector pipe for every shape
 //   MTS_NO_JOINT_SCHEDULE = 1     units and dX tiles of the joint backward launch are dealt round-robin / in equal ranges
-//   MTS_NO_FUSED_CAST = 1         fp32 expert weights are cast by one launch per weight instead of one for both
 // A switch is on when its value parses to a non-zero integer ("0" and the empty string leave it off).
 #pragma once
 
@@ -22,7 +21,6 @@ struct MtsTuning {
     int tile_order_mask;        // ORDER_* bits
     bool tail_split;
     bool mfma_router;
-    bool fused_cast;
     bool joint_schedule;
 };
 

@@ -25,7 +25,6 @@ MtsTuning read_environment() {
     t.tile_order_mask = flag("MTS_NO_TILE_ORDER") ? 0 : (pick && *pick ? atoi(pick) & 15 : 15);
     t.tail_split = !flag("MTS_NO_TAIL_SPLIT");
     t.mfma_router = !flag("MTS_NO_MFMA_ROUTER");
-    t.fused_cast = !flag("MTS_NO_FUSED_CAST");
     t.joint_schedule = !flag("MTS_NO_JOINT_SCHEDULE");
     return t;
 }

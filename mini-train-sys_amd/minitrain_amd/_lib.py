@@ -41,6 +41,7 @@ SIGNATURES = {
     "mts_moe_capacity_workspace_bytes": (_l, [_l, _i, _i]),
     "mts_moe_capacity_mask": (_i, [_p, _p, _l, _i, _i, _l, _p, _p, _p, _p, _l, _p]),
     "mts_moe_stage_weights": (_i, [_p, _i, _p, _i, _i, _l, _l, _i, _p]),
+    "mts_moe_cast_weights_pair": (_i, [_p, _p, _l, _p, _p, _l, _i, _p]),
     "mts_moe_fwd_gateup_swiglu": (_i, [_p, _p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p, _p, _p]),
     "mts_moe_fwd_down": (_i, [_p, _p, _p, _l, _i, _i, _i, _i, _p, _p]),
     "mts_moe_combine": (_i, [_p, _p, _p, _p, _l, _i, _i, _i, _p, _p]),

@@ -263,8 +263,18 @@ def moe_forward(x, gate_up_proj, down_proj, weights_flat, routing):
     act = _lib.dtype_code(x.dtype)
     stream = _lib.stream_of(x)
 
-    w1 = _stage(lib, gate_up_proj, False, x.dtype)
-    w2 = _stage(lib, down_proj, False, x.dtype)
+    if (gate_up_proj.dtype == down_proj.dtype == torch.float32 and x.dtype != torch.float32
+            and gate_up_proj.numel() % 8 == 0 and down_proj.numel() % 8 == 0):
+        # fp32 master weights: both casts in one launch (the backward pass reuses the copies)
+        w1, w2 = torch.empty_like(gate_up_proj, dtype=x.dtype), torch.empty_like(down_proj, dtype=x.dtype)
+        _lib.check(
+            lib.mts_moe_cast_weights_pair(gate_up_proj.data_ptr(), w1.data_ptr(), gate_up_proj.numel(), down_proj.data_ptr(),
+                                          w2.data_ptr(), down_proj.numel(), act, stream),
+            "mts_moe_cast_weights_pair",
+        )
+    else:
+        w1 = _stage(lib, gate_up_proj, False, x.dtype)
+        w2 = _stage(lib, down_proj, False, x.dtype)
     pre_act = torch.empty(TK, 2 * I, dtype=x.dtype, device=dev)
     post_act = torch.empty(TK, I, dtype=x.dtype, device=dev)
     # The routing weight is applied where the activation is formed: post_act = s * silu(g) * u.  The
