@@ -5,12 +5,11 @@ Counterpart of the reference's ``TritonOpsBackend``
 that class there is no fallback: an unsupported tensor contract raises.
 """
 
-import os
-
 from minitrain_amd.kernels.dense_ops import DenseTorchOps
 from minitrain_amd.kernels.hip.capacity import capacity_mask, is_capacity_mask_supported
 from minitrain_amd.kernels.hip.fused_moe import expert_counts, fused_moe, is_fused_moe_supported
 from minitrain_amd.kernels.hip.moe_layer import moe_layer, moe_layer_violation
+from minitrain_amd.kernels.hip.switches import SWITCHES
 from minitrain_amd.kernels.hip.router import (
     is_router_logits_supported,
     is_router_postprocess_supported,
@@ -25,8 +24,8 @@ class HipOpsBackend(DenseTorchOps):
     drops_routes = True
 
     # router_postprocess takes ``weights_dtype`` and then also returns the weights rounded to it
-    # (MTS_NO_ROUTER_CAST=1 leaves the cast to the caller, for comparisons)
-    casts_router_weights = os.environ.get("MTS_NO_ROUTER_CAST", "0") != "1"
+    # (a comparison switch leaves the cast to the caller, see switches.py)
+    casts_router_weights = SWITCHES.router_cast
 
     def router_postprocess(self, logits, top_k, *, normalize, weights_dtype=None):
         return router_postprocess(logits, top_k, normalize=normalize, weights_dtype=weights_dtype)
@@ -45,8 +44,10 @@ class HipOpsBackend(DenseTorchOps):
             return None
         return capacity_mask(expert_indices, expert_weights, num_experts, capacity)
 
-    # MTS_NO_LAYER_NODE=1 keeps the layer on the three separate operators (for comparisons)
-    offers_moe_layer = os.environ.get("MTS_NO_LAYER_NODE", "0") != "1"
+    # a comparison switch keeps the layer on the three separate operators (switches.py); an instance may also set
+    # this attribute to False, e.g. to have forward hooks on the router module fire (the one-node path does not
+    # call that module)
+    offers_moe_layer = SWITCHES.layer_node
 
     def moe_layer(self, x, router_weight, gate_up_proj, down_proj, top_k, *, normalize):
         """Extension: router projection, post-process, routing metadata and the experts as one autograd

@@ -9,11 +9,12 @@ another and joins them before it returns.
 """
 
 import functools
-import os
+import warnings
 
 import torch
 
 from minitrain_amd import _lib
+from minitrain_amd.kernels.hip.switches import SWITCHES
 
 _MAX_EXPERTS = 65534   # MTS_MAX_MOE_EXPERTS
 BLOCK_M_TOKEN = 64
@@ -188,18 +189,6 @@ def expert_counts(topk_indices: torch.Tensor, E: int) -> torch.Tensor:
     return out[:E]
 
 
-# MTS_NO_OVERLAP=1 keeps every kernel of the backward pass on the caller's stream
-_OVERLAP = os.environ.get("MTS_NO_OVERLAP", "0") != "1"
-# MTS_NO_JOINT_BWD=1 launches dW2, dW1 and dX separately (on the side streams) even where one launch could hold them
-_JOINT = os.environ.get("MTS_NO_JOINT_BWD", "0") != "1"
-# MTS_NO_TAIL_IN_JOINT=1 keeps the router's backward of the layer node in launches of its own
-_TAIL_IN_JOINT = os.environ.get("MTS_NO_TAIL_IN_JOINT", "0") != "1"
-# MTS_NO_COMBINE_IN_TAIL=1 keeps the dX combine behind that launch in a launch of its own
-_COMBINE_IN_TAIL = os.environ.get("MTS_NO_COMBINE_IN_TAIL", "0") != "1"
-# MTS_NO_JOINT_SCHEDULE=1: that launch deals its blocks out to the XCDs without looking at the routes per expert
-_SCHEDULE = os.environ.get("MTS_NO_JOINT_SCHEDULE", "0") != "1"
-# MTS_WEIGHTED_POST=0: the forward pass writes the unweighted activation and dY1 writes s * a again (tuning runs only)
-_WEIGHTED_POST = os.environ.get("MTS_WEIGHTED_POST", "1") != "0"
 _SIDE_STREAMS: dict = {}
 
 
@@ -216,8 +205,18 @@ def _side_stream(device: torch.device, index: int) -> torch.cuda.Stream:
 _DW_WORKSPACE_LIMIT = 512 * 2**20
 
 
+_warned_shapes: set = set()
+
+
 def _dw_workspace(lib, which: int, E: int, H: int, I: int, dtype: torch.dtype, device):
     nbytes = lib.mts_moe_bwd_dw_workspace_bytes(which, E, H, I) if dtype != torch.float32 else 0
+    if nbytes > _DW_WORKSPACE_LIMIT and (E, H, I) not in _warned_shapes:
+        # said once per shape: from here on an over-full expert is not cut into row chunks and the joint launch gets no
+        # schedule, so skewed routing costs these widths more time than it has to (the results are the same)
+        _warned_shapes.add((E, H, I))
+        warnings.warn(f"hip fused MoE: the row-chunk workspace of the weight-gradient GEMMs for E={E}, H={H}, I={I} would take "
+                      f"{nbytes / 2**20:.0f} MiB (limit {_DW_WORKSPACE_LIMIT / 2**20:.0f} MiB); running without it", RuntimeWarning,
+                      stacklevel=3)
     if nbytes <= 0 or nbytes > _DW_WORKSPACE_LIMIT:
         return None, 0, 0
     ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
@@ -281,7 +280,7 @@ def moe_forward(x, gate_up_proj, down_proj, weights_flat, routing):
     # down projection then yields s * y, the combine is a plain sum, and post_act is at the same time
     # the `weighted_act` operand of the dW2 GEMM, so it is kept for the backward pass instead of being
     # written again there (TK * I elements held from forward to backward, and as many fewer written).
-    weighted = _WEIGHTED_POST
+    weighted = SWITCHES.weighted_post
     _lib.check(
         lib.mts_moe_fwd_gateup_swiglu(
             x.data_ptr(), w1.data_ptr(), x_gather.data_ptr(), expert_start.data_ptr(),
@@ -354,7 +353,7 @@ def moe_backward(tensors, state, dO, needs, x_addend=None, router_tail=None):
     # streams (default priority) are forked from and joined to the caller's stream with events;
     # everything they read stays referenced until the join has been enqueued.
     main = torch.cuda.current_stream(dev)
-    overlap = _OVERLAP
+    overlap = SWITCHES.overlap
     side = [_side_stream(dev, 0), _side_stream(dev, 1)] if overlap else [main, main]
 
     def fork(*to):
@@ -399,13 +398,13 @@ def moe_backward(tensors, state, dO, needs, x_addend=None, router_tail=None):
     # order starts the long weight-gradient tiles first; no side stream is involved.  Which XCD runs which of
     # its units and dX tiles follows a table that the dO * W2 launch writes on the side (uneven routing).
     joint = (
-        _JOINT and need_x and need_w1 and need_w2 and need_s and as_stored
+        SWITCHES.joint_bwd and need_x and need_w1 and need_w2 and need_s and as_stored
         and gate_up_proj.dtype == down_proj.dtype and bool(lib.mts_moe_bwd_joint_supported(act, H, I))
     )
     ws1, ws1_ptr, ws1_bytes = _dw_workspace(lib, 1, E, H, I, x.dtype, dev) if need_w1 else (None, 0, 0)
     ws2, ws2_ptr, ws2_bytes = _dw_workspace(lib, 2, E, H, I, x.dtype, dev) if need_w2 else (None, 0, 0)
     schedule = None
-    if joint and _SCHEDULE and ws1 is not None and ws2 is not None:
+    if joint and SWITCHES.joint_schedule and ws1 is not None and ws2 is not None:
         sched_bytes = lib.mts_moe_bwd_schedule_bytes(E)
         if sched_bytes > 0:
             schedule = torch.empty(sched_bytes // 4, dtype=torch.int32, device=dev)
@@ -444,10 +443,10 @@ def moe_backward(tensors, state, dO, needs, x_addend=None, router_tail=None):
         )
         sched_ptr = _lib.ptr(schedule)
         rt = router_tail
-        if rt is not None and _TAIL_IN_JOINT and lib.mts_moe_bwd_joint_router_supported(act, T, H, I, E):
+        if rt is not None and SWITCHES.tail_in_joint and lib.mts_moe_bwd_joint_router_supported(act, T, H, I, E):
             # the router's backward as trailing blocks of the same launch: it needs nothing the launch writes
             dx_r, dw_r = torch.empty_like(x), torch.empty_like(rt.router_weight)
-            dx = torch.empty_like(x) if _COMBINE_IN_TAIL else None
+            dx = torch.empty_like(x) if SWITCHES.combine_in_tail else None
             rws_bytes = lib.mts_moe_head_bwd_workspace_bytes(T, H, E)
             rws = torch.empty(rws_bytes, dtype=torch.uint8, device=dev)
             _lib.check(

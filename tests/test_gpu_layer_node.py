@@ -202,13 +202,13 @@ def test_router_backward_inside_the_joint_launch_equals_its_own_launches(T, H, E
     ops = hip_backend()
     x, w_r, w1, w2, g = O.make_inputs(900 + T, T, H, E, I)
     case = dict(x=x, w_r=w_r, w1=w1, w2=w2, g=g)
-    monkeypatch.setattr(F, "_JOINT", True)
-    monkeypatch.setattr(F, "_TAIL_IN_JOINT", True)
-    monkeypatch.setattr(F, "_COMBINE_IN_TAIL", True)   # the dX combine too (inside the library: with the partial sums
+    monkeypatch.setattr(F.SWITCHES, "joint_bwd", True)
+    monkeypatch.setattr(F.SWITCHES, "tail_in_joint", True)
+    monkeypatch.setattr(F.SWITCHES, "combine_in_tail", True)   # the dX combine too (inside the library: with the partial sums
     inside = _layer_grads(ops, case, K, True, dtype, fp32_params)[1]   # for two routes per token, else one more launch)
-    monkeypatch.setattr(F, "_COMBINE_IN_TAIL", False)
+    monkeypatch.setattr(F.SWITCHES, "combine_in_tail", False)
     own_combine = _layer_grads(ops, case, K, True, dtype, fp32_params)[1]
-    monkeypatch.setattr(F, "_TAIL_IN_JOINT", False)
+    monkeypatch.setattr(F.SWITCHES, "tail_in_joint", False)
     apart = _layer_grads(ops, case, K, True, dtype, fp32_params)[1]
     for other in (own_combine, apart):
         for name, a, b in zip(("dx", "dW_r", "dW1", "dW2"), inside, other):

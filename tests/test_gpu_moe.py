@@ -201,9 +201,9 @@ def test_joint_backward_launch_equals_separate_launches(T, H, E, I, dtype, fp32_
         idx[heavy & (idx[:, 1] == 1), 1] = 0
         case.update(idx=idx)
     args = (case["x"], case["w1"], case["w2"], case["idx"], case["w"], case["g"])
-    monkeypatch.setattr(F, "_JOINT", True)    # the default, whatever the environment says
+    monkeypatch.setattr(F.SWITCHES, "joint_bwd", True)    # the default, whatever the environment says
     joint = hip_moe_grads(*args)
-    monkeypatch.setattr(F, "_JOINT", False)
+    monkeypatch.setattr(F.SWITCHES, "joint_bwd", False)
     separate = hip_moe_grads(*args)
     for name, a, b in zip(NAMES, joint[1], separate[1]):
         assert a.dtype == b.dtype and torch.equal(a, b), name
@@ -290,10 +290,10 @@ def test_unweighted_post_act_path(monkeypatch):
         case = routed_case(81, *shape)
         args = (case["x"], case["w1"], case["w2"], case["idx"], case["w"], case["g"])
         with monkeypatch.context() as m:
-            m.setattr(F, "_WEIGHTED_POST", True)    # the default, whatever the environment says
+            m.setattr(F.SWITCHES, "weighted_post", True)    # the default, whatever the environment says
             a = hip_moe_grads(*args)
         with monkeypatch.context() as m:
-            m.setattr(F, "_WEIGHTED_POST", False)
+            m.setattr(F.SWITCHES, "weighted_post", False)
             _compare(case)
             b = hip_moe_grads(*args)
         assert_close_scaled(a[0], b[0], 1e-2, "out, weight in the epilogue vs in the combine")
@@ -487,15 +487,15 @@ def test_scheduled_joint_launch_equals_the_unscheduled_one(dtype, fp32_params, m
     if fp32_params:
         case["w1"], case["w2"] = case["w1"].float(), case["w2"].float()
     args = (case["x"], case["w1"], case["w2"], case["idx"], case["w"], case["g"])
-    monkeypatch.setattr(F, "_JOINT", True)
-    monkeypatch.setattr(F, "_SCHEDULE", True)
+    monkeypatch.setattr(F.SWITCHES, "joint_bwd", True)
+    monkeypatch.setattr(F.SWITCHES, "joint_schedule", True)
     with_table = hip_moe_grads(*args)
-    monkeypatch.setattr(F, "_SCHEDULE", False)
+    monkeypatch.setattr(F.SWITCHES, "joint_schedule", False)
     without = hip_moe_grads(*args)
     assert torch.equal(with_table[0], without[0])
     for name, a, b in zip(NAMES, with_table[1], without[1]):
         assert a.dtype == b.dtype and torch.equal(a, b), name
-    monkeypatch.setattr(F, "_SCHEDULE", True)
+    monkeypatch.setattr(F.SWITCHES, "joint_schedule", True)
     _compare(case)
 
 
