@@ -281,7 +281,7 @@ int mts_moe_bwd_dx(const void* d_pre_act, const void* w1, int w1_as_stored,
  *
  * workspace (both weight-gradient entry points): NULL, or at least
  * mts_moe_bwd_dw_workspace_bytes(which, E, H, I) bytes (which = 1 for dW1, 2 for dW2).
- * With a workspace, an expert that holds more than 1.25 times the balanced share of the
+ * With a workspace, an expert that holds more than 1.15 times the balanced share of the
  * routes has its rows cut into chunks that run as separate blocks and are added in a
  * fixed order by a second kernel, so that skewed routing does not leave the GPU waiting
  * for the tiles of the fullest expert; results stay run-to-run identical.  Without one,

@@ -446,7 +446,7 @@ def test_joint_launch_schedule(E, K, shares):
         parts = sorted(by_expert.get(e, []))
         assert parts and parts[0][0] == start[e] and parts[-1][1] == start[e + 1]            # every expert is covered ...
         assert all(a[1] == b[0] for a, b in zip(parts, parts[1:]))                            # ... by consecutive ranges
-        cut = c[e] > share + share // 4
+        cut = c[e] > share + share * 3 // 20
         assert len(parts) == (-(-c[e] // share) if cut else 1)
         assert all((p[2] >= 0) == cut for p in parts)
         slot_seen += [p[2] for p in parts if cut]
