@@ -49,9 +49,9 @@ RIDGE_FLOP_PER_BYTE = PEAK_BF16_TFLOPS * 1e12 / (PEAK_HBM_GBS * 1e9)   # 312.5: 
 # line names the file that holds the runs' commands and tables.
 TRAFFIC_SOURCE = "profiles/moe_layer_24x1024_hbm_traffic.txt"
 MEASURED_TRAFFIC_BYTES = {
-    "fwd_gateup_swiglu": 546.9e6, "fwd_down": 224.1e6, "bwd_dy1": 539.7e6,
-    "bwd_joint": 1232.3e6,   # the joint launch (1067.2) and the launch of partial sums with the dX combine behind it (165.1)
-    "combine": 114.6e6,
+    "fwd_gateup_swiglu": 546.9e6, "fwd_down": 224.1e6, "bwd_dy1": 539.6e6,
+    "bwd_joint": 1244.4e6,   # the joint launch (1079.2) and the launch of partial sums with the dX combine behind it (165.1)
+    "combine": 114.7e6,
 }
 
 WORKLOAD = dict(name="moe_layer_24x1024_d768_e8_top2_ff1024_bf16", seed=1, T=24576, H=768, E=8, K=2, I=1024)

@@ -10,8 +10,12 @@ expert loop on the same GPU, and the correctness columns ``max_abs``, ``max_rel`
 
     python -m minitrain_amd.benchmarks.moe_rows --tokens 24576 --zipf --capacity-factor 1.0
 
+    python -m minitrain_amd.benchmarks.moe_rows --tokens 24576 --expert-shares 4862,12086,3507,3153,6471,5392,7811,5870 --no-torch
+
 prints one JSON row per provider (``hip``, ``torch``).  ``--zipf`` skews the routing towards the
-low expert ids (probability ~ rank^-1.2); with ``--capacity-factor`` every expert accepts at most
+low expert ids (probability ~ rank^-1.2); ``--expert-shares`` draws every token's experts one after the
+other with odds proportional to the given numbers (e.g. the routes per expert a trained router produced),
+so that the routes per expert come out close to those proportions; with ``--capacity-factor`` every expert accepts at most
 ``ceil(factor*T*K/E)`` routes (minitrain/model/moe_router.py:38-42), the ``hip`` row runs the compacted
 dispatch (dropped routes carry index -1), a ``hip_zero_weight`` row runs the same weights with every
 route still dispatched, which is what masking the weights alone amounts to, and the selection kernel
@@ -45,7 +49,7 @@ def torch_expert_loop(x, gate_up, down, idx, w):
     return out
 
 
-def make_case(tokens, H, I, E, K, dtype, seed, zipf=False):
+def make_case(tokens, H, I, E, K, dtype, seed, zipf=False, shares=None):
     g = torch.Generator(device="cuda").manual_seed(seed)
     rn = lambda *s, std=1.0: (torch.randn(*s, generator=g, device="cuda") * std).to(dtype)
     x, gate_up, down = rn(tokens, H), rn(E, 2 * I, H, std=0.02), rn(E, H, I, std=0.02)
@@ -54,6 +58,16 @@ def make_case(tokens, H, I, E, K, dtype, seed, zipf=False):
         rank = torch.arange(1, E + 1, device="cuda", dtype=torch.float32)
         logits = logits + torch.log(rank ** -1.2 / (rank ** -1.2).sum())
     p, idx = torch.topk(torch.softmax(logits, dim=-1), K, dim=-1)
+    if shares is not None:
+        # K distinct experts per token, drawn one after the other with odds proportional to `shares`
+        odds = torch.tensor(shares, dtype=torch.float64, device="cuda").expand(tokens, E).clone()
+        cols = []
+        for _ in range(K):
+            c = torch.multinomial(odds, 1, generator=g)
+            odds.scatter_(1, c, 0.0)
+            cols.append(c)
+        idx = torch.cat(cols, 1)
+        p = torch.gather(torch.softmax(logits, dim=-1), 1, idx)
     w32 = p / p.sum(dim=-1, keepdim=True)
     grad = rn(tokens, H)
     idx = idx.int()
@@ -188,16 +202,17 @@ def correctness(op, case):
 
 
 def operator_rows(profile="layer", tokens=24576, iters=20, warmup=5, seed=1, with_torch=True, zipf=False,
-                  capacity_factor=None):
+                  capacity_factor=None, shares=None):
     """The benchmark rows as dictionaries: ``hip`` first, then ``hip_zero_weight`` (capacity runs) and ``torch``."""
     from minitrain_amd.model.ops import get_ops_backend
 
     H, I, E, K = PROFILES[profile]
     ops = get_ops_backend("hip")
-    case = make_case(tokens, H, I, E, K, torch.bfloat16, seed, zipf=zipf)
+    case = make_case(tokens, H, I, E, K, torch.bfloat16, seed, zipf=zipf, shares=shares)
     common = dict(op="fused_moe", profile=profile, size=tokens, hidden=H, expert_width=I, experts=E,
                   top_k=K, dtype="bf16", device=torch.cuda.get_device_name(0), timer="cuda_events",
-                  routing="zipf" if zipf else "uniform")
+                  routing="shares" if shares is not None else ("zipf" if zipf else "uniform"),
+                  routes_per_expert=torch.bincount(case["idx"].flatten().long(), minlength=E).tolist())
     extra_rows = []
     if capacity_factor is not None:
         capacity, dropped, accepted = limit_capacity(case, ops, E, capacity_factor)
@@ -227,9 +242,14 @@ def main():
     ap.add_argument("--no-torch", action="store_true", help="skip the PyTorch expert-loop baseline rows")
     ap.add_argument("--zipf", action="store_true", help="routing skewed towards the low expert ids")
     ap.add_argument("--capacity-factor", type=float, default=None)
+    ap.add_argument("--expert-shares", type=str, default=None,
+                    help="comma-separated odds per expert: the routes per expert come out close to these proportions")
     args = ap.parse_args()
+    shares = [float(v) for v in args.expert_shares.split(",")] if args.expert_shares else None
+    if shares is not None and len(shares) != PROFILES[args.profile][2]:
+        ap.error(f"--expert-shares needs {PROFILES[args.profile][2]} numbers")
     for row in operator_rows(args.profile, args.tokens, args.iters, args.warmup, args.seed, not args.no_torch, args.zipf,
-                             args.capacity_factor):
+                             args.capacity_factor, shares):
         print(json.dumps(row))
 
 
