@@ -21,7 +21,11 @@ from dataclasses import dataclass
 
 
 def _off(name: str) -> bool:
-    return os.environ.get(name, "0") == "1"
+    """A switch is set when its value parses to a non-zero integer ("0" and the empty string leave it alone)."""
+    try:
+        return int(os.environ.get(name, "0") or "0") != 0
+    except ValueError:
+        return False
 
 
 @dataclass
