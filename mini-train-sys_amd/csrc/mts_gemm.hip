@@ -595,14 +595,22 @@ __device__ __forceinline__ bool find_rows_tile(const RowsParams& p, int b, int& 
     ntile = j % p.n_tiles;
     parts = 1;      // pieces the tile is cut into: this block computes piece `part`
     int part = 0;
-    if (p.xcd_ranges) {
+    if (p.xcd_ranges && p.sched) {
+        // the XCD's range of m-tiles comes from the table (n-tile groups and cut tiles are not combined with it); a block
+        // the table leaves without work finds that out with one load
+        const int my = p.sched[kXcds + xcd];
+        int k = j / p.n_tiles;
+        if (k >= my) return false;
+        if (p.reverse) k = my - 1 - k;
+        tile = p.sched[xcd] + k;
+    } else if (p.xcd_ranges) {
         // m-tiles of the launch: the first (total % 8) XCDs take one more than the others
         int mine = 0;
         for (int le = lane; le < p.E; le += MTS_WAVE) mine += (p.expert_start[le + 1] - p.expert_start[le] + BM - 1) / BM;
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) mine += __shfl_xor(mine, o, MTS_WAVE);
         const int per = mine / kXcds, rem = mine % kXcds;
-        const int my = p.sched ? p.sched[kXcds + xcd] : per + (xcd < rem ? 1 : 0);
+        const int my = per + (xcd < rem ? 1 : 0);
         if (p.tail_slots > 0) {
             // the blocks behind the last whole round of this XCD: two per tile, the upper and the lower half (cutting
             // into four where a quarter of the slots is filled gains another 0.15 % of the layer step: not done)
@@ -626,7 +634,7 @@ __device__ __forceinline__ bool find_rows_tile(const RowsParams& p, int b, int& 
         }
         if (k >= my) return false;
         if (p.reverse) k = my - 1 - k;
-        tile = (p.sched ? p.sched[xcd] : xcd * per + (xcd < rem ? xcd : rem)) + k;
+        tile = xcd * per + (xcd < rem ? xcd : rem) + k;
     }
     int seen = 0;
     for (int e0 = 0; e0 < p.E; e0 += MTS_WAVE) {
@@ -2238,13 +2246,16 @@ bool bwd_joint_ok(int H, int I) {
 // function is compiled for that) and whole 16-byte chunks per row
 bool combine_in_tail(const BwdJointParams& q) { return q.c_out && q.n_router && q.c_K == 2 && q.rH % 8 == 0; }
 
-// table entries per XCD and the most dX m-tiles one XCD is given (twice the even share): the dO*W2 launch that writes
-// the table and the joint launch that sizes its grid by it must agree
+// Table entries per XCD and the most dX m-tiles one XCD is given: the dO*W2 launch that writes the table and the joint
+// launch that sizes its grid by it must agree.  One and a half even shares: the routing of a trained router asks for up
+// to 1.3; every block beyond an XCD's tiles costs the launch a microsecond of one CU in front of the router's blocks
+// (twice the even share: 640 such blocks at the 24576-token layer, 2.7 us of the whole chip).
 void schedule_shape(int64_t TK, int E, int& slots, int& cap) {
     slots = (2 * E + kXcds - 1) / kXcds;
     const int64_t upper = m_tiles<WsWide>(TK, E);
     const int64_t even = (upper + kXcds - 1) / kXcds;
-    cap = (int)(2 * even + 1 < upper ? 2 * even + 1 : upper);
+    const int64_t most = even + (even / 2 > 2 ? even / 2 : 2);
+    cap = (int)(most < upper ? most : upper);
 }
 
 int launch_bwd_joint(BwdJointParams q, int E, int grad_dtype, void* ws1, int64_t ws1_bytes, void* ws2, int64_t ws2_bytes,
@@ -2281,6 +2292,7 @@ int launch_bwd_joint(BwdJointParams q, int E, int grad_dtype, void* ws1, int64_t
         q.dw1.sched_slots = q.dw2.sched_slots = slots;
         if (q.dx.xcd_ranges) {
             q.dx.sched = schedule;
+            q.dx.n_groups = 1;
             q.n_dx = cap * q.dx.n_tiles * kXcds;
         }
     }
