@@ -54,6 +54,9 @@ MEASURED_TRAFFIC_BYTES = {
     "combine": 114.7e6,
 }
 
+# the forward GEMMs as the layer node issues them: one launch unless the comparison switch asks for two
+JOINT_FWD = os.environ.get("MTS_NO_JOINT_FWD", "0") in ("", "0")
+
 WORKLOAD = dict(name="moe_layer_24x1024_d768_e8_top2_ff1024_bf16", seed=1, T=24576, H=768, E=8, K=2, I=1024)
 
 
@@ -152,6 +155,15 @@ def time_layer(layer, steps, warmup):
     return (time.perf_counter() - t0) / steps
 
 
+def check_forward_status():
+    """The joint gate/up + down launches of the steps so far all ran through (their outputs would be invalid otherwise)."""
+    from minitrain_amd.kernels.hip.fused_moe import joint_forward_status
+
+    status = joint_forward_status()
+    if status != 0:
+        raise RuntimeError(f"the joint gate/up + down launch reported status {status}")
+
+
 def stage_breakdown(layer, steps):
     """Launch every stage of the layer step through the C ABI, in the order the layer node issues them,
     with HIP events (recorded on the launching stream) around each call.
@@ -193,18 +205,32 @@ def stage_breakdown(layer, steps):
     dx_r, dw_r = torch.empty(T, H, **bf), torch.empty_like(w_r)
     sched = torch.empty(lib.mts_moe_bwd_schedule_bytes(E) // 4, **i32)   # written by the dO*W2 launch, read by the joint one
 
+    status_words = []
     unit = 2.0 * TK * H * I                  # FLOPs of one [TK,H] x [H,I] product
     w1_b, w2_b = E * 2 * I * H * esz, E * H * I * esz
     rows_h, rows_i = TK * H * esz, TK * I * esz
+    if JOINT_FWD and lib.mts_moe_fwd_joint_supported(B, H, I):
+        # gate/up and down in one launch, as the layer node issues them: post_act is written once and read inside the launch
+        jws = torch.zeros(lib.mts_moe_fwd_joint_workspace_bytes(TK, E) // 4, **i32)
+        status_words.append(jws)
+        fwd_gemm_stages = [
+            ("fwd_gateup_down", 3 * unit, rows_h + w1_b + 3 * rows_i + TK * (4 + 4 + esz) + w2_b + rows_h,
+             lambda: lib.mts_moe_fwd_gateup_down(p(x), p(w1), p(w2), p(xg), p(es), p(r_wa), p(ss), T, K, E, H, I, B, p(pre), p(post),
+                                                 p(y), p(jws), jws.numel() * 4, st)),
+        ]
+    else:
+        fwd_gemm_stages = [
+            ("fwd_gateup_swiglu", 2 * unit, rows_h + w1_b + 3 * rows_i + TK * (4 + 4 + esz),
+             lambda: lib.mts_moe_fwd_gateup_swiglu(p(x), p(w1), p(xg), p(es), p(r_wa), p(ss), T, K, E, H, I, B, p(pre), p(post), st)),
+            ("fwd_down", unit, rows_i + w2_b + rows_h, lambda: lib.mts_moe_fwd_down(p(post), p(w2), p(es), TK, E, H, I, B, p(y), st)),
+        ]
     stages = [
         # name, FLOPs, algorithmic bytes, call
         ("head_fwd", 2.0 * T * H * E, T * H * esz + E * H * 4 + T * E * 4 + T * K * (4 + 4 + esz) + TK * 4 * 4,
          lambda: lib.mts_moe_head_fwd(p(x), p(w_r), T, H, E, K, 1, B, p(logits), p(r_w), p(r_i), p(r_wa), p(r_stats),
                                       p(r_stats) + 4 * E, p(r_stats) + 4 * E + 4, p(cnt), p(r_stats) + 4 * E + 8,
                                       p(r_stats) + 4 * E + 12, p(es), p(ss), p(sr), p(xg), p(hws), hws.numel(), st)),
-        ("fwd_gateup_swiglu", 2 * unit, rows_h + w1_b + 3 * rows_i + TK * (4 + 4 + esz),
-         lambda: lib.mts_moe_fwd_gateup_swiglu(p(x), p(w1), p(xg), p(es), p(r_wa), p(ss), T, K, E, H, I, B, p(pre), p(post), st)),
-        ("fwd_down", unit, rows_i + w2_b + rows_h, lambda: lib.mts_moe_fwd_down(p(post), p(w2), p(es), TK, E, H, I, B, p(y), st)),
+        *fwd_gemm_stages,
         ("combine", 1.0 * TK * H, rows_h + T * H * esz + TK * 4,
          lambda: lib.mts_moe_combine(p(y), None, None, p(sr), T, K, H, B, p(out), st)),
         ("bwd_dy1", unit, rows_h + w2_b + 2 * rows_i + 2 * rows_i + TK * npart * 4 + TK * (4 + 4 + esz),
@@ -237,6 +263,9 @@ def stage_breakdown(layer, steps):
             if it:
                 elapsed[j].append((e0, e1))
     torch.cuda.synchronize()
+    for words in status_words:
+        if int(words[0]) != 0:
+            raise RuntimeError(f"the joint gate/up + down launch reported status {int(words[0])}")
     rows = []
     for j, (name, flops, nbytes, _) in enumerate(stages):
         ms = float(np.mean([a.elapsed_time(b) for a, b in elapsed[j]]))
@@ -327,6 +356,7 @@ def run_config(ops, seed, T, steps, warmup, **layer_kwargs):
     settle(layer, seconds=0.2, at_least=10)
     torch.cuda.reset_peak_memory_stats()
     sec = time_layer(layer, steps, warmup)
+    check_forward_status()
     rec = {"tokens": T, "seed": seed, "ms_per_step": round(sec * 1e3, 4), "tokens_per_s": round(T / sec, 1),
            "layer_gemm_tflops": round(18.0 * T * w["K"] * w["H"] * w["I"] / sec / 1e12, 2),
            "peak_hbm_allocated_mb": round(torch.cuda.max_memory_allocated() / 2**20, 1),
@@ -425,6 +455,7 @@ def main():
     layer = Layer(ops, *make_inputs(w["seed"], w["T"], w["H"], w["E"], w["I"]), w["K"])
     settled = 0 if args.no_settle else settle(layer)
     sec = time_layer(layer, args.steps, args.warmup)
+    check_forward_status()
     tokens_per_s = w["T"] / sec
     gemm_flops = 18.0 * w["T"] * w["K"] * w["H"] * w["I"]
 
@@ -460,7 +491,7 @@ def main():
                               "frac_mfma": dom["frac_mfma"], "frac_hbm": dom["frac_hbm"],
                               "traffic": traffic, "traffic_source": TRAFFIC_SOURCE if traffic is not None else None,
                               "traffic_over_algorithmic": round(traffic / dom["algorithmic_bytes"], 3) if traffic else None}
-        gemm_rows = [r for r in rows if r["stage"] in ("fwd_gateup_swiglu", "fwd_down", "bwd_dy1", "bwd_joint")]
+        gemm_rows = [r for r in rows if r["stage"] in ("fwd_gateup_down", "fwd_gateup_swiglu", "fwd_down", "bwd_dy1", "bwd_joint")]
         g_ms = sum(r["avg_ms"] for r in gemm_rows)
         g_ach = sum(r["flops"] for r in gemm_rows) / (g_ms * 1e-3) / 1e12
         result["gemm_roofline"] = {"bound": "mfma", "achieved": round(g_ach, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",

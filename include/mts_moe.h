@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define MTS_VERSION 3
+#define MTS_VERSION 4
 
 /* element types of activations / weights / weight gradients */
 #define MTS_BF16 0
@@ -232,6 +232,31 @@ int mts_moe_fwd_gateup_swiglu(const void* x, const void* w1, const int32_t* x_ga
  * y[r] = W2[e] a[r];  post_act [TK,I], w2 [E,H,I] -> y [TK,H].                */
 int mts_moe_fwd_down(const void* post_act, const void* w2, const int32_t* expert_start,
                      int64_t TK, int E, int H, int I, int act_dtype, void* y, void* stream);
+
+/* The two launches above as ONE (the pair of launches in _FusedMoEFunction.forward,
+ * minitrain/kernels/triton/fused_moe.py:203-249): same arguments, same tiles, bit-identical pre_act,
+ * post_act and y.  On their own both GEMMs end in a round of tiles that fills a fraction of the chip;
+ * in one launch the down tiles take the CUs as the gate/up tiles leave them (forward GEMMs -5 %).
+ * A down tile reads post_act rows that gate/up tiles of the same launch write: the m-tiles of both
+ * parts go to the XCDs in the same contiguous ranges, so writers and readers of a row share an L2, and
+ * a counter per m-tile in `workspace` tells the readers when the rows are complete.
+ *   mts_moe_fwd_joint_supported: 1 where the launch exists (bf16 / fp16, H and I multiples of 64, one
+ *     expert's W1 no larger than an XCD's L2); elsewhere mts_moe_fwd_gateup_down returns MTS_ERR_SHAPE.
+ *   workspace: mts_moe_fwd_joint_workspace_bytes(TK, E) bytes of int32, 16-byte aligned, ALL ZERO on the
+ *     first call.  A launch that ran through leaves it all zero, so calls that follow one another on a
+ *     stream share one workspace (larger and smaller problems alike); calls that may overlap need one each.
+ *   status: word 0 of the workspace stays 0.  A block that waited longer than 200 ms for its rows gives
+ *     up and sets bit 0 (every other wait then ends at once: no launch hangs); a block that finds rows
+ *     written on another XCD than its own sets bit 1.  Either way the outputs of that call are invalid
+ *     and the workspace must be cleared before it is used again.  Reading the word is the caller's
+ *     business (after a synchronisation, or from a copy made on the stream).                          */
+int mts_moe_fwd_joint_supported(int act_dtype, int H, int I);
+int64_t mts_moe_fwd_joint_workspace_bytes(int64_t TK, int E);
+int mts_moe_fwd_gateup_down(const void* x, const void* w1, const void* w2, const int32_t* x_gather,
+                            const int32_t* expert_start, const void* weights,
+                            const int32_t* s_scatter, int64_t T, int K, int E, int H, int I,
+                            int act_dtype, void* pre_act, void* post_act, void* y,
+                            int32_t* workspace, int64_t workspace_bytes, void* stream);
 
 /* Replaces _token_gather_weighted_sum_kernel (fused_moe_kernels.py:451-498):
  * out[t] = addend[t] + sum_k w[t,k] * y[s_reverse[t*K+k]]  (fp32 sum, one rounding);

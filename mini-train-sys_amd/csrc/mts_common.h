@@ -48,6 +48,10 @@ int mts_moe_fwd_gateup_swiglu_f16(const void* x, const void* w1, const int32_t* 
                                   void* stream);
 int mts_moe_fwd_down_f16(const void* post_act, const void* w2, const int32_t* expert_start, int64_t TK, int E, int H,
                          int I, int act_dtype, void* y, void* stream);
+int mts_moe_fwd_gateup_down_f16(const void* x, const void* w1, const void* w2, const int32_t* x_gather,
+                                const int32_t* expert_start, const void* weights, const int32_t* s_scatter, int64_t T, int K,
+                                int E, int H, int I, int act_dtype, void* pre_act, void* post_act, void* y,
+                                int32_t* workspace, int64_t workspace_bytes, void* stream);
 int mts_moe_bwd_dy1_f16(const void* d_out, const void* w2, int w2_as_stored, const void* pre_act, const void* weights,
                         const int32_t* x_gather, const int32_t* s_scatter, const int32_t* expert_start, int64_t T,
                         int K, int E, int H, int I, int act_dtype, void* d_pre_act, void* weighted_act,

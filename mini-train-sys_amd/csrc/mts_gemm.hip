@@ -145,6 +145,8 @@ struct RowsParams {
     int reverse;               // with xcd_ranges: the range's m-tiles are walked from the last to the first
     int tail_slots;            // with xcd_ranges: blocks an XCD runs at a time; when the tiles behind its last whole round
                                // fill at most half of them, each of those is cut into two tiles of half the height (0: never)
+    int tail_tiles;            // with xcd_ranges: this many tiles at the end of every XCD's list are cut in two whatever the rounds
+                               // come to (a launch whose blocks start behind another part's: its rounds are not aligned)
     const int32_t* sched;      // with xcd_ranges: the m-tile range of every XCD (first[8], count[8]) from the schedule of the joint
                                // backward launch, or NULL: equal ranges
     int32_t* sched_out;        // dO*W2 launch: one more block writes the schedule of the joint backward launch here (NULL: none)
@@ -586,8 +588,12 @@ constexpr int kXcds = 8;
 // expert_start[l] and [l+1], a wave scan turns tile counts into tile offsets, and a
 // ballot picks the first expert whose offset range contains the tile (63 experts per
 // round; more experts take more rounds).
+// mtile: the m-tile's index in expert order, -1 where the block has none; a block that has the empty half of a cut tile
+// (the tile's rows end in the other half) gets the index and the answer false.
 template <int BM>
-__device__ __forceinline__ bool find_rows_tile(const RowsParams& p, int b, int& e, int& row0, int& rend, int& ntile, int& parts) {
+__device__ __forceinline__ bool find_rows_tile(const RowsParams& p, int b, int& e, int& row0, int& rend, int& ntile, int& parts,
+                                               int& mtile) {
+    mtile = -1;
     const int xcd = b % kXcds;
     int j = b / kXcds;
     const int lane = threadIdx.x % MTS_WAVE;
@@ -611,11 +617,12 @@ __device__ __forceinline__ bool find_rows_tile(const RowsParams& p, int b, int& 
         for (int o = 32; o > 0; o >>= 1) mine += __shfl_xor(mine, o, MTS_WAVE);
         const int per = mine / kXcds, rem = mine % kXcds;
         const int my = per + (xcd < rem ? 1 : 0);
-        if (p.tail_slots > 0) {
+        if (p.tail_slots > 0 || p.tail_tiles > 0) {
             // the blocks behind the last whole round of this XCD: two per tile, the upper and the lower half (cutting
             // into four where a quarter of the slots is filled gains another 0.15 % of the layer step: not done)
-            const int total = my * p.n_tiles, whole = total / p.tail_slots * p.tail_slots;
-            const int cut = 2 * (total - whole) <= p.tail_slots ? 2 : 1;
+            const int total = my * p.n_tiles;
+            const int whole = p.tail_tiles > 0 ? (total > p.tail_tiles ? total - p.tail_tiles : 0) : total / p.tail_slots * p.tail_slots;
+            const int cut = p.tail_tiles > 0 || 2 * (total - whole) <= p.tail_slots ? 2 : 1;
             if (cut > 1 && j >= whole) {
                 parts = cut;
                 part = (j - whole) % cut;
@@ -655,6 +662,7 @@ __device__ __forceinline__ bool find_rows_tile(const RowsParams& p, int b, int& 
             e = e0 + w;
             row0 = __shfl(s0, w, MTS_WAVE) + (tile - first) * BM;
             rend = __shfl(s1, w, MTS_WAVE);
+            mtile = tile;
             if (parts > 1) {
                 row0 += part * (BM / parts);
                 if (row0 + BM / parts < rend) rend = row0 + BM / parts;
@@ -671,15 +679,22 @@ __device__ __forceinline__ bool find_rows_tile(const RowsParams& p, int b, int& 
 // and LDS addresses built from these values then stay in scalar registers (a buffer instruction whose
 // descriptor sits in vector registers is wrapped in a loop over its distinct values).
 template <int BM>
-__device__ __forceinline__ bool locate_rows_tile(const RowsParams& p, int b, int& e, int& row0, int& rend, int& ntile, int& parts) {
-    int fe = 0, frow0 = 0, frend = 0, fn = 0, fh = 1;
-    const bool found = find_rows_tile<BM>(p, b, fe, frow0, frend, fn, fh);
+__device__ __forceinline__ bool locate_rows_tile(const RowsParams& p, int b, int& e, int& row0, int& rend, int& ntile, int& parts,
+                                                 int& mtile) {
+    int fe = 0, frow0 = 0, frend = 0, fn = 0, fh = 1, fm = -1;
+    const bool found = find_rows_tile<BM>(p, b, fe, frow0, frend, fn, fh, fm);
     e = __builtin_amdgcn_readfirstlane(fe);
     row0 = __builtin_amdgcn_readfirstlane(frow0);
     rend = __builtin_amdgcn_readfirstlane(frend);
     ntile = __builtin_amdgcn_readfirstlane(fn);
     parts = __builtin_amdgcn_readfirstlane(fh);
+    mtile = __builtin_amdgcn_readfirstlane(fm);
     return __builtin_amdgcn_readfirstlane((int)found) != 0;
+}
+template <int BM>
+__device__ __forceinline__ bool locate_rows_tile(const RowsParams& p, int b, int& e, int& row0, int& rend, int& ntile, int& parts) {
+    int mtile;
+    return locate_rows_tile<BM>(p, b, e, row0, rend, ntile, parts, mtile);
 }
 template <int BM>
 __device__ __forceinline__ bool locate_rows_tile(const RowsParams& p, int b, int& e, int& row0, int& rend, int& ntile) {
@@ -993,8 +1008,11 @@ constexpr int ws_lds_elems() {
 }
 
 // one output tile: rows [row0, rend) of expert e (at most T::BM of them), column tile ntile
-template <class T, int EPI, bool BKM>
-__device__ __forceinline__ void rows_gemm_ws_tile(const RowsParams& p, bf16_t* smem, int e, int row0, int rend, int ntile) {
+// `rows_ready` runs in the producer waves of a tile on three activation buffers, behind the first loads of the weights and
+// in front of the first loads of the activation rows (a launch whose rows are written by other blocks of the same launch).
+template <class T, int EPI, bool BKM, class RowsReady = NoHook>
+__device__ __forceinline__ void rows_gemm_ws_tile(const RowsParams& p, bf16_t* smem, int e, int row0, int rend, int ntile,
+                                                  RowsReady rows_ready = RowsReady()) {
     constexpr bool SWIGLU = (EPI == EPI_SWIGLU);
     constexpr int S = T::STAGES, L = T::A_INSTR + T::B_INSTR;
     const int n0 = ntile * (SWIGLU ? T::BN / 2 : T::BN);
@@ -1072,8 +1090,10 @@ __device__ __forceinline__ void rows_gemm_ws_tile(const RowsParams& p, bf16_t* s
                 for (int j = 0; j < T::B_INSTR; ++j)
                     __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_b, MTS_LDS_PTR(sb + j * 512), 16, (int)voff_b[j], soff_b, 0, 0);
             };
-            issue_a(0, 0);
+            // in this order the loads that the first barrier does not wait for are still the youngest
             issue_b(0, 0);
+            rows_ready(0);
+            issue_a(0, 0);
             if (nk > 1) issue_a(1, 1);
             int abuf = 2;   // activation buffer of tile kt+2
             for (int kt = 0; kt < nk; ++kt) {
@@ -1175,16 +1195,23 @@ __device__ __forceinline__ void rows_gemm_ws_tile(const RowsParams& p, bf16_t* s
 
 // the work of block `block` of a launch; `smem` holds ws_lds_elems<T, EPI>() elements, 1 KiB aligned.
 // TH (same block shape and columns, half the rows) runs the halves of the tiles that a launch with tail_slots cuts up.
+// a located tile, whole (T) or one of `parts` = 2 halves (TH)
+template <class T, int EPI, bool BKM, class TH, class RowsReady = NoHook>
+__device__ __forceinline__ void rows_gemm_ws_run(const RowsParams& p, bf16_t* smem, int e, int row0, int rend, int ntile, int parts,
+                                                 RowsReady rows_ready = RowsReady()) {
+    if constexpr (TH::BM != T::BM) {
+        if (parts == 2) return rows_gemm_ws_tile<TH, EPI, BKM>(p, smem, e, row0, rend, ntile, rows_ready);
+    }
+    rows_gemm_ws_tile<T, EPI, BKM>(p, smem, e, row0, rend, ntile, rows_ready);
+}
+
 template <class T, int EPI, bool BKM, class TH = T>
 __device__ __forceinline__ void rows_gemm_ws_block(const RowsParams& p, bf16_t* smem, int block) {
     static_assert(TH::NT == T::NT && TH::BN == T::BN && (TH::BM == T::BM || 2 * TH::BM == T::BM), "half tile shape");
     static_assert(ws_lds_elems<TH, EPI>() <= ws_lds_elems<T, EPI>(), "the half tile fits the same LDS");
     int e, row0, rend, ntile, parts;
     if (!locate_rows_tile<T::BM>(p, block, e, row0, rend, ntile, parts)) return;
-    if constexpr (TH::BM != T::BM) {
-        if (parts == 2) return rows_gemm_ws_tile<TH, EPI, BKM>(p, smem, e, row0, rend, ntile);
-    }
-    rows_gemm_ws_tile<T, EPI, BKM>(p, smem, e, row0, rend, ntile);
+    rows_gemm_ws_run<T, EPI, BKM, TH>(p, smem, e, row0, rend, ntile, parts);
 }
 
 template <class T, int EPI, bool BKM = false, class TH = T>
@@ -2034,6 +2061,124 @@ __global__ __launch_bounds__(WsLarge::NT, WsLarge::WAVES_PER_EU) void bwd_joint_
 }
 
 // ---------------------------------------------------------------------------
+// gate/up and down as one launch.
+//
+// On their own the two forward GEMMs each end in a round that fills a fraction of the chip (6.1 and 2.3 tiles of
+// 256 x 256 per CU at the 24576-token layer: an eighth and a seventh of their CU time idles).  In one launch the
+// down tiles take the CUs as the gate/up tiles leave them, and only the end of the down part is ragged.
+//
+// A down tile reads the post_act rows of its m-tile, which the gate/up tiles of that m-tile (all column tiles)
+// write in the same launch.  The m-tiles of both parts are dealt to the XCDs in the same contiguous ranges, so
+// the writers and the readers of an m-tile run on the SAME XCD and meet in that XCD's L2:
+//   * a consumer wave of a gate/up tile waits until its stores are acknowledged (s_waitcnt vmcnt(0): the
+//     vector cache writes through, the acknowledgement comes from the L2) and then adds one to the m-tile's
+//     counter with a relaxed device-scope atomic, which the L2 executes;
+//   * the producer waves of a down tile poll the counter with loads that bypass the vector cache until it
+//     holds (consumer waves x column tiles), invalidate the vector cache (acquire fence) and start loading.
+// No L2 is written back for this: the release that device scope formally asks for (it writes the whole L2
+// back, for readers on OTHER XCDs) would cost three times the GEMM.  The counter's upper bits carry the sum of
+// the writers' XCC_ID; a reader that finds another XCD's id there than its own - a placement this code does
+// not expect - raises the status word instead of trusting the data.
+// Deadlock: blocks are placed in the order of their index, XCD by XCD; every gate/up block has a smaller index
+// than every down block, so the tiles that a waiting down block needs are running or done, whatever else waits.
+// The wait is bounded all the same: after spin_ticks of the 100 MHz wall clock a block gives up, raises the
+// status word (which ends every other block's wait at once) and computes on what is there; the call's outputs
+// are then invalid, and the status word says so.
+// Counters: ready[t] as above, done[t] counts the down blocks of m-tile t; the last of them puts both back
+// to zero, so a launch that ran through leaves the workspace as it found it (all zeros).
+// ---------------------------------------------------------------------------
+struct FwdJointParams {
+    RowsParams gu, down;
+    int n_gu;                  // blocks of the gate/up part (the down part's follow)
+    int32_t* ready;            // [max m-tiles]
+    int32_t* done;             // [max m-tiles]
+    int32_t* status;           // one word, sticky: FWD_JOINT_TIMEOUT | FWD_JOINT_PLACEMENT
+    int ready_count;           // consumer waves x column tiles of gate/up
+    int64_t spin_ticks;
+};
+enum { FWD_JOINT_TIMEOUT = 1, FWD_JOINT_PLACEMENT = 2 };
+constexpr int kReadyCountBits = 16;   // arrivals below, the sum of the writers' XCC_ID (at most 7 each) above
+constexpr int kReadyCountMax = 4096;
+
+__device__ __forceinline__ int xcc_id() { return (int)__builtin_amdgcn_s_getreg(20 | (0 << 6) | (3 << 11)); }   // HW_REG_XCC_ID[3:0]
+
+__device__ __forceinline__ void wait_rows_ready(const FwdJointParams& q, const int32_t* ctr, int v);
+// The wait of a down tile's producer waves.  The counter is read when the object is made (in front of the tile's address
+// arithmetic and its first weight loads, which cover the load's latency); the call returns once the counter holds
+// all arrivals (or the wait was given up).
+struct RowsReadyWait {
+    const FwdJointParams& q;
+    const int32_t* ctr;
+    int first;
+    __device__ __forceinline__ RowsReadyWait(const FwdJointParams& q_, int mtile) : q(q_), ctr(q_.ready + mtile) {
+        first = __hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __device__ __forceinline__ void operator()(int) const { wait_rows_ready(q, ctr, first); }
+};
+__device__ __forceinline__ void wait_rows_ready(const FwdJointParams& q, const int32_t* ctr, int v) {
+    const int mask = (1 << kReadyCountBits) - 1;
+    if ((v & mask) != q.ready_count) {
+        const uint64_t t0 = wall_clock64();
+        for (;;) {
+            __builtin_amdgcn_s_sleep(16);
+            v = __hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if ((v & mask) == q.ready_count) break;
+            if (__hip_atomic_load(q.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) return;
+            if ((int64_t)(wall_clock64() - t0) > q.spin_ticks) {
+                __hip_atomic_fetch_or(q.status, FWD_JOINT_TIMEOUT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                return;
+            }
+        }
+    }
+    if ((int)((uint32_t)v >> kReadyCountBits) != q.ready_count * xcc_id())
+        __hip_atomic_fetch_or(q.status, FWD_JOINT_PLACEMENT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // This CU's vector cache is invalidated (what an acquire costs between CUs that share an L2; also the compiler's
+    // barrier for the loads that follow).  The acquire that device scope formally asks for walks the L2 as well,
+    // 3.7 us per tile, for lines that only a writer on another XCD could have made stale.
+    asm volatile("buffer_inv sc0" ::: "memory");
+}
+
+typedef WsWideGu FwdGuTile;
+typedef WsDeep FwdDownTile;
+typedef WsDeepHalf FwdDownHalf;
+template <class GuTile>
+__global__ __launch_bounds__(FwdGuTile::NT, FwdGuTile::WAVES_PER_EU) void fwd_joint_kernel(FwdJointParams q) {
+    static_assert(FwdGuTile::NT == FwdDownTile::NT && FwdDownHalf::NT == FwdDownTile::NT, "one block shape");
+    static_assert(FwdGuTile::BM == FwdDownTile::BM, "both parts count the same m-tiles");
+    constexpr int GU_LDS = ws_lds_elems<FwdGuTile, EPI_SWIGLU>(), DOWN_LDS = ws_lds_elems<FwdDownTile, EPI_PLAIN>();
+    constexpr int LDS_ELEMS = GU_LDS > DOWN_LDS ? GU_LDS : DOWN_LDS;
+    static_assert(LDS_ELEMS * 2 <= 160 * 1024, "LDS capacity");
+    __shared__ __attribute__((aligned(1024))) bf16_t smem[LDS_ELEMS];
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / MTS_WAVE), lane = threadIdx.x % MTS_WAVE;
+    int b = blockIdx.x;
+    int e, row0, rend, ntile, parts, mtile;
+    if (b < q.n_gu) {
+        if (!locate_rows_tile<FwdGuTile::BM>(q.gu, b, e, row0, rend, ntile, parts, mtile)) return;   // whole tiles only
+        rows_gemm_ws_run<FwdGuTile, EPI_SWIGLU, false, FwdGuTile>(q.gu, smem, e, row0, rend, ntile, 1);
+        if (wave < FwdGuTile::NWAVES) {
+            wait_vmcnt<0>();   // this wave's rows of pre_act and post_act are in the L2
+            if (lane == 0)
+                __hip_atomic_fetch_add(q.ready + mtile, 1 + (xcc_id() << kReadyCountBits), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        return;
+    }
+    b -= q.n_gu;
+    const bool found = locate_rows_tile<FwdDownTile::BM>(q.down, b, e, row0, rend, ntile, parts, mtile);
+    if (mtile < 0) return;
+    if (found)
+        rows_gemm_ws_run<FwdDownTile, EPI_PLAIN, false, FwdDownHalf>(q.down, smem, e, row0, rend, ntile, parts, RowsReadyWait(q, mtile));
+    // the last block of the m-tile (the empty half of a cut tile counts as one) clears its counters; all other readers
+    // of ready[mtile] have had their answer by then: they add to done[] behind their loads
+    if (wave == FwdDownTile::NWAVES && lane == 0) {
+        const int blocks = q.down.n_tiles * parts;
+        if (__hip_atomic_fetch_add(q.done + mtile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1 == blocks) {
+            __hip_atomic_store(q.ready + mtile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(q.done + mtile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
 
@@ -2110,7 +2255,7 @@ dim3 rows_grid(RowsParams& p, int64_t TK) {
     const int64_t m_groups = (m_tiles<T>(TK, p.E) + kXcds - 1) / kXcds;
     if (!p.xcd_ranges) p.tail_slots = 0;
     // tiles that are cut in two add at most tail_slots / 2 blocks per XCD; one more block writes the schedule (dO*W2 only)
-    return dim3((unsigned)((m_groups * p.n_tiles + p.tail_slots / 2) * kXcds + (p.sched_out ? 1 : 0)));
+    return dim3((unsigned)((m_groups * p.n_tiles + p.tail_slots / 2 + p.tail_tiles) * kXcds + (p.sched_out ? 1 : 0)));
 }
 
 // does launch_rows_any take B in the weights' stored layout for this kind and reduction length?
@@ -2230,6 +2375,44 @@ int launch_dw_any(int kind, DwParams p, int E, int grad_dtype, void* workspace, 
         if (grad_dtype == MTS_GEMM_DTYPE) dw_gemm_kernel<StagedSmall, bf16_t><<<grid, StagedSmall::NT, 0, s>>>(p);
         else dw_gemm_kernel<StagedSmall, float><<<grid, StagedSmall::NT, 0, s>>>(p);
     }
+    MTS_CHECK_LAUNCH();
+    return MTS_OK;
+}
+
+// gate/up + down as one launch: both on the 256 x 256 tiles with specialised waves, both dealt to the XCDs in
+// contiguous ranges of the same m-tiles (an expert's W1 fits an L2)
+bool fwd_joint_ok(int H, int I) {
+    const int n_tiles_gu = (I + FwdGuTile::BN / 2 - 1) / (FwdGuTile::BN / 2);
+    return tile_choice(K_GATEUP) == 4 && tile_choice(K_DOWN) == 4 && H % 64 == 0 && I % 64 == 0 &&
+           xcd_ranges_choice((int64_t)2 * I * H * (int64_t)sizeof(bf16_t)) == 1 &&
+           xcd_ranges_choice((int64_t)I * H * (int64_t)sizeof(bf16_t)) == 1 && FwdGuTile::NWAVES * n_tiles_gu <= kReadyCountMax;
+}
+int64_t fwd_joint_counters(int64_t TK, int E) { return m_tiles<FwdGuTile>(TK, E); }
+
+int launch_fwd_joint(RowsParams gu, RowsParams down, int64_t TK, int32_t* workspace, hipStream_t s) {
+    FwdJointParams q = {};
+    gu.reverse = down.reverse = 0;   // the down part follows the gate/up part through the range, oldest rows first
+    gu.tail_slots = down.tail_slots = 0;
+    q.n_gu = (int)rows_grid<FwdGuTile, EPI_SWIGLU>(gu, TK).x;
+    // Only the end of the down part is ragged: its last m-tiles (per XCD) are cut into tiles of half the height, as many
+    // as make about 3/8 of a round of whole tiles (measured at 768/1024: 2, 4 and 6 m-tiles of 3 tiles each give 276, 272
+    // and 281 us; none 277).
+    down.n_tiles = (down.N + FwdDownTile::BN - 1) / FwdDownTile::BN;
+    const int forced = mts_tuning().fwd_joint_tail;
+    const int by_rule = (kCusPerXcd * 3 / 8 + down.n_tiles / 2) / down.n_tiles;
+    const int tail_mtiles = forced >= 0 ? forced : (by_rule > 1 ? by_rule : 1);
+    down.tail_tiles = tail_mtiles * down.n_tiles;
+    const int n_down = (int)rows_grid<FwdDownTile, EPI_PLAIN>(down, TK).x;
+    if (!gu.xcd_ranges || !down.xcd_ranges || down.n_groups != 1) return MTS_ERR_SHAPE;
+    q.gu = gu;
+    q.down = down;
+    const int64_t n = fwd_joint_counters(TK, gu.E);
+    q.status = workspace;           // word 0; the counters start 16 bytes in
+    q.ready = workspace + 4;
+    q.done = q.ready + n;
+    q.ready_count = FwdGuTile::NWAVES * gu.n_tiles;
+    q.spin_ticks = mts_tuning().fwd_joint_spin_us * 100;   // the wall clock counts at 100 MHz
+    fwd_joint_kernel<FwdGuTile><<<dim3((unsigned)(q.n_gu + n_down)), FwdGuTile::NT, 0, s>>>(q);
     MTS_CHECK_LAUNCH();
     return MTS_OK;
 }
@@ -2398,6 +2581,48 @@ extern "C" int MTS_GEMM_ENTRY(mts_moe_fwd_down)(const void* post_act, const void
     p.N = H; p.Kdim = I; p.expert_start = expert_start; p.E = E;
     p.C = (bf16_t*)y; p.TK = TK;
     return launch_rows_any<EPI_PLAIN>(K_DOWN, p, TK, (hipStream_t)stream);
+}
+
+#ifndef MTS_GEMM_F16
+extern "C" int mts_moe_fwd_joint_supported(int act_dtype, int H, int I) {
+    return (act_dtype == MTS_BF16 || act_dtype == MTS_F16) && H >= 64 && I >= 64 && fwd_joint_ok(H, I) ? 1 : 0;
+}
+extern "C" int64_t mts_moe_fwd_joint_workspace_bytes(int64_t TK, int E) {
+    if (TK <= 0 || E < 1) return 0;
+    return ((2 * fwd_joint_counters(TK, E) + 4) * (int64_t)sizeof(int32_t) + 15) / 16 * 16;
+}
+#endif
+
+extern "C" int MTS_GEMM_ENTRY(mts_moe_fwd_gateup_down)(const void* x, const void* w1, const void* w2, const int32_t* x_gather,
+                                       const int32_t* expert_start, const void* weights, const int32_t* s_scatter,
+                                       int64_t T, int K, int E, int H, int I, int act_dtype, void* pre_act, void* post_act,
+                                       void* y, int32_t* workspace, int64_t workspace_bytes, void* stream) {
+#ifndef MTS_GEMM_F16
+    if (act_dtype == MTS_F16) return mts_moe_fwd_gateup_down_f16(x, w1, w2, x_gather, expert_start, weights, s_scatter, T, K, E, H, I, act_dtype, pre_act, post_act, y, workspace, workspace_bytes, stream);
+#endif
+    if (!x || !w1 || !w2 || !x_gather || !expert_start || !pre_act || !post_act || !y || !workspace) return MTS_ERR_NULL;
+    if ((weights != nullptr) != (s_scatter != nullptr)) return MTS_ERR_NULL;
+    if (T <= 0 || K < 1) return MTS_ERR_SHAPE;
+    if (act_dtype != MTS_GEMM_DTYPE) return MTS_ERR_DTYPE;
+    int rc = check_common(T * K, E, H, I, T);
+    if (rc) return rc;
+    if (!fwd_joint_ok(H, I)) return MTS_ERR_SHAPE;
+    if (!mts_aligned16(x) || !mts_aligned16(w1) || !mts_aligned16(w2) || !mts_aligned16(pre_act) || !mts_aligned16(post_act) ||
+        !mts_aligned16(y) || !mts_aligned16(workspace))
+        return MTS_ERR_ALIGN;
+    if (workspace_bytes < (2 * fwd_joint_counters(T * K, E) + 4) * (int64_t)sizeof(int32_t)) return MTS_ERR_WORKSPACE;
+    RowsParams g = {};
+    g.A = (const bf16_t*)x; g.a_rows = T; g.lda = H; g.a_gather = x_gather;
+    g.B = (const bf16_t*)w1; g.b_rows = 2 * I;
+    g.N = I; g.Kdim = H; g.expert_start = expert_start; g.E = E;
+    g.C = (bf16_t*)pre_act; g.C2 = (bf16_t*)post_act; g.TK = T * K;
+    g.route_w = (const bf16_t*)weights; g.s_scatter = s_scatter;
+    RowsParams d = {};
+    d.A = (const bf16_t*)post_act; d.a_rows = T * K; d.lda = I; d.a_gather = nullptr;
+    d.B = (const bf16_t*)w2; d.b_rows = H;
+    d.N = H; d.Kdim = I; d.expert_start = expert_start; d.E = E;
+    d.C = (bf16_t*)y; d.TK = T * K;
+    return launch_fwd_joint(g, d, T * K, workspace, (hipStream_t)stream);
 }
 
 #ifndef MTS_GEMM_F16

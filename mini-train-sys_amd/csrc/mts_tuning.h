@@ -10,6 +10,8 @@
 //   MTS_NO_TAIL_SPLIT = 1         every tile whole (the tiles behind an XCD's last whole round are not cut in two)
 //   MTS_NO_MFMA_ROUTER = 1        router projection on the vector pipe for every shape
 //   MTS_NO_JOINT_SCHEDULE = 1     units and dX tiles of the joint backward launch are dealt round-robin / in equal ranges
+//   MTS_FWD_JOINT_TAIL = n        gate/up + down as one launch: the last n m-tiles of every XCD's down part are cut in two
+//   MTS_FWD_JOINT_SPIN_US = n     ... and a down block gives up waiting for its rows after n microseconds (0: at once)
 // A switch is on when its value parses to a non-zero integer ("0" and the empty string leave it off).
 #pragma once
 
@@ -22,6 +24,8 @@ struct MtsTuning {
     bool tail_split;
     bool mfma_router;
     bool joint_schedule;
+    int fwd_joint_tail;         // -1: the launcher's own choice
+    long long fwd_joint_spin_us;
 };
 
 const MtsTuning& mts_tuning();

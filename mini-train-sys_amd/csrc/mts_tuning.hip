@@ -26,6 +26,10 @@ MtsTuning read_environment() {
     t.tail_split = !flag("MTS_NO_TAIL_SPLIT");
     t.mfma_router = !flag("MTS_NO_MFMA_ROUTER");
     t.joint_schedule = !flag("MTS_NO_JOINT_SCHEDULE");
+    const char* tail = getenv("MTS_FWD_JOINT_TAIL");
+    t.fwd_joint_tail = tail && *tail && atoi(tail) >= 0 ? atoi(tail) : -1;
+    const char* spin = getenv("MTS_FWD_JOINT_SPIN_US");
+    t.fwd_joint_spin_us = spin && *spin && atoll(spin) >= 0 ? atoll(spin) : 200000;
     return t;
 }
 

@@ -44,6 +44,9 @@ SIGNATURES = {
     "mts_moe_cast_weights_pair": (_i, [_p, _p, _l, _p, _p, _l, _i, _p]),
     "mts_moe_fwd_gateup_swiglu": (_i, [_p, _p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p, _p, _p]),
     "mts_moe_fwd_down": (_i, [_p, _p, _p, _l, _i, _i, _i, _i, _p, _p]),
+    "mts_moe_fwd_joint_supported": (_i, [_i, _i, _i]),
+    "mts_moe_fwd_joint_workspace_bytes": (_l, [_l, _i]),
+    "mts_moe_fwd_gateup_down": (_i, [_p] * 7 + [_l, _i, _i, _i, _i, _i, _p, _p, _p, _p, _l, _p]),
     "mts_moe_combine": (_i, [_p, _p, _p, _p, _l, _i, _i, _i, _p, _p]),
     "mts_moe_head_workspace_bytes": (_l, [_l, _i, _i]),
     "mts_moe_head_fwd": (_i, [_p, _p, _l, _i, _i, _i, _i, _i] + [_p] * 14 + [_p, _l, _p]),

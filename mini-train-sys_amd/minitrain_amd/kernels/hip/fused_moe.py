@@ -223,6 +223,71 @@ def _dw_workspace(lib, which: int, E: int, H: int, I: int, dtype: torch.dtype, d
     return ws, ws.data_ptr(), nbytes
 
 
+class _JointForwardWorkspace:
+    """Counters of the launch that holds gate/up and down (``mts_moe_fwd_gateup_down``), one per device and stream.
+
+    The launch needs them zero and leaves them zero, so the layers of a model that run one after the other on a stream
+    share one buffer.  Word 0 is the launch's status: it stays zero unless a block gave up waiting for the rows it reads
+    (or found them written on another XCD than its own); the outputs of that call are then invalid.  Nothing here
+    waits for the GPU: every ``CHECK_EVERY`` calls the word is copied to pinned host memory, and the copy of an earlier
+    call is looked at once its event has passed, so an error is raised a few calls late rather than never."""
+
+    CHECK_EVERY = 16
+
+    def __init__(self, device: torch.device):
+        self.device = device
+        self.buf = None
+        self.host = torch.zeros(1, dtype=torch.int32, pin_memory=True)
+        self.event = None
+        self.calls = 0
+
+    def get(self, nbytes: int) -> torch.Tensor:
+        if self.buf is None or self.buf.numel() * 4 < nbytes:
+            self.buf = torch.zeros((nbytes + 3) // 4, dtype=torch.int32, device=self.device)
+        return self.buf
+
+    def _raise(self, status: int):
+        self.buf = None     # the counters of a failed launch are not trusted again
+        raise RuntimeError(f"hip fused MoE: the joint gate/up + down launch reported status {status} "
+                           "(1: a block gave up waiting for its rows, 2: rows written on another XCD); the outputs of "
+                           "that call are invalid. MTS_NO_JOINT_FWD=1 runs the two GEMMs as launches of their own.")
+
+    def before_launch(self):
+        if self.event is not None and self.event.query():
+            self.event = None
+            if int(self.host[0]) != 0:
+                self._raise(int(self.host[0]))
+
+    def after_launch(self):
+        self.calls += 1
+        if self.event is None and self.calls % self.CHECK_EVERY == 1:
+            self.host.copy_(self.buf[:1], non_blocking=True)
+            self.event = torch.cuda.Event()
+            self.event.record()
+
+    def status(self) -> int:
+        """The status word now (waits for the stream)."""
+        return 0 if self.buf is None else int(self.buf[0].item())
+
+
+_JOINT_FWD: dict = {}
+
+
+def _joint_forward_workspace(device: torch.device) -> _JointForwardWorkspace:
+    key = (device.index if device.index is not None else torch.cuda.current_device(), torch.cuda.current_stream(device).cuda_stream)
+    ws = _JOINT_FWD.get(key)
+    if ws is None:
+        ws = _JOINT_FWD[key] = _JointForwardWorkspace(device)
+    return ws
+
+
+def joint_forward_status(device=None) -> int:
+    """Status of the joint gate/up + down launches on the current stream of ``device`` (0: all of them ran through).
+    Synchronises; for tests, benchmarks and the points where a training loop reads a value back anyway."""
+    device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    return _joint_forward_workspace(device).status()
+
+
 def _stage(lib, w: torch.Tensor, transpose: bool, dtype: torch.dtype, stream: int | None = None) -> torch.Tensor:
     """Copy of an expert weight ``[E,R,C]`` in the activation dtype, optionally as ``[E,C,R]``."""
     if not transpose and w.dtype == dtype:
@@ -281,21 +346,37 @@ def moe_forward(x, gate_up_proj, down_proj, weights_flat, routing):
     # the `weighted_act` operand of the dW2 GEMM, so it is kept for the backward pass instead of being
     # written again there (TK * I elements held from forward to backward, and as many fewer written).
     weighted = SWITCHES.weighted_post
-    _lib.check(
-        lib.mts_moe_fwd_gateup_swiglu(
-            x.data_ptr(), w1.data_ptr(), x_gather.data_ptr(), expert_start.data_ptr(),
-            weights_flat.data_ptr() if weighted else None, s_scatter.data_ptr() if weighted else None,
-            T, K, E, H, I, act, pre_act.data_ptr(), post_act.data_ptr(), stream,
-        ),
-        "mts_moe_fwd_gateup_swiglu",
-    )
     y = torch.empty(TK, H, dtype=x.dtype, device=dev)
-    _lib.check(
-        lib.mts_moe_fwd_down(
-            post_act.data_ptr(), w2.data_ptr(), expert_start.data_ptr(), TK, E, H, I, act, y.data_ptr(), stream
-        ),
-        "mts_moe_fwd_down",
-    )
+    if SWITCHES.joint_fwd and x.dtype != torch.float32 and lib.mts_moe_fwd_joint_supported(act, H, I):
+        # one launch: the down tiles take the CUs as the gate/up tiles leave them
+        jw = _joint_forward_workspace(dev)
+        jw.before_launch()
+        nbytes = lib.mts_moe_fwd_joint_workspace_bytes(TK, E)
+        counters = jw.get(nbytes)
+        _lib.check(
+            lib.mts_moe_fwd_gateup_down(
+                x.data_ptr(), w1.data_ptr(), w2.data_ptr(), x_gather.data_ptr(), expert_start.data_ptr(),
+                weights_flat.data_ptr() if weighted else None, s_scatter.data_ptr() if weighted else None,
+                T, K, E, H, I, act, pre_act.data_ptr(), post_act.data_ptr(), y.data_ptr(), counters.data_ptr(), nbytes, stream,
+            ),
+            "mts_moe_fwd_gateup_down",
+        )
+        jw.after_launch()
+    else:
+        _lib.check(
+            lib.mts_moe_fwd_gateup_swiglu(
+                x.data_ptr(), w1.data_ptr(), x_gather.data_ptr(), expert_start.data_ptr(),
+                weights_flat.data_ptr() if weighted else None, s_scatter.data_ptr() if weighted else None,
+                T, K, E, H, I, act, pre_act.data_ptr(), post_act.data_ptr(), stream,
+            ),
+            "mts_moe_fwd_gateup_swiglu",
+        )
+        _lib.check(
+            lib.mts_moe_fwd_down(
+                post_act.data_ptr(), w2.data_ptr(), expert_start.data_ptr(), TK, E, H, I, act, y.data_ptr(), stream
+            ),
+            "mts_moe_fwd_down",
+        )
     out = torch.empty(T, H, dtype=x.dtype, device=dev)
     _lib.check(
         lib.mts_moe_combine(

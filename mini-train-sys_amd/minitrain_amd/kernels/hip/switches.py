@@ -10,6 +10,7 @@ inside the library when it is loaded (``csrc/mts_tuning.h``).
     MTS_NO_JOINT_BWD=1        dW2, dW1 and dX as launches of their own even where one launch could hold them
     MTS_NO_TAIL_IN_JOINT=1    the router's backward of the layer node in launches of its own
     MTS_NO_COMBINE_IN_TAIL=1  the dX combine behind the joint launch in a launch of its own
+    MTS_NO_JOINT_FWD=1        gate/up and down as two launches even where one launch could hold them
     MTS_NO_JOINT_SCHEDULE=1   no table for the joint launch: its blocks are dealt to the XCDs without regard to routing
     MTS_WEIGHTED_POST=0       the forward pass writes the unweighted activation and dO*W2 writes s * a again
     MTS_NO_ROUTER_CAST=1      router_postprocess leaves the cast of the routing weights to the caller
@@ -32,6 +33,7 @@ def _off(name: str) -> bool:
 class Switches:
     overlap: bool
     joint_bwd: bool
+    joint_fwd: bool
     tail_in_joint: bool
     combine_in_tail: bool
     joint_schedule: bool
@@ -43,6 +45,7 @@ class Switches:
 SWITCHES = Switches(
     overlap=not _off("MTS_NO_OVERLAP"),
     joint_bwd=not _off("MTS_NO_JOINT_BWD"),
+    joint_fwd=not _off("MTS_NO_JOINT_FWD"),
     tail_in_joint=not _off("MTS_NO_TAIL_IN_JOINT"),
     combine_in_tail=not _off("MTS_NO_COMBINE_IN_TAIL"),
     joint_schedule=not _off("MTS_NO_JOINT_SCHEDULE"),

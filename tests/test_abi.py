@@ -22,7 +22,7 @@ def _declared():
 
 def test_header_declares_the_expected_entry_points():
     names = _declared()
-    for must in ("mts_router_fwd", "mts_router_bwd", "mts_moe_route", "mts_moe_fwd_gateup_swiglu", "mts_moe_fwd_down",
+    for must in ("mts_router_fwd", "mts_router_bwd", "mts_moe_route", "mts_moe_fwd_gateup_swiglu", "mts_moe_fwd_down", "mts_moe_fwd_gateup_down",
                  "mts_moe_combine", "mts_moe_bwd_dy1", "mts_moe_bwd_dx", "mts_moe_bwd_dw1", "mts_moe_bwd_dw2",
                  "mts_moe_bwd_joint"):
         assert must in names
@@ -37,7 +37,7 @@ def test_library_exports_every_declared_symbol():
     for name in _declared():
         assert hasattr(lib, name), f"{name} is declared in include/ but not exported"
         assert name in _lib.SIGNATURES, f"{name} has no ctypes prototype"
-    assert lib.mts_version() == 3
+    assert lib.mts_version() == 4
     assert lib.mts_error_string(0) == b"ok"
     # argument checks run on the host before any launch: safe without a GPU
     assert lib.mts_router_fwd(None, 4, 8, 2, 1, None, None, None, None, None, None, None, None, None, 0, None, 0, None) == -1
@@ -53,6 +53,24 @@ def test_contract_violations_are_reported_before_any_launch():
     lib = _lib.load()
     NULL, SHAPE, WORKSPACE = -1, -2, -4
     fake = 4096   # any non-null, 16-byte aligned value: nothing is dereferenced before the checks fail
+    # gate/up + down as one launch: required pointers, the shapes it exists for, workspace size
+    BF16, F32 = 0, 1
+    assert lib.mts_moe_fwd_joint_supported(BF16, 768, 1024) == 1
+    assert lib.mts_moe_fwd_joint_supported(BF16, 768, 1000) == 0      # I not a multiple of 64
+    assert lib.mts_moe_fwd_joint_supported(BF16, 4096, 14336) == 0    # an expert's W1 beyond an L2: the two launches
+    assert lib.mts_moe_fwd_joint_supported(F32, 768, 1024) == 0
+    need = lib.mts_moe_fwd_joint_workspace_bytes(49152, 8)
+    assert need % 16 == 0 and need >= (2 * (49152 // 256 + 7) + 1) * 4
+    args = lambda **kw: [kw.get(k, v) for k, v in dict(x=fake, w1=fake, w2=fake, x_gather=fake, expert_start=fake, weights=fake,
+                                                         s_scatter=fake, T=24576, K=2, E=8, H=768, I=1024, act=BF16, pre=fake,
+                                                         post=fake, y=fake, ws=fake, ws_bytes=need, stream=None).items()]
+    assert lib.mts_moe_fwd_gateup_down(*args(ws=None)) == NULL
+    assert lib.mts_moe_fwd_gateup_down(*args(w2=None)) == NULL
+    assert lib.mts_moe_fwd_gateup_down(*args(s_scatter=None)) == NULL     # the routing weight needs the row -> entry map
+    assert lib.mts_moe_fwd_gateup_down(*args(I=1000)) == SHAPE
+    assert lib.mts_moe_fwd_gateup_down(*args(ws_bytes=need - 16)) == WORKSPACE
+    assert lib.mts_moe_fwd_gateup_down(*args(act=F32)) == -3
+    assert lib.mts_moe_fwd_gateup_down(*args(y=fake + 4)) == -5
     # capacity mask: required pointers, expert limit, workspace size
     assert lib.mts_moe_capacity_mask(None, fake, 8, 2, 4, 3, fake, None, fake, fake, 1 << 20, None) == NULL
     assert lib.mts_moe_capacity_mask(fake, fake, 8, 2, 4096, 3, fake, None, fake, fake, 1 << 20, None) == SHAPE

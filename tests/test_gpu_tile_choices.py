@@ -28,6 +28,9 @@ CONFIGURATIONS = {
     "64-wide k-tiles for dX and the weight gradients on their own, every tile whole": dict(MTS_NO_JOINT_BWD="1",
                                                                                            MTS_NO_TAIL_SPLIT="1"),
     "router projection on the vector pipe": dict(MTS_NO_MFMA_ROUTER="1"),
+    "gate/up and down as two launches": dict(MTS_NO_JOINT_FWD="1"),
+    "gate/up and down as one launch, every down tile whole": dict(MTS_FWD_JOINT_TAIL="0"),
+    "gate/up and down as one launch, every down tile cut in two": dict(MTS_FWD_JOINT_TAIL="1000"),
     "ranges per XCD, plain order, tail launches apart": dict(MTS_XCD_RANGES="1", MTS_NO_TILE_ORDER="1",
                                                              MTS_NO_TAIL_IN_JOINT="1"),
 }
