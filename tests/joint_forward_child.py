@@ -1,6 +1,7 @@
-"""Child process of tests/test_gpu_joint_forward.py: the joint gate/up + down launch at a size where down blocks start
-while gate/up tiles are still running, with whatever wait limit the environment holds (it is read once per process).
-Prints the status word; the outputs are compared with the two launches when the status is zero."""
+"""Child process of tests/test_gpu_joint_forward.py: the joint gate/up + down launch at a size whose tiles all fit the
+chip at once, so that every down block starts while the gate/up tiles it reads from are still running, with whatever
+wait limit the environment holds (it is read once per process).  Prints the status word; the outputs are compared
+with the two launches when the status is zero."""
 
 import sys
 from pathlib import Path
@@ -16,7 +17,7 @@ from minitrain_amd import _lib   # noqa: E402
 
 if __name__ == "__main__":
     lib = _lib.load()
-    T, H, E, I, K, dtype = 24576, 768, 8, 1024, 2, torch.bfloat16
+    T, H, E, I, K, dtype = 2000, 768, 8, 1024, 2, torch.bfloat16
     x, w1, w2, idx, weights = J._case(5, T, H, E, I, K, dtype)
     routing = J._routing(lib, idx, E)
     ws = torch.zeros(lib.mts_moe_fwd_joint_workspace_bytes(T * K, E) // 4, dtype=torch.int32, device="cuda")

@@ -169,10 +169,10 @@ def test_host_side_raises_on_a_status_word(monkeypatch):
 
 def test_a_wait_that_is_given_up_ends_the_launch_and_is_reported(tmp_path):
     """With a wait limit of zero (set from the host, read when the library is loaded) a down block that finds its rows
-    unfinished gives up at once instead of waiting: the launch still ends, the status word says 1 (or 0, if no block
-    came early; the outputs are compared in that case)."""
+    unfinished gives up at once instead of waiting: the launch still ends and the status word says 1."""
     env = dict(os.environ, MTS_FWD_JOINT_SPIN_US="0")
     run = subprocess.run([sys.executable, str(ROOT / "tests" / "joint_forward_child.py")], env=env, capture_output=True, text=True,
                          timeout=300, cwd=str(ROOT))
     assert run.returncode == 0, run.stderr[-2000:]
-    assert "status after a limit of zero:" in run.stdout and "cleared workspace: equal" in run.stdout, run.stdout
+    # at the child's size every down block comes early, so with no time to wait the word must say so
+    assert "status after a limit of zero: 1" in run.stdout and "cleared workspace: equal" in run.stdout, run.stdout
