@@ -594,6 +594,11 @@ template <int BM>
 __device__ __forceinline__ bool find_rows_tile(const RowsParams& p, int b, int& e, int& row0, int& rend, int& ntile, int& parts,
                                                int& mtile) {
     mtile = -1;
+    // up to 64 experts: lane l reads expert_start[l] and [l + 1] once, for the count of m-tiles and for the search
+    const bool in_regs = p.E <= MTS_WAVE;
+    const int lane_ = threadIdx.x % MTS_WAVE;
+    const int w0 = in_regs && lane_ < p.E ? p.expert_start[lane_] : 0;
+    const int w1 = in_regs && lane_ < p.E ? p.expert_start[lane_ + 1] : 0;
     const int xcd = b % kXcds;
     int j = b / kXcds;
     const int lane = threadIdx.x % MTS_WAVE;
@@ -612,7 +617,9 @@ __device__ __forceinline__ bool find_rows_tile(const RowsParams& p, int b, int& 
     } else if (p.xcd_ranges) {
         // m-tiles of the launch: the first (total % 8) XCDs take one more than the others
         int mine = 0;
-        for (int le = lane; le < p.E; le += MTS_WAVE) mine += (p.expert_start[le + 1] - p.expert_start[le] + BM - 1) / BM;
+        if (in_regs) mine = (w1 - w0 + BM - 1) / BM;
+        else
+            for (int le = lane; le < p.E; le += MTS_WAVE) mine += (p.expert_start[le + 1] - p.expert_start[le] + BM - 1) / BM;
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) mine += __shfl_xor(mine, o, MTS_WAVE);
         const int per = mine / kXcds, rem = mine % kXcds;
@@ -646,8 +653,8 @@ __device__ __forceinline__ bool find_rows_tile(const RowsParams& p, int b, int& 
     int seen = 0;
     for (int e0 = 0; e0 < p.E; e0 += MTS_WAVE) {
         const int le = e0 + lane;
-        const int s0 = le < p.E ? p.expert_start[le] : 0;
-        const int s1 = le < p.E ? p.expert_start[le + 1] : 0;
+        const int s0 = in_regs ? w0 : (le < p.E ? p.expert_start[le] : 0);
+        const int s1 = in_regs ? w1 : (le < p.E ? p.expert_start[le + 1] : 0);
         const int nt = (s1 - s0 + BM - 1) / BM;
         int incl = nt;
 #pragma unroll
