@@ -82,6 +82,9 @@ def _case(seed, T, H, E, I, K, dtype, skew=0.0, empty_expert=None):
     (130, 64, 3, 64, 2, torch.float16, 0.0, True),          # m-tiles of at most 128 rows cut in two: empty halves
     (2048, 768, 8, 1024, 2, torch.float16, 0.3, True),
     (5000, 192, 64, 128, 2, torch.bfloat16, 0.5, True),     # more experts than XCDs, most with a single short tile
+    (4096, 64, 1, 64, 1, torch.bfloat16, 0.0, True),        # one expert, one k-tile per GEMM, one column tile each
+    (9000, 512, 16, 1984, 2, torch.bfloat16, 0.2, True),    # 15.5 column tiles of gate/up: the last one half empty
+    (3000, 320, 130, 64, 2, torch.float16, 0.0, True),      # more experts than a wave holds: the search walks two groups
 ])
 def test_joint_forward_launch_equals_two_launches(T, H, E, I, K, dtype, skew, weighted):
     print(f"joint forward T={T} H={H} E={E} I={I} K={K} {dtype} skew={skew} weighted={weighted}", flush=True)
