@@ -124,6 +124,38 @@ def test_joint_forward_consecutive_sizes_on_one_workspace():
             assert torch.equal(a, b), T
 
 
+def test_joint_forward_while_another_stream_keeps_the_chip_busy():
+    """Blocks of other kernels take CUs and cache lines while the launch runs (large copies and GEMMs on a second stream):
+    the hand-over of rows between the launch's blocks does not depend on having the chip to itself."""
+    from minitrain_amd import _lib
+
+    lib = _lib.load()
+    T, H, E, I, K = 24576, 768, 8, 1024, 2
+    side = torch.cuda.Stream()
+    a = torch.randn(4096, 4096, device="cuda", dtype=torch.bfloat16)
+    big = torch.empty(128 * 2**20, device="cuda", dtype=torch.uint8)
+    big2 = torch.empty_like(big)
+    ws = torch.zeros(lib.mts_moe_fwd_joint_workspace_bytes(T * K, E) // 4, dtype=torch.int32, device="cuda")
+    for seed in range(4):
+        print(f"joint forward beside another stream: seed {seed}", flush=True)
+        x, w1, w2, idx, weights = _case(2000 + seed, T, H, E, I, K, torch.bfloat16, skew=0.2 * seed)
+        routing = _routing(lib, idx, E)
+        want = _forward(lib, False, x, w1, w2, weights.flatten(), routing)
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(8):
+                if seed % 2:
+                    torch.mm(a, a)
+                else:
+                    big2.copy_(big)
+        for _ in range(3):
+            got = _forward(lib, True, x, w1, w2, weights.flatten(), routing, ws)
+            assert int((ws != 0).sum()) == 0, f"status {int(ws[0])}"
+            for u, v in zip(got, want):
+                assert torch.equal(u, v)
+        torch.cuda.synchronize()
+
+
 @pytest.mark.parametrize("dtype,fp32_weights", [(torch.bfloat16, False), (torch.float16, True)])
 def test_operator_with_and_without_the_joint_forward_launch(dtype, fp32_weights, monkeypatch):
     """The operator's output and every gradient are bit-identical whichever way the forward GEMMs are launched."""
