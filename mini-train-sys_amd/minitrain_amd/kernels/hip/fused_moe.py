@@ -237,7 +237,7 @@ class _JointForwardWorkspace:
     def __init__(self, device: torch.device):
         self.device = device
         self.buf = None
-        self.host = torch.zeros(1, dtype=torch.int32, pin_memory=True)
+        self.host = None     # pinned word, allocated with the first copy (not while a graph is being captured)
         self.event = None
         self.calls = 0
 
@@ -253,6 +253,10 @@ class _JointForwardWorkspace:
                            "that call are invalid. MTS_NO_JOINT_FWD=1 runs the two GEMMs as launches of their own.")
 
     def before_launch(self):
+        # (a stream that is being captured into a graph admits neither the query nor the copy: the word is then left
+        # to joint_forward_status())
+        if torch.cuda.is_current_stream_capturing():
+            return
         if self.event is not None and self.event.query():
             self.event = None
             if int(self.host[0]) != 0:
@@ -260,7 +264,11 @@ class _JointForwardWorkspace:
 
     def after_launch(self):
         self.calls += 1
+        if torch.cuda.is_current_stream_capturing():
+            return
         if self.event is None and self.calls % self.CHECK_EVERY == 1:
+            if self.host is None:
+                self.host = torch.zeros(1, dtype=torch.int32, pin_memory=True)
             self.host.copy_(self.buf[:1], non_blocking=True)
             self.event = torch.cuda.Event()
             self.event.record()

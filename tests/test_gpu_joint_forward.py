@@ -156,6 +156,40 @@ def test_joint_forward_while_another_stream_keeps_the_chip_busy():
         torch.cuda.synchronize()
 
 
+def test_operator_forward_replayed_from_a_graph():
+    """The operator's forward pass captured into a graph and replayed with other activations and another routing in
+    the same buffers, with eager calls and synchronisations between the replays: every replay gives what the eager call
+    gives.  (The launch's counters are cleared by a fill kernel inside the graph and left clear by the launch; the host
+    side does not look at the status word while a stream is being captured.)"""
+    from tests.helpers import hip_backend, routed_case
+    from minitrain_amd.kernels.hip.fused_moe import joint_forward_status
+
+    ops = hip_backend()
+    T, H, E, I, K = 4096, 768, 8, 1024, 2
+    case = routed_case(5, T, H, E, I, K)
+    x, w1, w2, idx, w = (case[k].cuda() for k in ("x", "w1", "w2", "idx", "w"))
+    gen = torch.Generator().manual_seed(17)
+    with torch.no_grad():
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                ops.fused_moe(x, w1, w2, idx, w)
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out = ops.fused_moe(x, w1, w2, idx, w)
+        for replay in range(4):
+            print(f"graph replay {replay}", flush=True)
+            x.copy_(torch.randn(T, H, generator=gen).to(x.dtype))
+            idx.copy_(torch.stack([torch.randperm(E, generator=gen)[:K] for _ in range(T)]).int())
+            graph.replay()
+            torch.cuda.synchronize()
+            eager = ops.fused_moe(x, w1, w2, idx, w)
+            assert torch.equal(out, eager), replay
+    assert joint_forward_status() == 0
+
+
 @pytest.mark.parametrize("dtype,fp32_weights", [(torch.bfloat16, False), (torch.float16, True)])
 def test_operator_with_and_without_the_joint_forward_launch(dtype, fp32_weights, monkeypatch):
     """The operator's output and every gradient are bit-identical whichever way the forward GEMMs are launched."""
