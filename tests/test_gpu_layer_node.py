@@ -268,3 +268,47 @@ def test_block_uses_the_layer_node_and_falls_back_when_it_must():
     assert set(one.router_metrics) == set(three.router_metrics)
     for key in one.router_metrics:
         torch.testing.assert_close(one.router_metrics[key].float(), three.router_metrics[key].float(), rtol=2e-5, atol=2e-6)
+
+
+def test_layer_step_replayed_from_a_graph():
+    """Forward and backward of the layer node captured into one graph and replayed, with eager steps and
+    synchronisations between the replays: outputs and all four gradients equal the eager step's, bit for bit.  No
+    kernel of the step needs the host between launches (grids follow from the sizes, not from the routing), nothing is
+    cleared with a memset, and the host side leaves the joint forward launch's status word alone while capturing."""
+    ops = hip_backend()
+    T, H, E, I, K = 4096, 768, 8, 1024, 2
+    x, w_r, w1, w2, g = O.make_inputs(7, T, H, E, I)
+    x, w1, w2, g = (t.bfloat16().cuda() for t in (x, w1, w2, g))
+    w_r = w_r.cuda()
+    g_aux, g_z = torch.tensor(0.01, device="cuda"), torch.tensor(0.001, device="cuda")
+    leaves = [t.requires_grad_(True) for t in (x, w_r, w1, w2)]
+
+    def step():
+        for leaf in leaves:
+            leaf.grad = None
+        out, aux, z = ops.moe_layer(*leaves, K, normalize=True)[:3]
+        torch.autograd.backward([out, aux, z], [g, g_aux, g_z])
+        return out.detach(), [leaf.grad for leaf in leaves]
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out, grads = step()
+    gen = torch.Generator().manual_seed(3)
+    for replay in range(3):
+        print(f"layer step graph replay {replay}", flush=True)
+        with torch.no_grad():
+            x.copy_(torch.randn(T, H, generator=gen).bfloat16())   # other activations, hence another routing
+        graph.replay()
+        torch.cuda.synchronize()
+        got_out, got_grads = out.clone(), [t.clone() for t in grads]
+        want_out, want_grads = step()
+        torch.cuda.synchronize()
+        assert torch.equal(got_out, want_out), replay
+        for a, b in zip(got_grads, want_grads):
+            assert torch.equal(a, b), replay
