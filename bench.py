@@ -345,18 +345,38 @@ def zipf_ties_transform(T, E, seed, s=1.2, tie_fraction=0.01):
     return transform
 
 
+class Replayed:
+    """A layer's step captured into a graph once (forward and backward on the layer's own buffers); `step` replays it."""
+
+    def __init__(self, layer):
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                layer.step()
+        torch.cuda.current_stream().wait_stream(side)
+        self.layer, self.graph = layer, torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            layer.step()
+
+    def step(self):
+        self.graph.replay()
+
+
 def run_config(ops, seed, T, steps, warmup, **layer_kwargs):
     """tokens/s and peak allocation of one more workload of the same layer shape."""
     w = WORKLOAD
+    replayed = layer_kwargs.pop("replayed", False)
     transform = layer_kwargs.pop("transform_factory", None)
     if transform is not None:
         layer_kwargs["logit_transform"] = transform(T, w["E"], seed)
     layer = Layer(ops, *make_inputs(seed, T, w["H"], w["E"], w["I"]), w["K"], **layer_kwargs)
     torch.cuda.synchronize()
     resident = torch.cuda.memory_allocated()
-    settle(layer, seconds=0.2, at_least=10)
+    runner = Replayed(layer) if replayed else layer   # (captured before the clocks are settled: a capture leaves the GPU idle)
+    settle(runner, seconds=0.2, at_least=10)
     torch.cuda.reset_peak_memory_stats()
-    sec = time_layer(layer, steps, warmup)
+    sec = time_layer(runner, steps, warmup)
     check_forward_status()
     rec = {"tokens": T, "seed": seed, "ms_per_step": round(sec * 1e3, 4), "tokens_per_s": round(T / sec, 1),
            "layer_gemm_tflops": round(18.0 * T * w["K"] * w["H"] * w["I"] / sec / 1e12, 2),
@@ -374,13 +394,16 @@ def run_config(ops, seed, T, steps, warmup, **layer_kwargs):
 
 def other_configs(ops, steps, warmup):
     """The benchmark workloads besides the headline one, each a short run of its own: the headline layer through
-    the unchanged operator protocol, the 98304-token batch with its peak allocation, imbalanced routing with
+    the unchanged operator protocol, the headline step replayed from a graph, the 98304-token batch with its peak allocation, imbalanced routing with
     exact ties, and the 12-layer decoder's training step with the MoE share of it."""
     w = WORKLOAD
     out = {}
     out["layer_24x1024_protocol_only"] = dict(
         run_config(ops, w["seed"], w["T"], steps, warmup, protocol_only=True),
         path="F.linear + OpsBackend.router_postprocess + torch.bincount + OpsBackend.fused_moe, autograd sums dx; no extension hooks")
+    out["layer_24x1024_graph_replay"] = dict(
+        run_config(ops, w["seed"], w["T"], steps, warmup, replayed=True),
+        path="the headline step (one autograd node, forward and backward) captured into a graph once and replayed")
     out["layer_96x1024"] = dict(run_config(ops, 2, 98304, max(3, steps // 2), max(1, warmup // 2)), path="one autograd node (as the headline)")
     out["layer_24x1024_zipf_ties"] = dict(
         run_config(ops, 3, w["T"], steps, warmup, transform_factory=zipf_ties_transform),

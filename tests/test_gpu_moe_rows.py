@@ -125,11 +125,14 @@ def test_bench_line_carries_the_contract():
     assert 0.3 < rec["mfma_sustained"]["frac_of_peak"] < 1.0
     # the other workloads of the benchmark contract
     cfg = rec["configs"]
-    assert set(cfg) == {"layer_24x1024_protocol_only", "layer_96x1024", "layer_24x1024_zipf_ties", "decoder_12layer_24x1024"}
+    assert set(cfg) == {"layer_24x1024_protocol_only", "layer_24x1024_graph_replay", "layer_96x1024", "layer_24x1024_zipf_ties",
+                        "decoder_12layer_24x1024"}
     for name, row in cfg.items():
         assert row["tokens_per_s"] > 0 and row["ms_per_step"] > 0 and row["peak_hbm_allocated_mb"] > 0, name
     proto = cfg["layer_24x1024_protocol_only"]
     assert proto["tokens"] == 24576 and proto["ms_per_step"] >= 0.97 * rec["ms_per_step"]   # the hooks only take work away
+    replay = cfg["layer_24x1024_graph_replay"]
+    assert replay["tokens"] == 24576 and 0.9 * rec["ms_per_step"] < replay["ms_per_step"] < 1.05 * rec["ms_per_step"]   # the same kernels
     assert cfg["layer_96x1024"]["tokens"] == 98304 and cfg["layer_96x1024"]["peak_hbm_allocated_mb"] > cfg["layer_96x1024"]["resident_inputs_mb"]
     skew = cfg["layer_24x1024_zipf_ties"]
     assert 0.33 < skew["top_expert_share"] < 0.5 and skew["tied_tokens"] == 246
