@@ -49,9 +49,9 @@ RIDGE_FLOP_PER_BYTE = PEAK_BF16_TFLOPS * 1e12 / (PEAK_HBM_GBS * 1e9)   # 312.5: 
 # line names the file that holds the runs' commands and tables.
 TRAFFIC_SOURCE = "profiles/moe_layer_24x1024_hbm_traffic.txt"
 MEASURED_TRAFFIC_BYTES = {
-    "fwd_gateup_down": 774.6e6,   # gate/up and down as one launch; as two launches: 546.9 and 224.1
-    "fwd_gateup_swiglu": 546.9e6, "fwd_down": 224.1e6, "bwd_dy1": 539.6e6,
-    "bwd_joint": 1245.3e6,   # the joint launch (1080.2) and the launch of partial sums with the dX combine behind it (165.1)
+    "fwd_gateup_down": 772.7e6,   # gate/up and down as one launch; as two launches: 546.9 and 224.1
+    "fwd_gateup_swiglu": 546.9e6, "fwd_down": 224.1e6, "bwd_dy1": 538.8e6,
+    "bwd_joint": 1248.1e6,   # the joint launch (1083.0) and the launch of partial sums with the dX combine behind it (165.1)
     "combine": 114.7e6,
 }
 
